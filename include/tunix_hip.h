@@ -1,0 +1,320 @@
+/*
+ * tunix_hip.h -- C ABI of libtunix_hip.so: hand-written gfx950 (MI355X) kernels for the
+ * quantized rollout-decode path of google/tunix (Sampler decode step on int4/NF4 QLoRA
+ * models + per-token logps).
+ *
+ * Conventions (all entry points):
+ *   - extern "C"; `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *   - every pointer is a DEVICE pointer unless its name starts with `h_`;
+ *   - no allocation, no synchronisation, no host callback inside; outputs are caller-allocated;
+ *   - in-place updates (KV cache, token buffer) use the same pointer for input and output;
+ *   - return 0 on success, a negative TNX_E* code otherwise; tnx_last_error() returns the
+ *     calling thread's last message;
+ *   - bf16 values are raw uint16_t bit patterns; all matrices are row-major;
+ *   - scalars that change from one decode step to the next (step index, positions) are read
+ *     from device memory so that a captured HIP graph of one step can be replayed unchanged.
+ *
+ * Each declaration cites the reference code (paths relative to the google/tunix tree) whose
+ * arithmetic the entry point replaces.
+ */
+#ifndef TUNIX_HIP_H_
+#define TUNIX_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TNX_OK 0
+#define TNX_EINVAL (-22)  /* bad shape / alignment / enum                         */
+#define TNX_ELAUNCH (-5)  /* hipGetLastError() != hipSuccess after a kernel launch */
+#define TNX_ENOSYS (-38)  /* combination not built                                 */
+
+/* Weight code books. INT4: code u in [0,15] means the integer u-8. NF4: the 16 QLoRA levels. */
+#define TNX_Q_INT4 0
+#define TNX_Q_NF4 1
+
+/* RMSNorm dtype flows (tunix/models/llama3/model.py:290-297, qwen3/model.py:450-456,
+ * gemma3/model.py:940-950). */
+#define TNX_NORM_LLAMA 0
+#define TNX_NORM_QWEN3 1
+#define TNX_NORM_GEMMA3 2
+
+/* RoPE dtype flows (llama3/model.py:249-270 fp32 sin/cos; qwen3/model.py:404-425 sin/cos
+ * rounded to bf16 first; gemma3/model.py:402-430 fp32 with base frequency + scale factor). */
+#define TNX_ROPE_LLAMA 0
+#define TNX_ROPE_QWEN3 1
+#define TNX_ROPE_GEMMA3 2
+
+/* Epilogues of tnx_qlinear_lora. */
+#define TNX_EPI_STORE 0     /* y = bf16(acc)                                               */
+#define TNX_EPI_RESIDUAL 1  /* y = bf16(bf16(acc) + residual)      (llama3/model.py:560-563) */
+#define TNX_EPI_SILU_MUL 2  /* y = bf16(bf16(silu(bf16 g)) * bf16 u) (llama3/model.py:493)    */
+#define TNX_EPI_GELU_MUL 3  /* y = bf16(bf16(gelu_tanh(bf16 g)) * bf16 u) (gemma3/model.py:785-797) */
+#define TNX_EPI_F32 4       /* y(fp32) = acc, no rounding                                   */
+
+const char* tnx_last_error(void);
+/* Library/ABI version: (major << 16) | minor. */
+int tnx_version(void);
+
+/* ---------------------------------------------------------------------------------------
+ * Packed weight format ("QW"), defined by this library (qwix's QArray layout is third-party
+ * and not part of the reference tree; tunix only passes weight_qtype / tile_size through at
+ * tunix/cli/utils/model.py:31-77).
+ *
+ * A linear y[M,N] = x[M,K] . W[K,N] is quantized in groups of `group` consecutive K indices
+ * per output column: scale[g,n] = bf16(absmax / 7) (INT4) or bf16(absmax) (NF4); the code of
+ * an element is the nearest code-book entry of w / f32(scale) (round-half-even for INT4,
+ * clamped to [-8,7]; nearest level, ties to the lower code, for NF4).  The value a kernel
+ * uses is   level(code) * f32(scale)   with products accumulated in fp32 per group:
+ *     y[m,n] = sum_g f32(scale[g,n]) * ( sum_{k in g} x[m,k] * bf16(level(code[k,n])) ).
+ *
+ * Storage: N is padded to a multiple of 16 and K to a multiple of 128. Codes are tiled as
+ * [N/16][K/128][64 lanes][4 dwords]; lane l of a tile owns column n = 16*nt + l%16; its dword
+ * j holds the 8 codes of k = 128*kt + 32*j + 8*(l/16) + i, i = 0..7, code i in bits 4i..4i+3.
+ * Scales are tiled as [N/16][K/128][S][16] bf16 with S = max(1, 128/group) scales per tile
+ * and column (group > 128: the tile's scale is repeated).
+ * tnx_qw_sizes() gives the byte sizes; tnx_quantize_pack() produces both arrays on device.
+ * ------------------------------------------------------------------------------------- */
+int tnx_qw_sizes(int64_t K, int64_t N, int group, size_t* codes_bytes, size_t* scales_bytes);
+
+/* w: bf16 or fp32 [K,N] row-major (w_is_f32 selects).  If `interleave2` != 0 the N columns
+ * are the concatenation [gate | up] of two N/2-wide matrices and are stored interleaved in
+ * blocks of 16 (gate block, up block, ...) so that TNX_EPI_*_MUL sees matching columns in
+ * adjacent tiles.  Replaces qwix's quantizer reached from tunix/cli/utils/model.py:51-68. */
+int tnx_quantize_pack(void* stream, const void* w, int w_is_f32, int64_t K, int64_t N,
+                      int group, int qtype, int interleave2, uint32_t* codes, uint16_t* scales);
+
+/* Inverse of the packing for tests and export: w_out fp32 [K,N] = level * scale. */
+int tnx_qw_dequant(void* stream, const uint32_t* codes, const uint16_t* scales, int64_t K,
+                   int64_t N, int group, int qtype, int interleave2, float* w_out);
+
+/* ---------------------------------------------------------------------------------------
+ * Quantized linear fused with the LoRA delta:  y = epi( x . dequant(W) + lora_scale * t . B )
+ * replaces Einsum.__call__ / nnx.Linear as rewritten by qwix (llama3/model.py:216-218,
+ * :461-496; qwen3/model.py:361-365; gemma3/model.py:398-399) and the merge formula
+ * W + (A @ B) * alpha / rank pinned at tunix/models/safetensors_saver.py:107.
+ * ------------------------------------------------------------------------------------- */
+typedef struct tnx_qlinear_desc {
+  int64_t M, K, N;          /* N counts packed columns (after interleave2 it is 2*F)        */
+  int group, qtype;
+  const uint16_t* x;        /* bf16 [M,K]                                                   */
+  const uint32_t* codes;    /* QW codes                                                     */
+  const uint16_t* scales;   /* QW scales                                                    */
+  /* LoRA (optional: lora_rank == 0 disables). t = bf16(x . A) comes from tnx_lora_down.    */
+  int lora_rank;            /* r, multiple of 32                                            */
+  int lora_nseg;            /* 1..4 column segments, each with its own t columns; -1: the
+                               columns are an interleaved gate/up pair (even tiles use t
+                               columns [0,r), odd tiles [r,2r))                             */
+  int64_t lora_seg_end[4];  /* exclusive end column (packed order) of each segment, %16==0  */
+  int lora_seg_toff[4];     /* first t column of each segment                               */
+  int64_t t_ld;             /* row stride of t in elements                                  */
+  const uint16_t* t;        /* bf16 [M, t_ld]                                               */
+  const uint16_t* lora_b;   /* bf16 [N, r] (B transposed: r contiguous)                     */
+  float lora_scale;         /* alpha / rank                                                 */
+  int epilogue;             /* TNX_EPI_*                                                    */
+  const uint16_t* residual; /* bf16 [M, N] for TNX_EPI_RESIDUAL                             */
+  void* y;                  /* bf16 [M,N]; *_MUL: bf16 [M,N/2]; TNX_EPI_F32: fp32 [M,N]     */
+  int split_k;              /* >1: partial sums are atomically added into `ws`              */
+  float* ws;                /* fp32 [M,N] workspace, all zero on entry; required when
+                               split_k > 1; tnx_splitk_finish applies the epilogue and
+                               leaves it zero again                                         */
+} tnx_qlinear_desc;
+
+int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* h_desc);
+/* Epilogue for split_k > 1 (same desc): y = epi(ws); ws := 0. */
+int tnx_splitk_finish(void* stream, const tnx_qlinear_desc* h_desc);
+
+/* t[M, R] = bf16( x[M,K] . A ), a_t = A transposed: bf16 [R, K].  R multiple of 16.
+ * The LoRA "down" half of qwix's x @ lora_a @ lora_b (shapes at
+ * tunix/models/llama3/mapping_sglang_jax.py:64-145). */
+int tnx_lora_down(void* stream, const uint16_t* x, int64_t M, int64_t K, const uint16_t* a_t,
+                  int R, uint16_t* t, int64_t t_ld);
+
+/* ---------------------------------------------------------------------------------------
+ * Embedding gather: out[m,:] = table[ids[m],:] * scale_bf16  (scale 1.0 = plain copy).
+ * Embedder.encode llama3/model.py:238-242, qwen3/model.py:390-395, gemma3/model.py:353-358
+ * (gemma3 multiplies by bf16(sqrt(D))).  ids are read as ids[row_stride*b + col(+t)].
+ * ------------------------------------------------------------------------------------- */
+int tnx_embed(void* stream, const uint16_t* table, int64_t V, int64_t D, const int32_t* ids,
+              int64_t ids_ld, const int32_t* col_ptr, int64_t B, int64_t T, float scale,
+              uint16_t* out);
+
+/* RMSNorm over the last axis, three dtype flows.
+ *   h = (res_pre ? bf16(x + res_pre) : x);  if (h_out) h_out = h;
+ *   y = norm(h) ;  if (res_post) y = bf16(y + res_post)
+ * llama3/model.py:290-297, qwen3/model.py:450-456, gemma3/model.py:940-950; residual adds
+ * llama3/model.py:560-563, gemma3/model.py:875-898. */
+int tnx_rmsnorm(void* stream, const uint16_t* x, const uint16_t* res_pre, uint16_t* h_out,
+                const uint16_t* w, const uint16_t* res_post, uint16_t* y, int64_t M, int64_t D,
+                float eps, int flavor);
+
+/* ---------------------------------------------------------------------------------------
+ * Per-head q/k RMSNorm (optional) + RoPE + KV-cache write for T tokens per row.
+ *   qkv: bf16 [B*T, (Hq+2*Hkv)*dh] (q heads, then k heads, then v heads)
+ *   positions[b*pos_ld + col + t], col = *col_ptr (device) : RoPE position of token t of row b
+ *   cache slot of token t = (*col_ptr + t) % S
+ *   q_out: bf16 [B*T, Hq*dh];  kcache/vcache: bf16 [B, Hkv, S, dh]
+ * apply_rope llama3/model.py:249-270 (call sites :356-365 never pass rope_theta, so theta is
+ * 1e6), qwen3/model.py:404-425 (+ q_norm/k_norm :531-532), gemma3/model.py:402-430 (+ q/k
+ * norm :586-587, query pre-scale :596); cache write llama3/model.py:367-377.
+ * ------------------------------------------------------------------------------------- */
+typedef struct tnx_rope_desc {
+  int64_t B, T, S;
+  int Hq, Hkv, dh;
+  int rope_flavor;           /* TNX_ROPE_*                                                  */
+  float rope_scale;          /* gemma3: angles are divided by this scale factor (>= 1)      */
+  const float* timescale;    /* fp32 [dh/2] device: theta^(2i/dh), computed once by the host */
+  int qk_norm;               /* -1 none, else TNX_NORM_* flavour applied per head to q and k */
+  float norm_eps;
+  const uint16_t* q_norm_w;  /* bf16 [dh] or NULL                                           */
+  const uint16_t* k_norm_w;
+  float q_prescale;          /* 0 = none; gemma3 multiplies q by bf16(this) after RoPE      */
+  const uint16_t* qkv;
+  const int32_t* positions;
+  int64_t pos_ld;
+  const int32_t* col_ptr;    /* device int32: first token-buffer column of this call        */
+  uint16_t* q_out;
+  uint16_t* kcache;
+  uint16_t* vcache;
+} tnx_rope_desc;
+int tnx_qknorm_rope_kvwrite(void* stream, const tnx_rope_desc* h_desc);
+
+/* ---------------------------------------------------------------------------------------
+ * GQA attention over the KV cache for T query tokens per row (T = 1: decode).
+ * Query token t of row b sits in cache slot c = *col_ptr + t and attends slot j iff
+ *   j <= c  and  tokens[b*tok_ld + j] != pad_id  and (window == 0 or j > c - window),
+ * i.e. the mask of compute_attention_masks (tunix/generate/utils.py:34-58) /
+ * make_causal_attn_mask (:61-83) and create_sliding_window_mask (gemma3/model.py:477-496),
+ * evaluated from the token buffer instead of a dense [B,T,S] mask.
+ * scores: s = bf16(q.k) ; s = bf16(s * bf16(scale)) (scale 0: skip, gemma3 pre-scales q);
+ * softmax in fp32, probabilities rounded to bf16 before the PV product, fp32 accumulation,
+ * output rounded to bf16 (llama3/model.py:379-396, qwen3/model.py:674-686,
+ * gemma3/model.py:618-660).
+ *   q: bf16 [B*T, Hq*dh]; out: bf16 [B*T, Hq*dh]; caches bf16 [B,Hkv,S,dh]
+ *   ws: fp32 workspace of tnx_attn_ws_bytes() bytes (only touched when the key range is split)
+ * ------------------------------------------------------------------------------------- */
+typedef struct tnx_attn_desc {
+  int64_t B, T, S;
+  int Hq, Hkv, dh;
+  float scale;
+  int window;
+  int32_t pad_id;
+  const uint16_t* q;
+  const uint16_t* kcache;
+  const uint16_t* vcache;
+  const int32_t* tokens;
+  int64_t tok_ld;
+  const int32_t* col_ptr;
+  int kv_chunk;              /* keys per work-group when splitting (multiple of 32); 0: no split */
+  float* ws;
+  uint16_t* out;
+} tnx_attn_desc;
+size_t tnx_attn_ws_bytes(int64_t B, int64_t T, int64_t S, int Hq, int dh, int kv_chunk);
+int tnx_gqa_attn(void* stream, const tnx_attn_desc* h_desc);
+
+/* ---------------------------------------------------------------------------------------
+ * Fused lm_head -> fp32 log-softmax statistics, never writing [M,V] logits:
+ *   logit[m,v] = f32(bf16( x[m,:] . W[v,:] (+ lora) )) / temperature
+ * per row m: best id (first maximal index), best logit, logsumexp, and optionally the logit
+ * of a given target id.  compute_final_logits llama3/model.py:688-697; sample_best
+ * tunix/generate/sampler.py:151-161; selective_log_softmax tunix/rl/common.py:187-203;
+ * compute_chunked_logps :485-571.
+ *   head weights: dense bf16 [V,D] (w_bf16 != NULL; also the tied embedding table), or QW
+ *   part: fp32 workspace [M, n_vblocks, 4]; n_vblocks from tnx_lmhead_nblocks(V)
+ * ------------------------------------------------------------------------------------- */
+typedef struct tnx_lmhead_desc {
+  int64_t M, D, V;
+  const uint16_t* x;          /* bf16 [M,D]                                                  */
+  const uint16_t* w_bf16;     /* bf16 [V,D] or NULL                                          */
+  const uint32_t* codes;      /* QW (K = D, N = V) when w_bf16 == NULL                       */
+  const uint16_t* scales;
+  int group, qtype;
+  int lora_rank;
+  const uint16_t* t;          /* bf16 [M, t_ld]                                              */
+  int64_t t_ld;
+  const uint16_t* lora_b;     /* bf16 [V, r]                                                 */
+  float lora_scale;
+  float temperature;          /* fp32 logits are divided by this (0 or 1.0 = no scaling)     */
+  const int32_t* forbidden;   /* device list of ids forced to -inf, or NULL                  */
+  int n_forbidden;
+  const int32_t* targets;     /* int32 [M] or NULL                                           */
+  float* part;
+  int32_t* best_id;           /* int32 [M] or NULL                                           */
+  float* best_logp;           /* fp32 [M]: log-softmax at best_id, or NULL                   */
+  float* target_logp;         /* fp32 [M]: log-softmax at targets[m], or NULL                */
+  float* lse;                 /* fp32 [M] or NULL                                            */
+  float* logits_out;          /* fp32 [M,V] or NULL: materialise logits (return_logits /
+                                 top-k sampling path)                                       */
+} tnx_lmhead_desc;
+int64_t tnx_lmhead_nblocks(int64_t V);
+int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* h_desc);
+
+/* Top-k / top-p sampling from materialised fp32 logits (already divided by temperature):
+ * sample_top_p tunix/generate/sampler.py:105-148.  The k largest logits per row (descending,
+ * lower index first among equals) are softmaxed, entries whose exclusive cumulative
+ * probability exceeds top_p are dropped, and one is drawn by Gumbel-max (jax.random.categorical)
+ * with noise from threefry2x32 keyed by fold_in((key0,key1), *step_ptr) (sampler.py:516).
+ * rng_variant selects jax's random_bits layout: 1 = partitionable (counter (0,n), x0^x1),
+ * 0 = original (counter array split in halves).  k <= 0 or k >= V with top_p >= 1 draws from
+ * the whole vocabulary.  logp_out = full-vocabulary log-softmax at the drawn id (:141-144).
+ * k <= 1024.  `ws` is unused (reserved). */
+int tnx_sample_topk(void* stream, const float* logits, int64_t M, int64_t V, int k, float top_p,
+                    uint32_t key0, uint32_t key1, int rng_variant, const int32_t* step_ptr,
+                    float* ws, int32_t* ids_out, float* logp_out);
+
+/* Sampler bookkeeping of one step (tunix/generate/sampler.py:529-535, :692-703):
+ *   col = *step_ptr; tokens[b, col+1] = ids[b]; logprobs[b, col+1] = logp[b] (if given);
+ *   done[b] |= ids[b] in eos[];  then *step_ptr = col + 1 (by the last thread). */
+int tnx_sample_commit(void* stream, const int32_t* ids, const float* logp, int64_t B,
+                      int32_t* tokens, int64_t tok_ld, float* logprobs, int32_t* done,
+                      const int32_t* eos, int n_eos, int32_t* step_ptr);
+
+/* ---------------------------------------------------------------------------------------
+ * MoE (qwen3/model.py:787-832): router softmax -> top-k -> renormalise (weights bf16), and an
+ * int4/NF4 grouped GEMM over routed tokens (operator shape of megablox.gmm, :975-995).
+ * ------------------------------------------------------------------------------------- */
+/* scores: bf16 [M,E] router outputs.  topk_w: bf16 [M,k]; topk_id: int32 [M,k] (descending
+ * probability, lower expert id first among equals). */
+int tnx_moe_route_topk(void* stream, const uint16_t* scores, int64_t M, int E, int k,
+                       uint16_t* topk_w, int32_t* topk_id);
+/* Builds the expert-sorted route list: counts[E], offsets[E+1], sorted_route[M*k] (route =
+ * m*k + j).  Single work-group; M*k <= 1<<20. */
+int tnx_moe_sort_routes(void* stream, const int32_t* topk_id, int64_t M, int k, int E,
+                        int32_t* counts, int32_t* offsets, int32_t* sorted_route);
+typedef struct tnx_moe_gmm_desc {
+  int64_t n_routes;          /* M*k                                                          */
+  int E, k;
+  int64_t K, N;              /* per-expert linear: x[.,K] . W_e[K,N]                          */
+  int group, qtype;
+  const uint16_t* x;         /* bf16 rows; row of route r is r / x_div (x_div = k for the
+                                token activations, 1 for per-route activations)             */
+  int x_div;
+  const uint32_t* codes;     /* QW per expert, expert stride = tnx_qw_sizes().codes_bytes    */
+  const uint16_t* scales;
+  const int32_t* offsets;    /* int32 [E+1]                                                  */
+  const int32_t* sorted_route;
+  int epilogue;              /* TNX_EPI_STORE or TNX_EPI_SILU_MUL (interleave2 packing)      */
+  uint16_t* y;               /* bf16 [n_routes, N or N/2], indexed by route                  */
+} tnx_moe_gmm_desc;
+int tnx_moe_int4_gmm(void* stream, const tnx_moe_gmm_desc* h_desc);
+/* out[m,:] = bf16( sum_j f32(topk_w[m,j]) * f32(y[m*k+j,:]) )  (qwen3/model.py:827-832). */
+int tnx_moe_combine(void* stream, const uint16_t* y, const uint16_t* topk_w, int64_t M, int k,
+                    int64_t D, const uint16_t* residual, uint16_t* out);
+
+/* GRPO clipped ratio (tunix/rl/algo_core.py:440-489): lr = clip(logp - old, -20, 20);
+ * ratio = exp(lr); loss = max(-A*ratio, -A*clip(ratio, 1-eps_lo, 1+eps_hi)).
+ * adv has one value per sequence: adv[n / tokens_per_seq].  Outputs may be NULL. */
+int tnx_grpo_ratio(void* stream, const float* logp, const float* old_logp, const float* adv,
+                   int64_t N, int64_t tokens_per_seq, float eps_lo, float eps_hi, float* ratio,
+                   float* loss, int32_t* clipped);
+
+/* Fill n 32-bit words with `value` (graph-capturable replacement for hipMemsetAsync). */
+int tnx_fill_u32(void* stream, uint32_t* p, int64_t n, uint32_t value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TUNIX_HIP_H_ */

@@ -1,0 +1,268 @@
+"""Decoder forward passes of the three model families on the path (oracle; tests only).
+
+Restates tunix/models/llama3/model.py:199-697, tunix/models/qwen3/model.py:338-832,:1045-1335
+and tunix/models/gemma3/model.py:318-950,:997-1063 with torch on the CPU.  Tensors are fp32
+storage; in `bf16` mode every value that the reference holds in bf16 is rounded with rb() at
+the point where the reference's dtype flow rounds it, matmuls accumulate in `acc` (fp64 by
+default: the order-free ideal of an fp32 accumulation).  `bf16=False` is the fp32 reference
+mode: same formulas, no rounding.
+
+Weights come as a flat dict of 2-D tensors (see tunix_amd.weights for the naming); quantised
+linears are (codes, scales) pairs produced by oracle.quant_ref.quantize.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+
+from . import quant_ref as Q
+
+K_MASK = -2.3819763e38  # tunix/models/llama3/model.py:37, qwen3/model.py, gemma3/model.py:434
+
+
+class RefModel:
+  """Oracle model: holds prepared weights and runs prefill / decode with a dense KV cache."""
+
+  def __init__(self, cfg, weights: dict, bf16: bool = True, acc=torch.float64):
+    self.cfg = cfg
+    self.bf16 = bf16
+    self.acc = acc
+    self.w = {}
+    self.q = {}     # name -> (dequantised fp32 [K,N])
+    self.lora = {}  # name -> (A [K,r], B [r,N])
+    for name, v in weights.items():
+      self.w[name] = v if isinstance(v, torch.Tensor) else torch.as_tensor(v)
+    self._prepare()
+
+  # ---- helpers -----------------------------------------------------------------------------
+  def r(self, x):
+    return Q.rb(x) if self.bf16 else x
+
+  def _prepare(self):
+    cfg = self.cfg
+    for name in list(self.w):
+      if name.endswith(".lora_a"):
+        base = name[:-7]
+        self.lora[base] = (self.w[name].float(), self.w[base + ".lora_b"].float())
+    for name in cfg.quantized_names():
+      wt = self.w[name].float().numpy()
+      if wt.ndim == 3:  # experts [E,K,N]
+        deq = []
+        for e in range(wt.shape[0]):
+          c, s = Q.quantize(wt[e], cfg.group, cfg.qtype)
+          deq.append(Q.dequantize(c, s, cfg.group, cfg.qtype, round_levels=self.bf16))
+        self.q[name] = torch.from_numpy(np.stack(deq))
+      else:
+        c, s = Q.quantize(wt, cfg.group, cfg.qtype)
+        self.q[name] = torch.from_numpy(Q.dequantize(c, s, cfg.group, cfg.qtype,
+                                                     round_levels=self.bf16))
+
+  def linear(self, x, name):
+    """x [.., K] -> fp32 [.., N] (unrounded): quantised (or dense) matmul + LoRA delta."""
+    wd = self.q[name] if name in self.q else self.w[name].float()
+    y = x.to(self.acc) @ wd.to(self.acc)
+    if name in self.lora:
+      a, b = self.lora[name]
+      t = (x.to(self.acc) @ a.to(self.acc)).float()
+      t = self.r(t)
+      y = y + float(self.cfg.lora_alpha) / float(self.cfg.lora_rank) * (t.to(self.acc) @ b.to(self.acc))
+    return y.float()
+
+  # ---- RMSNorm flavours ----------------------------------------------------------------------
+  def rmsnorm(self, x, w, flavor=None, eps=None):
+    cfg = self.cfg
+    flavor = flavor or cfg.family
+    eps = cfg.norm_eps if eps is None else eps
+    if flavor == "llama3":
+      # tunix/models/llama3/model.py:290-297: astype(w * x / rms): bf16 product, fp32 division
+      rms = torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+      return self.r(self.r(w * x) / rms)
+    if flavor == "qwen3":
+      # tunix/models/qwen3/model.py:450-456: everything in fp32
+      rms = torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+      return self.r(w * (x / rms))
+    # tunix/models/gemma3/model.py:940-950: every op in the activation dtype
+    var = self.r(self.r(x * x).mean(-1, keepdim=True))
+    normed = self.r(x * self.r(torch.rsqrt(self.r(var + 1e-6))))
+    return self.r(normed * self.r(1.0 + w))
+
+  # ---- RoPE flavours -------------------------------------------------------------------------
+  @staticmethod
+  def timescale(head_dim: int, theta: float) -> np.ndarray:
+    fraction = (np.float32(2.0) * np.arange(0, head_dim // 2, dtype=np.float32)
+                / np.float32(head_dim)).astype(np.float32)
+    return np.power(np.float32(theta), fraction).astype(np.float32)
+
+  def rope(self, x, positions, theta, flavor=None, scale_factor=1.0):
+    """x [B,T,H,dh]; positions [B,T] int.  llama3/model.py:249-270, qwen3/model.py:404-425,
+    gemma3/model.py:402-430."""
+    flavor = flavor or self.cfg.family
+    dh = x.shape[-1]
+    ts = torch.from_numpy(self.timescale(dh, theta))
+    ang = positions.to(torch.float32)[..., None] / ts[None, None, :]
+    if flavor == "gemma3":
+      ang = ang / np.float32(scale_factor)
+    ang = ang[..., None, :]
+    sin, cos = torch.sin(ang), torch.cos(ang)
+    x1, x2 = x[..., : dh // 2], x[..., dh // 2:]
+    if flavor == "qwen3":
+      sin, cos = self.r(sin), self.r(cos)
+      o1 = self.r(self.r(x1 * cos) - self.r(x2 * sin))
+      o2 = self.r(self.r(x2 * cos) + self.r(x1 * sin))
+    else:
+      o1 = self.r(x1 * cos - x2 * sin)
+      o2 = self.r(x2 * cos + x1 * sin)
+    return torch.cat([o1, o2], dim=-1)
+
+  # ---- attention -----------------------------------------------------------------------------
+  def attention(self, q, k_all, v_all, mask, scale, softmax_bf16_flow=False):
+    """q [B,T,Hq,dh], k_all/v_all [B,S,Hkv,dh], mask [B,T,S] bool.
+
+    llama3/model.py:379-396, qwen3/model.py:674-686, gemma3/model.py:618-660: scores are a
+    bf16 einsum, scaled in bf16 (scale=None: q was pre-scaled), masked with K_MASK, softmaxed
+    in fp32, cast to bf16, then a bf16 einsum with V.
+    """
+    B, T, Hq, dh = q.shape
+    Hkv = k_all.shape[2]
+    G = Hq // Hkv
+    qg = q.reshape(B, T, Hkv, G, dh)
+    s = torch.einsum("bthgd,bshd->bhgts", qg.to(self.acc), k_all.to(self.acc)).float()
+    s = self.r(s)
+    if scale is not None:
+      s = self.r(s * (self.r(torch.tensor(scale, dtype=torch.float32)) if self.bf16 else scale))
+    s = torch.where(mask[:, None, None, :, :], s, torch.tensor(K_MASK))
+    p = torch.softmax(s.to(torch.float32), dim=-1)
+    p = self.r(p)
+    o = torch.einsum("bhgts,bshd->bthgd", p.to(self.acc), v_all.to(self.acc)).float()
+    return self.r(o).reshape(B, T, Hq, dh)
+
+  # ---- one decoder layer ---------------------------------------------------------------------
+  def layer(self, i, x, positions, cache, mask, slot0):
+    cfg = self.cfg
+    p = f"l{i}."
+    B, T, D = x.shape
+    Hq, Hkv, dh = cfg.num_heads, cfg.num_kv_heads, cfg.head_dim
+    fam = cfg.family
+    xn = self.rmsnorm(x, self.w[p + "attn_norm"].float())
+    q = self.r(self.linear(xn, p + "wq")).reshape(B, T, Hq, dh)
+    k = self.r(self.linear(xn, p + "wk")).reshape(B, T, Hkv, dh)
+    v = self.r(self.linear(xn, p + "wv")).reshape(B, T, Hkv, dh)
+    if fam in ("qwen3", "gemma3"):
+      q = self.rmsnorm(q, self.w[p + "q_norm"].float(), eps=cfg.norm_eps if fam == "qwen3" else 1e-6)
+      k = self.rmsnorm(k, self.w[p + "k_norm"].float(), eps=cfg.norm_eps if fam == "qwen3" else 1e-6)
+    theta, sf = cfg.rope_params(i)
+    q = self.rope(q, positions, theta, scale_factor=sf)
+    k = self.rope(k, positions, theta, scale_factor=sf)
+    scale = dh ** -0.5
+    if fam == "gemma3":
+      qs = cfg.query_pre_attn_scalar
+      q = self.r(q * (self.r(torch.tensor(qs, dtype=torch.float32)) if self.bf16 else qs))
+      scale = None
+    # cache write at slot end_index % S (llama3/model.py:367-377); all rows share the slot
+    kc, vc = cache[i]
+    S = kc.shape[1]
+    for t in range(T):
+      kc[:, (slot0 + t) % S] = k[:, t]
+      vc[:, (slot0 + t) % S] = v[:, t]
+    m = mask
+    if fam == "gemma3" and cfg.is_local_layer(i):
+      m = self.sliding_mask(mask, cfg.sliding_window, T)
+    o = self.attention(q, kc, vc, m, scale)
+    attn_out = self.r(self.linear(o.reshape(B, T, Hq * dh), p + "wo"))
+    if fam == "gemma3":
+      # gemma3/model.py:875-898: post-norms before each residual add
+      attn_out = self.rmsnorm(attn_out, self.w[p + "post_attn_norm"].float())
+      h = self.r(attn_out + x)
+      y = self.rmsnorm(h, self.w[p + "mlp_norm"].float())
+      y = self.mlp(i, y)
+      y = self.rmsnorm(y, self.w[p + "post_ffw_norm"].float())
+      return self.r(y + h)
+    h = self.r(attn_out + x)  # llama3/model.py:560-563
+    y = self.rmsnorm(h, self.w[p + "mlp_norm"].float())
+    y = self.moe(i, y) if cfg.num_experts else self.mlp(i, y)
+    return self.r(h + y)
+
+  def sliding_mask(self, mask, window, T):
+    """gemma3/model.py:632-643."""
+    if T == 1:
+      from .utils_ref import create_sliding_window_mask
+      sm = torch.from_numpy(create_sliding_window_mask(mask.numpy(), window))
+      return sm & mask
+    ones = torch.ones_like(mask)
+    sm = torch.triu(ones, -window + 1) & torch.tril(ones, window - 1)
+    return sm & mask
+
+  def act(self, g):
+    if self.cfg.family == "gemma3":
+      # nnx.gelu (tanh approximation) on a bf16 tensor; one rounding at the end
+      return self.r(torch.nn.functional.gelu(g, approximate="tanh"))
+    # jax.nn.silu = x * sigmoid(x): two bf16 ops
+    return self.r(g * self.r(torch.sigmoid(g)))
+
+  def mlp(self, i, x):
+    p = f"l{i}."
+    g = self.r(self.linear(x, p + "w_gate"))
+    u = self.r(self.linear(x, p + "w_up"))
+    a = self.r(self.act(g) * u)
+    return self.r(self.linear(a, p + "w_down"))
+
+  def moe(self, i, x):
+    """qwen3/model.py:787-832 (dense-over-experts semantics, computed per routed token)."""
+    cfg = self.cfg
+    p = f"l{i}."
+    B, T, D = x.shape
+    scores = self.r(self.linear(x, p + "router"))            # bf16 Linear output, cast to fp32
+    probs = torch.softmax(scores.float(), dim=-1)
+    kk = cfg.num_experts_per_tok
+    # top_k: descending, lower index first among equals
+    order = torch.sort(probs, dim=-1, descending=True, stable=True).indices[..., :kk]
+    wts = torch.gather(probs, -1, order)
+    wts = self.r(wts / wts.sum(-1, keepdim=True))
+    out = torch.zeros(B, T, D, dtype=torch.float64)
+    xf = x.reshape(B * T, D)
+    of = out.reshape(B * T, D)
+    order_f, wts_f = order.reshape(B * T, kk), wts.reshape(B * T, kk)
+    wg, wu, wdn = self.q[p + "e_gate"], self.q[p + "e_up"], self.q[p + "e_down"]
+    for n in range(B * T):
+      for j in range(kk):
+        e = int(order_f[n, j])
+        g = self.r((xf[n].to(self.acc) @ wg[e].to(self.acc)).float())
+        u = self.r((xf[n].to(self.acc) @ wu[e].to(self.acc)).float())
+        a = self.r(self.act(g) * u)
+        y = self.r((a.to(self.acc) @ wdn[e].to(self.acc)).float())
+        of[n] += (wts_f[n, j] * y).double()
+    return self.r(out.float())
+
+  # ---- whole model ---------------------------------------------------------------------------
+  def init_cache(self, B, S):
+    cfg = self.cfg
+    return [(torch.zeros(B, S, cfg.num_kv_heads, cfg.head_dim),
+             torch.zeros(B, S, cfg.num_kv_heads, cfg.head_dim)) for _ in range(cfg.num_layers)]
+
+  def embed(self, tokens):
+    cfg = self.cfg
+    ids = tokens.long().clamp(0, cfg.vocab_size - 1)
+    x = self.w["embed"].float()[ids]
+    if cfg.family == "gemma3":
+      # gemma3/model.py:353-358: x *= sqrt(D).astype(x.dtype)
+      s = torch.tensor(math.sqrt(cfg.embed_dim), dtype=torch.float32)
+      x = self.r(x * self.r(s))
+    return x
+
+  def hidden(self, tokens, positions, cache, mask, slot0):
+    """tokens/positions [B,T]; mask [B,T,S] -> final-normed hidden [B,T,D]."""
+    x = self.embed(tokens)
+    for i in range(self.cfg.num_layers):
+      x = self.layer(i, x, positions, cache, mask, slot0)
+    return self.rmsnorm(x, self.w["final_norm"].float())
+
+  def logits(self, h):
+    """compute_final_logits (llama3/model.py:688-697): bf16 einsum, cast to fp32."""
+    if self.cfg.tied_embedding:
+      return self.r((h.to(self.acc) @ self.w["embed"].float().t().to(self.acc)).float())
+    return self.r(self.linear(h, "lm_head"))
+
+  def __call__(self, tokens, positions, cache, mask, slot0=0):
+    return self.logits(self.hidden(tokens, positions, cache, mask, slot0))

@@ -1,0 +1,292 @@
+// GQA attention over the KV cache with a wavefront-level online softmax.
+//
+// One wave owns a tile of 16 query vectors that share a (batch row, kv head): the G query
+// heads of the group (decode), or G heads x 16/G consecutive positions (prefill).  Scores are
+// computed transposed, S^T[key, query] = K . q^T, so that every lane ends up holding the
+// probabilities of ONE query column for 8 keys -- exactly the A fragment of the P.V MFMA --
+// and the max / sum of the online softmax are per-lane scalars reduced over 4 lanes.  V rows
+// are loaded in their natural [key][dh] layout (256 B contiguous per key) and transposed
+// inside each lane with v_perm_b32 to form B fragments; nothing goes through LDS.
+#include <string.h>
+
+#include "common.h"
+
+namespace {
+
+struct AttnArgs {
+  int64_t B, T, S;
+  int Hq, Hkv, dh, G, Gp;
+  float scale_bf;  // bf16-rounded scale, 0 = none
+  int window;
+  int32_t pad_id;
+  const uint16_t* q;
+  const uint16_t* k;
+  const uint16_t* v;
+  const int32_t* tokens;
+  int64_t tok_ld;
+  const int32_t* col_ptr;
+  int kv_chunk, n_chunks;
+  float* ws;
+  uint16_t* out;
+};
+
+constexpr float kNegBig = -1.0e30f;
+
+template <int DH>
+__global__ __launch_bounds__(64) void attn_kernel(const AttnArgs a) {
+  constexpr int KS = DH / 32;                 // k-steps of the QK product
+  constexpr int NH = DH > 128 ? DH / 128 : 1; // 128-column halves of V / O
+  const int lane = threadIdx.x, lm = lane & 15, lq = lane >> 4;
+  const int chunk = blockIdx.x, hkv = blockIdx.y;
+  const int PT = 16 / a.Gp;                              // positions per query tile
+  const int QT = (int)((a.T + PT - 1) / PT);
+  const int64_t b = blockIdx.z / QT;
+  const int qt = blockIdx.z % QT;
+  const int col0 = *a.col_ptr;
+
+  // query column of this lane (as B-fragment column and as softmax owner)
+  const int g = lm % a.Gp, tq = qt * PT + lm / a.Gp;
+  const bool qvalid = g < a.G && tq < a.T;
+  const int c_n = col0 + tq;                              // cache slot of the query token
+  const int lo_n = a.window > 0 ? max(0, c_n - a.window + 1) : 0;
+  const int64_t qvec = (b * a.T + (qvalid ? tq : 0)) * a.Hq + hkv * a.G + (qvalid ? g : 0);
+
+  // key range of the tile
+  const int t_last = min((int)a.T - 1, qt * PT + PT - 1);
+  int k_hi = col0 + t_last;                               // inclusive
+  int k_lo = a.window > 0 ? max(0, col0 + qt * PT - a.window + 1) : 0;
+  if (a.kv_chunk > 0) {
+    k_lo = max(k_lo, chunk * a.kv_chunk);
+    k_hi = min(k_hi, chunk * a.kv_chunk + a.kv_chunk - 1);
+  }
+
+  u32x4 qf[KS];
+#pragma unroll
+  for (int j = 0; j < KS; ++j) {
+    qf[j] = u32x4{0, 0, 0, 0};
+    if (qvalid) qf[j] = *reinterpret_cast<const u32x4*>(a.q + qvec * DH + j * 32 + lq * 8);
+  }
+
+  f32x4 O[NH][8];
+#pragma unroll
+  for (int h = 0; h < NH; ++h)
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) O[h][jj] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = kNegBig, l_run = 0.f;
+
+  const uint16_t* kbase = a.k + ((b * a.Hkv + hkv) * a.S) * DH;
+  const uint16_t* vbase = a.v + ((b * a.Hkv + hkv) * a.S) * DH;
+  const int32_t* tok = a.tokens + b * a.tok_ld;
+  const int vcol = (8 * lm) % (DH < 128 ? DH : 128);     // DH=64: upper lanes duplicate
+
+  for (int kb = k_lo & ~31; kb <= k_hi; kb += 32) {
+    // ---- loads: K as A fragments (two tiles of 16 keys), V rows of this lane's 8 keys ----
+    u32x4 kf[2][KS];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      const int key = min(kb + 16 * tt + lm, (int)a.S - 1);
+#pragma unroll
+      for (int j = 0; j < KS; ++j)
+        kf[tt][j] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)key * DH + j * 32 + lq * 8);
+    }
+    u32x4 vf[NH][8];
+    int keys[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      keys[s] = kb + (s < 4 ? 4 * lq + s : 16 + 4 * lq + (s - 4));
+      const int key = min(keys[s], (int)a.S - 1);
+#pragma unroll
+      for (int h = 0; h < NH; ++h)
+        vf[h][s] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)key * DH + h * 128 + vcol);
+    }
+    bool kvalid[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int key = keys[s];
+      bool ok = qvalid && key >= max(k_lo, lo_n) && key <= min(k_hi, c_n);
+      if (ok) ok = tok[key] != a.pad_id;
+      kvalid[s] = ok;
+    }
+    // ---- S^T = K . q^T ----
+    f32x4 st[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      st[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < KS; ++j) st[tt] = mfma16(kf[tt][j], qf[j], st[tt]);
+    }
+    float sv[8];
+    float bmax = kNegBig;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      float x = rbf(st[s >> 2][s & 3]);
+      if (a.scale_bf != 0.f) x = rbf(x * a.scale_bf);
+      sv[s] = x;
+      if (kvalid[s]) bmax = fmaxf(bmax, x);
+    }
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
+    bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+    const float m_new = fmaxf(m_run, bmax);
+    const float alpha = __expf(m_run - m_new);
+    m_run = m_new;
+    float p[8], psum = 0.f;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      p[s] = kvalid[s] ? __expf(sv[s] - m_new) : 0.f;
+      psum += p[s];
+    }
+    l_run = l_run * alpha + psum;
+    u32x4 pa;
+    pa[0] = pack2bf(p[0], p[1]);
+    pa[1] = pack2bf(p[2], p[3]);
+    pa[2] = pack2bf(p[4], p[5]);
+    pa[3] = pack2bf(p[6], p[7]);
+    // ---- O = O * alpha + P . V ----
+    float ar[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ar[i] = __shfl(alpha, 4 * lq + i, 64);
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) {
+        const uint32_t sel = (jj & 1) ? 0x07060302u : 0x05040100u;
+        u32x4 bfrag;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          bfrag[r] = __builtin_amdgcn_perm(vf[h][2 * r + 1][jj >> 1], vf[h][2 * r][jj >> 1], sel);
+        f32x4 o = O[h][jj];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] *= ar[i];
+        O[h][jj] = mfma16(pa, bfrag, o);
+      }
+  }
+
+  l_run += __shfl_xor(l_run, 16, 64);
+  l_run += __shfl_xor(l_run, 32, 64);
+
+  // O rows are query columns 4*lq + i; columns are d = h*128 + 8*lm + jj.
+  const bool dvalid = 8 * lm < (DH < 128 ? DH : 128);
+  if (a.kv_chunk <= 0 || a.n_chunks == 1) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = 4 * lq + i;
+      const float l = __shfl(l_run, n, 64);
+      const int gi = n % a.Gp, ti = qt * PT + n / a.Gp;
+      if (!(gi < a.G && ti < a.T) || !dvalid) continue;
+      const float inv = l > 0.f ? 1.0f / l : 0.f;
+      uint16_t* o = a.out + ((b * a.T + ti) * a.Hq + hkv * a.G + gi) * DH;
+#pragma unroll
+      for (int h = 0; h < NH; ++h) {
+        u32x4 w;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          w[r] = pack2bf(O[h][2 * r][i] * inv, O[h][2 * r + 1][i] * inv);
+        *reinterpret_cast<u32x4*>(o + h * 128 + 8 * lm) = w;
+      }
+    }
+    return;
+  }
+  // split: partial (m, l, O[dh]) per (query vector, chunk)
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = 4 * lq + i;
+    const float l = __shfl(l_run, n, 64);
+    const float m = __shfl(m_run, n, 64);
+    const int gi = n % a.Gp, ti = qt * PT + n / a.Gp;
+    if (!(gi < a.G && ti < a.T)) continue;
+    const int64_t qv = (b * a.T + ti) * a.Hq + hkv * a.G + gi;
+    float* p = a.ws + (qv * a.n_chunks + chunk) * (DH + 2);
+    if (lm == 0) {
+      p[0] = m;
+      p[1] = l;
+    }
+    if (!dvalid || l <= 0.f) continue;
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) p[2 + h * 128 + 8 * lm + jj] = O[h][jj][i];
+  }
+}
+
+// out[qv, d] = bf16( sum_c e^{m_c - M} O_c[d] / sum_c e^{m_c - M} l_c )
+__global__ void attn_combine_kernel(const float* ws, int64_t n_qvec, int dh, int n_chunks,
+                                    uint16_t* out) {
+  const int64_t qv = blockIdx.x;
+  const int d = threadIdx.x;
+  if (d >= dh) return;
+  const float* p = ws + qv * n_chunks * (dh + 2);
+  float M = kNegBig;
+  for (int c = 0; c < n_chunks; ++c)
+    if (p[c * (dh + 2) + 1] > 0.f) M = fmaxf(M, p[c * (dh + 2)]);
+  float L = 0.f, o = 0.f;
+  for (int c = 0; c < n_chunks; ++c) {
+    const float l = p[c * (dh + 2) + 1];
+    if (l <= 0.f) continue;
+    const float w = __expf(p[c * (dh + 2)] - M);
+    L += w * l;
+    o += w * p[c * (dh + 2) + 2 + d];
+  }
+  out[qv * dh + d] = f2bf(L > 0.f ? o / L : 0.f);
+}
+
+int next_pow2(int x) {
+  int p = 1;
+  while (p < x) p <<= 1;
+  return p;
+}
+
+}  // namespace
+
+extern "C" size_t tnx_attn_ws_bytes(int64_t B, int64_t T, int64_t S, int Hq, int dh,
+                                    int kv_chunk) {
+  if (kv_chunk <= 0) return 0;
+  const int64_t n_chunks = cdiv(S, kv_chunk);
+  return (size_t)(B * T * Hq * n_chunks * (dh + 2)) * sizeof(float);
+}
+
+extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
+  TNX_REQUIRE(d, "attn: null descriptor");
+  TNX_REQUIRE(d->B > 0 && d->T > 0 && d->S > 0, "attn: B,T,S must be positive");
+  TNX_REQUIRE(d->dh == 64 || d->dh == 128 || d->dh == 256, "attn: head_dim %d not in {64,128,256}", d->dh);
+  TNX_REQUIRE(d->Hkv > 0 && d->Hq % d->Hkv == 0, "attn: Hq=%d not a multiple of Hkv=%d", d->Hq, d->Hkv);
+  const int G = d->Hq / d->Hkv;
+  TNX_REQUIRE(G <= 16, "attn: group size %d > 16 not supported", G);
+  TNX_REQUIRE(d->q && d->kcache && d->vcache && d->tokens && d->col_ptr && d->out, "attn: null pointer");
+  TNX_REQUIRE(d->kv_chunk >= 0 && d->kv_chunk % 32 == 0, "attn: kv_chunk must be a multiple of 32");
+  TNX_REQUIRE(d->tok_ld >= d->S || d->tok_ld > 0, "attn: bad tok_ld");
+  AttnArgs a;
+  a.B = d->B; a.T = d->T; a.S = d->S; a.Hq = d->Hq; a.Hkv = d->Hkv; a.dh = d->dh;
+  a.G = G; a.Gp = next_pow2(G);
+  // bf16(scale), as a weak-typed python float multiplied into a bf16 array
+  if (d->scale != 0.f) {
+    uint32_t u; float f = d->scale; memcpy(&u, &f, 4);
+    u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+    memcpy(&a.scale_bf, &u, 4);
+  } else {
+    a.scale_bf = 0.f;
+  }
+  a.window = d->window; a.pad_id = d->pad_id;
+  a.q = d->q; a.k = d->kcache; a.v = d->vcache; a.tokens = d->tokens; a.tok_ld = d->tok_ld;
+  a.col_ptr = d->col_ptr; a.kv_chunk = d->kv_chunk;
+  a.n_chunks = d->kv_chunk > 0 ? (int)cdiv(d->S, d->kv_chunk) : 1;
+  a.ws = d->ws; a.out = d->out;
+  if (a.n_chunks > 1) TNX_REQUIRE(d->ws, "attn: split key range needs a workspace");
+  const int PT = 16 / a.Gp;
+  const int64_t QT = cdiv(d->T, PT);
+  TNX_REQUIRE(d->B * QT <= 65535 * 32, "attn: too many query tiles");
+  dim3 grid((unsigned)a.n_chunks, (unsigned)d->Hkv, (unsigned)(d->B * QT));
+  hipStream_t st = as_stream(stream);
+  switch (d->dh) {
+    case 64: hipLaunchKernelGGL(attn_kernel<64>, grid, dim3(64), 0, st, a); break;
+    case 128: hipLaunchKernelGGL(attn_kernel<128>, grid, dim3(64), 0, st, a); break;
+    default: hipLaunchKernelGGL(attn_kernel<256>, grid, dim3(64), 0, st, a); break;
+  }
+  TNX_CHECK_LAUNCH("gqa_attn");
+  if (a.n_chunks > 1) {
+    const int64_t nq = d->B * d->T * d->Hq;
+    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)nq), dim3(d->dh), 0, st, a.ws, nq, d->dh,
+                       a.n_chunks, a.out);
+    TNX_CHECK_LAUNCH("gqa_attn_combine");
+  }
+  return TNX_OK;
+}

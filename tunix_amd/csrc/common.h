@@ -1,0 +1,95 @@
+// Shared device helpers for the gfx950 kernels of libtunix_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "tunix_hip.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define TNX_WAVE 64
+
+// ---- error plumbing (host) -------------------------------------------------------------
+void tnx_set_error(const char* fmt, ...);
+#define TNX_REQUIRE(cond, ...)      \
+  do {                              \
+    if (!(cond)) {                  \
+      tnx_set_error(__VA_ARGS__);   \
+      return TNX_EINVAL;            \
+    }                               \
+  } while (0)
+#define TNX_CHECK_LAUNCH(name)                                                  \
+  do {                                                                          \
+    hipError_t e_ = hipGetLastError();                                          \
+    if (e_ != hipSuccess) {                                                     \
+      tnx_set_error("%s: launch failed: %s", name, hipGetErrorString(e_));      \
+      return TNX_ELAUNCH;                                                       \
+    }                                                                           \
+  } while (0)
+
+// ---- bf16 <-> f32 ----------------------------------------------------------------------
+__device__ __forceinline__ float bf2f(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+__device__ __forceinline__ uint16_t f2bf(float f) {
+  return __builtin_bit_cast(uint16_t, (__bf16)f);  // round-to-nearest-even (v_cvt_pk_bf16_f32)
+}
+__device__ __forceinline__ float rbf(float f) { return bf2f(f2bf(f)); }
+__device__ __forceinline__ uint32_t pack2bf(float lo, float hi) {
+  return (uint32_t)f2bf(lo) | ((uint32_t)f2bf(hi) << 16);
+}
+__device__ __forceinline__ float bflo(uint32_t p) { return __uint_as_float(p << 16); }
+__device__ __forceinline__ float bfhi(uint32_t p) { return __uint_as_float(p & 0xffff0000u); }
+
+__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+  // D[16x16] += A[16x32] * B[32x16]; lane l holds A row l%16 / B column l%16, k = 8*(l/16)..+7;
+  // D: column l%16, rows 4*(l/16)..+3.
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                 __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// ---- code books ------------------------------------------------------------------------
+// The 16 NF4 levels of QLoRA (Dettmers et al. 2023), fp32.
+__device__ __constant__ const float kNf4Levels[16] = {
+    -1.0f,        -0.6961928f,  -0.52507305f, -0.39491749f, -0.28444138f, -0.18477343f,
+    -0.09105004f, 0.0f,         0.0795803f,   0.1609302f,   0.2461123f,   0.33791524f,
+    0.44070983f,  0.562617f,    0.72295684f,  1.0f};
+
+__device__ __forceinline__ float code_level(int qtype, int code) {
+  return qtype == TNX_Q_NF4 ? kNf4Levels[code] : (float)(code - 8);
+}
+
+// LDS look-up table: byte (two codes) -> two bf16 levels, replicated so that lane l reads
+// entry [byte][l % 32] and every lane of a half-wave hits its own bank.
+#define TNX_LUT_COPIES 32
+#define TNX_LUT_WORDS (256 * TNX_LUT_COPIES)
+__device__ __forceinline__ void build_lut(uint32_t* lut, int qtype, int tid, int nthreads) {
+  for (int e = tid; e < TNX_LUT_WORDS; e += nthreads) {
+    int byte = e / TNX_LUT_COPIES;
+    lut[e] = pack2bf(code_level(qtype, byte & 15), code_level(qtype, byte >> 4));
+  }
+}
+__device__ __forceinline__ u32x4 dequant8(uint32_t w, const uint32_t* lut_lane) {
+  u32x4 r;
+  r[0] = lut_lane[(w & 0xffu) * TNX_LUT_COPIES];
+  r[1] = lut_lane[((w >> 8) & 0xffu) * TNX_LUT_COPIES];
+  r[2] = lut_lane[((w >> 16) & 0xffu) * TNX_LUT_COPIES];
+  r[3] = lut_lane[(w >> 24) * TNX_LUT_COPIES];
+  return r;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+static inline hipStream_t as_stream(void* s) { return (hipStream_t)s; }
+static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }

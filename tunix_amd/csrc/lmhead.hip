@@ -1,0 +1,249 @@
+// Fused lm_head -> log-softmax statistics.  Every work-group computes a [16*MT x 128] tile of
+// bf16-rounded logits with the shared skinny-GEMM main loop and reduces it on the spot to
+// (max, first arg-max, sum of exponentials, logit of the row's target id); a second small
+// kernel merges the per-block statistics of a row.  Full-vocabulary logits reach HBM only when
+// the caller asks for them (logits_out).
+#include <string.h>
+
+#include <mutex>
+
+#include "gemm_tile.h"
+
+namespace {
+
+struct LHArgs {
+  int64_t M, D, V;
+  const uint16_t* x;
+  const uint16_t* w_bf16;
+  const uint32_t* codes;
+  const uint16_t* scales;
+  int group, qtype;
+  int lora_rank;
+  const uint16_t* t;
+  int64_t t_ld;
+  const uint16_t* lora_b;
+  float lora_scale;
+  float temperature;
+  const int32_t* forbidden;
+  int n_forbidden;
+  const int32_t* targets;
+  float* part;
+  int64_t nvb;
+  float* logits_out;
+};
+
+constexpr float kNegInf = -__builtin_inff();
+
+struct Stat {
+  float mx;
+  int idx;
+  float sum;
+  float tgt;
+};
+// Merge two statistics; `a` covers lower column indices than `b`.
+__device__ __forceinline__ Stat merge(const Stat& a, const Stat& b) {
+  Stat r;
+  r.mx = fmaxf(a.mx, b.mx);
+  r.idx = (b.mx > a.mx) ? b.idx : a.idx;  // equal maxima: keep the lower index
+  const float wa = a.mx == kNegInf ? 0.f : __expf(a.mx - r.mx);
+  const float wb = b.mx == kNegInf ? 0.f : __expf(b.mx - r.mx);
+  r.sum = a.sum * wa + b.sum * wb;
+  r.tgt = fmaxf(a.tgt, b.tgt);
+  return r;
+}
+
+template <int MT, bool DENSE>
+__global__ __launch_bounds__(256) void lmhead_kernel(const LHArgs a) {
+  constexpr int NT = 2;
+  extern __shared__ __align__(16) unsigned char smem[];
+  uint16_t* sA = reinterpret_cast<uint16_t*>(smem);
+  uint32_t* sLut = reinterpret_cast<uint32_t*>(smem + MT * 16 * A_LD * sizeof(uint16_t));
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lm = lane & 15, lq = lane >> 4;
+  const int64_t vb = blockIdx.x;
+  const int64_t m0 = (int64_t)blockIdx.y * (MT * 16);
+  const int64_t ntile0 = (vb * 4 + wave) * NT;
+
+  const uint32_t* lut_lane = nullptr;
+  if constexpr (!DENSE) {
+    build_lut(sLut, a.qtype, tid, 256);
+    lut_lane = sLut + (lane & (TNX_LUT_COPIES - 1));
+  }
+  TileSrc s;
+  s.M = a.M; s.K = a.D; s.x = a.x; s.row_index = nullptr; s.row_div = 1; s.w_bf16 = a.w_bf16;
+  s.codes = a.codes; s.scales = a.scales; s.group = a.group; s.qtype = a.qtype;
+  s.ntiles = a.V / 16; s.lora_rank = a.lora_rank; s.t = a.t; s.t_ld = a.t_ld;
+  s.lora_b = a.lora_b; s.lora_scale = a.lora_scale;
+
+  f32x4 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) zero_acc(acc[mt][nt]);
+  tile_mainloop<MT, NT, DENSE>(s, m0, ntile0, 0, (int)(a.D / KTILE), sA, lut_lane, acc);
+  if (a.lora_rank > 0) {
+    int toff[NT] = {0, 0};
+    tile_lora<MT, NT>(s, m0, ntile0, toff, acc);
+  }
+
+  __syncthreads();  // sA is reused for the cross-wave reduction
+  Stat* sRed = reinterpret_cast<Stat*>(smem);  // [4 waves][16*MT rows]
+  const int64_t colA = (ntile0 + 0) * 16 + lm, colB = (ntile0 + 1) * 16 + lm;
+  bool okA = (ntile0 + 0) < s.ntiles, okB = (ntile0 + 1) < s.ntiles;
+  for (int f = 0; f < a.n_forbidden; ++f) {
+    const int64_t fid = a.forbidden[f];
+    if (fid == colA) okA = false;
+    if (fid == colB) okB = false;
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int rl = mt * 16 + lq * 4 + i;
+      const int64_t row = m0 + rl;
+      const bool rok = row < a.M;
+      // logits are the bf16 einsum output cast to fp32, then divided by the temperature
+      const float la = okA ? __fdiv_rn(rbf(acc[mt][0][i]), a.temperature) : kNegInf;
+      const float lb = okB ? __fdiv_rn(rbf(acc[mt][1][i]), a.temperature) : kNegInf;
+      if (a.logits_out && rok) {
+        if ((ntile0 + 0) < s.ntiles) a.logits_out[row * a.V + colA] = la;
+        if ((ntile0 + 1) < s.ntiles) a.logits_out[row * a.V + colB] = lb;
+      }
+      Stat st;
+      st.mx = fmaxf(la, lb);
+      st.idx = (lb > la) ? (int)colB : (int)colA;
+      const int tg = (a.targets && rok) ? a.targets[row] : -1;
+      st.tgt = tg == (int)colA ? la : (tg == (int)colB ? lb : kNegInf);
+      // arg-max over the 16 lanes of the row (columns grow with lm)
+      float mx = st.mx;
+      int idx = st.idx;
+#pragma unroll
+      for (int o = 1; o < 16; o <<= 1) {
+        const float omx = __shfl_xor(mx, o, 64);
+        const int oidx = __shfl_xor(idx, o, 64);
+        if (omx > mx || (omx == mx && oidx < idx)) {
+          mx = omx;
+          idx = oidx;
+        }
+        st.tgt = fmaxf(st.tgt, __shfl_xor(st.tgt, o, 64));
+      }
+      float se = 0.f;
+      if (mx != kNegInf) se = (la == kNegInf ? 0.f : __expf(la - mx)) + (lb == kNegInf ? 0.f : __expf(lb - mx));
+#pragma unroll
+      for (int o = 1; o < 16; o <<= 1) se += __shfl_xor(se, o, 64);
+      if (lm == 0) {
+        Stat r;
+        r.mx = mx; r.idx = idx; r.sum = se; r.tgt = st.tgt;
+        sRed[wave * (MT * 16) + rl] = r;
+      }
+    }
+  __syncthreads();
+  if (tid < MT * 16 && m0 + tid < a.M) {
+    Stat r = sRed[tid];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) r = merge(r, sRed[w * (MT * 16) + tid]);
+    float* p = a.part + ((m0 + tid) * a.nvb + vb) * 4;
+    p[0] = r.mx;
+    p[1] = __int_as_float(r.idx);
+    p[2] = r.sum;
+    p[3] = r.tgt;
+  }
+}
+
+// One wave per row merges the per-block statistics in column order.
+__global__ __launch_bounds__(64) void lmhead_finish_kernel(const float* part, int64_t nvb,
+                                                           int32_t* best_id, float* best_logp,
+                                                           float* target_logp, float* lse_out) {
+  const int64_t row = blockIdx.x;
+  const int lane = threadIdx.x;
+  const float* p = part + row * nvb * 4;
+  // lane l owns the contiguous block range [l*per, (l+1)*per): merges stay in column order
+  const int64_t per = (nvb + 63) / 64;
+  Stat r;
+  r.mx = kNegInf; r.idx = 0x7fffffff; r.sum = 0.f; r.tgt = kNegInf;
+  for (int64_t c = lane * per; c < min(nvb, (lane + 1) * per); ++c) {
+    Stat b;
+    b.mx = p[c * 4]; b.idx = __float_as_int(p[c * 4 + 1]); b.sum = p[c * 4 + 2]; b.tgt = p[c * 4 + 3];
+    r = merge(r, b);
+  }
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    Stat b;
+    b.mx = __shfl_xor(r.mx, o, 64);
+    b.idx = __shfl_xor(r.idx, o, 64);
+    b.sum = __shfl_xor(r.sum, o, 64);
+    b.tgt = __shfl_xor(r.tgt, o, 64);
+    r = (lane & o) ? merge(b, r) : merge(r, b);  // the lower lane holds the lower columns
+  }
+  if (lane == 0) {
+    const float lse = r.mx + logf(r.sum);
+    if (best_id) best_id[row] = r.idx;
+    if (best_logp) best_logp[row] = r.mx - lse;
+    if (target_logp) target_logp[row] = r.tgt - lse;
+    if (lse_out) lse_out[row] = lse;
+  }
+}
+
+template <class Kern>
+int raise_lds_limit(Kern kern, size_t bytes) {
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e != hipSuccess) {
+    tnx_set_error("cannot raise dynamic LDS limit: %s", hipGetErrorString(e));
+    return TNX_ELAUNCH;
+  }
+  return TNX_OK;
+}
+
+template <int MT, bool DENSE>
+int launch_lmhead(hipStream_t st, const LHArgs& a) {
+  static std::once_flag once;
+  static int attr_rc = TNX_OK;
+  std::call_once(once, [] { attr_rc = raise_lds_limit(&lmhead_kernel<MT, DENSE>, tile_smem_bytes(MT)); });
+  if (attr_rc) return attr_rc;
+  dim3 grid((unsigned)a.nvb, (unsigned)cdiv(a.M, MT * 16));
+  hipLaunchKernelGGL((lmhead_kernel<MT, DENSE>), grid, dim3(256), tile_smem_bytes(MT), st, a);
+  TNX_CHECK_LAUNCH("lmhead");
+  return TNX_OK;
+}
+
+}  // namespace
+
+extern "C" int64_t tnx_lmhead_nblocks(int64_t V) { return cdiv(V, 128); }
+
+extern "C" int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* d) {
+  TNX_REQUIRE(d, "lmhead: null descriptor");
+  TNX_REQUIRE(d->M > 0 && d->D > 0 && d->V > 0, "lmhead: bad shape");
+  TNX_REQUIRE(d->D % KTILE == 0 && d->V % 16 == 0, "lmhead: D %% 128 and V %% 16 must be 0 (D=%lld V=%lld)",
+              (long long)d->D, (long long)d->V);
+  TNX_REQUIRE(d->M <= 65535LL * 128, "lmhead: too many rows in one call");
+  TNX_REQUIRE(d->x && d->part, "lmhead: null pointer");
+  TNX_REQUIRE(d->w_bf16 || (d->codes && d->scales), "lmhead: no head weights");
+  if (!d->w_bf16) {
+    int rc = tnx_qw_sizes(d->D, d->V, d->group, nullptr, nullptr);
+    if (rc) return rc;
+    TNX_REQUIRE(d->qtype == TNX_Q_INT4 || d->qtype == TNX_Q_NF4, "lmhead: bad qtype");
+  }
+  if (d->lora_rank > 0)
+    TNX_REQUIRE(d->lora_rank % 32 == 0 && d->t && d->lora_b && d->t_ld % 8 == 0, "lmhead: bad LoRA arguments");
+  LHArgs a;
+  a.M = d->M; a.D = d->D; a.V = d->V; a.x = d->x; a.w_bf16 = d->w_bf16; a.codes = d->codes;
+  a.scales = d->scales; a.group = d->group; a.qtype = d->qtype; a.lora_rank = d->lora_rank;
+  a.t = d->t; a.t_ld = d->t_ld; a.lora_b = d->lora_b; a.lora_scale = d->lora_scale;
+  a.temperature = d->temperature == 0.f ? 1.0f : d->temperature;
+  a.forbidden = d->forbidden; a.n_forbidden = d->forbidden ? d->n_forbidden : 0;
+  a.targets = d->targets; a.part = d->part; a.nvb = tnx_lmhead_nblocks(d->V);
+  a.logits_out = d->logits_out;
+  hipStream_t st = as_stream(stream);
+  int rc;
+  const bool dense = d->w_bf16 != nullptr;
+  if (d->M <= 16) rc = dense ? launch_lmhead<1, true>(st, a) : launch_lmhead<1, false>(st, a);
+  else if (d->M <= 32) rc = dense ? launch_lmhead<2, true>(st, a) : launch_lmhead<2, false>(st, a);
+  else if (d->M <= 64) rc = dense ? launch_lmhead<4, true>(st, a) : launch_lmhead<4, false>(st, a);
+  else rc = dense ? launch_lmhead<8, true>(st, a) : launch_lmhead<8, false>(st, a);
+  if (rc) return rc;
+  hipLaunchKernelGGL(lmhead_finish_kernel, dim3((unsigned)d->M), dim3(64), 0, st, a.part, a.nvb,
+                     d->best_id, d->best_logp, d->target_logp, d->lse);
+  TNX_CHECK_LAUNCH("lmhead_finish");
+  return TNX_OK;
+}

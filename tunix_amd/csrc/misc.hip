@@ -1,0 +1,214 @@
+// Error plumbing, small element-wise kernels (fill, sampler bookkeeping, GRPO ratio) and the
+// MoE routing helpers.
+#include <stdarg.h>
+#include <string.h>
+
+#include "common.h"
+
+namespace {
+thread_local char g_err[512] = "";
+}
+
+void tnx_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+extern "C" const char* tnx_last_error(void) { return g_err; }
+extern "C" int tnx_version(void) { return (1 << 16) | 0; }
+
+namespace {
+
+__global__ void fill_kernel(uint32_t* p, int64_t n, uint32_t v) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+__global__ void sample_commit_kernel(const int32_t* ids, const float* logp, int64_t B,
+                                     int32_t* tokens, int64_t tok_ld, float* logprobs,
+                                     int32_t* done, const int32_t* eos, int n_eos,
+                                     int32_t* step_ptr) {
+  // single work-group: every thread reads the step before anyone advances it
+  const int col = *step_ptr;
+  __syncthreads();
+  for (int64_t b = threadIdx.x; b < B; b += blockDim.x) {
+    const int32_t id = ids[b];
+    tokens[b * tok_ld + col + 1] = id;
+    if (logprobs && logp) logprobs[b * tok_ld + col + 1] = logp[b];
+    if (done) {
+      int hit = 0;
+      for (int e = 0; e < n_eos; ++e) hit |= (id == eos[e]);
+      if (hit) done[b] = 1;
+    }
+  }
+  if (threadIdx.x == 0) *step_ptr = col + 1;
+}
+
+__global__ void grpo_ratio_kernel(const float* logp, const float* old_logp, const float* adv,
+                                  int64_t N, int64_t tokens_per_seq, float eps_lo, float eps_hi,
+                                  float* ratio, float* loss, int32_t* clipped) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= N) return;
+  float lr = logp[i] - (old_logp ? old_logp[i] : logp[i]);
+  lr = fminf(fmaxf(lr, -20.0f), 20.0f);
+  const float r = expf(lr);
+  const float a = adv[i / tokens_per_seq];
+  const float l1 = -a * r;
+  const float l2 = -a * fminf(fmaxf(r, 1.0f - eps_lo), 1.0f + eps_hi);
+  if (ratio) ratio[i] = r;
+  if (loss) loss[i] = fmaxf(l1, l2);
+  if (clipped) clipped[i] = l2 > l1 ? 1 : 0;
+}
+
+// Router: fp32 softmax of the bf16 scores, top-k (descending, lower expert id first among
+// equals), renormalise, cast to bf16.  One wave per token; E <= 1024.
+__global__ __launch_bounds__(64) void moe_route_kernel(const uint16_t* scores, int E, int k,
+                                                       uint16_t* topk_w, int32_t* topk_id) {
+  __shared__ float prob[1024];
+  const int64_t m = blockIdx.x;
+  const int lane = threadIdx.x;
+  const uint16_t* sr = scores + m * E;
+  float mx = -__builtin_inff();
+  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, bf2f(sr[e]));
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int e = lane; e < E; e += 64) {
+    const float p = expf(bf2f(sr[e]) - mx);
+    prob[e] = p;
+    sum += p;
+  }
+  sum = wave_sum(sum);
+  __syncthreads();
+  for (int e = lane; e < E; e += 64) prob[e] = prob[e] / sum;
+  __syncthreads();
+  float wsum = 0.f;
+  float sel_w = 0.f;   // lane j keeps the j-th selected weight (k <= 64)
+  int sel_id = 0;
+  for (int j = 0; j < k; ++j) {
+    float best = -1.f;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float p = prob[e];
+      if (p > best) { best = p; bi = e; }
+    }
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const float ob = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+    }
+    if (lane == j) { sel_w = best; sel_id = bi; }
+    wsum += best;
+    if (lane == 0) prob[bi] = -1.f;
+    __syncthreads();
+  }
+  if (lane < k) {
+    topk_w[m * k + lane] = f2bf(sel_w / wsum);
+    topk_id[m * k + lane] = sel_id;
+  }
+}
+
+// Counting sort of routes by expert; single work-group, stable in route order.
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* topk_id, int64_t n_routes,
+                                                        int E, int32_t* counts, int32_t* offsets,
+                                                        int32_t* sorted_route) {
+  extern __shared__ int32_t sh[];  // [E] counts, then [E] cursors
+  int32_t* cnt = sh;
+  int32_t* cur = sh + E;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int64_t r = threadIdx.x; r < n_routes; r += blockDim.x) atomicAdd(&cnt[topk_id[r]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t acc = 0;
+    for (int e = 0; e < E; ++e) {
+      offsets[e] = acc;
+      cur[e] = acc;
+      counts[e] = cnt[e];
+      acc += cnt[e];
+    }
+    offsets[E] = acc;
+  }
+  __syncthreads();
+  // stable placement: expert e's routes in increasing route id, one thread per expert
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    int32_t pos = cur[e];
+    for (int64_t r = 0; r < n_routes; ++r)
+      if (topk_id[r] == e) sorted_route[pos++] = (int32_t)r;
+  }
+}
+
+__global__ void moe_combine_kernel(const uint16_t* y, const uint16_t* topk_w, int k, int64_t D,
+                                   const uint16_t* residual, uint16_t* out) {
+  const int64_t m = blockIdx.x;
+  for (int64_t d = threadIdx.x; d < D; d += blockDim.x) {
+    float acc = 0.f;
+    for (int j = 0; j < k; ++j) acc += bf2f(topk_w[m * k + j]) * bf2f(y[(m * k + j) * D + d]);
+    float v = rbf(acc);
+    if (residual) v = rbf(v + bf2f(residual[m * D + d]));
+    out[m * D + d] = f2bf(v);
+  }
+}
+
+}  // namespace
+
+extern "C" int tnx_fill_u32(void* stream, uint32_t* p, int64_t n, uint32_t value) {
+  TNX_REQUIRE(p && n >= 0, "fill: bad arguments");
+  if (n == 0) return TNX_OK;
+  hipLaunchKernelGGL(fill_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, as_stream(stream), p, n, value);
+  TNX_CHECK_LAUNCH("fill");
+  return TNX_OK;
+}
+
+extern "C" int tnx_sample_commit(void* stream, const int32_t* ids, const float* logp, int64_t B,
+                                 int32_t* tokens, int64_t tok_ld, float* logprobs, int32_t* done,
+                                 const int32_t* eos, int n_eos, int32_t* step_ptr) {
+  TNX_REQUIRE(ids && tokens && step_ptr && B > 0, "sample_commit: bad arguments");
+  TNX_REQUIRE(n_eos == 0 || eos, "sample_commit: eos list is null");
+  hipLaunchKernelGGL(sample_commit_kernel, dim3(1), dim3(256), 0, as_stream(stream), ids, logp, B,
+                     tokens, tok_ld, logprobs, done, eos, n_eos, step_ptr);
+  TNX_CHECK_LAUNCH("sample_commit");
+  return TNX_OK;
+}
+
+extern "C" int tnx_grpo_ratio(void* stream, const float* logp, const float* old_logp,
+                              const float* adv, int64_t N, int64_t tokens_per_seq, float eps_lo,
+                              float eps_hi, float* ratio, float* loss, int32_t* clipped) {
+  TNX_REQUIRE(logp && adv && N > 0 && tokens_per_seq > 0, "grpo_ratio: bad arguments");
+  hipLaunchKernelGGL(grpo_ratio_kernel, dim3((unsigned)cdiv(N, 256)), dim3(256), 0,
+                     as_stream(stream), logp, old_logp, adv, N, tokens_per_seq, eps_lo, eps_hi,
+                     ratio, loss, clipped);
+  TNX_CHECK_LAUNCH("grpo_ratio");
+  return TNX_OK;
+}
+
+extern "C" int tnx_moe_route_topk(void* stream, const uint16_t* scores, int64_t M, int E, int k,
+                                  uint16_t* topk_w, int32_t* topk_id) {
+  TNX_REQUIRE(scores && topk_w && topk_id, "moe_route: null pointer");
+  TNX_REQUIRE(M > 0 && E > 0 && E <= 1024 && k > 0 && k <= 64 && k <= E, "moe_route: bad shape E=%d k=%d", E, k);
+  hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)M), dim3(64), 0, as_stream(stream), scores, E,
+                     k, topk_w, topk_id);
+  TNX_CHECK_LAUNCH("moe_route");
+  return TNX_OK;
+}
+
+extern "C" int tnx_moe_sort_routes(void* stream, const int32_t* topk_id, int64_t M, int k, int E,
+                                   int32_t* counts, int32_t* offsets, int32_t* sorted_route) {
+  TNX_REQUIRE(topk_id && counts && offsets && sorted_route, "moe_sort: null pointer");
+  TNX_REQUIRE(M > 0 && k > 0 && E > 0 && E <= 4096 && M * k <= (1 << 20), "moe_sort: bad shape");
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), (size_t)(2 * E) * sizeof(int32_t),
+                     as_stream(stream), topk_id, M * k, E, counts, offsets, sorted_route);
+  TNX_CHECK_LAUNCH("moe_sort");
+  return TNX_OK;
+}
+
+extern "C" int tnx_moe_combine(void* stream, const uint16_t* y, const uint16_t* topk_w, int64_t M,
+                               int k, int64_t D, const uint16_t* residual, uint16_t* out) {
+  TNX_REQUIRE(y && topk_w && out && M > 0 && k > 0 && D > 0, "moe_combine: bad arguments");
+  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)M), dim3(256), 0, as_stream(stream), y,
+                     topk_w, k, D, residual, out);
+  TNX_CHECK_LAUNCH("moe_combine");
+  return TNX_OK;
+}

@@ -1,0 +1,230 @@
+// Embedding gather, RMSNorm (three dtype flows), per-head q/k norm + RoPE + KV-cache write.
+// All of these move a few bytes per decode step compared with the weights and the cache; they
+// are written for exact dtype-flow parity and few launches, not for peak bandwidth.
+#include <string.h>
+
+#include "common.h"
+
+namespace {
+
+// ---- block reductions --------------------------------------------------------------------
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+  if (nw == 1) return v;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[wave] = v;
+  __syncthreads();
+  float s = 0.f;
+  for (int w = 0; w < nw; ++w) s += red[w];
+  return s;
+}
+
+// One normalised element, given the row statistics.  `ms` is mean(x^2) (llama/qwen3: fp32 of
+// fp32 squares; gemma3: bf16-rounded mean of bf16-rounded squares).
+__device__ __forceinline__ float norm_elem(float x, float w, float ms, float eps, int flavor) {
+  if (flavor == TNX_NORM_LLAMA) {
+    // astype(w * x / rms): w*x is a bf16 product, the division is fp32.
+    const float rms = sqrtf(ms + eps);
+    return rbf(rbf(w * x) / rms);
+  } else if (flavor == TNX_NORM_QWEN3) {
+    const float rms = sqrtf(ms + eps);
+    return rbf(w * (x / rms));
+  } else {
+    // gemma3: every op in bf16: x * rsqrt(var + eps) * (1 + scale)
+    const float r = rbf(1.0f / sqrtf(rbf(ms + eps)));
+    return rbf(rbf(x * r) * rbf(1.0f + w));
+  }
+}
+__device__ __forceinline__ float sq_term(float x, int flavor) {
+  return flavor == TNX_NORM_GEMMA3 ? rbf(x * x) : x * x;
+}
+__device__ __forceinline__ float finish_ms(float ss, float n, int flavor) {
+  const float ms = ss / n;
+  return flavor == TNX_NORM_GEMMA3 ? rbf(ms) : ms;
+}
+
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* x, const uint16_t* res_pre,
+                                                      uint16_t* h_out, const uint16_t* w,
+                                                      const uint16_t* res_post, uint16_t* y,
+                                                      int64_t D, float eps, int flavor) {
+  __shared__ float red[4];
+  extern __shared__ __align__(16) unsigned char smem_dyn[];
+  float* hrow = reinterpret_cast<float*>(smem_dyn);  // [D]
+  const int64_t row = blockIdx.x;
+  const uint16_t* xr = x + row * D;
+  float ss = 0.f;
+  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
+    float h = bf2f(xr[i]);
+    if (res_pre) h = rbf(h + bf2f(res_pre[row * D + i]));
+    if (h_out) h_out[row * D + i] = f2bf(h);
+    hrow[i] = h;
+    ss += sq_term(h, flavor);
+  }
+  ss = block_sum(ss, red);
+  const float ms = finish_ms(ss, (float)D, flavor);
+  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
+    float v = norm_elem(hrow[i], bf2f(w[i]), ms, eps, flavor);
+    if (res_post) v = rbf(v + bf2f(res_post[row * D + i]));
+    y[row * D + i] = f2bf(v);
+  }
+}
+
+__global__ void embed_kernel(const uint16_t* table, int64_t V, int64_t D, const int32_t* ids,
+                             int64_t ids_ld, const int32_t* col_ptr, int64_t T, float scale_bf,
+                             uint16_t* out) {
+  const int64_t row = blockIdx.x;  // b*T + t
+  const int64_t b = row / T, t = row % T;
+  const int col = col_ptr ? *col_ptr : 0;
+  int64_t id = ids[b * ids_ld + col + t];
+  if (id < 0 || id >= V) id = 0;  // pad sentinels outside the vocabulary read row 0 (masked later)
+  const uint16_t* src = table + id * D;
+  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
+    uint16_t v = src[i];
+    if (scale_bf != 1.0f) v = f2bf(bf2f(v) * scale_bf);
+    out[row * D + i] = v;
+  }
+}
+
+struct RopeArgs {
+  int64_t B, T, S;
+  int Hq, Hkv, dh;
+  int rope_flavor;
+  float rope_scale;
+  int qk_norm;
+  float norm_eps;
+  const uint16_t* q_norm_w;
+  const uint16_t* k_norm_w;
+  float q_prescale_bf;
+  const uint16_t* qkv;
+  const int32_t* positions;
+  int64_t pos_ld;
+  const int32_t* col_ptr;
+  const float* timescale;
+  uint16_t* q_out;
+  uint16_t* kcache;
+  uint16_t* vcache;
+};
+
+// grid (B*T, Hq + 2*Hkv); max(64, dh/2) threads: thread i < dh/2 owns elements i and i + dh/2
+// of one head; the other threads only take part in the reductions.
+__global__ void rope_kernel(const RopeArgs a) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const int64_t b = row / a.T, t = row % a.T;
+  const int head = blockIdx.y;
+  const int half = a.dh / 2, i = threadIdx.x;
+  const bool live = i < half;
+  const int col = *a.col_ptr;
+  const int ld = (a.Hq + 2 * a.Hkv) * a.dh;
+  const uint16_t* src = a.qkv + row * ld + (int64_t)head * a.dh;
+  const int slot = (int)((col + t) % a.S);
+  if (head >= a.Hq + a.Hkv) {  // V: plain copy into the cache slot
+    const int hk = head - a.Hq - a.Hkv;
+    uint16_t* dst = a.vcache + (((b * a.Hkv + hk) * a.S) + slot) * a.dh;
+    if (live) {
+      dst[i] = src[i];
+      dst[i + half] = src[i + half];
+    }
+    return;
+  }
+  const bool is_q = head < a.Hq;
+  float x1 = live ? bf2f(src[i]) : 0.f, x2 = live ? bf2f(src[i + half]) : 0.f;
+  if (a.qk_norm >= 0) {
+    const float ss = block_sum(sq_term(x1, a.qk_norm) + sq_term(x2, a.qk_norm), red);
+    const float ms = finish_ms(ss, (float)a.dh, a.qk_norm);
+    const uint16_t* w = is_q ? a.q_norm_w : a.k_norm_w;
+    if (live) {
+      x1 = norm_elem(x1, bf2f(w[i]), ms, a.norm_eps, a.qk_norm);
+      x2 = norm_elem(x2, bf2f(w[i + half]), ms, a.norm_eps, a.qk_norm);
+    }
+  }
+  if (!live) return;
+  const float pos = (float)a.positions[b * a.pos_ld + col + t];
+  float ang = __fdiv_rn(pos, a.timescale[i]);
+  if (a.rope_flavor == TNX_ROPE_GEMMA3) ang = __fdiv_rn(ang, a.rope_scale);
+  float sn = sinf(ang), cs = cosf(ang);
+  float o1, o2;
+  if (a.rope_flavor == TNX_ROPE_QWEN3) {
+    sn = rbf(sn);
+    cs = rbf(cs);
+    o1 = rbf(rbf(x1 * cs) - rbf(x2 * sn));
+    o2 = rbf(rbf(x2 * cs) + rbf(x1 * sn));
+  } else {
+    // fp32 products and sum, one rounding at the end (no fused multiply-add)
+    o1 = rbf(__fsub_rn(__fmul_rn(x1, cs), __fmul_rn(x2, sn)));
+    o2 = rbf(__fadd_rn(__fmul_rn(x2, cs), __fmul_rn(x1, sn)));
+  }
+  if (is_q) {
+    if (a.q_prescale_bf != 0.f) {
+      o1 = rbf(o1 * a.q_prescale_bf);
+      o2 = rbf(o2 * a.q_prescale_bf);
+    }
+    uint16_t* dst = a.q_out + (row * a.Hq + head) * a.dh;
+    dst[i] = f2bf(o1);
+    dst[i + half] = f2bf(o2);
+  } else {
+    const int hk = head - a.Hq;
+    uint16_t* dst = a.kcache + (((b * a.Hkv + hk) * a.S) + slot) * a.dh;
+    dst[i] = f2bf(o1);
+    dst[i + half] = f2bf(o2);
+  }
+}
+
+float host_round_bf16(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+}  // namespace
+
+extern "C" int tnx_embed(void* stream, const uint16_t* table, int64_t V, int64_t D,
+                         const int32_t* ids, int64_t ids_ld, const int32_t* col_ptr, int64_t B,
+                         int64_t T, float scale, uint16_t* out) {
+  TNX_REQUIRE(table && ids && out, "embed: null pointer");
+  TNX_REQUIRE(V > 0 && D > 0 && B > 0 && T > 0, "embed: bad shape");
+  hipLaunchKernelGGL(embed_kernel, dim3((unsigned)(B * T)), dim3(256), 0, as_stream(stream), table,
+                     V, D, ids, ids_ld, col_ptr, T, host_round_bf16(scale), out);
+  TNX_CHECK_LAUNCH("embed");
+  return TNX_OK;
+}
+
+extern "C" int tnx_rmsnorm(void* stream, const uint16_t* x, const uint16_t* res_pre,
+                           uint16_t* h_out, const uint16_t* w, const uint16_t* res_post,
+                           uint16_t* y, int64_t M, int64_t D, float eps, int flavor) {
+  TNX_REQUIRE(x && w && y, "rmsnorm: null pointer");
+  TNX_REQUIRE(M > 0 && D > 0 && D <= 16384, "rmsnorm: D=%lld out of range (1..16384)", (long long)D);
+  TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm: bad flavor %d", flavor);
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)M), dim3(256), (size_t)D * sizeof(float),
+                     as_stream(stream), x, res_pre, h_out, w, res_post, y, D, eps, flavor);
+  TNX_CHECK_LAUNCH("rmsnorm");
+  return TNX_OK;
+}
+
+extern "C" int tnx_qknorm_rope_kvwrite(void* stream, const tnx_rope_desc* d) {
+  TNX_REQUIRE(d, "rope: null descriptor");
+  TNX_REQUIRE(d->B > 0 && d->T > 0 && d->S > 0, "rope: bad shape");
+  TNX_REQUIRE(d->dh % 2 == 0 && d->dh >= 2 && d->dh <= 512, "rope: bad head_dim %d", d->dh);
+  TNX_REQUIRE(d->qkv && d->positions && d->col_ptr && d->timescale && d->q_out && d->kcache &&
+                  d->vcache,
+              "rope: null pointer");
+  TNX_REQUIRE(d->rope_flavor >= TNX_ROPE_LLAMA && d->rope_flavor <= TNX_ROPE_GEMMA3, "rope: bad flavor");
+  TNX_REQUIRE(d->qk_norm >= -1 && d->qk_norm <= TNX_NORM_GEMMA3, "rope: bad qk_norm");
+  if (d->qk_norm >= 0) TNX_REQUIRE(d->q_norm_w && d->k_norm_w, "rope: qk_norm weights are null");
+  if (d->rope_flavor == TNX_ROPE_GEMMA3)
+    TNX_REQUIRE(d->rope_scale >= 1.0f, "rope: scale_factor must be >= 1.0, got %f", d->rope_scale);
+  RopeArgs a;
+  a.B = d->B; a.T = d->T; a.S = d->S; a.Hq = d->Hq; a.Hkv = d->Hkv; a.dh = d->dh;
+  a.rope_flavor = d->rope_flavor; a.rope_scale = d->rope_scale; a.qk_norm = d->qk_norm;
+  a.norm_eps = d->norm_eps; a.q_norm_w = d->q_norm_w; a.k_norm_w = d->k_norm_w;
+  a.q_prescale_bf = d->q_prescale != 0.f ? host_round_bf16(d->q_prescale) : 0.f;
+  a.qkv = d->qkv; a.positions = d->positions; a.pos_ld = d->pos_ld; a.col_ptr = d->col_ptr;
+  a.timescale = d->timescale; a.q_out = d->q_out; a.kcache = d->kcache; a.vcache = d->vcache;
+  dim3 grid((unsigned)(d->B * d->T), (unsigned)(d->Hq + 2 * d->Hkv));
+  hipLaunchKernelGGL(rope_kernel, grid, dim3(d->dh / 2 < 64 ? 64 : d->dh / 2), 0, as_stream(stream), a);
+  TNX_CHECK_LAUNCH("qknorm_rope_kvwrite");
+  return TNX_OK;
+}

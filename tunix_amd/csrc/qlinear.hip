@@ -1,0 +1,526 @@
+// Quantized (int4 / NF4, group scales) skinny GEMM fused with the rank-r LoRA delta, the MoE
+// grouped variant, the LoRA down-projection, the QW packer and its inverse.  The main loop is
+// in gemm_tile.h.
+#include <string.h>
+
+#include <mutex>
+
+#include "gemm_tile.h"
+
+namespace {
+
+struct QLArgs {
+  int64_t M, K, N;
+  int group, qtype;
+  const uint16_t* x;
+  const uint32_t* codes;
+  const uint16_t* scales;
+  int lora_rank, lora_nseg;
+  int64_t lora_seg_end[4];
+  int lora_seg_toff[4];
+  int64_t t_ld;
+  const uint16_t* t;
+  const uint16_t* lora_b;
+  float lora_scale;
+  int epilogue;
+  const uint16_t* residual;
+  void* y;
+  int split_k;
+  float* ws;
+  int ktiles_per_split;
+  // grouped (MoE) mode: blockIdx.x = expert; rows are routes sorted by expert
+  const int32_t* offsets;
+  const int32_t* sorted_route;
+  int x_div;
+  int64_t codes_stride, scales_stride;  // per-expert strides in elements
+};
+
+__device__ __forceinline__ float silu_bf16(float g) {
+  // jax.nn.silu = x * sigmoid(x) as two bf16 HLO ops.
+  float s = rbf(1.0f / (1.0f + __expf(-g)));
+  return rbf(g * s);
+}
+__device__ __forceinline__ float gelu_tanh_bf16(float g) {
+  const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+  float inner = k0 * (g + k1 * g * g * g);
+  return rbf(0.5f * g * (1.0f + tanhf(inner)));
+}
+
+// Epilogue shared by the plain and the grouped kernel.  `out_row(r)` maps a tile row to the
+// output row (identity, or the route id in grouped mode).
+template <int MT, int NT, class RowMap>
+__device__ __forceinline__ void store_tile(const QLArgs& a, int64_t m0, int64_t m_end,
+                                           int64_t ntile0, int64_t ntiles, f32x4 (&acc)[MT][NT],
+                                           RowMap out_row) {
+  const int lane = threadIdx.x & 63, lm = lane & 15, lq = lane >> 4;
+  if (a.split_k > 1) {  // partial sums; tnx_splitk_finish applies the epilogue
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      if (ntile0 + nt >= ntiles) continue;
+      const int64_t col = (ntile0 + nt) * 16 + lm;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int64_t row = m0 + mt * 16 + lq * 4 + i;
+          if (row < m_end) atomicAdd(a.ws + out_row(row) * a.N + col, acc[mt][nt][i]);
+        }
+    }
+    return;
+  }
+  if (a.epilogue == TNX_EPI_SILU_MUL || a.epilogue == TNX_EPI_GELU_MUL) {
+    if constexpr (NT % 2 == 0) {
+      uint16_t* y = reinterpret_cast<uint16_t*>(a.y);
+      const int64_t ldy = a.N / 2;
+#pragma unroll
+      for (int p = 0; p < NT / 2; ++p) {
+        if (ntile0 + 2 * p >= ntiles) continue;
+        const int64_t col = ((ntile0 + 2 * p) / 2) * 16 + lm;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int64_t row = m0 + mt * 16 + lq * 4 + i;
+            if (row >= m_end) continue;
+            const float g = rbf(acc[mt][2 * p][i]);
+            const float u = rbf(acc[mt][2 * p + 1][i]);
+            const float act = a.epilogue == TNX_EPI_SILU_MUL ? silu_bf16(g) : gelu_tanh_bf16(g);
+            y[out_row(row) * ldy + col] = f2bf(rbf(act) * u);
+          }
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    if (ntile0 + nt >= ntiles) continue;
+    const int64_t col = (ntile0 + nt) * 16 + lm;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int64_t row = m0 + mt * 16 + lq * 4 + i;
+        if (row >= m_end) continue;
+        const float v = acc[mt][nt][i];
+        const int64_t o = out_row(row) * a.N + col;
+        if (a.epilogue == TNX_EPI_F32) {
+          reinterpret_cast<float*>(a.y)[o] = v;
+        } else if (a.epilogue == TNX_EPI_RESIDUAL) {
+          reinterpret_cast<uint16_t*>(a.y)[o] = f2bf(rbf(v) + bf2f(a.residual[o]));
+        } else {
+          reinterpret_cast<uint16_t*>(a.y)[o] = f2bf(v);
+        }
+      }
+  }
+}
+
+template <int MT, int NT>
+__global__ __launch_bounds__(256) void qlinear_kernel(const QLArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  uint16_t* sA = reinterpret_cast<uint16_t*>(smem);  // [16*MT][A_LD]
+  uint32_t* sLut = reinterpret_cast<uint32_t*>(smem + MT * 16 * A_LD * sizeof(uint16_t));
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t m0 = (int64_t)blockIdx.x * (MT * 16);
+  const int64_t ntile0 = ((int64_t)blockIdx.y * 4 + wave) * NT;
+  const int ktiles = (int)(a.K / KTILE);
+  const int kt_begin = blockIdx.z * a.ktiles_per_split;
+  const int kt_end = min(ktiles, kt_begin + a.ktiles_per_split);
+
+  build_lut(sLut, a.qtype, tid, 256);
+  const uint32_t* lut_lane = sLut + (lane & (TNX_LUT_COPIES - 1));
+
+  TileSrc s;
+  s.M = a.M; s.K = a.K; s.x = a.x; s.row_index = nullptr; s.row_div = 1; s.w_bf16 = nullptr;
+  s.codes = a.codes; s.scales = a.scales; s.group = a.group; s.qtype = a.qtype;
+  s.ntiles = a.N / 16; s.lora_rank = a.lora_rank; s.t = a.t; s.t_ld = a.t_ld;
+  s.lora_b = a.lora_b; s.lora_scale = a.lora_scale;
+
+  f32x4 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) zero_acc(acc[mt][nt]);
+
+  tile_mainloop<MT, NT, false>(s, m0, ntile0, kt_begin, kt_end, sA, lut_lane, acc);
+
+  if (a.lora_rank > 0 && blockIdx.z == 0) {
+    int toff[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int64_t col0 = (ntile0 + nt) * 16;
+      if (a.lora_nseg < 0) {
+        toff[nt] = (int)((ntile0 + nt) & 1) * a.lora_rank;  // interleaved gate/up pair
+      } else {
+        toff[nt] = a.lora_seg_toff[0];
+        for (int q = 1; q < a.lora_nseg; ++q)
+          if (col0 >= a.lora_seg_end[q - 1]) toff[nt] = a.lora_seg_toff[q];
+      }
+    }
+    tile_lora<MT, NT>(s, m0, ntile0, toff, acc);
+  }
+  store_tile<MT, NT>(a, m0, a.M, ntile0, s.ntiles, acc, [](int64_t r) { return r; });
+}
+
+// Grouped GEMM over routed tokens: blockIdx.x = expert, blockIdx.z = 16*MT-row block inside
+// the expert's route list.  Rows are gathered through sorted_route; outputs are indexed by
+// route.
+template <int MT, int NT>
+__global__ __launch_bounds__(256) void moe_gmm_kernel(const QLArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  uint16_t* sA = reinterpret_cast<uint16_t*>(smem);
+  uint32_t* sLut = reinterpret_cast<uint32_t*>(smem + MT * 16 * A_LD * sizeof(uint16_t));
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int e = blockIdx.x;
+  const int r_begin = a.offsets[e], r_end = a.offsets[e + 1];
+  const int64_t m0 = (int64_t)blockIdx.z * (MT * 16);
+  if (m0 >= r_end - r_begin) return;
+  const int64_t ntile0 = ((int64_t)blockIdx.y * 4 + wave) * NT;
+
+  build_lut(sLut, a.qtype, tid, 256);
+  const uint32_t* lut_lane = sLut + (lane & (TNX_LUT_COPIES - 1));
+
+  TileSrc s;
+  s.M = r_end - r_begin; s.K = a.K; s.x = a.x; s.row_index = a.sorted_route + r_begin;
+  s.row_div = a.x_div; s.w_bf16 = nullptr;
+  s.codes = a.codes + (int64_t)e * a.codes_stride; s.scales = a.scales + (int64_t)e * a.scales_stride;
+  s.group = a.group; s.qtype = a.qtype; s.ntiles = a.N / 16; s.lora_rank = 0; s.t = nullptr;
+  s.t_ld = 0; s.lora_b = nullptr; s.lora_scale = 0.f;
+
+  f32x4 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) zero_acc(acc[mt][nt]);
+  tile_mainloop<MT, NT, false>(s, m0, ntile0, 0, (int)(a.K / KTILE), sA, lut_lane, acc);
+  const int32_t* routes = s.row_index;
+  store_tile<MT, NT>(a, m0, s.M, ntile0, s.ntiles, acc,
+                     [routes](int64_t r) { return (int64_t)routes[r]; });
+}
+
+// y = epi(ws); ws = 0.  One thread per output element.
+__global__ void splitk_finish_kernel(const QLArgs a) {
+  const bool mul = a.epilogue == TNX_EPI_SILU_MUL || a.epilogue == TNX_EPI_GELU_MUL;
+  const int64_t ncol = mul ? a.N / 2 : a.N;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= a.M * ncol) return;
+  const int64_t row = idx / ncol, c = idx % ncol;
+  if (mul) {
+    const int64_t cg = (c / 16) * 32 + (c % 16);
+    float* pg = a.ws + row * a.N + cg;
+    float* pu = pg + 16;
+    const float g = rbf(*pg), u = rbf(*pu);
+    *pg = 0.f;
+    *pu = 0.f;
+    const float act = a.epilogue == TNX_EPI_SILU_MUL ? silu_bf16(g) : gelu_tanh_bf16(g);
+    reinterpret_cast<uint16_t*>(a.y)[idx] = f2bf(act * u);
+    return;
+  }
+  float* p = a.ws + idx;
+  const float v = *p;
+  *p = 0.f;
+  if (a.epilogue == TNX_EPI_F32)
+    reinterpret_cast<float*>(a.y)[idx] = v;
+  else if (a.epilogue == TNX_EPI_RESIDUAL)
+    reinterpret_cast<uint16_t*>(a.y)[idx] = f2bf(rbf(v) + bf2f(a.residual[idx]));
+  else
+    reinterpret_cast<uint16_t*>(a.y)[idx] = f2bf(v);
+}
+
+// t[M,R] = bf16(x . A): one 16x16 output tile per work-group, K split over 8 waves.
+__global__ __launch_bounds__(512) void lora_down_kernel(const uint16_t* x, int64_t M, int64_t K,
+                                                        const uint16_t* a_t, int R, uint16_t* t,
+                                                        int64_t t_ld) {
+  __shared__ float red[8][64][4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lm = lane & 15, lq = lane >> 4;
+  const int64_t m0 = (int64_t)blockIdx.x * 16;
+  const int n0 = blockIdx.y * 16;
+  const int64_t row = m0 + lm;
+  const uint16_t* xr = x + row * K + lq * 8;
+  const uint16_t* ar = a_t + (int64_t)(n0 + lm) * K + lq * 8;
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int ksteps = (int)(K / 32);
+#pragma unroll 4
+  for (int ks = wave; ks < ksteps; ks += 8) {
+    u32x4 af = u32x4{0, 0, 0, 0};
+    if (row < M) af = *reinterpret_cast<const u32x4*>(xr + (int64_t)ks * 32);
+    const u32x4 bf = *reinterpret_cast<const u32x4*>(ar + (int64_t)ks * 32);
+    acc = mfma16(af, bf, acc);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) red[wave][lane][i] = acc[i];
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float s = 0.f;
+#pragma unroll
+      for (int w = 0; w < 8; ++w) s += red[w][lane][i];
+      const int64_t r = m0 + lq * 4 + i;
+      if (r < M) t[r * t_ld + n0 + lm] = f2bf(s);
+    }
+  }
+}
+
+// ---- QW packer ---------------------------------------------------------------------------
+__device__ __forceinline__ int64_t packed_col(int64_t c, int64_t N, int interleave2) {
+  if (!interleave2) return c;
+  const int64_t half = N / 2;
+  const int64_t h = c / half, cc = c % half;
+  return (cc / 16) * 32 + h * 16 + (cc % 16);
+}
+
+// One thread per (group of `group` consecutive k, source column).
+__global__ void quantize_pack_kernel(const void* w, int w_is_f32, int64_t K, int64_t N, int group,
+                                     int qtype, int interleave2, uint32_t* codes,
+                                     uint16_t* scales) {
+  const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t g = blockIdx.y;
+  if (c >= N) return;
+  const int64_t k0 = g * group;
+  auto ld = [&](int64_t k) -> float {
+    return w_is_f32 ? reinterpret_cast<const float*>(w)[k * N + c]
+                    : bf2f(reinterpret_cast<const uint16_t*>(w)[k * N + c]);
+  };
+  float amax = 0.f;
+  for (int i = 0; i < group; ++i) amax = fmaxf(amax, fabsf(ld(k0 + i)));
+  const uint16_t sbits = f2bf(qtype == TNX_Q_NF4 ? amax : amax / 7.0f);
+  const float s = bf2f(sbits);
+  const int64_t pc = packed_col(c, N, interleave2);
+  const int64_t nt = pc / 16, lm = pc % 16;
+  const int64_t ktiles = K / KTILE;
+  const int spt = group >= KTILE ? 1 : KTILE / group;
+  // scales: [nt][kt][spt][16]; a group larger than a k-tile repeats its scale in every tile.
+  for (int64_t k = k0; k < k0 + group; k += (group >= KTILE ? KTILE : group)) {
+    const int64_t kt = k / KTILE;
+    const int si = group >= KTILE ? 0 : (int)((k % KTILE) / group);
+    scales[((nt * ktiles + kt) * spt + si) * 16 + lm] = sbits;
+  }
+  for (int i0 = 0; i0 < group; i0 += 8) {
+    uint32_t word = 0;
+    for (int i = 0; i < 8; ++i) {
+      const float v = ld(k0 + i0 + i);
+      int code;
+      if (qtype == TNX_Q_NF4) {
+        code = 7;
+        if (s != 0.f) {
+          const float xn = v / s;
+          code = 0;
+          for (int e = 0; e < 15; ++e)
+            code += xn > 0.5f * (kNf4Levels[e] + kNf4Levels[e + 1]) ? 1 : 0;
+        }
+      } else {
+        code = 8;
+        if (s != 0.f) {
+          float q = rintf(v / s);
+          q = fminf(fmaxf(q, -8.f), 7.f);
+          code = (int)q + 8;
+        }
+      }
+      word |= (uint32_t)code << (4 * i);
+    }
+    const int64_t k = k0 + i0;
+    const int64_t kt = k / KTILE;
+    const int j = (int)((k % KTILE) / 32), lq = (int)((k % 32) / 8);
+    codes[((nt * ktiles + kt) * 64 + lq * 16 + lm) * 4 + j] = word;
+  }
+}
+
+__global__ void qw_dequant_kernel(const uint32_t* codes, const uint16_t* scales, int64_t K,
+                                  int64_t N, int group, int qtype, int interleave2, float* out) {
+  const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t k = blockIdx.y;
+  if (c >= N) return;
+  const int64_t pc = packed_col(c, N, interleave2);
+  const int64_t nt = pc / 16, lm = pc % 16, ktiles = K / KTILE, kt = k / KTILE;
+  const int spt = group >= KTILE ? 1 : KTILE / group;
+  const int si = group >= KTILE ? 0 : (int)((k % KTILE) / group);
+  const int j = (int)((k % KTILE) / 32), lq = (int)((k % 32) / 8), i = (int)(k % 8);
+  const uint32_t word = codes[((nt * ktiles + kt) * 64 + lq * 16 + lm) * 4 + j];
+  const float s = bf2f(scales[((nt * ktiles + kt) * spt + si) * 16 + lm]);
+  out[k * N + c] = rbf(code_level(qtype, (word >> (4 * i)) & 15)) * s;
+}
+
+QLArgs to_args(const tnx_qlinear_desc* d) {
+  QLArgs a;
+  a.M = d->M; a.K = d->K; a.N = d->N; a.group = d->group; a.qtype = d->qtype;
+  a.x = d->x; a.codes = d->codes; a.scales = d->scales;
+  a.lora_rank = d->lora_rank; a.lora_nseg = d->lora_nseg;
+  for (int i = 0; i < 4; ++i) { a.lora_seg_end[i] = d->lora_seg_end[i]; a.lora_seg_toff[i] = d->lora_seg_toff[i]; }
+  a.t_ld = d->t_ld; a.t = d->t; a.lora_b = d->lora_b; a.lora_scale = d->lora_scale;
+  a.epilogue = d->epilogue; a.residual = d->residual; a.y = d->y;
+  a.split_k = d->split_k < 1 ? 1 : d->split_k; a.ws = d->ws;
+  const int ktiles = (int)(d->K / KTILE);
+  a.ktiles_per_split = (ktiles + a.split_k - 1) / a.split_k;
+  a.offsets = nullptr; a.sorted_route = nullptr; a.x_div = 1; a.codes_stride = 0; a.scales_stride = 0;
+  return a;
+}
+
+int check_desc(const tnx_qlinear_desc* d) {
+  TNX_REQUIRE(d != nullptr, "qlinear: null descriptor");
+  TNX_REQUIRE(d->M > 0 && d->K > 0 && d->N > 0, "qlinear: M,K,N must be positive");
+  TNX_REQUIRE(d->K % KTILE == 0, "qlinear: K=%lld must be a multiple of 128", (long long)d->K);
+  TNX_REQUIRE(d->N % 16 == 0, "qlinear: N=%lld must be a multiple of 16", (long long)d->N);
+  TNX_REQUIRE(d->group >= 32 && d->group % 32 == 0 &&
+                  (d->group <= KTILE ? KTILE % d->group == 0 : d->group % KTILE == 0) &&
+                  d->K % d->group == 0,
+              "qlinear: unsupported group size %d for K=%lld", d->group, (long long)d->K);
+  TNX_REQUIRE(d->qtype == TNX_Q_INT4 || d->qtype == TNX_Q_NF4, "qlinear: bad qtype %d", d->qtype);
+  TNX_REQUIRE(d->x && d->codes && d->scales && d->y, "qlinear: null pointer");
+  TNX_REQUIRE(d->epilogue >= TNX_EPI_STORE && d->epilogue <= TNX_EPI_F32, "qlinear: bad epilogue");
+  if (d->epilogue == TNX_EPI_RESIDUAL) TNX_REQUIRE(d->residual, "qlinear: residual is null");
+  if (d->epilogue == TNX_EPI_SILU_MUL || d->epilogue == TNX_EPI_GELU_MUL)
+    TNX_REQUIRE(d->N % 32 == 0, "qlinear: *_MUL epilogue needs N %% 32 == 0");
+  if (d->lora_rank > 0) {
+    TNX_REQUIRE(d->lora_rank % 32 == 0, "qlinear: lora_rank %d must be a multiple of 32 (zero-pad)",
+                d->lora_rank);
+    TNX_REQUIRE(d->t && d->lora_b, "qlinear: LoRA pointers are null");
+    TNX_REQUIRE(d->lora_nseg == -1 || (d->lora_nseg >= 1 && d->lora_nseg <= 4),
+                "qlinear: lora_nseg must be -1 (interleaved pair) or 1..4");
+    TNX_REQUIRE(d->t_ld % 8 == 0, "qlinear: t_ld must be a multiple of 8");
+    for (int s = 0; s < d->lora_nseg; ++s)
+      TNX_REQUIRE(d->lora_seg_end[s] % 16 == 0 && d->lora_seg_toff[s] % 8 == 0,
+                  "qlinear: LoRA segment %d misaligned", s);
+  }
+  if (d->split_k > 1) TNX_REQUIRE(d->ws, "qlinear: split_k > 1 needs a workspace");
+  return TNX_OK;
+}
+
+template <class Kern>
+int raise_lds_limit(Kern kern, size_t bytes) {
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e != hipSuccess) {
+    tnx_set_error("cannot raise dynamic LDS limit: %s", hipGetErrorString(e));
+    return TNX_ELAUNCH;
+  }
+  return TNX_OK;
+}
+
+template <int MT, int NT>
+int launch_qlinear(hipStream_t st, const QLArgs& a) {
+  static std::once_flag once;
+  static int attr_rc = TNX_OK;
+  std::call_once(once, [] { attr_rc = raise_lds_limit(&qlinear_kernel<MT, NT>, tile_smem_bytes(MT)); });
+  if (attr_rc) return attr_rc;
+  dim3 grid((unsigned)cdiv(a.M, MT * 16), (unsigned)cdiv(a.N, 64 * NT), (unsigned)a.split_k);
+  hipLaunchKernelGGL((qlinear_kernel<MT, NT>), grid, dim3(256), tile_smem_bytes(MT), st, a);
+  TNX_CHECK_LAUNCH("qlinear");
+  return TNX_OK;
+}
+
+template <int MT, int NT>
+int launch_moe(hipStream_t st, const QLArgs& a, int E, int64_t max_rows) {
+  static std::once_flag once;
+  static int attr_rc = TNX_OK;
+  std::call_once(once, [] { attr_rc = raise_lds_limit(&moe_gmm_kernel<MT, NT>, tile_smem_bytes(MT)); });
+  if (attr_rc) return attr_rc;
+  dim3 grid((unsigned)E, (unsigned)cdiv(a.N, 64 * NT), (unsigned)cdiv(max_rows, MT * 16));
+  hipLaunchKernelGGL((moe_gmm_kernel<MT, NT>), grid, dim3(256), tile_smem_bytes(MT), st, a);
+  TNX_CHECK_LAUNCH("moe_gmm");
+  return TNX_OK;
+}
+
+}  // namespace
+
+extern "C" int tnx_qw_sizes(int64_t K, int64_t N, int group, size_t* codes_bytes,
+                            size_t* scales_bytes) {
+  TNX_REQUIRE(K > 0 && N > 0 && K % KTILE == 0 && N % 16 == 0,
+              "qw_sizes: K %% 128 and N %% 16 must be 0 (K=%lld N=%lld)", (long long)K, (long long)N);
+  TNX_REQUIRE(group >= 32 && group % 32 == 0 && K % group == 0 &&
+                  (group <= KTILE ? KTILE % group == 0 : group % KTILE == 0),
+              "qw_sizes: unsupported group %d", group);
+  const int spt = group >= KTILE ? 1 : KTILE / group;
+  if (codes_bytes) *codes_bytes = (size_t)(K * N / 2);
+  if (scales_bytes) *scales_bytes = (size_t)((N / 16) * (K / KTILE) * spt * 16 * 2);
+  return TNX_OK;
+}
+
+extern "C" int tnx_quantize_pack(void* stream, const void* w, int w_is_f32, int64_t K, int64_t N,
+                                 int group, int qtype, int interleave2, uint32_t* codes,
+                                 uint16_t* scales) {
+  int rc = tnx_qw_sizes(K, N, group, nullptr, nullptr);
+  if (rc) return rc;
+  TNX_REQUIRE(w && codes && scales, "quantize_pack: null pointer");
+  TNX_REQUIRE(qtype == TNX_Q_INT4 || qtype == TNX_Q_NF4, "quantize_pack: bad qtype %d", qtype);
+  if (interleave2) TNX_REQUIRE(N % 32 == 0, "quantize_pack: interleave2 needs N %% 32 == 0");
+  dim3 grid((unsigned)cdiv(N, 128), (unsigned)(K / group));
+  hipLaunchKernelGGL(quantize_pack_kernel, grid, dim3(128), 0, as_stream(stream), w, w_is_f32, K, N,
+                     group, qtype, interleave2, codes, scales);
+  TNX_CHECK_LAUNCH("quantize_pack");
+  return TNX_OK;
+}
+
+extern "C" int tnx_qw_dequant(void* stream, const uint32_t* codes, const uint16_t* scales,
+                              int64_t K, int64_t N, int group, int qtype, int interleave2,
+                              float* w_out) {
+  int rc = tnx_qw_sizes(K, N, group, nullptr, nullptr);
+  if (rc) return rc;
+  TNX_REQUIRE(codes && scales && w_out, "qw_dequant: null pointer");
+  dim3 grid((unsigned)cdiv(N, 128), (unsigned)K);
+  hipLaunchKernelGGL(qw_dequant_kernel, grid, dim3(128), 0, as_stream(stream), codes, scales, K, N,
+                     group, qtype, interleave2, w_out);
+  TNX_CHECK_LAUNCH("qw_dequant");
+  return TNX_OK;
+}
+
+extern "C" int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* d) {
+  int rc = check_desc(d);
+  if (rc) return rc;
+  const QLArgs a = to_args(d);
+  hipStream_t st = as_stream(stream);
+  if (a.M <= 16) return launch_qlinear<1, 2>(st, a);
+  if (a.M <= 32) return launch_qlinear<2, 2>(st, a);
+  if (a.M <= 64) return launch_qlinear<4, 2>(st, a);
+  return launch_qlinear<8, 2>(st, a);
+}
+
+extern "C" int tnx_splitk_finish(void* stream, const tnx_qlinear_desc* d) {
+  int rc = check_desc(d);
+  if (rc) return rc;
+  TNX_REQUIRE(d->ws, "splitk_finish: null workspace");
+  const QLArgs a = to_args(d);
+  const bool mul = a.epilogue == TNX_EPI_SILU_MUL || a.epilogue == TNX_EPI_GELU_MUL;
+  const int64_t n = a.M * (mul ? a.N / 2 : a.N);
+  hipLaunchKernelGGL(splitk_finish_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0,
+                     as_stream(stream), a);
+  TNX_CHECK_LAUNCH("splitk_finish");
+  return TNX_OK;
+}
+
+extern "C" int tnx_lora_down(void* stream, const uint16_t* x, int64_t M, int64_t K,
+                             const uint16_t* a_t, int R, uint16_t* t, int64_t t_ld) {
+  TNX_REQUIRE(x && a_t && t, "lora_down: null pointer");
+  TNX_REQUIRE(M > 0 && K > 0 && K % 32 == 0, "lora_down: K=%lld must be a multiple of 32", (long long)K);
+  TNX_REQUIRE(R > 0 && R % 16 == 0 && t_ld >= R, "lora_down: R=%d must be a multiple of 16 and <= t_ld", R);
+  dim3 grid((unsigned)cdiv(M, 16), (unsigned)(R / 16));
+  hipLaunchKernelGGL(lora_down_kernel, grid, dim3(512), 0, as_stream(stream), x, M, K, a_t, R, t, t_ld);
+  TNX_CHECK_LAUNCH("lora_down");
+  return TNX_OK;
+}
+
+extern "C" int tnx_moe_int4_gmm(void* stream, const tnx_moe_gmm_desc* d) {
+  TNX_REQUIRE(d, "moe_gmm: null descriptor");
+  TNX_REQUIRE(d->n_routes > 0 && d->E > 0 && d->k > 0, "moe_gmm: bad shape");
+  size_t cb = 0, sb = 0;
+  int rc = tnx_qw_sizes(d->K, d->N, d->group, &cb, &sb);
+  if (rc) return rc;
+  TNX_REQUIRE(d->x && d->codes && d->scales && d->offsets && d->sorted_route && d->y, "moe_gmm: null pointer");
+  TNX_REQUIRE(d->x_div >= 1, "moe_gmm: x_div must be >= 1");
+  TNX_REQUIRE(d->epilogue == TNX_EPI_STORE || d->epilogue == TNX_EPI_SILU_MUL, "moe_gmm: bad epilogue");
+  if (d->epilogue == TNX_EPI_SILU_MUL) TNX_REQUIRE(d->N % 32 == 0, "moe_gmm: SILU_MUL needs N %% 32 == 0");
+  QLArgs a;
+  memset(&a, 0, sizeof(a));
+  a.M = d->n_routes; a.K = d->K; a.N = d->N; a.group = d->group; a.qtype = d->qtype;
+  a.x = d->x; a.codes = d->codes; a.scales = d->scales; a.epilogue = d->epilogue; a.y = d->y;
+  a.split_k = 1; a.ktiles_per_split = (int)(d->K / KTILE);
+  a.offsets = d->offsets; a.sorted_route = d->sorted_route; a.x_div = d->x_div;
+  a.codes_stride = (int64_t)(cb / 4); a.scales_stride = (int64_t)(sb / 2);
+  // Any expert can receive up to all rows (one route per token and expert): the grid covers
+  // that bound and blocks past an expert's count exit at once.
+  const int64_t max_rows = d->n_routes / d->k;
+  hipStream_t st = as_stream(stream);
+  if (max_rows <= 16) return launch_moe<1, 2>(st, a, d->E, max_rows);
+  if (max_rows <= 32) return launch_moe<2, 2>(st, a, d->E, max_rows);
+  return launch_moe<4, 2>(st, a, d->E, max_rows);
+}

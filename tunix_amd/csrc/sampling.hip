@@ -1,0 +1,294 @@
+// Top-k / top-p sampling from materialised fp32 logits with the threefry2x32 bit stream of
+// jax.random (fold_in -> random_bits -> uniform -> gumbel -> argmax), one work-group per row.
+#include "common.h"
+
+namespace {
+
+constexpr int NTH = 1024;
+constexpr float kNegInf = -__builtin_inff();
+
+__device__ __forceinline__ uint32_t rotl(uint32_t x, int r) { return (x << r) | (x >> (32 - r)); }
+
+// Threefry-2x32, 20 rounds (Salmon et al. 2011), as used by jax.random's default PRNG.
+__device__ __forceinline__ void threefry2x32(uint32_t k0, uint32_t k1, uint32_t& x0, uint32_t& x1) {
+  const uint32_t ks[3] = {k0, k1, k0 ^ k1 ^ 0x1BD11BDAu};
+  const int rot[8] = {13, 15, 26, 6, 17, 29, 16, 24};
+  x0 += ks[0];
+  x1 += ks[1];
+#pragma unroll
+  for (int g = 0; g < 5; ++g) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      x0 += x1;
+      x1 = rotl(x1, rot[(g & 1) * 4 + r]);
+      x1 ^= x0;
+    }
+    x0 += ks[(g + 1) % 3];
+    x1 += ks[(g + 2) % 3] + (uint32_t)(g + 1);
+  }
+}
+
+// 32 random bits of element n of an array of `total` elements.
+//   variant 1: counters (0, n), output x0 ^ x1       (jax_threefry_partitionable = True)
+//   variant 0: the array of counters is split in two halves (first half -> x0, second -> x1)
+__device__ __forceinline__ uint32_t random_bits(uint32_t k0, uint32_t k1, uint64_t n, uint64_t total,
+                                                int variant) {
+  if (variant == 1) {
+    uint32_t x0 = (uint32_t)(n >> 32), x1 = (uint32_t)n;
+    threefry2x32(k0, k1, x0, x1);
+    return x0 ^ x1;
+  }
+  const uint64_t half = (total + 1) / 2;
+  const uint64_t i = n < half ? n : n - half;
+  uint32_t x0 = (uint32_t)i;
+  uint32_t x1 = (i + half < total) ? (uint32_t)(i + half) : 0u;
+  threefry2x32(k0, k1, x0, x1);
+  return n < half ? x0 : x1;
+}
+
+// jax.random.gumbel: -log(-log(uniform(minval=tiny, maxval=1)))
+__device__ __forceinline__ float gumbel_from_bits(uint32_t bits) {
+  const float tiny = 1.17549435e-38f;
+  float u = __uint_as_float((bits >> 9) | 0x3f800000u) - 1.0f;
+  u = fmaxf(tiny, u * (1.0f - tiny) + tiny);
+  return -logf(-logf(u));
+}
+
+__device__ __forceinline__ uint32_t order_key(float f) {
+  const uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+struct ArgMax {
+  float v;
+  int i;
+};
+__device__ __forceinline__ ArgMax better(ArgMax a, ArgMax b) {  // larger value, then lower index
+  return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a;
+}
+
+__device__ ArgMax block_argmax(ArgMax x, ArgMax* red) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    ArgMax y;
+    y.v = __shfl_xor(x.v, o, 64);
+    y.i = __shfl_xor(x.i, o, 64);
+    x = better(x, y);
+  }
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = x;
+  __syncthreads();
+  ArgMax r = red[0];
+  for (int w = 1; w < NTH / 64; ++w) r = better(r, red[w]);
+  __syncthreads();
+  return r;
+}
+
+__device__ float block_sum_f(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float s = 0.f;
+  for (int w = 0; w < NTH / 64; ++w) s += red[w];
+  __syncthreads();
+  return s;
+}
+
+__global__ __launch_bounds__(NTH) void sample_topk_kernel(const float* logits, int64_t V, int k,
+                                                          float top_p, uint32_t key0, uint32_t key1,
+                                                          int variant, const int32_t* step_ptr,
+                                                          int64_t M, int32_t* ids_out,
+                                                          float* logp_out) {
+  __shared__ uint32_t hist[256];
+  __shared__ float cval[NTH];
+  __shared__ int cidx[NTH];
+  __shared__ ArgMax red_am[NTH / 64];
+  __shared__ float red_f[NTH / 64];
+  __shared__ uint32_t s_sel, s_rem, s_cnt, s_base;
+  __shared__ uint32_t wave_cnt[NTH / 64];
+  const int tid = threadIdx.x;
+  const int64_t row = blockIdx.x;
+  const float* lr = logits + row * V;
+
+  // fold_in(key, step): threefry of the key over the counter pair (0, step)
+  uint32_t ks0 = 0u, ks1 = (uint32_t)(*step_ptr);
+  threefry2x32(key0, key1, ks0, ks1);
+
+  // ---- log-sum-exp of the row (for the log-probability of the drawn token) ----
+  ArgMax am;
+  am.v = kNegInf;
+  am.i = 0x7fffffff;
+  for (int64_t v = tid; v < V; v += NTH) {
+    ArgMax c;
+    c.v = lr[v];
+    c.i = (int)v;
+    am = better(am, c);
+  }
+  am = block_argmax(am, red_am);
+  float se = 0.f;
+  for (int64_t v = tid; v < V; v += NTH) se += expf(lr[v] - am.v);
+  se = block_sum_f(se, red_f);
+  const float lse = am.v + logf(se);
+
+  if (k <= 0) {
+    // categorical over the whole vocabulary: arg-max of logit + gumbel noise
+    ArgMax g;
+    g.v = kNegInf;
+    g.i = 0x7fffffff;
+    for (int64_t v = tid; v < V; v += NTH) {
+      ArgMax c;
+      c.v = lr[v] + gumbel_from_bits(random_bits(ks0, ks1, (uint64_t)(row * V + v), (uint64_t)(M * V), variant));
+      c.i = (int)v;
+      g = better(g, c);
+    }
+    g = block_argmax(g, red_am);
+    if (tid == 0) {
+      ids_out[row] = g.i;
+      if (logp_out) logp_out[row] = lr[g.i] - lse;
+    }
+    return;
+  }
+
+  // ---- radix select: key of the k-th largest logit ----
+  uint32_t prefix = 0, mask = 0;
+  if (tid == 0) s_rem = (uint32_t)k;
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    if (tid < 256) hist[tid] = 0;
+    __syncthreads();
+    for (int64_t v = tid; v < V; v += NTH) {
+      const uint32_t kk = order_key(lr[v]);
+      if ((kk & mask) == prefix) atomicAdd(&hist[(kk >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    if (tid == 0) {
+      uint32_t cum = 0, rem = s_rem;
+      int b = 255;
+      for (; b > 0; --b) {
+        if (cum + hist[b] >= rem) break;
+        cum += hist[b];
+      }
+      s_sel = (uint32_t)b;
+      s_rem = rem - cum;
+    }
+    __syncthreads();
+    prefix |= s_sel << shift;
+    mask |= 0xffu << shift;
+  }
+  const uint32_t thr = prefix;
+  const uint32_t r_eq = s_rem;  // how many elements equal to the threshold are taken
+  if (tid == 0) {
+    s_cnt = 0;
+    s_base = 0;
+  }
+  cval[tid] = kNegInf;
+  cidx[tid] = 0x7fffffff;
+  __syncthreads();
+  // elements above the threshold: any order (sorted below)
+  for (int64_t v = tid; v < V; v += NTH) {
+    const float x = lr[v];
+    if (order_key(x) > thr) {
+      const uint32_t p = atomicAdd(&s_cnt, 1u);
+      cval[p] = x;
+      cidx[p] = (int)v;
+    }
+  }
+  __syncthreads();
+  const uint32_t n_gt = s_cnt;
+  // elements equal to the threshold: the r_eq lowest indices, by an ordered block scan
+  for (int64_t v0 = 0; v0 < V; v0 += NTH) {
+    if (s_base >= r_eq) break;
+    const int64_t v = v0 + tid;
+    const bool eq = v < V && order_key(lr[v]) == thr;
+    const uint64_t bal = __ballot(eq);
+    const int lane = tid & 63, wave = tid >> 6;
+    const uint32_t before = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_cnt[wave] = (uint32_t)__popcll(bal);
+    __syncthreads();
+    uint32_t woff = 0, tot = 0;
+    for (int w = 0; w < NTH / 64; ++w) {
+      if (w < wave) woff += wave_cnt[w];
+      tot += wave_cnt[w];
+    }
+    const uint32_t pos = s_base + woff + before;
+    if (eq && pos < r_eq) {
+      cval[n_gt + pos] = lr[v];
+      cidx[n_gt + pos] = (int)v;
+    }
+    __syncthreads();
+    if (tid == 0) s_base += tot;
+    __syncthreads();
+  }
+  __syncthreads();
+  // ---- bitonic sort of the candidates: descending value, ascending index ----
+  for (int size = 2; size <= NTH; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      const int partner = tid ^ stride;
+      if (partner > tid) {
+        ArgMax a{cval[tid], cidx[tid]}, b{cval[partner], cidx[partner]};
+        const bool a_first = (a.v > b.v) || (a.v == b.v && a.i < b.i);
+        const bool up = (tid & size) == 0;  // this pair sorts "best first" when up
+        if (up != a_first) {
+          cval[tid] = b.v; cidx[tid] = b.i;
+          cval[partner] = a.v; cidx[partner] = a.i;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  // ---- softmax over the k sorted logits, top-p cut, gumbel arg-max ----
+  const float mx = cval[0];
+  float e = tid < k ? expf(cval[tid] - mx) : 0.f;
+  const float tot = block_sum_f(e, red_f);
+  __shared__ float prob[NTH];
+  prob[tid] = e / tot;
+  __syncthreads();
+  __shared__ float excl[NTH];
+  if (tid == 0) {
+    float c = 0.f;
+    for (int j = 0; j < k; ++j) {
+      c += prob[j];
+      excl[j] = c - prob[j];  // cumsum - p, as in the reference
+    }
+  }
+  __syncthreads();
+  ArgMax g;
+  g.v = kNegInf;
+  g.i = 0x7fffffff;
+  if (tid < k) {
+    const float lg = excl[tid] > top_p ? kNegInf : cval[tid];
+    g.v = lg + gumbel_from_bits(random_bits(ks0, ks1, (uint64_t)(row * k + tid), (uint64_t)(M * k), variant));
+    g.i = tid;
+  }
+  g = block_argmax(g, red_am);
+  if (tid == 0) {
+    const int tokid = cidx[g.i];
+    ids_out[row] = tokid;
+    if (logp_out) logp_out[row] = lr[tokid] - lse;
+  }
+}
+
+}  // namespace
+
+extern "C" int tnx_sample_topk(void* stream, const float* logits, int64_t M, int64_t V, int k,
+                               float top_p, uint32_t key0, uint32_t key1, int rng_variant,
+                               const int32_t* step_ptr, float* ws, int32_t* ids_out,
+                               float* logp_out) {
+  (void)ws;
+  TNX_REQUIRE(logits && step_ptr && ids_out, "sample_topk: null pointer");
+  TNX_REQUIRE(M > 0 && V > 0 && V < (1ll << 31), "sample_topk: bad shape");
+  TNX_REQUIRE(rng_variant == 0 || rng_variant == 1, "sample_topk: rng_variant must be 0 or 1");
+  if (k <= 0 || k >= V) {
+    if (top_p < 1.0f) {
+      tnx_set_error("sample_topk: top_p < 1 without top_k needs a full-vocabulary sort (not built)");
+      return TNX_ENOSYS;
+    }
+    k = 0;
+  }
+  TNX_REQUIRE(k <= NTH, "sample_topk: top_k=%d exceeds %d", k, NTH);
+  hipLaunchKernelGGL(sample_topk_kernel, dim3((unsigned)M), dim3(NTH), 0, as_stream(stream), logits,
+                     V, k, top_p, key0, key1, rng_variant, step_ptr, M, ids_out, logp_out);
+  TNX_CHECK_LAUNCH("sample_topk");
+  return TNX_OK;
+}

@@ -1,0 +1,401 @@
+"""Device-resident QLoRA decoder: packed int4/NF4 weights + separate LoRA tensors, and the
+kernel sequence of one forward pass over T tokens per row (T = 1: a decode step).
+
+Mirrors the layer structure of tunix/models/llama3/model.py:546-564, qwen3/model.py:1161-1182
+(+ MoELayer :787-832) and gemma3/model.py:875-898; every arithmetic step is a libtunix_hip.so
+kernel.  LoRA A/B stay separate buffers so that `update_lora` can swap them between rollouts
+(tunix/generate/sampler.py:333-352, tunix/rl/rollout/vanilla_rollout.py:92-121).
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+
+from . import _lib as L
+from . import ops
+from .config import ModelConfig
+
+_NORM = {"llama3": L.TNX_NORM_LLAMA, "qwen3": L.TNX_NORM_QWEN3, "gemma3": L.TNX_NORM_GEMMA3}
+_ROPE = {"llama3": L.TNX_ROPE_LLAMA, "qwen3": L.TNX_ROPE_QWEN3, "gemma3": L.TNX_ROPE_GEMMA3}
+
+
+def _pad32(r: int) -> int:
+  return (r + 31) // 32 * 32 if r > 0 else 0
+
+
+def rope_timescale(head_dim: int, theta: float) -> np.ndarray:
+  """theta ** (2i / head_dim) in fp32, as apply_rope computes it (llama3/model.py:256-257)."""
+  fraction = (np.float32(2.0) * np.arange(0, head_dim // 2, dtype=np.float32)
+              / np.float32(head_dim)).astype(np.float32)
+  return np.power(np.float32(theta), fraction).astype(np.float32)
+
+
+class FusedLinear:
+  """One quantised projection (possibly several reference linears sharing an input) with its
+  LoRA tensors in kernel layout."""
+
+  def __init__(self, cfg: ModelConfig, weights: dict, names: list[str], device,
+               interleave2: bool = False):
+    ws = [weights[n].to(device=device, dtype=torch.bfloat16) for n in names]
+    self.names = names
+    self.K = ws[0].shape[0]
+    self.widths = [w.shape[1] for w in ws]
+    self.N = sum(self.widths)
+    self.interleave2 = interleave2
+    self.group, self.qtype = cfg.group, cfg.qtype
+    w = torch.cat(ws, dim=1).contiguous() if len(ws) > 1 else ws[0].contiguous()
+    self.codes, self.scales = ops.quantize_pack(w, cfg.group, cfg.qtype, interleave2)
+    del w
+    r = cfg.lora_rank
+    self.has_lora = any((n + ".lora_a") in weights for n in names)
+    self.rp = _pad32(r) if self.has_lora else 0
+    self.r = r
+    self.lora_scale = float(cfg.lora_alpha) / float(r) if self.has_lora else 0.0
+    self.seg_end, self.seg_toff = [], []
+    off = 0
+    for i, wd in enumerate(self.widths):
+      off += wd
+      self.seg_end.append(off)
+      self.seg_toff.append(i * self.rp)
+    if self.has_lora:
+      self.a_t = torch.zeros(len(names) * self.rp, self.K, dtype=torch.bfloat16, device=device)
+      self.b_t = torch.zeros(self.N, self.rp, dtype=torch.bfloat16, device=device)
+      self._row_perm = None
+      if interleave2:
+        c = torch.arange(self.N, device=device)
+        half = self.N // 2
+        h, cc = c // half, c % half
+        self._row_perm = (cc // 16) * 32 + h * 16 + (cc % 16)
+      self.load_lora(weights)
+
+  def load_lora(self, weights: dict):
+    """Copies lora_a [K,r] / lora_b [r,N_i] of every member into the kernel layout."""
+    if not self.has_lora:
+      return
+    b_full = torch.zeros(self.N, self.rp, dtype=torch.bfloat16, device=self.b_t.device)
+    off = 0
+    for i, (n, wd) in enumerate(zip(self.names, self.widths)):
+      a = weights.get(n + ".lora_a")
+      if a is not None:
+        b = weights[n + ".lora_b"]
+        if tuple(a.shape) != (self.K, self.r) or tuple(b.shape) != (self.r, wd):
+          raise ValueError(
+              f"New state must have the same shape as the old state: {n} lora_a {tuple(a.shape)}"
+              f" lora_b {tuple(b.shape)} vs {(self.K, self.r)} / {(self.r, wd)}")
+        self.a_t[i * self.rp: i * self.rp + self.r].copy_(a.to(self.a_t.device, torch.bfloat16).t())
+        b_full[off: off + wd, : self.r].copy_(b.to(self.b_t.device, torch.bfloat16).t())
+      off += wd
+    if self._row_perm is not None:
+      self.b_t[self._row_perm] = b_full
+    else:
+      self.b_t.copy_(b_full)
+
+  @property
+  def t_cols(self) -> int:
+    return len(self.names) * self.rp
+
+
+class ExpertBank:
+  """Per-expert QW weights of one MoE layer: fused gate|up (interleaved) and down."""
+
+  def __init__(self, cfg: ModelConfig, weights: dict, prefix: str, device):
+    g, u, d = weights[prefix + "e_gate"], weights[prefix + "e_up"], weights[prefix + "e_down"]
+    E = g.shape[0]
+    self.E, self.D, self.F = E, g.shape[1], g.shape[2]
+    cb, sb = ops.qw_sizes(self.D, 2 * self.F, cfg.group)
+    self.gu_codes = torch.empty(E * cb // 4, dtype=torch.int32, device=device)
+    self.gu_scales = torch.empty(E * sb // 2, dtype=torch.bfloat16, device=device)
+    cb2, sb2 = ops.qw_sizes(self.F, self.D, cfg.group)
+    self.dn_codes = torch.empty(E * cb2 // 4, dtype=torch.int32, device=device)
+    self.dn_scales = torch.empty(E * sb2 // 2, dtype=torch.bfloat16, device=device)
+    for e in range(E):
+      w = torch.cat([g[e], u[e]], dim=1).to(device, torch.bfloat16).contiguous()
+      c, s = ops.quantize_pack(w, cfg.group, cfg.qtype, True)
+      self.gu_codes[e * cb // 4:(e + 1) * cb // 4].copy_(c)
+      self.gu_scales[e * sb // 2:(e + 1) * sb // 2].copy_(s)
+      c, s = ops.quantize_pack(d[e].to(device, torch.bfloat16).contiguous(), cfg.group, cfg.qtype)
+      self.dn_codes[e * cb2 // 4:(e + 1) * cb2 // 4].copy_(c)
+      self.dn_scales[e * sb2 // 2:(e + 1) * sb2 // 2].copy_(s)
+    self.router_t = weights[prefix + "router"].to(device, torch.bfloat16).t().contiguous()
+
+
+class QLoRAModel:
+  """Packed weights of one model on one GPU."""
+
+  def __init__(self, cfg: ModelConfig, weights: dict, device="cuda"):
+    L.lib()  # fail loudly when the HIP library is missing
+    self.cfg = cfg
+    self.device = torch.device(device)
+    dev = self.device
+    bf = torch.bfloat16
+    self.embed = weights["embed"].to(dev, bf).contiguous()
+    self.final_norm = weights["final_norm"].to(dev, bf).contiguous()
+    self.head = None
+    self.head_w = None
+    if not cfg.tied_embedding:
+      if cfg.quantize_head:
+        self.head = FusedLinear(cfg, weights, ["lm_head"], dev)
+      else:
+        self.head_w = weights["lm_head"].to(dev, bf).t().contiguous()  # [V, D]
+    self.layers = []
+    for i in range(cfg.num_layers):
+      p = f"l{i}."
+      ly = {}
+      ly["attn_norm"] = weights[p + "attn_norm"].to(dev, bf).contiguous()
+      ly["mlp_norm"] = weights[p + "mlp_norm"].to(dev, bf).contiguous()
+      for extra in ("q_norm", "k_norm", "post_attn_norm", "post_ffw_norm"):
+        if p + extra in weights:
+          ly[extra] = weights[p + extra].to(dev, bf).contiguous()
+      ly["qkv"] = FusedLinear(cfg, weights, [p + "wq", p + "wk", p + "wv"], dev)
+      ly["o"] = FusedLinear(cfg, weights, [p + "wo"], dev)
+      if cfg.num_experts:
+        ly["experts"] = ExpertBank(cfg, weights, p, dev)
+      else:
+        ly["gu"] = FusedLinear(cfg, weights, [p + "w_gate", p + "w_up"], dev, interleave2=True)
+        ly["down"] = FusedLinear(cfg, weights, [p + "w_down"], dev)
+      theta, sf = cfg.rope_params(i)
+      ly["timescale"] = torch.from_numpy(rope_timescale(cfg.head_dim, theta)).to(dev)
+      ly["rope_scale"] = sf
+      self.layers.append(ly)
+    torch.cuda.synchronize(dev)
+
+  # weight sync: LoRA-only replacement (tunix/generate/sampler.py:333-352)
+  def update_lora(self, new_lora: dict):
+    expected = set()
+    for n in self.cfg.lora_names():
+      expected.add(n + ".lora_a")
+      expected.add(n + ".lora_b")
+    if set(new_lora) != expected:
+      raise ValueError(
+          "New state must have the same structure as the old state. "
+          f"missing={sorted(expected - set(new_lora))} extra={sorted(set(new_lora) - expected)}")
+    for ly in self.layers:
+      for key in ("qkv", "o", "gu", "down"):
+        if key in ly:
+          ly[key].load_lora(new_lora)
+    if self.head is not None:
+      self.head.load_lora(new_lora)
+    torch.cuda.synchronize(self.device)
+
+  def weight_bytes(self) -> dict:
+    """Bytes one decode step reads: codes+scales, LoRA, head (algorithmic traffic)."""
+    q = lora = 0
+    for ly in self.layers:
+      for key in ("qkv", "o", "gu", "down"):
+        if key in ly:
+          f = ly[key]
+          q += f.codes.numel() * 4 + f.scales.numel() * 2
+          if f.has_lora:
+            lora += (f.K * f.r * len(f.names) + f.N * f.r) * 2
+      if "experts" in ly:
+        ex = ly["experts"]
+        q += (ex.gu_codes.numel() + ex.dn_codes.numel()) * 4
+        q += (ex.gu_scales.numel() + ex.dn_scales.numel()) * 2
+    if self.head_w is not None:
+      head = self.head_w.numel() * 2
+    elif self.head is not None:
+      head = self.head.codes.numel() * 4 + self.head.scales.numel() * 2
+    else:
+      head = self.embed.numel() * 2
+    return {"quantized": q, "lora": lora, "head": head}
+
+
+class Runner:
+  """Workspaces + the kernel sequence for up to `max_rows` = B*T token rows.
+
+  State tensors (token buffer, positions, KV cache, step counter) are owned by the caller and
+  bound with `bind`; all kernels read the step / column from device memory so that a decode step
+  can be captured once into a HIP graph and replayed.
+  """
+
+  def __init__(self, model: QLoRAModel, B: int, T: int, S: int, pad_id: int, kv_chunk=None,
+               want_logits: bool = False):
+    cfg = model.cfg
+    self.model, self.cfg, self.B, self.T, self.S = model, cfg, B, T, S
+    self.pad_id = int(pad_id)
+    dev = model.device
+    M = B * T
+    self.M = M
+    bf = torch.bfloat16
+    D, F = cfg.embed_dim, cfg.hidden_dim
+    nqkv = cfg.q_dim + 2 * cfg.kv_dim
+    rp = _pad32(cfg.lora_rank)
+    self.h = torch.empty(M, D, dtype=bf, device=dev)
+    self.xn = torch.empty(M, D, dtype=bf, device=dev)
+    self.tmp = torch.empty(M, D, dtype=bf, device=dev)
+    self.qkv = torch.empty(M, nqkv, dtype=bf, device=dev)
+    self.q = torch.empty(M, cfg.q_dim, dtype=bf, device=dev)
+    self.attn = torch.empty(M, cfg.q_dim, dtype=bf, device=dev)
+    self.t = torch.zeros(M, max(3 * rp, 32), dtype=bf, device=dev)
+    if cfg.num_experts:
+      k = cfg.num_experts_per_tok
+      self.scores = torch.empty(M, cfg.num_experts, dtype=bf, device=dev)
+      self.topk_w = torch.empty(M, k, dtype=bf, device=dev)
+      self.topk_id = torch.empty(M, k, dtype=torch.int32, device=dev)
+      self.counts = torch.empty(cfg.num_experts, dtype=torch.int32, device=dev)
+      self.offsets = torch.empty(cfg.num_experts + 1, dtype=torch.int32, device=dev)
+      self.sorted_route = torch.empty(M * k, dtype=torch.int32, device=dev)
+      self.act = torch.empty(M * k, F, dtype=bf, device=dev)
+      self.y_route = torch.empty(M * k, D, dtype=bf, device=dev)
+    else:
+      self.act = torch.empty(M, F, dtype=bf, device=dev)
+    nmax = max(nqkv, D, 2 * F if not cfg.num_experts else D)
+    self.splitk_ws = torch.zeros(M * nmax, dtype=torch.float32, device=dev)
+    if kv_chunk is None:
+      kv_chunk = 256 if (T == 1 and S > 256) else 0
+    self.kv_chunk = kv_chunk
+    nb = ops.attn_ws_bytes(B, T, S, cfg.num_heads, cfg.head_dim, kv_chunk)
+    self.attn_ws = torch.empty(max(nb // 4, 1), dtype=torch.float32, device=dev)
+    self.zero = torch.zeros(1, dtype=torch.int32, device=dev)
+    # head
+    self.nvb = ops.lmhead_nblocks(cfg.vocab_size)
+    self.head_rows = B
+    self.xlast = torch.empty(B, D, dtype=bf, device=dev)
+    self.part = torch.empty(B * self.nvb * 4, dtype=torch.float32, device=dev)
+    self.best_id = torch.empty(B, dtype=torch.int32, device=dev)
+    self.best_logp = torch.empty(B, dtype=torch.float32, device=dev)
+    self.logits = (torch.empty(B, cfg.vocab_size, dtype=torch.float32, device=dev)
+                   if want_logits else None)
+    self.split_k_override = {}
+
+  # ---- building blocks -----------------------------------------------------------------------
+  def _split_k(self, f: FusedLinear, M: int) -> int:
+    if f.names[0] in self.split_k_override:
+      return self.split_k_override[f.names[0]]
+    key = f.names[0].split(".")[-1]
+    if key in self.split_k_override:
+      return self.split_k_override[key]
+    blocks = math.ceil(f.N / 128) * math.ceil(M / 128)
+    ktiles = f.K // 128
+    if blocks >= 200 or M > 128:
+      return 1
+    return int(max(1, min(8, ktiles, 256 // blocks)))
+
+  def linear(self, f: FusedLinear, x, y, M, epilogue=L.TNX_EPI_STORE, residual=None):
+    if f.has_lora:
+      ops.lora_down(x, f.a_t, self.t, M=M)
+    split = self._split_k(f, M)
+    d = ops.make_qlinear_desc(
+        M=M, K=f.K, N=f.N, group=f.group, qtype=f.qtype, x=x, codes=f.codes, scales=f.scales, y=y,
+        epilogue=epilogue, residual=residual, lora_rank=f.rp,
+        lora_nseg=(-1 if f.interleave2 else len(f.names)), lora_seg_end=f.seg_end,
+        lora_seg_toff=f.seg_toff, t=self.t if f.has_lora else None, t_ld=self.t.shape[1],
+        lora_b=f.b_t if f.has_lora else None, lora_scale=f.lora_scale, split_k=split,
+        ws=self.splitk_ws if split > 1 else None)
+    ops.qlinear(d)
+
+  def forward_hidden(self, tokens, positions, col_ptr, kcache, vcache, B=None, T=None):
+    """Runs all layers for tokens[b, col .. col+T) of each row; leaves the final-normed hidden
+    state in self.xn[:B*T].  kcache/vcache: lists of [B,Hkv,S,dh] tensors."""
+    cfg, m = self.cfg, self.model
+    B = self.B if B is None else B
+    T = self.T if T is None else T
+    M = B * T
+    flavor = _NORM[cfg.family]
+    emb_scale = math.sqrt(cfg.embed_dim) if cfg.family == "gemma3" else 1.0
+    ops.embed(m.embed, tokens, col_ptr, B, T, emb_scale, self.h)
+    for i, ly in enumerate(m.layers):
+      ops.rmsnorm(self.h, ly["attn_norm"], self.xn, cfg.norm_eps, flavor, M=M)
+      self.linear(ly["qkv"], self.xn, self.qkv, M)
+      rd = L.RopeDesc()
+      rd.B, rd.T, rd.S = B, T, self.S
+      rd.Hq, rd.Hkv, rd.dh = cfg.num_heads, cfg.num_kv_heads, cfg.head_dim
+      rd.rope_flavor, rd.rope_scale = _ROPE[cfg.family], ly["rope_scale"]
+      rd.timescale = ly["timescale"].data_ptr()
+      if "q_norm" in ly:
+        rd.qk_norm = flavor
+        rd.norm_eps = cfg.norm_eps if cfg.family == "qwen3" else 1e-6
+        rd.q_norm_w, rd.k_norm_w = ly["q_norm"].data_ptr(), ly["k_norm"].data_ptr()
+      else:
+        rd.qk_norm = -1
+      rd.q_prescale = cfg.query_pre_attn_scalar if cfg.family == "gemma3" else 0.0
+      rd.qkv, rd.positions, rd.pos_ld = self.qkv.data_ptr(), positions.data_ptr(), positions.shape[1]
+      rd.col_ptr = col_ptr.data_ptr()
+      rd.q_out, rd.kcache, rd.vcache = self.q.data_ptr(), kcache[i].data_ptr(), vcache[i].data_ptr()
+      ops.rope_kvwrite(rd)
+      ad = L.AttnDesc()
+      ad.B, ad.T, ad.S = B, T, self.S
+      ad.Hq, ad.Hkv, ad.dh = cfg.num_heads, cfg.num_kv_heads, cfg.head_dim
+      ad.scale = 0.0 if cfg.family == "gemma3" else cfg.head_dim ** -0.5
+      ad.window = cfg.sliding_window if cfg.is_local_layer(i) else 0
+      ad.pad_id = self.pad_id
+      ad.q, ad.kcache, ad.vcache = self.q.data_ptr(), kcache[i].data_ptr(), vcache[i].data_ptr()
+      ad.tokens, ad.tok_ld, ad.col_ptr = tokens.data_ptr(), tokens.shape[1], col_ptr.data_ptr()
+      ad.kv_chunk = self.kv_chunk if T == 1 else 0
+      ad.ws, ad.out = self.attn_ws.data_ptr(), self.attn.data_ptr()
+      ops.gqa_attn(ad)
+      if cfg.family == "gemma3":
+        self.linear(ly["o"], self.attn, self.tmp, M)
+        ops.rmsnorm(self.tmp, ly["post_attn_norm"], self.h, cfg.norm_eps, flavor, M=M,
+                    res_post=self.h)
+      else:
+        self.linear(ly["o"], self.attn, self.h, M, epilogue=L.TNX_EPI_RESIDUAL, residual=self.h)
+      ops.rmsnorm(self.h, ly["mlp_norm"], self.xn, cfg.norm_eps, flavor, M=M)
+      if cfg.num_experts:
+        self._moe(ly["experts"], M)
+      elif cfg.family == "gemma3":
+        self.linear(ly["gu"], self.xn, self.act, M, epilogue=L.TNX_EPI_GELU_MUL)
+        self.linear(ly["down"], self.act, self.tmp, M)
+        ops.rmsnorm(self.tmp, ly["post_ffw_norm"], self.h, cfg.norm_eps, flavor, M=M,
+                    res_post=self.h)
+      else:
+        self.linear(ly["gu"], self.xn, self.act, M, epilogue=L.TNX_EPI_SILU_MUL)
+        self.linear(ly["down"], self.act, self.h, M, epilogue=L.TNX_EPI_RESIDUAL, residual=self.h)
+    ops.rmsnorm(self.h, m.final_norm, self.xn, cfg.norm_eps, flavor, M=M)
+    return self.xn
+
+  def _moe(self, ex: ExpertBank, M: int):
+    cfg = self.cfg
+    k, E = cfg.num_experts_per_tok, cfg.num_experts
+    ops.lora_down(self.xn, ex.router_t, self.scores, M=M)          # dense bf16 router
+    ops.moe_route_topk(self.scores[:M], k, self.topk_w, self.topk_id)
+    ops.moe_sort_routes(self.topk_id[:M], E, self.counts, self.offsets, self.sorted_route)
+    d = L.MoeGmmDesc()
+    d.n_routes, d.E, d.k, d.K, d.N = M * k, E, k, ex.D, 2 * ex.F
+    d.group, d.qtype = cfg.group, cfg.qtype
+    d.x, d.x_div = self.xn.data_ptr(), k
+    d.codes, d.scales = ex.gu_codes.data_ptr(), ex.gu_scales.data_ptr()
+    d.offsets, d.sorted_route = self.offsets.data_ptr(), self.sorted_route.data_ptr()
+    d.epilogue, d.y = L.TNX_EPI_SILU_MUL, self.act.data_ptr()
+    ops.moe_gmm(d)
+    d2 = L.MoeGmmDesc()
+    d2.n_routes, d2.E, d2.k, d2.K, d2.N = M * k, E, k, ex.F, ex.D
+    d2.group, d2.qtype = cfg.group, cfg.qtype
+    d2.x, d2.x_div = self.act.data_ptr(), 1
+    d2.codes, d2.scales = ex.dn_codes.data_ptr(), ex.dn_scales.data_ptr()
+    d2.offsets, d2.sorted_route = self.offsets.data_ptr(), self.sorted_route.data_ptr()
+    d2.epilogue, d2.y = L.TNX_EPI_STORE, self.y_route.data_ptr()
+    ops.moe_gmm(d2)
+    ops.moe_combine(self.y_route, self.topk_w, M, k, cfg.embed_dim, self.h, self.h)
+
+  def head_desc(self, x, rows, part, temperature=1.0, targets=None, best_id=None, best_logp=None,
+                target_logp=None, lse=None, logits_out=None, forbidden=None) -> L.LmHeadDesc:
+    cfg, m = self.cfg, self.model
+    d = L.LmHeadDesc()
+    d.M, d.D, d.V = rows, cfg.embed_dim, cfg.vocab_size
+    d.x = x.data_ptr()
+    if m.head is not None:
+      f = m.head
+      d.codes, d.scales, d.group, d.qtype = f.codes.data_ptr(), f.scales.data_ptr(), f.group, f.qtype
+      if f.has_lora:
+        d.lora_rank, d.t, d.t_ld = f.rp, self.t.data_ptr(), self.t.shape[1]
+        d.lora_b, d.lora_scale = f.b_t.data_ptr(), f.lora_scale
+    else:
+      d.w_bf16 = (m.head_w if m.head_w is not None else m.embed).data_ptr()
+    d.temperature = float(temperature)
+    if forbidden is not None:
+      d.forbidden, d.n_forbidden = forbidden.data_ptr(), forbidden.numel()
+    for name, tns in (("targets", targets), ("best_id", best_id), ("best_logp", best_logp),
+                      ("target_logp", target_logp), ("lse", lse), ("logits_out", logits_out)):
+      if tns is not None:
+        setattr(d, name, tns.data_ptr())
+    d.part = part.data_ptr()
+    return d
+
+  def run_head(self, x, rows, **kw):
+    m = self.model
+    if m.head is not None and m.head.has_lora:
+      ops.lora_down(x, m.head.a_t, self.t, M=rows)
+    ops.lmhead(self.head_desc(x, rows, self.part, **kw))

@@ -1,0 +1,172 @@
+"""Thin Python wrappers over the C ABI: torch tensors in, kernels launched on torch's current
+stream.  torch is used for device memory and streams only; every computation below happens in
+libtunix_hip.so.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib as L
+
+
+def _stream() -> int:
+  return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+  if t is None:
+    return None
+  if not t.is_cuda:
+    raise ValueError("expected a tensor on the GPU")
+  if not t.is_contiguous():
+    raise ValueError("expected a contiguous tensor")
+  return t.data_ptr()
+
+
+def _expect(t: torch.Tensor, dtype, what: str):
+  if t.dtype != dtype:
+    raise ValueError(f"{what}: expected {dtype}, got {t.dtype}")
+
+
+def qw_sizes(K: int, N: int, group: int) -> tuple[int, int]:
+  cb, sb = C.c_size_t(0), C.c_size_t(0)
+  L.check(L.lib().tnx_qw_sizes(K, N, group, C.byref(cb), C.byref(sb)), "tnx_qw_sizes")
+  return cb.value, sb.value
+
+
+def quantize_pack(w: torch.Tensor, group: int, qtype: int, interleave2: bool = False):
+  """w [K,N] bf16 or fp32 on the GPU -> (codes int32 [K*N/8], scales bf16 [...])."""
+  K, N = w.shape
+  cb, sb = qw_sizes(K, N, group)
+  codes = torch.empty(cb // 4, dtype=torch.int32, device=w.device)
+  scales = torch.empty(sb // 2, dtype=torch.bfloat16, device=w.device)
+  is_f32 = 1 if w.dtype == torch.float32 else 0
+  if not is_f32:
+    _expect(w, torch.bfloat16, "quantize_pack")
+  L.check(L.lib().tnx_quantize_pack(_stream(), _ptr(w), is_f32, K, N, group, qtype,
+                                    1 if interleave2 else 0, _ptr(codes), _ptr(scales)),
+          "tnx_quantize_pack")
+  return codes, scales
+
+
+def qw_dequant(codes, scales, K, N, group, qtype, interleave2=False) -> torch.Tensor:
+  out = torch.empty(K, N, dtype=torch.float32, device=codes.device)
+  L.check(L.lib().tnx_qw_dequant(_stream(), _ptr(codes), _ptr(scales), K, N, group, qtype,
+                                 1 if interleave2 else 0, _ptr(out)), "tnx_qw_dequant")
+  return out
+
+
+def make_qlinear_desc(*, M, K, N, group, qtype, x, codes, scales, y, epilogue=L.TNX_EPI_STORE,
+                      residual=None, lora_rank=0, lora_nseg=1, lora_seg_end=(), lora_seg_toff=(),
+                      t=None, t_ld=0, lora_b=None, lora_scale=0.0, split_k=1, ws=None):
+  d = L.QLinearDesc()
+  d.M, d.K, d.N, d.group, d.qtype = M, K, N, group, qtype
+  d.x, d.codes, d.scales, d.y = _ptr(x), _ptr(codes), _ptr(scales), _ptr(y)
+  d.epilogue, d.residual = epilogue, _ptr(residual)
+  d.lora_rank, d.lora_nseg = lora_rank, lora_nseg
+  for i, v in enumerate(lora_seg_end):
+    d.lora_seg_end[i] = v
+  for i, v in enumerate(lora_seg_toff):
+    d.lora_seg_toff[i] = v
+  d.t, d.t_ld, d.lora_b, d.lora_scale = _ptr(t), t_ld, _ptr(lora_b), lora_scale
+  d.split_k, d.ws = split_k, _ptr(ws)
+  return d
+
+
+def qlinear(desc: L.QLinearDesc):
+  L.check(L.lib().tnx_qlinear_lora(_stream(), C.byref(desc)), "tnx_qlinear_lora")
+  if desc.split_k > 1:
+    L.check(L.lib().tnx_splitk_finish(_stream(), C.byref(desc)), "tnx_splitk_finish")
+
+
+def lora_down(x, a_t, t, M=None):
+  """t[M, :R] = bf16(x @ a_t.T); x [M,K], a_t [R,K], t [M, t_ld]."""
+  M = x.shape[0] if M is None else M
+  K = x.shape[1]
+  R = a_t.shape[0]
+  L.check(L.lib().tnx_lora_down(_stream(), _ptr(x), M, K, _ptr(a_t), R, _ptr(t), t.shape[1]),
+          "tnx_lora_down")
+
+
+def embed(table, ids, col_ptr, B, T, scale, out):
+  V, D = table.shape
+  L.check(L.lib().tnx_embed(_stream(), _ptr(table), V, D, _ptr(ids), ids.shape[1], _ptr(col_ptr),
+                            B, T, float(scale), _ptr(out)), "tnx_embed")
+
+
+def rmsnorm(x, w, y, eps, flavor, M=None, res_pre=None, h_out=None, res_post=None):
+  M = x.shape[0] if M is None else M
+  D = x.shape[1]
+  L.check(L.lib().tnx_rmsnorm(_stream(), _ptr(x), _ptr(res_pre), _ptr(h_out), _ptr(w),
+                              _ptr(res_post), _ptr(y), M, D, float(eps), flavor), "tnx_rmsnorm")
+
+
+def rope_kvwrite(desc: L.RopeDesc):
+  L.check(L.lib().tnx_qknorm_rope_kvwrite(_stream(), C.byref(desc)), "tnx_qknorm_rope_kvwrite")
+
+
+def attn_ws_bytes(B, T, S, Hq, dh, kv_chunk) -> int:
+  return int(L.lib().tnx_attn_ws_bytes(B, T, S, Hq, dh, kv_chunk))
+
+
+def gqa_attn(desc: L.AttnDesc):
+  L.check(L.lib().tnx_gqa_attn(_stream(), C.byref(desc)), "tnx_gqa_attn")
+
+
+def lmhead_nblocks(V: int) -> int:
+  return int(L.lib().tnx_lmhead_nblocks(V))
+
+
+def lmhead(desc: L.LmHeadDesc):
+  L.check(L.lib().tnx_lmhead_logp(_stream(), C.byref(desc)), "tnx_lmhead_logp")
+
+
+def sample_topk(logits, k, top_p, key, rng_variant, step_ptr, ws, ids_out, logp_out):
+  M, V = logits.shape
+  L.check(L.lib().tnx_sample_topk(_stream(), _ptr(logits), M, V, k, float(top_p), key[0], key[1],
+                                  rng_variant, _ptr(step_ptr), _ptr(ws), _ptr(ids_out),
+                                  _ptr(logp_out)), "tnx_sample_topk")
+
+
+def sample_commit(ids, logp, tokens, logprobs, done, eos, step_ptr):
+  B = ids.shape[0]
+  L.check(L.lib().tnx_sample_commit(_stream(), _ptr(ids), _ptr(logp), B, _ptr(tokens),
+                                    tokens.shape[1], _ptr(logprobs), _ptr(done), _ptr(eos),
+                                    0 if eos is None else eos.numel(), _ptr(step_ptr)),
+          "tnx_sample_commit")
+
+
+def moe_route_topk(scores, k, topk_w, topk_id):
+  M, E = scores.shape
+  L.check(L.lib().tnx_moe_route_topk(_stream(), _ptr(scores), M, E, k, _ptr(topk_w),
+                                     _ptr(topk_id)), "tnx_moe_route_topk")
+
+
+def moe_sort_routes(topk_id, E, counts, offsets, sorted_route):
+  M, k = topk_id.shape
+  L.check(L.lib().tnx_moe_sort_routes(_stream(), _ptr(topk_id), M, k, E, _ptr(counts),
+                                      _ptr(offsets), _ptr(sorted_route)), "tnx_moe_sort_routes")
+
+
+def moe_gmm(desc: L.MoeGmmDesc):
+  L.check(L.lib().tnx_moe_int4_gmm(_stream(), C.byref(desc)), "tnx_moe_int4_gmm")
+
+
+def moe_combine(y, topk_w, M, k, D, residual, out):
+  L.check(L.lib().tnx_moe_combine(_stream(), _ptr(y), _ptr(topk_w), M, k, D, _ptr(residual),
+                                  _ptr(out)), "tnx_moe_combine")
+
+
+def grpo_ratio(logp, old_logp, adv, tokens_per_seq, eps_lo, eps_hi, ratio=None, loss=None,
+               clipped=None):
+  N = logp.numel()
+  L.check(L.lib().tnx_grpo_ratio(_stream(), _ptr(logp), _ptr(old_logp), _ptr(adv), N,
+                                 tokens_per_seq, float(eps_lo), float(eps_hi), _ptr(ratio),
+                                 _ptr(loss), _ptr(clipped)), "tnx_grpo_ratio")
+
+
+def fill_u32(t: torch.Tensor, value: int = 0):
+  assert t.element_size() == 4
+  L.check(L.lib().tnx_fill_u32(_stream(), _ptr(t), t.numel(), value), "tnx_fill_u32")
