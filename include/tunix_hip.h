@@ -117,14 +117,15 @@ typedef struct tnx_qlinear_desc {
   int epilogue;             /* TNX_EPI_*                                                    */
   const uint16_t* residual; /* bf16 [M, N] for TNX_EPI_RESIDUAL                             */
   void* y;                  /* bf16 [M,N]; *_MUL: bf16 [M,N/2]; TNX_EPI_F32: fp32 [M,N]     */
-  int split_k;              /* >1: partial sums are atomically added into `ws`              */
-  float* ws;                /* fp32 [M,N] workspace, all zero on entry; required when
-                               split_k > 1; tnx_splitk_finish applies the epilogue and
-                               leaves it zero again                                         */
+  int split_k;              /* >1: the K range is split over work-groups, each writing its
+                               partial tile into `ws`                                       */
+  float* ws;                /* fp32 [split_k, M, N] workspace (need not be initialised);
+                               required when split_k > 1; tnx_splitk_finish adds the
+                               partial tiles in split order and applies the epilogue        */
 } tnx_qlinear_desc;
 
 int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* h_desc);
-/* Epilogue for split_k > 1 (same desc): y = epi(ws); ws := 0. */
+/* Epilogue for split_k > 1 (same desc): y = epi(sum_z ws[z]). */
 int tnx_splitk_finish(void* stream, const tnx_qlinear_desc* h_desc);
 
 /* t[M, R] = bf16( x[M,K] . A ), a_t = A transposed: bf16 [R, K].  R multiple of 16.
@@ -224,6 +225,8 @@ int tnx_gqa_attn(void* stream, const tnx_attn_desc* h_desc);
  * compute_chunked_logps :485-571.
  *   head weights: dense bf16 [V,D] (w_bf16 != NULL; also the tied embedding table), or QW
  *   part: fp32 workspace [M, n_vblocks, 4]; n_vblocks from tnx_lmhead_nblocks(V)
+ *   logits_out (optional) receives the raw logits f32(bf16(x . W)): neither the temperature nor
+ *   the forbidden mask is applied to it (the sampler's logits buffer, sampler.py:724-728)
  * ------------------------------------------------------------------------------------- */
 typedef struct tnx_lmhead_desc {
   int64_t M, D, V;
@@ -252,8 +255,9 @@ typedef struct tnx_lmhead_desc {
 int64_t tnx_lmhead_nblocks(int64_t V);
 int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* h_desc);
 
-/* Top-k / top-p sampling from materialised fp32 logits (already divided by temperature):
- * sample_top_p tunix/generate/sampler.py:105-148.  The k largest logits per row (descending,
+/* Top-k / top-p sampling from materialised raw fp32 logits, which are divided by `temperature`
+ * on the fly: sample_top_p tunix/generate/sampler.py:105-148.  `forbidden` ids (may be NULL) are
+ * treated as -inf (:490-491).  The k largest logits per row (descending,
  * lower index first among equals) are softmaxed, entries whose exclusive cumulative
  * probability exceeds top_p are dropped, and one is drawn by Gumbel-max (jax.random.categorical)
  * with noise from threefry2x32 keyed by fold_in((key0,key1), *step_ptr) (sampler.py:516).
@@ -262,8 +266,9 @@ int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* h_desc);
  * the whole vocabulary.  logp_out = full-vocabulary log-softmax at the drawn id (:141-144).
  * k <= 1024.  `ws` is unused (reserved). */
 int tnx_sample_topk(void* stream, const float* logits, int64_t M, int64_t V, int k, float top_p,
-                    uint32_t key0, uint32_t key1, int rng_variant, const int32_t* step_ptr,
-                    float* ws, int32_t* ids_out, float* logp_out);
+                    float temperature, uint32_t key0, uint32_t key1, int rng_variant,
+                    const int32_t* forbidden, int n_forbidden, const int32_t* step_ptr, float* ws,
+                    int32_t* ids_out, float* logp_out);
 
 /* Sampler bookkeeping of one step (tunix/generate/sampler.py:529-535, :692-703):
  *   col = *step_ptr; tokens[b, col+1] = ids[b]; logprobs[b, col+1] = logp[b] (if given);

@@ -1,0 +1,88 @@
+"""Per-token log-probabilities, KL estimators and the GRPO clipped ratio (oracle; tests only).
+
+Follows tunix/rl/common.py:135-203, :234-291, :326-571 and tunix/rl/algo_core.py:440-489.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from . import utils_ref as U
+
+
+def compute_kl_divergence(logps, ref_logps, method="low_var_kl", clamp_value=None):
+  """tunix/rl/common.py:135-184."""
+  logps = np.asarray(logps, dtype=np.float32)
+  ref = np.asarray(ref_logps, dtype=np.float32)
+  if method == "kl":
+    kl = logps - ref
+  elif method == "mse_kl":
+    kl = 0.5 * np.square(logps - ref)
+  elif method == "low_var_kl":
+    diff = ref - logps
+    kl = np.exp(diff) - diff - 1
+  else:
+    raise ValueError("`method` must be one of 'kl', 'mse_kl', 'low_var_kl'. Received:"
+                     f" {method}")
+  if clamp_value is not None:
+    kl = np.clip(kl, -clamp_value, clamp_value)
+  return kl
+
+
+def selective_log_softmax(logits: torch.Tensor, input_ids: torch.Tensor) -> torch.Tensor:
+  """tunix/rl/common.py:187-203: f32(logit[target]) - logsumexp(f32(logits))."""
+  lg = logits.to(torch.float32)
+  tgt = torch.gather(lg, -1, input_ids.long()[..., None]).squeeze(-1)
+  return tgt - torch.logsumexp(lg, dim=-1)
+
+
+def process_ids(prompt_tokens: np.ndarray, completion_tokens: np.ndarray, pad_id: int):
+  """tunix/rl/common.py:234-291 (unpacked branch)."""
+  ids = np.concatenate([prompt_tokens, completion_tokens], axis=1)
+  mask = np.concatenate([prompt_tokens != pad_id, completion_tokens != pad_id], axis=-1)
+  positions = U.build_positions_from_mask(mask)
+  attn_mask = U.make_causal_attn_mask(mask)
+  return ids, positions, attn_mask
+
+
+def compute_per_token_logps(ref_model, prompt_tokens, completion_tokens, pad_id,
+                            temperature: float = 1.0, chunk_size: int = 0):
+  """tunix/rl/common.py:326-482: one full forward without cache, logits[:, -T-1:-1],
+  optional temperature, gather - logsumexp.  chunk_size > 0 follows compute_chunked_logps
+  (:485-571): the head is applied per sequence chunk."""
+  ids, positions, attn_mask = process_ids(np.asarray(prompt_tokens), np.asarray(completion_tokens),
+                                          pad_id)
+  B, Ltot = ids.shape
+  T = completion_tokens.shape[1]
+  cache = ref_model.init_cache(B, Ltot)
+  tok = torch.from_numpy(ids.astype(np.int64))
+  h = ref_model.hidden(tok, torch.from_numpy(positions.astype(np.int64)), cache,
+                       torch.from_numpy(attn_mask), 0)
+  hk = h[:, -T - 1:-1]
+  targets = tok[:, -T:]
+
+  def head(hh):
+    lg = ref_model.logits(hh).to(torch.float32)
+    if temperature != 0.0 and temperature != 1.0:
+      lg = lg / np.float32(temperature)
+    return lg
+
+  if chunk_size > 0:
+    outs = []
+    for s in range(0, T, chunk_size):
+      outs.append(selective_log_softmax(head(hk[:, s:s + chunk_size]), targets[:, s:s + chunk_size]))
+    return torch.cat(outs, dim=1)
+  return selective_log_softmax(head(hk), targets)
+
+
+def grpo_ratio(logp, old_logp, adv, eps_lo, eps_hi):
+  """tunix/rl/algo_core.py:440-489: clipped importance ratio and per-token loss."""
+  logp = np.asarray(logp, dtype=np.float32)
+  old = logp if old_logp is None else np.asarray(old_logp, dtype=np.float32)
+  lr = np.clip(logp - old, -20.0, 20.0).astype(np.float32)
+  ratio = np.exp(lr).astype(np.float32)
+  a = np.asarray(adv, dtype=np.float32)
+  a = a if a.ndim == logp.ndim else a[..., None]
+  l1 = -a * ratio
+  l2 = -a * np.clip(ratio, np.float32(1 - eps_lo), np.float32(1 + eps_hi))
+  return ratio, np.maximum(l1, l2).astype(np.float32), (l2 > l1)

@@ -1,0 +1,553 @@
+"""GPU parity of every kernel family against the CPU oracle, called through the C ABI.
+
+Bars: bit-exact for integer / index outputs (codes, scales, arg-max ids, routes); for bf16
+outputs the kernel and the oracle round the same fp32 value, so they may differ by one bf16 ulp
+where the accumulation order moves a sum across a rounding boundary: the tests allow
+|diff| <= 2^-7 * |ref| + atol (one ulp) and require the bulk of the elements to be bit-equal.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import model_ref as MR
+from oracle import quant_ref as Q
+from oracle import rl_ref, threefry as TF
+from oracle import sampler_ref as SR
+
+pytestmark = pytest.mark.gpu
+
+
+def bf(x):
+  return x.to(torch.bfloat16)
+
+
+def rnd(shape, seed, scale=1.0):
+  g = torch.Generator().manual_seed(seed)
+  return (torch.randn(*shape, generator=g) * scale).to(torch.bfloat16).float()
+
+
+def assert_bf16_close(got, ref, atol=1e-6, min_equal=0.97, what=""):
+  got, ref = got.float().cpu(), ref.float().cpu()
+  diff = (got - ref).abs()
+  tol = ref.abs() * 2.0 ** -7 + atol
+  bad = (diff > tol).sum().item()
+  eq = (got == ref).float().mean().item()
+  assert bad == 0, f"{what}: {bad} elements beyond one bf16 ulp, max diff {diff.max().item()}"
+  assert eq >= min_equal, f"{what}: only {eq:.4f} of the elements are bit-equal"
+
+
+@pytest.mark.parametrize("qtype", [Q.INT4, Q.NF4])
+@pytest.mark.parametrize("group", [32, 64, 128, 256])
+@pytest.mark.parametrize("interleave", [False, True])
+def test_quantize_pack_bit_exact(gpu, qtype, group, interleave):
+  from tunix_amd import ops
+  K, N = 512, 96 if not interleave else 128
+  w = rnd((K, N), 11 + group, 0.02)
+  w[0:group, 3] = 0.0  # an all-zero group
+  codes, scale = Q.quantize(w.numpy(), group, qtype)
+  ref_c, ref_s = Q.pack_qw(codes, scale, group, interleave)
+  c, s = ops.quantize_pack(bf(w).to(gpu), group, qtype, interleave)
+  np.testing.assert_array_equal(c.cpu().numpy().view(np.uint32), ref_c)
+  np.testing.assert_array_equal(s.cpu().view(torch.int16).numpy().view(np.uint16), ref_s)
+  deq = ops.qw_dequant(c, s, K, N, group, qtype, interleave).cpu().numpy()
+  np.testing.assert_array_equal(deq, Q.dequantize(codes, scale, group, qtype))
+
+
+def _lora(K, N, r, seed):
+  return rnd((K, r), seed, 0.02), rnd((r, N), seed + 1, 0.01)
+
+
+def _pad_lora(a, b, rp):
+  K, r = a.shape
+  N = b.shape[1]
+  a_t = torch.zeros(rp, K)
+  a_t[:r] = a.t()
+  b_t = torch.zeros(N, rp)
+  b_t[:, :r] = b.t()
+  return a_t, b_t
+
+
+@pytest.mark.parametrize("M,K,N,group,qtype,r,split", [
+    (8, 512, 512, 64, Q.INT4, 8, 1),
+    (128, 4096, 1024, 64, Q.NF4, 64, 1),
+    (128, 4096, 1024, 64, Q.NF4, 64, 4),
+    (64, 1152, 1024, 128, Q.INT4, 16, 3),
+    (33, 768, 208, 256, Q.NF4, 0, 1),
+    (130, 256, 48, 32, Q.INT4, 32, 1),
+])
+def test_qlinear_lora_matches_oracle(gpu, M, K, N, group, qtype, r, split):
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  x = rnd((M, K), 1)
+  w = rnd((K, N), 2, 0.02)
+  codes, scale = Q.quantize(w.numpy(), group, qtype)
+  a = b = None
+  if r:
+    a, b = _lora(K, N, r, 3)
+  ref = Q.rb(Q.qlinear_lora(x, codes, scale, group, qtype, a, b, lora_scale=2.0))
+  c, s = ops.quantize_pack(bf(w).to(gpu), group, qtype)
+  y = torch.empty(M, N, dtype=torch.bfloat16, device=gpu)
+  kw = {}
+  if r:
+    rp = (r + 31) // 32 * 32
+    a_t, b_t = _pad_lora(a, b, rp)
+    t = torch.zeros(M, rp, dtype=torch.bfloat16, device=gpu)
+    ops.lora_down(bf(x).to(gpu), bf(a_t).to(gpu), t)
+    t_ref = Q.rb((x.double() @ a.double()).float())
+    assert_bf16_close(t[:, :r], t_ref, what="lora_down")
+    kw = dict(lora_rank=rp, lora_nseg=1, lora_seg_end=[N], lora_seg_toff=[0], t=t, t_ld=rp,
+              lora_b=bf(b_t).to(gpu), lora_scale=2.0)
+  ws = torch.full((split * M * N,), float('nan'), dtype=torch.float32, device=gpu) if split > 1 else None
+  d = ops.make_qlinear_desc(M=M, K=K, N=N, group=group, qtype=qtype, x=bf(x).to(gpu), codes=c,
+                            scales=s, y=y, split_k=split, ws=ws, **kw)
+  ops.qlinear(d)
+  torch.cuda.synchronize()
+  assert_bf16_close(y, ref, what="qlinear")
+
+
+def test_qlinear_invariants(gpu):
+  """Zero codes give zero; B = 0 leaves the base result; scale linearity (exact powers of 2)."""
+  from tunix_amd import ops
+  M, K, N, g = 16, 256, 64, 64
+  x = rnd((M, K), 5)
+  w = rnd((K, N), 6, 0.02)
+
+  def run(wt, lora=None):
+    c, s = ops.quantize_pack(bf(wt).to(gpu), g, Q.NF4)
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=gpu)
+    kw = {}
+    if lora is not None:
+      a_t, b_t = lora
+      t = torch.zeros(M, 32, dtype=torch.bfloat16, device=gpu)
+      ops.lora_down(bf(x).to(gpu), bf(a_t).to(gpu), t)
+      kw = dict(lora_rank=32, lora_nseg=1, lora_seg_end=[N], lora_seg_toff=[0], t=t, t_ld=32,
+                lora_b=bf(b_t).to(gpu), lora_scale=1.0)
+    ops.qlinear(ops.make_qlinear_desc(M=M, K=K, N=N, group=g, qtype=Q.NF4, x=bf(x).to(gpu),
+                                      codes=c, scales=s, y=y, **kw))
+    return y.float().cpu()
+
+  assert run(torch.zeros(K, N)).abs().max().item() == 0.0
+  base = run(w)
+  a_t = rnd((32, K), 7, 0.02)
+  assert torch.equal(run(w, (a_t, torch.zeros(N, 32))), base)
+  assert torch.equal(run(w * 4.0), base * 4.0)
+
+
+@pytest.mark.parametrize("epi", ["silu", "gelu", "residual"])
+def test_qlinear_epilogues(gpu, epi):
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  M, K, F, g = 40, 512, 256, 64
+  x = rnd((M, K), 8)
+  if epi == "residual":
+    w = rnd((K, F), 9, 0.02)
+    res = rnd((M, F), 10)
+    codes, scale = Q.quantize(w.numpy(), g, Q.INT4)
+    ref = Q.rb(Q.rb(Q.qlinear_lora(x, codes, scale, g, Q.INT4)) + res)
+    c, s = ops.quantize_pack(bf(w).to(gpu), g, Q.INT4)
+    y = torch.empty(M, F, dtype=torch.bfloat16, device=gpu)
+    ops.qlinear(ops.make_qlinear_desc(M=M, K=K, N=F, group=g, qtype=Q.INT4, x=bf(x).to(gpu), codes=c,
+                                      scales=s, y=y, epilogue=L.TNX_EPI_RESIDUAL,
+                                      residual=bf(res).to(gpu)))
+    assert_bf16_close(y, ref, what="residual epilogue")
+    return
+  wg, wu = rnd((K, F), 9, 0.05), rnd((K, F), 10, 0.05)
+  cg, sg = Q.quantize(wg.numpy(), g, Q.INT4)
+  cu, su = Q.quantize(wu.numpy(), g, Q.INT4)
+  gte = Q.rb(Q.qlinear_lora(x, cg, sg, g, Q.INT4))
+  up = Q.rb(Q.qlinear_lora(x, cu, su, g, Q.INT4))
+  if epi == "silu":
+    act = Q.rb(gte * Q.rb(torch.sigmoid(gte)))
+  else:
+    act = Q.rb(torch.nn.functional.gelu(gte, approximate="tanh"))
+  ref = Q.rb(act * up)
+  c, s = ops.quantize_pack(bf(torch.cat([wg, wu], 1)).to(gpu), g, Q.INT4, True)
+  y = torch.empty(M, F, dtype=torch.bfloat16, device=gpu)
+  ops.qlinear(ops.make_qlinear_desc(
+      M=M, K=K, N=2 * F, group=g, qtype=Q.INT4, x=bf(x).to(gpu), codes=c, scales=s, y=y,
+      epilogue=L.TNX_EPI_SILU_MUL if epi == "silu" else L.TNX_EPI_GELU_MUL))
+  assert_bf16_close(y, ref, atol=1e-5, min_equal=0.9, what=f"{epi} epilogue")
+
+
+class _Cfg:
+  def __init__(self, family, eps=1e-6):
+    self.family, self.norm_eps = family, eps
+
+
+@pytest.mark.parametrize("family", ["llama3", "qwen3", "gemma3"])
+def test_rmsnorm_flavours(gpu, family):
+  from tunix_amd import ops
+  from tunix_amd.model import _NORM
+  M, D = 37, 1152
+  x, res = rnd((M, D), 20, 2.0), rnd((M, D), 21)
+  w = rnd((D,), 22, 0.5) + (0.0 if family == "gemma3" else 1.0)
+  w = Q.rb(w)
+  ref_m = MR.RefModel.__new__(MR.RefModel)
+  ref_m.cfg, ref_m.bf16 = _Cfg(family, 1e-5), True
+  ref = ref_m.rmsnorm(x, w)
+  y = torch.empty(M, D, dtype=torch.bfloat16, device=gpu)
+  ops.rmsnorm(bf(x).to(gpu), bf(w).to(gpu), y, 1e-5 if family != "gemma3" else 1e-6, _NORM[family])
+  assert_bf16_close(y, ref, min_equal=0.95, what=f"rmsnorm {family}")
+  # residual variants
+  h = Q.rb(x + res)
+  ref2 = Q.rb(ref_m.rmsnorm(h, w) + res)
+  y2 = torch.empty_like(y)
+  hout = torch.empty_like(y)
+  ops.rmsnorm(bf(x).to(gpu), bf(w).to(gpu), y2, 1e-5 if family != "gemma3" else 1e-6, _NORM[family],
+              res_pre=bf(res).to(gpu), h_out=hout, res_post=bf(res).to(gpu))
+  assert torch.equal(hout.float().cpu(), h)
+  assert_bf16_close(y2, ref2, min_equal=0.95, what=f"rmsnorm+residual {family}")
+
+
+@pytest.mark.parametrize("family,dh,Hq,Hkv", [("llama3", 128, 8, 2), ("qwen3", 64, 8, 2),
+                                               ("gemma3", 256, 4, 1)])
+def test_rope_kvwrite(gpu, family, dh, Hq, Hkv):
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  from tunix_amd.model import _NORM, _ROPE, rope_timescale
+  B, T, S = 3, 5, 16
+  col = 4
+  theta = 1e6 if family != "gemma3" else 1e4
+  qkv = rnd((B * T, (Hq + 2 * Hkv) * dh), 30)
+  pos = torch.randint(0, 900, (B, S), generator=torch.Generator().manual_seed(31), dtype=torch.int32)
+  qn, kn = Q.rb(rnd((dh,), 32, 0.3) + 1), Q.rb(rnd((dh,), 33, 0.3) + 1)
+  rm = MR.RefModel.__new__(MR.RefModel)
+  rm.cfg, rm.bf16 = _Cfg(family), True
+  x = qkv.view(B, T, Hq + 2 * Hkv, dh)
+  q, k, v = x[:, :, :Hq], x[:, :, Hq:Hq + Hkv], x[:, :, Hq + Hkv:]
+  if family != "llama3":
+    q, k = rm.rmsnorm(q, qn), rm.rmsnorm(k, kn)
+  p = pos[:, col:col + T].long()
+  sf = 8.0 if family == "gemma3" else 1.0
+  q, k = rm.rope(q, p, theta, scale_factor=sf), rm.rope(k, p, theta, scale_factor=sf)
+  if family == "gemma3":
+    q = Q.rb(q * Q.rb(torch.tensor(dh ** -0.5)))
+  d = L.RopeDesc()
+  d.B, d.T, d.S, d.Hq, d.Hkv, d.dh = B, T, S, Hq, Hkv, dh
+  d.rope_flavor, d.rope_scale = _ROPE[family], sf
+  ts = torch.from_numpy(rope_timescale(dh, theta)).to(gpu)
+  d.timescale = ts.data_ptr()
+  wq, wk = bf(qn).to(gpu), bf(kn).to(gpu)
+  if family != "llama3":
+    d.qk_norm, d.norm_eps, d.q_norm_w, d.k_norm_w = _NORM[family], 1e-6, wq.data_ptr(), wk.data_ptr()
+  else:
+    d.qk_norm = -1
+  d.q_prescale = dh ** -0.5 if family == "gemma3" else 0.0
+  g_qkv, g_pos = bf(qkv).to(gpu), pos.to(gpu)
+  colp = torch.tensor([col], dtype=torch.int32, device=gpu)
+  qo = torch.empty(B * T, Hq * dh, dtype=torch.bfloat16, device=gpu)
+  kc = torch.zeros(B, Hkv, S, dh, dtype=torch.bfloat16, device=gpu)
+  vc = torch.zeros_like(kc)
+  d.qkv, d.positions, d.pos_ld, d.col_ptr = g_qkv.data_ptr(), g_pos.data_ptr(), S, colp.data_ptr()
+  d.q_out, d.kcache, d.vcache = qo.data_ptr(), kc.data_ptr(), vc.data_ptr()
+  ops.rope_kvwrite(d)
+  torch.cuda.synchronize()
+  assert_bf16_close(qo.view(B, T, Hq, dh), q, min_equal=0.9, what="rope q")
+  assert_bf16_close(kc[:, :, col:col + T].permute(0, 2, 1, 3), k, min_equal=0.9, what="rope k")
+  assert torch.equal(vc[:, :, col:col + T].permute(0, 2, 1, 3).float().cpu(), v)
+  assert kc[:, :, :col].abs().max().item() == 0 and kc[:, :, col + T:].abs().max().item() == 0
+
+
+def _attn_ref(q, kc, vc, tokens, pad_id, col, T, scale, window):
+  """Oracle attention with the dense masks of the reference."""
+  from oracle import utils_ref as U
+  B, S = kc.shape[0], kc.shape[2]
+  rm = MR.RefModel.__new__(MR.RefModel)
+  rm.bf16, rm.acc = True, torch.float64
+  k_all, v_all = kc.permute(0, 2, 1, 3), vc.permute(0, 2, 1, 3)
+  tok = tokens.numpy()
+  if T == 1:
+    mask = U.compute_attention_masks(col, S, tok == pad_id)
+    if window:
+      mask = U.create_sliding_window_mask(mask, window) & mask
+  else:
+    assert col == 0
+    mask = U.make_causal_attn_mask(tok[:, :T] != pad_id, S)
+    if window:
+      ones = torch.ones(T, S, dtype=torch.bool)
+      sm = (torch.triu(ones, -window + 1) & torch.tril(ones, window - 1)).numpy()
+      mask = mask & sm[None]
+  return rm.attention(q, k_all, v_all, torch.from_numpy(mask), scale)
+
+
+@pytest.mark.parametrize("B,T,S,Hq,Hkv,dh,col,chunk,window", [
+    (4, 1, 64, 8, 2, 64, 37, 0, 0),
+    (4, 1, 320, 8, 2, 128, 300, 64, 0),
+    (3, 1, 128, 4, 1, 256, 100, 32, 48),
+    (2, 1, 96, 32, 4, 128, 95, 32, 0),
+    (2, 1, 64, 6, 2, 128, 20, 0, 0),
+    (3, 24, 32, 8, 2, 64, 0, 0, 0),
+    (2, 40, 64, 4, 1, 256, 0, 0, 16),
+])
+def test_gqa_attention_matches_oracle(gpu, B, T, S, Hq, Hkv, dh, col, chunk, window):
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  pad = 0
+  g = torch.Generator().manual_seed(40 + S)
+  tokens = torch.randint(1, 100, (B, S), generator=g, dtype=torch.int32)
+  tokens[0, :5] = pad            # left padding
+  tokens[1, 7] = pad             # a pad id inside the sequence is masked as well
+  q = rnd((B, T, Hq, dh), 41)
+  kc, vc = rnd((B, Hkv, S, dh), 42), rnd((B, Hkv, S, dh), 43)
+  scale = dh ** -0.5
+  ref = _attn_ref(q, kc, vc, tokens, pad, col, T, scale, window)
+  # slots above the current column hold garbage that must not matter
+  kc_g, vc_g = kc.clone(), vc.clone()
+  kc_g[:, :, col + T:] = 1e4
+  vc_g[:, :, col + T:] = 1e4
+  d = L.AttnDesc()
+  d.B, d.T, d.S, d.Hq, d.Hkv, d.dh = B, T, S, Hq, Hkv, dh
+  d.scale, d.window, d.pad_id = scale, window, pad
+  gq, gk, gv = bf(q).reshape(B * T, Hq * dh).to(gpu), bf(kc_g).to(gpu), bf(vc_g).to(gpu)
+  gt = tokens.to(gpu)
+  colp = torch.tensor([col], dtype=torch.int32, device=gpu)
+  out = torch.zeros(B * T, Hq * dh, dtype=torch.bfloat16, device=gpu)
+  nb = ops.attn_ws_bytes(B, T, S, Hq, dh, chunk)
+  ws = torch.empty(max(nb // 4, 1), dtype=torch.float32, device=gpu)
+  d.q, d.kcache, d.vcache, d.tokens, d.tok_ld = gq.data_ptr(), gk.data_ptr(), gv.data_ptr(), gt.data_ptr(), S
+  d.col_ptr, d.kv_chunk, d.ws, d.out = colp.data_ptr(), chunk, ws.data_ptr(), out.data_ptr()
+  ops.gqa_attn(d)
+  torch.cuda.synchronize()
+  got = out.view(B, T, Hq, dh).float().cpu()
+  # rows whose query token is itself pad attend nothing in the reference's mask: skip them
+  valid = torch.ones(B, T, dtype=torch.bool)
+  for b in range(B):
+    for t in range(T):
+      c = col + t
+      if not ((tokens[b, :c + 1] != pad).any()):
+        valid[b, t] = False
+  diff = (got - ref).abs()[valid]
+  # probabilities are rounded to bf16 before (oracle) or after (kernel, online softmax) the
+  # normalisation, so outputs agree to bf16 resolution of O(1) values, not bit for bit
+  assert diff.max().item() <= 2.0 ** -6 * max(1.0, ref.abs().max().item()), diff.max().item()
+  assert diff.mean().item() <= 2e-3
+
+
+@pytest.mark.parametrize("M,D,V,dense", [(8, 512, 32000, True), (128, 512, 4096, True),
+                                         (50, 256, 1040, False), (130, 256, 4096, False)])
+def test_lmhead_greedy_and_logp(gpu, M, D, V, dense):
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  x = rnd((M, D), 50)
+  w = rnd((D, V), 51, 0.05)
+  g = torch.Generator().manual_seed(52)
+  targets = torch.randint(0, V, (M,), generator=g, dtype=torch.int32)
+  d = L.LmHeadDesc()
+  d.M, d.D, d.V = M, D, V
+  gx = bf(x).to(gpu)
+  d.x = gx.data_ptr()
+  keep = []
+  if dense:
+    logits = Q.rb((x.double() @ w.double()).float())
+    gw = bf(w).t().contiguous().to(gpu)
+    d.w_bf16 = gw.data_ptr()
+  else:
+    codes, scale = Q.quantize(w.numpy(), 128, Q.INT4)
+    a, b = _lora(D, V, 32, 53)
+    logits = Q.rb(Q.qlinear_lora(x, codes, scale, 128, Q.INT4, a, b, lora_scale=1.0))
+    c, s = ops.quantize_pack(bf(w).to(gpu), 128, Q.INT4)
+    a_t, b_t = _pad_lora(a, b, 32)
+    t = torch.zeros(M, 32, dtype=torch.bfloat16, device=gpu)
+    ops.lora_down(gx, bf(a_t).to(gpu), t)
+    gb = bf(b_t).to(gpu)
+    d.codes, d.scales, d.group, d.qtype = c.data_ptr(), s.data_ptr(), 128, Q.INT4
+    d.lora_rank, d.t, d.t_ld, d.lora_b, d.lora_scale = 32, t.data_ptr(), 32, gb.data_ptr(), 1.0
+    keep += [c, s, t, gb]
+  temperature = 0.7
+  d.temperature = temperature
+  nvb = ops.lmhead_nblocks(V)
+  part = torch.empty(M * nvb * 4, dtype=torch.float32, device=gpu)
+  best = torch.empty(M, dtype=torch.int32, device=gpu)
+  blp = torch.empty(M, dtype=torch.float32, device=gpu)
+  tlp = torch.empty(M, dtype=torch.float32, device=gpu)
+  lse = torch.empty(M, dtype=torch.float32, device=gpu)
+  lg_out = torch.empty(M, V, dtype=torch.float32, device=gpu)
+  gt = targets.to(gpu)
+  d.targets, d.part, d.best_id, d.best_logp = gt.data_ptr(), part.data_ptr(), best.data_ptr(), blp.data_ptr()
+  d.target_logp, d.lse, d.logits_out = tlp.data_ptr(), lse.data_ptr(), lg_out.data_ptr()
+  ops.lmhead(d)
+  torch.cuda.synchronize()
+  got_logits = lg_out.cpu()
+  scaled = logits / np.float32(temperature)
+  # the materialised logits are bf16 values / T: compare through the bf16 criterion
+  assert_bf16_close(Q.rb(got_logits * temperature), logits, atol=1e-6, min_equal=0.97, what="logits")
+  # the fused statistics must agree with the logits the kernel itself produced
+  ref_best = torch.from_numpy(np.argmax(got_logits.numpy(), axis=-1))
+  assert torch.equal(best.cpu().long(), ref_best), "arg-max (first maximal index)"
+  ref_lse = torch.logsumexp(got_logits, dim=-1)
+  np.testing.assert_allclose(lse.cpu().numpy(), ref_lse.numpy(), rtol=0, atol=2e-5)
+  ref_t = rl_ref.selective_log_softmax(got_logits, targets)
+  np.testing.assert_allclose(tlp.cpu().numpy(), ref_t.numpy(), rtol=0, atol=2e-5)
+  np.testing.assert_allclose(blp.cpu().numpy(), (got_logits.max(-1).values - ref_lse).numpy(), atol=2e-5)
+  # and with the oracle's logits within the bf16 tolerance of the path
+  ref_t2 = rl_ref.selective_log_softmax(scaled, targets)
+  assert (tlp.cpu() - ref_t2).abs().max().item() < 2e-2
+
+
+def test_lmhead_forbidden_and_ties(gpu):
+  """Equal maxima resolve to the lowest index; forbidden ids are never chosen."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  M, D, V = 4, 128, 512
+  x = torch.zeros(M, D)
+  x[:, 0] = 1.0
+  w = torch.zeros(D, V)
+  w[0, [5, 300, 511]] = 2.0      # three-way tie
+  d = L.LmHeadDesc()
+  d.M, d.D, d.V = M, D, V
+  gx, gw = bf(x).to(gpu), bf(w).t().contiguous().to(gpu)
+  d.x, d.w_bf16, d.temperature = gx.data_ptr(), gw.data_ptr(), 1.0
+  part = torch.empty(M * ops.lmhead_nblocks(V) * 4, dtype=torch.float32, device=gpu)
+  best = torch.empty(M, dtype=torch.int32, device=gpu)
+  d.part, d.best_id = part.data_ptr(), best.data_ptr()
+  ops.lmhead(d)
+  assert best.cpu().tolist() == [5] * M
+  fb = torch.tensor([5, 300], dtype=torch.int32, device=gpu)
+  d.forbidden, d.n_forbidden = fb.data_ptr(), 2
+  ops.lmhead(d)
+  assert best.cpu().tolist() == [511] * M
+
+
+@pytest.mark.parametrize("k,top_p,variant", [(50, 1.0, 0), (50, 0.7, 0), (8, 0.9, 1), (0, 1.0, 0)])
+def test_sample_topk_matches_oracle(gpu, k, top_p, variant):
+  from tunix_amd import ops
+  M, V = 16, 3000
+  g = torch.Generator().manual_seed(60)
+  logits = (torch.randn(M, V, generator=g) * 2).float()
+  logits[:, 17] = logits[:, 29]                      # ties inside the top-k
+  key = TF.prng_key(1234)
+  step = 77
+  tok_ref, lp_ref = SR.sample_top_p(logits, TF.fold_in(key, step), 1.0, top_p, k if k else None,
+                                    partitionable=bool(variant))
+  ids = torch.empty(M, dtype=torch.int32, device=gpu)
+  lp = torch.empty(M, dtype=torch.float32, device=gpu)
+  stp = torch.tensor([step], dtype=torch.int32, device=gpu)
+  ws = torch.empty(8, dtype=torch.float32, device=gpu)
+  ops.sample_topk(logits.to(gpu), k, top_p, (int(key[0]), int(key[1])), variant, stp, ws, ids, lp)
+  torch.cuda.synchronize()
+  assert ids.cpu().long().tolist() == tok_ref.tolist()
+  np.testing.assert_allclose(lp.cpu().numpy(), lp_ref.numpy(), atol=2e-5)
+
+
+def test_sample_commit_and_fill(gpu):
+  from tunix_amd import ops
+  B, Ld = 5, 12
+  tokens = torch.full((B, Ld), 9, dtype=torch.int32, device=gpu)
+  lps = torch.zeros(B, Ld, dtype=torch.float32, device=gpu)
+  done = torch.zeros(B, dtype=torch.int32, device=gpu)
+  step = torch.tensor([6], dtype=torch.int32, device=gpu)
+  ids = torch.tensor([3, 4, 2, 7, 2], dtype=torch.int32, device=gpu)
+  lp = torch.arange(B, dtype=torch.float32, device=gpu) * -0.5
+  eos = torch.tensor([2, 11], dtype=torch.int32, device=gpu)
+  ops.sample_commit(ids, lp, tokens, lps, done, eos, step)
+  assert step.item() == 7
+  assert tokens[:, 7].cpu().tolist() == [3, 4, 2, 7, 2] and tokens[:, 6].cpu().tolist() == [9] * B
+  assert lps[:, 7].cpu().tolist() == [0.0, -0.5, -1.0, -1.5, -2.0]
+  assert done.cpu().tolist() == [0, 0, 1, 0, 1]
+  buf = torch.ones(1000, dtype=torch.int32, device=gpu)
+  ops.fill_u32(buf, 0)
+  assert buf.sum().item() == 0
+
+
+def test_grpo_ratio_matches_oracle(gpu):
+  from tunix_amd import ops
+  N, T = 4096, 64
+  g = torch.Generator().manual_seed(70)
+  logp = -torch.rand(N, generator=g) * 5
+  old = logp + torch.randn(N, generator=g) * 0.05
+  old[:8] = logp[:8] - 30.0          # exercises the +-20 clamp
+  adv = torch.randn(N // T, generator=g)
+  r_ref, l_ref, c_ref = rl_ref.grpo_ratio(logp.view(-1, T).numpy(), old.view(-1, T).numpy(),
+                                          adv.numpy(), 0.2, 0.2)
+  ratio = torch.empty(N, dtype=torch.float32, device=gpu)
+  loss = torch.empty(N, dtype=torch.float32, device=gpu)
+  clipped = torch.empty(N, dtype=torch.int32, device=gpu)
+  ops.grpo_ratio(logp.to(gpu), old.to(gpu), adv.to(gpu), T, 0.2, 0.2, ratio, loss, clipped)
+  np.testing.assert_allclose(ratio.cpu().numpy(), r_ref.reshape(-1), rtol=2e-6)
+  np.testing.assert_allclose(loss.cpu().numpy(), l_ref.reshape(-1), rtol=2e-6, atol=1e-7)
+  assert (clipped.cpu().numpy().astype(bool) == c_ref.reshape(-1)).mean() > 0.999
+  # old = None: ratio is exactly one (tests/rl/algo_core_test.py:51-143 relies on it)
+  ops.grpo_ratio(logp.to(gpu), None, adv.to(gpu), T, 0.2, 0.2, ratio, loss, None)
+  assert torch.all(ratio == 1.0)
+
+
+def test_moe_route_sort_gmm_combine(gpu):
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  M, E, k, D, F, g = 12, 16, 4, 256, 128, 128
+  scores = rnd((M, E), 80)
+  scores[3, 5] = scores[3, 9]                          # tie between experts
+  probs = torch.softmax(scores, -1)
+  order = torch.sort(probs, dim=-1, descending=True, stable=True).indices[:, :k]
+  wts = torch.gather(probs, -1, order)
+  wts = Q.rb(wts / wts.sum(-1, keepdim=True))
+  tw = torch.empty(M, k, dtype=torch.bfloat16, device=gpu)
+  ti = torch.empty(M, k, dtype=torch.int32, device=gpu)
+  ops.moe_route_topk(bf(scores).to(gpu), k, tw, ti)
+  assert torch.equal(ti.cpu().long(), order)
+  assert_bf16_close(tw, wts, what="routing weights")
+  counts = torch.empty(E, dtype=torch.int32, device=gpu)
+  offs = torch.empty(E + 1, dtype=torch.int32, device=gpu)
+  sr = torch.empty(M * k, dtype=torch.int32, device=gpu)
+  ops.moe_sort_routes(ti, E, counts, offs, sr)
+  flat = order.reshape(-1).numpy()
+  ref_sorted = np.argsort(flat, kind="stable")
+  np.testing.assert_array_equal(sr.cpu().numpy(), ref_sorted)
+  np.testing.assert_array_equal(counts.cpu().numpy(), np.bincount(flat, minlength=E))
+  # grouped gate|up with SiLU-mul, then down, then the weighted combine
+  x = rnd((M, D), 81)
+  wg, wu, wd = rnd((E, D, F), 82, 0.05), rnd((E, D, F), 83, 0.05), rnd((E, F, D), 84, 0.05)
+  cb, sb = ops.qw_sizes(D, 2 * F, g)
+  gc = torch.empty(E * cb // 4, dtype=torch.int32, device=gpu)
+  gs = torch.empty(E * sb // 2, dtype=torch.bfloat16, device=gpu)
+  cb2, sb2 = ops.qw_sizes(F, D, g)
+  dc = torch.empty(E * cb2 // 4, dtype=torch.int32, device=gpu)
+  ds = torch.empty(E * sb2 // 2, dtype=torch.bfloat16, device=gpu)
+  deq = {}
+  for e in range(E):
+    c, s = ops.quantize_pack(bf(torch.cat([wg[e], wu[e]], 1)).to(gpu), g, Q.INT4, True)
+    gc[e * cb // 4:(e + 1) * cb // 4] = c
+    gs[e * sb // 2:(e + 1) * sb // 2] = s
+    c, s = ops.quantize_pack(bf(wd[e]).to(gpu), g, Q.INT4)
+    dc[e * cb2 // 4:(e + 1) * cb2 // 4] = c
+    ds[e * sb2 // 2:(e + 1) * sb2 // 2] = s
+    deq[e] = [torch.from_numpy(Q.dequantize(*Q.quantize(m.numpy(), g, Q.INT4), g, Q.INT4)).double()
+              for m in (wg[e], wu[e], wd[e])]
+  ref = torch.zeros(M, D, dtype=torch.float64)
+  for m in range(M):
+    for j in range(k):
+      e = int(order[m, j])
+      gg = Q.rb((x[m].double() @ deq[e][0]).float())
+      uu = Q.rb((x[m].double() @ deq[e][1]).float())
+      a = Q.rb(Q.rb(gg * Q.rb(torch.sigmoid(gg))) * uu)
+      y = Q.rb((a.double() @ deq[e][2]).float())
+      ref[m] += (wts[m, j] * y).double()
+  ref = Q.rb(ref.float())
+  gx = bf(x).to(gpu)
+  act = torch.empty(M * k, F, dtype=torch.bfloat16, device=gpu)
+  yr = torch.empty(M * k, D, dtype=torch.bfloat16, device=gpu)
+  d = L.MoeGmmDesc()
+  d.n_routes, d.E, d.k, d.K, d.N, d.group, d.qtype = M * k, E, k, D, 2 * F, g, Q.INT4
+  d.x, d.x_div, d.codes, d.scales = gx.data_ptr(), k, gc.data_ptr(), gs.data_ptr()
+  d.offsets, d.sorted_route, d.epilogue, d.y = offs.data_ptr(), sr.data_ptr(), L.TNX_EPI_SILU_MUL, act.data_ptr()
+  ops.moe_gmm(d)
+  d2 = L.MoeGmmDesc()
+  d2.n_routes, d2.E, d2.k, d2.K, d2.N, d2.group, d2.qtype = M * k, E, k, F, D, g, Q.INT4
+  d2.x, d2.x_div, d2.codes, d2.scales = act.data_ptr(), 1, dc.data_ptr(), ds.data_ptr()
+  d2.offsets, d2.sorted_route, d2.epilogue, d2.y = offs.data_ptr(), sr.data_ptr(), L.TNX_EPI_STORE, yr.data_ptr()
+  ops.moe_gmm(d2)
+  out = torch.empty(M, D, dtype=torch.bfloat16, device=gpu)
+  ops.moe_combine(yr, tw, M, k, D, None, out)
+  torch.cuda.synchronize()
+  assert_bf16_close(out, ref, atol=1e-5, min_equal=0.85, what="moe")
+
+
+def test_argument_errors_raise(gpu):
+  from tunix_amd import ops
+  with pytest.raises(ValueError, match="K % 128"):
+    ops.qw_sizes(100, 64, 64)
+  x = torch.zeros(4, 128, dtype=torch.bfloat16, device=gpu)
+  with pytest.raises(ValueError):
+    ops.quantize_pack(x.t().contiguous(), 48, 0)

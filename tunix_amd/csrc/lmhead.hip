@@ -103,11 +103,12 @@ __global__ __launch_bounds__(256) void lmhead_kernel(const LHArgs a) {
       const int64_t row = m0 + rl;
       const bool rok = row < a.M;
       // logits are the bf16 einsum output cast to fp32, then divided by the temperature
-      const float la = okA ? __fdiv_rn(rbf(acc[mt][0][i]), a.temperature) : kNegInf;
-      const float lb = okB ? __fdiv_rn(rbf(acc[mt][1][i]), a.temperature) : kNegInf;
-      if (a.logits_out && rok) {
-        if ((ntile0 + 0) < s.ntiles) a.logits_out[row * a.V + colA] = la;
-        if ((ntile0 + 1) < s.ntiles) a.logits_out[row * a.V + colB] = lb;
+      const float ra = rbf(acc[mt][0][i]), rb_ = rbf(acc[mt][1][i]);
+      const float la = okA ? __fdiv_rn(ra, a.temperature) : kNegInf;
+      const float lb = okB ? __fdiv_rn(rb_, a.temperature) : kNegInf;
+      if (a.logits_out && rok) {  // raw model logits: no temperature, no forbidden mask
+        if ((ntile0 + 0) < s.ntiles) a.logits_out[row * a.V + colA] = ra;
+        if ((ntile0 + 1) < s.ntiles) a.logits_out[row * a.V + colB] = rb_;
       }
       Stat st;
       st.mx = fmaxf(la, lb);

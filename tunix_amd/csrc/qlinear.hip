@@ -53,7 +53,7 @@ __device__ __forceinline__ void store_tile(const QLArgs& a, int64_t m0, int64_t 
                                            int64_t ntile0, int64_t ntiles, f32x4 (&acc)[MT][NT],
                                            RowMap out_row) {
   const int lane = threadIdx.x & 63, lm = lane & 15, lq = lane >> 4;
-  if (a.split_k > 1) {  // partial sums; tnx_splitk_finish applies the epilogue
+  if (a.split_k > 1) {  // partial tile of this k split; tnx_splitk_finish sums the splits and applies the epilogue
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       if (ntile0 + nt >= ntiles) continue;
@@ -63,7 +63,8 @@ __device__ __forceinline__ void store_tile(const QLArgs& a, int64_t m0, int64_t 
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int64_t row = m0 + mt * 16 + lq * 4 + i;
-          if (row < m_end) atomicAdd(a.ws + out_row(row) * a.N + col, acc[mt][nt][i]);
+          if (row < m_end)
+            a.ws[((int64_t)blockIdx.z * a.M + out_row(row)) * a.N + col] = acc[mt][nt][i];
         }
     }
     return;
@@ -197,27 +198,31 @@ __global__ __launch_bounds__(256) void moe_gmm_kernel(const QLArgs a) {
                      [routes](int64_t r) { return (int64_t)routes[r]; });
 }
 
-// y = epi(ws); ws = 0.  One thread per output element.
+// y = epi(sum of the split_k partial tiles, added in split order).  One thread per output
+// element; the fixed summation order makes split-k results reproducible run to run.
 __global__ void splitk_finish_kernel(const QLArgs a) {
   const bool mul = a.epilogue == TNX_EPI_SILU_MUL || a.epilogue == TNX_EPI_GELU_MUL;
   const int64_t ncol = mul ? a.N / 2 : a.N;
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= a.M * ncol) return;
   const int64_t row = idx / ncol, c = idx % ncol;
+  const int64_t plane = a.M * a.N;
   if (mul) {
     const int64_t cg = (c / 16) * 32 + (c % 16);
-    float* pg = a.ws + row * a.N + cg;
-    float* pu = pg + 16;
-    const float g = rbf(*pg), u = rbf(*pu);
-    *pg = 0.f;
-    *pu = 0.f;
+    const float* pg = a.ws + row * a.N + cg;
+    float g = 0.f, u = 0.f;
+    for (int z = 0; z < a.split_k; ++z) {
+      g += pg[z * plane];
+      u += pg[z * plane + 16];
+    }
+    g = rbf(g);
+    u = rbf(u);
     const float act = a.epilogue == TNX_EPI_SILU_MUL ? silu_bf16(g) : gelu_tanh_bf16(g);
     reinterpret_cast<uint16_t*>(a.y)[idx] = f2bf(act * u);
     return;
   }
-  float* p = a.ws + idx;
-  const float v = *p;
-  *p = 0.f;
+  float v = 0.f;
+  for (int z = 0; z < a.split_k; ++z) v += a.ws[z * plane + idx];
   if (a.epilogue == TNX_EPI_F32)
     reinterpret_cast<float*>(a.y)[idx] = v;
   else if (a.epilogue == TNX_EPI_RESIDUAL)

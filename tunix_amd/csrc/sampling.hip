@@ -98,8 +98,9 @@ __device__ float block_sum_f(float v, float* red) {
 __global__ __launch_bounds__(NTH) void sample_topk_kernel(const float* logits, int64_t V, int k,
                                                           float top_p, uint32_t key0, uint32_t key1,
                                                           int variant, const int32_t* step_ptr,
-                                                          int64_t M, int32_t* ids_out,
-                                                          float* logp_out) {
+                                                          int64_t M, float temperature,
+                                                          const int32_t* forbidden, int n_forbidden,
+                                                          int32_t* ids_out, float* logp_out) {
   __shared__ uint32_t hist[256];
   __shared__ float cval[NTH];
   __shared__ int cidx[NTH];
@@ -110,6 +111,12 @@ __global__ __launch_bounds__(NTH) void sample_topk_kernel(const float* logits, i
   const int tid = threadIdx.x;
   const int64_t row = blockIdx.x;
   const float* lr = logits + row * V;
+  // the caller passes raw logits; sampling works on f32(logit) / temperature
+  auto lg = [lr, temperature, forbidden, n_forbidden](int64_t v) {
+    for (int f = 0; f < n_forbidden; ++f)
+      if (forbidden[f] == (int32_t)v) return kNegInf;
+    return __fdiv_rn(lr[v], temperature);
+  };
 
   // fold_in(key, step): threefry of the key over the counter pair (0, step)
   uint32_t ks0 = 0u, ks1 = (uint32_t)(*step_ptr);
@@ -121,13 +128,13 @@ __global__ __launch_bounds__(NTH) void sample_topk_kernel(const float* logits, i
   am.i = 0x7fffffff;
   for (int64_t v = tid; v < V; v += NTH) {
     ArgMax c;
-    c.v = lr[v];
+    c.v = lg(v);
     c.i = (int)v;
     am = better(am, c);
   }
   am = block_argmax(am, red_am);
   float se = 0.f;
-  for (int64_t v = tid; v < V; v += NTH) se += expf(lr[v] - am.v);
+  for (int64_t v = tid; v < V; v += NTH) se += expf(lg(v) - am.v);
   se = block_sum_f(se, red_f);
   const float lse = am.v + logf(se);
 
@@ -138,14 +145,14 @@ __global__ __launch_bounds__(NTH) void sample_topk_kernel(const float* logits, i
     g.i = 0x7fffffff;
     for (int64_t v = tid; v < V; v += NTH) {
       ArgMax c;
-      c.v = lr[v] + gumbel_from_bits(random_bits(ks0, ks1, (uint64_t)(row * V + v), (uint64_t)(M * V), variant));
+      c.v = lg(v) + gumbel_from_bits(random_bits(ks0, ks1, (uint64_t)(row * V + v), (uint64_t)(M * V), variant));
       c.i = (int)v;
       g = better(g, c);
     }
     g = block_argmax(g, red_am);
     if (tid == 0) {
       ids_out[row] = g.i;
-      if (logp_out) logp_out[row] = lr[g.i] - lse;
+      if (logp_out) logp_out[row] = lg(g.i) - lse;
     }
     return;
   }
@@ -158,7 +165,7 @@ __global__ __launch_bounds__(NTH) void sample_topk_kernel(const float* logits, i
     if (tid < 256) hist[tid] = 0;
     __syncthreads();
     for (int64_t v = tid; v < V; v += NTH) {
-      const uint32_t kk = order_key(lr[v]);
+      const uint32_t kk = order_key(lg(v));
       if ((kk & mask) == prefix) atomicAdd(&hist[(kk >> shift) & 255u], 1u);
     }
     __syncthreads();
@@ -187,7 +194,7 @@ __global__ __launch_bounds__(NTH) void sample_topk_kernel(const float* logits, i
   __syncthreads();
   // elements above the threshold: any order (sorted below)
   for (int64_t v = tid; v < V; v += NTH) {
-    const float x = lr[v];
+    const float x = lg(v);
     if (order_key(x) > thr) {
       const uint32_t p = atomicAdd(&s_cnt, 1u);
       cval[p] = x;
@@ -200,7 +207,7 @@ __global__ __launch_bounds__(NTH) void sample_topk_kernel(const float* logits, i
   for (int64_t v0 = 0; v0 < V; v0 += NTH) {
     if (s_base >= r_eq) break;
     const int64_t v = v0 + tid;
-    const bool eq = v < V && order_key(lr[v]) == thr;
+    const bool eq = v < V && order_key(lg(v)) == thr;
     const uint64_t bal = __ballot(eq);
     const int lane = tid & 63, wave = tid >> 6;
     const uint32_t before = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
@@ -213,7 +220,7 @@ __global__ __launch_bounds__(NTH) void sample_topk_kernel(const float* logits, i
     }
     const uint32_t pos = s_base + woff + before;
     if (eq && pos < r_eq) {
-      cval[n_gt + pos] = lr[v];
+      cval[n_gt + pos] = lg(v);
       cidx[n_gt + pos] = (int)v;
     }
     __syncthreads();
@@ -265,20 +272,22 @@ __global__ __launch_bounds__(NTH) void sample_topk_kernel(const float* logits, i
   if (tid == 0) {
     const int tokid = cidx[g.i];
     ids_out[row] = tokid;
-    if (logp_out) logp_out[row] = lr[tokid] - lse;
+    if (logp_out) logp_out[row] = lg(tokid) - lse;
   }
 }
 
 }  // namespace
 
 extern "C" int tnx_sample_topk(void* stream, const float* logits, int64_t M, int64_t V, int k,
-                               float top_p, uint32_t key0, uint32_t key1, int rng_variant,
+                               float top_p, float temperature, uint32_t key0, uint32_t key1,
+                               int rng_variant, const int32_t* forbidden, int n_forbidden,
                                const int32_t* step_ptr, float* ws, int32_t* ids_out,
                                float* logp_out) {
   (void)ws;
   TNX_REQUIRE(logits && step_ptr && ids_out, "sample_topk: null pointer");
   TNX_REQUIRE(M > 0 && V > 0 && V < (1ll << 31), "sample_topk: bad shape");
   TNX_REQUIRE(rng_variant == 0 || rng_variant == 1, "sample_topk: rng_variant must be 0 or 1");
+  TNX_REQUIRE(temperature > 0.f, "sample_topk: temperature must be positive, got %f", temperature);
   if (k <= 0 || k >= V) {
     if (top_p < 1.0f) {
       tnx_set_error("sample_topk: top_p < 1 without top_k needs a full-vocabulary sort (not built)");
@@ -288,7 +297,8 @@ extern "C" int tnx_sample_topk(void* stream, const float* logits, int64_t M, int
   }
   TNX_REQUIRE(k <= NTH, "sample_topk: top_k=%d exceeds %d", k, NTH);
   hipLaunchKernelGGL(sample_topk_kernel, dim3((unsigned)M), dim3(NTH), 0, as_stream(stream), logits,
-                     V, k, top_p, key0, key1, rng_variant, step_ptr, M, ids_out, logp_out);
+                     V, k, top_p, key0, key1, rng_variant, step_ptr, M, temperature, forbidden,
+                     forbidden ? n_forbidden : 0, ids_out, logp_out);
   TNX_CHECK_LAUNCH("sample_topk");
   return TNX_OK;
 }

@@ -75,7 +75,7 @@ class Sampler:
     self.cache_config = cache_config
     self.use_graph = use_graph
     self.prefill_rows = prefill_rows
-    self.rng_variant = 1  # threefry "partitionable" bit stream (the jax default)
+    self.rng_variant = 0  # threefry random_bits layout that reproduces the reference's golden arrays
     self.last_stats: dict = {}
 
   @property
@@ -115,10 +115,10 @@ class Sampler:
                       forbidden=mode["forbidden"], logits_out=runner.logits)
       ids, lp = runner.best_id, (runner.best_logp if want_lp else None)
     else:
-      runner.run_head(x, runner.B, temperature=mode["temperature"], best_id=runner.best_id,
-                      forbidden=mode["forbidden"], logits_out=runner.logits)
-      ops.sample_topk(runner.logits, mode["top_k"], mode["top_p"], mode["key"], self.rng_variant,
-                      st.step, mode["ws"], mode["ids"], mode["logp"])
+      runner.run_head(x, runner.B, best_id=runner.best_id, logits_out=runner.logits)
+      ops.sample_topk(runner.logits, mode["top_k"], mode["top_p"], mode["temperature"], mode["key"],
+                      self.rng_variant, st.step, mode["ws"], mode["ids"], mode["logp"],
+                      forbidden=mode["forbidden"])
       ids, lp = mode["ids"], (mode["logp"] if want_lp else None)
     ops.sample_commit(ids, lp, st.token_buffer, st.logprobs_buffer, st.done, mode["eos"], st.step)
 

@@ -241,8 +241,15 @@ class Runner:
       self.y_route = torch.empty(M * k, D, dtype=bf, device=dev)
     else:
       self.act = torch.empty(M, F, dtype=bf, device=dev)
-    nmax = max(nqkv, D, 2 * F if not cfg.num_experts else D)
-    self.splitk_ws = torch.zeros(M * nmax, dtype=torch.float32, device=dev)
+    self.split_k_override = {}
+    need = 1
+    for ly in model.layers:
+      for key in ("qkv", "o", "gu", "down"):
+        if key in ly:
+          sk = self._split_k(ly[key], M)
+          if sk > 1:
+            need = max(need, sk * M * ly[key].N)
+    self.splitk_ws = torch.empty(need, dtype=torch.float32, device=dev)
     if kv_chunk is None:
       kv_chunk = 256 if (T == 1 and S > 256) else 0
     self.kv_chunk = kv_chunk
@@ -258,7 +265,6 @@ class Runner:
     self.best_logp = torch.empty(B, dtype=torch.float32, device=dev)
     self.logits = (torch.empty(B, cfg.vocab_size, dtype=torch.float32, device=dev)
                    if want_logits else None)
-    self.split_k_override = {}
 
   # ---- building blocks -----------------------------------------------------------------------
   def _split_k(self, f: FusedLinear, M: int) -> int:

@@ -123,11 +123,15 @@ def lmhead(desc: L.LmHeadDesc):
   L.check(L.lib().tnx_lmhead_logp(_stream(), C.byref(desc)), "tnx_lmhead_logp")
 
 
-def sample_topk(logits, k, top_p, key, rng_variant, step_ptr, ws, ids_out, logp_out):
+def sample_topk(logits, k, top_p, temperature, key, rng_variant, step_ptr, ws, ids_out, logp_out,
+                forbidden=None):
+  """logits: raw fp32 [M,V]; they are divided by `temperature` inside the kernel."""
   M, V = logits.shape
-  L.check(L.lib().tnx_sample_topk(_stream(), _ptr(logits), M, V, k, float(top_p), key[0], key[1],
-                                  rng_variant, _ptr(step_ptr), _ptr(ws), _ptr(ids_out),
-                                  _ptr(logp_out)), "tnx_sample_topk")
+  L.check(L.lib().tnx_sample_topk(_stream(), _ptr(logits), M, V, k, float(top_p),
+                                  float(temperature), key[0], key[1], rng_variant,
+                                  _ptr(forbidden), 0 if forbidden is None else forbidden.numel(),
+                                  _ptr(step_ptr), _ptr(ws), _ptr(ids_out), _ptr(logp_out)),
+          "tnx_sample_topk")
 
 
 def sample_commit(ids, logp, tokens, logprobs, done, eos, step_ptr):
