@@ -1,0 +1,274 @@
+"""Decode throughput of the quantized rollout path on one MI355X.
+
+`python bench.py --gpus 1 --steps K --warmup W` builds the Llama-3.1-8B-shaped NF4 QLoRA model
+(random-init weights, synthetic prompts), prefills batch 128 x prompt 512, runs W untimed decode
+steps and times exactly K decode steps (one captured HIP graph replayed K times), then prints ONE
+JSON line.  A "step" is one decode step of the whole batch: embedding -> 32 layers -> lm_head ->
+greedy sampling -> token commit.
+
+Extra objects on the line:
+  roofline      the kernel with the largest share of a step, timed in isolation with events on
+                the launch stream at the mean context of the timed region
+  kernels       the same measurement for every kernel family of the step
+  cpu_baseline  the CPU oracle (a port of the reference's JAX path) timed on this host on a
+                bounded sample and scaled linearly
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+  sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def log(*a):
+  print(*a, file=sys.stderr, flush=True)
+
+
+def time_loop(fn, iters, warm=3):
+  import torch
+  for _ in range(warm):
+    fn()
+  e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+  torch.cuda.synchronize()
+  e0.record()
+  for _ in range(iters):
+    fn()
+  e1.record()
+  torch.cuda.synchronize()
+  return e0.elapsed_time(e1) / iters  # ms
+
+
+def kernel_breakdown(model, runner, st, ctx, iters):
+  """Times each kernel family of one layer in isolation (events on the launch stream)."""
+  import torch
+
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  cfg = model.cfg
+  B, S = runner.B, runner.S
+  ly = model.layers[0]
+  col = torch.tensor([ctx - 1], dtype=torch.int32, device=model.device)
+  out = {}
+
+  def attn():
+    ad = L.AttnDesc()
+    ad.B, ad.T, ad.S = B, 1, S
+    ad.Hq, ad.Hkv, ad.dh = cfg.num_heads, cfg.num_kv_heads, cfg.head_dim
+    ad.scale, ad.window, ad.pad_id = cfg.head_dim ** -0.5, 0, runner.pad_id
+    ad.q, ad.kcache, ad.vcache = runner.q.data_ptr(), st.kcache[0].data_ptr(), st.vcache[0].data_ptr()
+    ad.tokens, ad.tok_ld, ad.col_ptr = st.token_buffer.data_ptr(), st.token_buffer.shape[1], col.data_ptr()
+    ad.kv_chunk, ad.ws, ad.out = runner.kv_chunk, runner.attn_ws.data_ptr(), runner.attn.data_ptr()
+    ops.gqa_attn(ad)
+
+  kv_bytes = B * cfg.num_kv_heads * ctx * cfg.head_dim * 2 * 2
+  out["gqa_attn"] = {"ms": time_loop(attn, iters), "bytes": kv_bytes, "flops": 0, "per_step": cfg.num_layers}
+
+  def lin(key, x, y, epi=L.TNX_EPI_STORE, residual=None):
+    f = ly[key]
+    nbytes = f.codes.numel() * 4 + f.scales.numel() * 2
+    if f.has_lora:
+      nbytes += (f.K * f.r * len(f.names) + f.N * f.r) * 2
+    nbytes += B * f.K * 2 + B * (f.N // (2 if f.interleave2 else 1)) * 2
+    ms = time_loop(lambda: runner.linear(f, x, y, B, epilogue=epi, residual=residual), iters)
+    return {"ms": ms, "bytes": nbytes, "flops": 2.0 * B * f.K * f.N, "per_step": cfg.num_layers}
+
+  out["qlinear_qkv"] = lin("qkv", runner.xn, runner.qkv)
+  out["qlinear_o"] = lin("o", runner.attn, runner.tmp)
+  out["qlinear_gate_up"] = lin("gu", runner.xn, runner.act, L.TNX_EPI_SILU_MUL)
+  out["qlinear_down"] = lin("down", runner.act, runner.tmp)
+  head_bytes = model.weight_bytes()["head"] + B * cfg.embed_dim * 2
+  ms = time_loop(lambda: runner.run_head(runner.xn, B, best_id=runner.best_id,
+                                         best_logp=runner.best_logp), iters)
+  out["lmhead_logp"] = {"ms": ms, "bytes": head_bytes, "flops": 2.0 * B * cfg.embed_dim * cfg.vocab_size,
+                        "per_step": 1}
+  for v in out.values():
+    v["gbs"] = v["bytes"] / (v["ms"] * 1e-3) / 1e9
+    v["tflops"] = v["flops"] / (v["ms"] * 1e-3) / 1e12
+    v["step_ms"] = v["ms"] * v["per_step"]
+  return out
+
+
+def cpu_baseline(cfg_full, B, ctx, S, threads):
+  """CPU oracle on a bounded sample: 1 layer x 2 decode steps at context `ctx` + the lm_head,
+  scaled linearly to the full depth."""
+  import dataclasses
+
+  import numpy as np
+  import torch
+
+  from oracle import model_ref
+  from oracle import utils_ref
+  from tunix_amd import dummy_model
+  torch.set_num_threads(threads)
+  cfg = dataclasses.replace(cfg_full, num_layers=1, vocab_size=1024)
+  w = dummy_model.create_dummy_weights(cfg, seed=3)
+  ref = model_ref.RefModel(cfg, w, bf16=True, acc=torch.float32)
+  cache = ref.init_cache(B, S)
+  for k, v in cache:
+    k.normal_()
+    v.normal_()
+  tokens = torch.randint(1, cfg.vocab_size, (B, 1))
+  positions = torch.full((B, 1), ctx - 1, dtype=torch.int64)
+  mask = torch.from_numpy(utils_ref.compute_attention_masks(ctx - 1, S, np.zeros((B, S), dtype=bool)))
+  x = ref.embed(tokens)
+  ref.layer(0, x, positions, cache, mask, ctx - 1)  # warm
+  t0 = time.perf_counter()
+  n = 2
+  for _ in range(n):
+    ref.layer(0, x, positions, cache, mask, ctx - 1)
+  t_layer = (time.perf_counter() - t0) / n
+  D, V = cfg_full.embed_dim, cfg_full.vocab_size
+  head = (torch.randn(D, V // 8) * 0.02).to(torch.bfloat16).float()
+  h = torch.randn(B, D).to(torch.bfloat16).float()
+  t0 = time.perf_counter()
+  for _ in range(2):
+    lg = (h @ head).to(torch.bfloat16).float()
+    lg.argmax(-1)
+  t_head = (time.perf_counter() - t0) / 2 * 8
+  t_step = cfg_full.num_layers * t_layer + t_head
+  return {"value": B / t_step, "unit": "tokens/s", "cores": threads, "kind": "port",
+          "sample": (f"1 of {cfg_full.num_layers} layers x {n} decode steps at context {ctx} "
+                     f"(dense mask over the {S}-slot cache, fp32 torch matmuls) + 1/8 of the lm_head "
+                     "columns, scaled linearly (extrapolated)"),
+          "layer_s": t_layer, "head_s": t_head}
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=508)
+  ap.add_argument("--warmup", type=int, default=3)
+  ap.add_argument("--batch", type=int, default=128)
+  ap.add_argument("--prompt", type=int, default=512)
+  ap.add_argument("--gen", type=int, default=512)
+  ap.add_argument("--layers", type=int, default=0, help="debug only: fewer layers (invalidates the metric)")
+  ap.add_argument("--no-cpu-baseline", action="store_true")
+  ap.add_argument("--kernel-iters", type=int, default=20)
+  args = ap.parse_args()
+  if args.gpus != 1:
+    print("bench.py measures one GPU: this build has no multi-GPU path (the decode path shards "
+          "by batch rows with no exchange); run with --gpus 1", file=sys.stderr)
+    sys.exit(2)
+
+  import numpy as np
+  import torch
+
+  from tunix_amd import config, dummy_model
+  from tunix_amd.generate import CacheConfig, Sampler
+  from tunix_amd.generate.sampler import _SamplingState
+  from tunix_amd.generate.utils import IdTokenizer
+  from tunix_amd.model import QLoRAModel, Runner
+
+  assert torch.cuda.is_available(), "bench.py needs a GPU"
+  dev = torch.device("cuda:0")
+  cfg = config.llama31_8b()
+  if args.layers:
+    cfg = config.llama31_8b(num_layers=args.layers)
+  B, P, T = args.batch, args.prompt, args.gen
+  S = P + T
+  W = max(1, args.warmup)
+  K = args.steps
+  if W + K > T - 1:
+    K = T - 1 - W
+    log(f"steps clamped to {K}: a rollout of {T} tokens has {T - 1} decode steps")
+
+  t0 = time.time()
+  weights = dummy_model.create_dummy_weights(cfg, seed=20253, device=dev)
+  model = QLoRAModel(cfg, weights, dev)
+  del weights
+  torch.cuda.empty_cache()
+  log(f"model built in {time.time() - t0:.1f}s; bytes per step {model.weight_bytes()}")
+
+  pad = 0
+  tok = IdTokenizer(cfg.vocab_size, pad_id=pad, eos_id=1)
+  sampler = Sampler(model, tok, CacheConfig(S, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim))
+  rng = np.random.Generator(np.random.PCG64(20253))
+  ids = rng.integers(1, cfg.vocab_size, size=(B, P)).astype(np.int32)
+  st = _SamplingState(model, ids, S, S, pad, False, False)
+  mode = {"name": "greedy", "forbidden": None, "eos": torch.tensor([-1], dtype=torch.int32, device=dev)}
+  runner = Runner(model, B, 1, S, pad)
+  torch.cuda.synchronize()
+  t0 = time.time()
+  sampler._prefill(st, runner, mode, False)
+  torch.cuda.synchronize()
+  prefill_s = time.time() - t0
+  log(f"prefill {B}x{P}: {prefill_s:.2f}s")
+
+  for _ in range(W):
+    sampler._decode_step(runner, st, mode)
+  graph = torch.cuda.CUDAGraph()
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):
+    with torch.cuda.graph(graph, stream=side):
+      sampler._decode_step(runner, st, mode)
+  torch.cuda.current_stream().wait_stream(side)
+  torch.cuda.synchronize()
+  step_first = int(st.step.item())
+  t0 = time.perf_counter()
+  for _ in range(K):
+    graph.replay()
+  torch.cuda.synchronize()
+  dt = time.perf_counter() - t0
+  step_last = int(st.step.item())
+  assert step_last - step_first == K, (step_first, step_last, K)
+  ms_per_step = dt / K * 1e3
+  value = B * K / dt
+  mean_ctx = (step_first + 1 + step_last) / 2.0 + 0.5
+  log(f"decode: {K} steps, {ms_per_step:.3f} ms/step, {value:.0f} tokens/s, mean context {mean_ctx:.1f}")
+
+  kern = kernel_breakdown(model, runner, st, int(round(mean_ctx)), args.kernel_iters)
+  for name, v in kern.items():
+    log(f"  {name:16s} {v['ms'] * 1e3:8.1f} us/launch  {v['gbs']:7.0f} GB/s  {v['tflops']:7.1f} TFLOP/s"
+        f"  x{v['per_step']} = {v['step_ms']:.3f} ms/step")
+  dom_name = max(kern, key=lambda k: kern[k]["step_ms"])
+  dom = kern[dom_name]
+  hbm_frac = dom["gbs"] / HBM_PEAK_GBS
+  roofline = {"kernel": dom_name, "bound": "hbm", "achieved": round(dom["gbs"], 1),
+              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(hbm_frac, 4), "traffic": None,
+              "us_per_launch": round(dom["ms"] * 1e3, 2), "algorithmic_bytes": dom["bytes"]}
+  lin_bytes = sum(kern[k]["bytes"] for k in kern if k.startswith("qlinear"))
+  lin_ms = sum(kern[k]["ms"] for k in kern if k.startswith("qlinear"))
+  lin_flops = sum(kern[k]["flops"] for k in kern if k.startswith("qlinear"))
+  roofline_linears = {
+      "bound": "hbm", "achieved": round(lin_bytes / (lin_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
+      "unit": "GB/s", "frac": round(lin_bytes / (lin_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+      "mfma_tflops": round(lin_flops / (lin_ms * 1e-3) / 1e12, 1),
+      "mfma_frac": round(lin_flops / (lin_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+  wb = model.weight_bytes()
+  step_bytes = (wb["quantized"] + wb["lora"] + wb["head"]
+                + B * cfg.num_kv_heads * mean_ctx * cfg.head_dim * 4 * cfg.num_layers)
+  result = {
+      "metric": "decode tokens/sec @1 MI355X (8B NF4 QLoRA, bs128); % HBM roofline",
+      "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
+      "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+      "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+      "config": {"workload": "Llama-3.1-8B-shaped NF4(g64)+LoRA r64 greedy rollout decode",
+                 "layers": cfg.num_layers, "global_batch": B, "prompt_len": P, "gen_len": T,
+                 "context_range": [step_first + 1, step_last + 1], "parallelism": "single GPU"},
+      "hbm_roofline_frac_step": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+      "step_bytes": int(step_bytes), "prefill_s": round(prefill_s, 3),
+      "roofline": roofline, "roofline_linears": roofline_linears,
+      "kernels": {k: {"us": round(v["ms"] * 1e3, 2), "GBps": round(v["gbs"], 1),
+                      "TFLOPs": round(v["tflops"], 1), "ms_per_step": round(v["step_ms"], 4)}
+                  for k, v in kern.items()},
+  }
+  if not args.no_cpu_baseline:
+    threads = min(16, os.cpu_count() or 1)
+    t0 = time.time()
+    result["cpu_baseline"] = cpu_baseline(cfg, B, int(round(mean_ctx)), S, threads)
+    log(f"cpu baseline took {time.time() - t0:.1f}s: {result['cpu_baseline']['value']:.2f} tokens/s")
+  print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+  main()

@@ -68,14 +68,15 @@ int tnx_version(void);
  * per output column: scale[g,n] = bf16(absmax / 7) (INT4) or bf16(absmax) (NF4); the code of
  * an element is the nearest code-book entry of w / f32(scale) (round-half-even for INT4,
  * clamped to [-8,7]; nearest level, ties to the lower code, for NF4).  The value a kernel
- * uses is   level(code) * f32(scale)   with products accumulated in fp32 per group:
- *     y[m,n] = sum_g f32(scale[g,n]) * ( sum_{k in g} x[m,k] * bf16(level(code[k,n])) ).
+ * uses is the weight dequantised to bf16,  w^[k,n] = bf16( bf16(level(code)) * scale[g(k),n] ),
+ * multiplied into bf16 activations with fp32 accumulation:  y[m,n] = sum_k x[m,k] * w^[k,n].
  *
  * Storage: N is padded to a multiple of 16 and K to a multiple of 128. Codes are tiled as
  * [N/16][K/128][64 lanes][4 dwords]; lane l of a tile owns column n = 16*nt + l%16; its dword
  * j holds the 8 codes of k = 128*kt + 32*j + 8*(l/16) + i, i = 0..7, code i in bits 4i..4i+3.
- * Scales are tiled as [N/16][K/128][S][16] bf16 with S = max(1, 128/group) scales per tile
- * and column (group > 128: the tile's scale is repeated).
+ * Scales are tiled as [N/16][K/128][16][S] bf16 with S = max(2, 128/group) slots per k-tile
+ * and column, slot s holding the scale of k = 128*kt + s*(128/S) .. (a group wider than a slot
+ * repeats its scale), so that a lane reads its scales as one aligned 4- or 8-byte word.
  * tnx_qw_sizes() gives the byte sizes; tnx_quantize_pack() produces both arrays on device.
  * ------------------------------------------------------------------------------------- */
 int tnx_qw_sizes(int64_t K, int64_t N, int group, size_t* codes_bytes, size_t* scales_bytes);
@@ -87,7 +88,7 @@ int tnx_qw_sizes(int64_t K, int64_t N, int group, size_t* codes_bytes, size_t* s
 int tnx_quantize_pack(void* stream, const void* w, int w_is_f32, int64_t K, int64_t N,
                       int group, int qtype, int interleave2, uint32_t* codes, uint16_t* scales);
 
-/* Inverse of the packing for tests and export: w_out fp32 [K,N] = level * scale. */
+/* Inverse of the packing for tests and export: w_out fp32 [K,N] = w^ (bf16 values). */
 int tnx_qw_dequant(void* stream, const uint32_t* codes, const uint16_t* scales, int64_t K,
                    int64_t N, int group, int qtype, int interleave2, float* w_out);
 

@@ -8,8 +8,9 @@ reference tree, so this file restates the format that include/tunix_hip.h define
                 consecutive K indices per output column n
   code        = clamp(rint(w / f32(scale)), -8, 7) + 8   (int4, round-half-even)
               = index of the nearest NF4 level of w / f32(scale), ties to the lower code
-  value       = bf16(level(code)) * f32(scale), products accumulated per group in fp32:
-                y[m, n] = sum_g scale[g, n] * sum_{k in g} x[m, k] * bf16(level(code[k, n]))
+  value       = w^[k, n] = bf16(bf16(level(code)) * scale): the weight "dequantised to bf16"
+                (qvalue.astype(scale dtype) * scale), then a bf16 matmul with fp32 accumulation:
+                y[m, n] = sum_k x[m, k] * w^[k, n]
   LoRA        y += (alpha / rank) * bf16(x @ A) @ B        (tunix/models/safetensors_saver.py:107
                                                             W_eff = W + (A @ B) * alpha / rank)
 
@@ -54,7 +55,8 @@ def quantize(w: np.ndarray, group: int, qtype: int) -> tuple[np.ndarray, np.ndar
   xn = (wg / safe[:, None, :]).astype(np.float32)
   if qtype == NF4:
     mids = (np.float32(0.5) * (NF4_LEVELS[:-1] + NF4_LEVELS[1:])).astype(np.float32)
-    codes = (xn[..., None] > mids).sum(axis=-1).astype(np.uint8)
+    # number of midpoints strictly below x == index of the nearest level, ties to the lower code
+    codes = np.searchsorted(mids, xn, side="left").astype(np.uint8)
     codes = np.where(scale[:, None, :] == 0, np.uint8(7), codes)
   else:
     q = np.clip(np.rint(xn), -8, 7)
@@ -65,13 +67,15 @@ def quantize(w: np.ndarray, group: int, qtype: int) -> tuple[np.ndarray, np.ndar
 
 def dequantize(codes: np.ndarray, scale: np.ndarray, group: int, qtype: int,
                round_levels: bool = True) -> np.ndarray:
-  """fp32 [K, N]: bf16(level) * scale (round_levels=False keeps the fp32 level)."""
+  """fp32 [K, N]: bf16(bf16(level) * scale); round_levels=False is the fp32 reference mode
+  (fp32 level * scale, no rounding)."""
   lv = levels(qtype)
   if round_levels:
     lv = rb_np(lv)
   K, N = codes.shape
   s = np.repeat(scale, group, axis=0)
-  return (lv[codes].astype(np.float64) * s.astype(np.float64)).astype(np.float32)
+  w = (lv[codes].astype(np.float64) * s.astype(np.float64)).astype(np.float32)
+  return rb_np(w) if round_levels else w
 
 
 def qlinear_lora(x: torch.Tensor, codes: np.ndarray, scale: np.ndarray, group: int, qtype: int,
@@ -82,11 +86,7 @@ def qlinear_lora(x: torch.Tensor, codes: np.ndarray, scale: np.ndarray, group: i
   bf16=True follows the kernel's dtype flow (bf16 level, bf16 t); bf16=False is the
   fp32 reference mode (fp32 levels, no rounding of t).
   """
-  lv = levels(qtype)
-  if bf16:
-    lv = rb_np(lv)
-  wd = torch.from_numpy(lv[codes].astype(np.float64)) * torch.from_numpy(
-      np.repeat(scale, group, axis=0).astype(np.float64))
+  wd = torch.from_numpy(dequantize(codes, scale, group, qtype, round_levels=bf16))
   y = x.to(acc) @ wd.to(acc)
   if lora_a is not None:
     t = (x.to(acc) @ lora_a.to(acc)).to(torch.float32)
@@ -110,7 +110,8 @@ def pack_qw(codes: np.ndarray, scale: np.ndarray, group: int, interleave2: bool 
   K, N = codes.shape
   assert K % 128 == 0 and N % 16 == 0
   ktiles, ntiles = K // 128, N // 16
-  spt = 1 if group >= 128 else 128 // group
+  spt = 2 if group >= 64 else 128 // group   # scale slots per k-tile and column
+  slot_w = 128 // spt
   pc = packed_col(np.arange(N), N, interleave2)
   cp = np.empty_like(codes)
   cp[:, pc] = codes
@@ -123,10 +124,7 @@ def pack_qw(codes: np.ndarray, scale: np.ndarray, group: int, interleave2: bool 
       torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
   sp = np.empty_like(sbits)
   sp[:, pc] = sbits
-  if group >= 128:
-    rep = np.repeat(sp, group // 128, axis=0)          # one scale per k-tile
-    st = rep.reshape(ktiles, 1, ntiles, 16)
-  else:
-    st = sp.reshape(ktiles, spt, ntiles, 16)
-  out_scales = st.transpose(2, 0, 1, 3).reshape(-1)
+  per_slot = np.repeat(sp, group, axis=0)[::slot_w]      # [K / slot_w, N]
+  st = per_slot.reshape(ktiles, spt, ntiles, 16)
+  out_scales = st.transpose(2, 0, 3, 1).reshape(-1)       # [nt][kt][16][spt]
   return out_codes, np.ascontiguousarray(out_scales)

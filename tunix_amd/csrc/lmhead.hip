@@ -57,7 +57,7 @@ __global__ __launch_bounds__(256) void lmhead_kernel(const LHArgs a) {
   constexpr int NT = 2;
   extern __shared__ __align__(16) unsigned char smem[];
   uint16_t* sA = reinterpret_cast<uint16_t*>(smem);
-  uint32_t* sLut = reinterpret_cast<uint32_t*>(smem + MT * 16 * A_LD * sizeof(uint16_t));
+  uint32_t* sLut = tile_lut(smem, MT);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lm = lane & 15, lq = lane >> 4;
   const int64_t vb = blockIdx.x;
@@ -70,7 +70,8 @@ __global__ __launch_bounds__(256) void lmhead_kernel(const LHArgs a) {
     lut_lane = sLut + (lane & (TNX_LUT_COPIES - 1));
   }
   TileSrc s;
-  s.M = a.M; s.K = a.D; s.x = a.x; s.row_index = nullptr; s.row_div = 1; s.w_bf16 = a.w_bf16;
+  s.M = a.M; s.K = a.D; s.x = a.x; s.row_index = nullptr; s.row_div = 1; s.x_rows = a.M;
+  s.w_bf16 = a.w_bf16;
   s.codes = a.codes; s.scales = a.scales; s.group = a.group; s.qtype = a.qtype;
   s.ntiles = a.V / 16; s.lora_rank = a.lora_rank; s.t = a.t; s.t_ld = a.t_ld;
   s.lora_b = a.lora_b; s.lora_scale = a.lora_scale;
@@ -219,6 +220,9 @@ extern "C" int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* d) {
               (long long)d->D, (long long)d->V);
   TNX_REQUIRE(d->M <= 65535LL * 128, "lmhead: too many rows in one call");
   TNX_REQUIRE(d->x && d->part, "lmhead: null pointer");
+  TNX_REQUIRE((uint64_t)(d->M + 128) * (uint64_t)d->D * 2 < (1ull << 32) &&
+                  (uint64_t)d->V * (uint64_t)d->D * 2 < (1ull << 32),
+              "lmhead: x and the head weights must stay below 4 GiB each (32-bit buffer offsets)");
   TNX_REQUIRE(d->w_bf16 || (d->codes && d->scales), "lmhead: no head weights");
   if (!d->w_bf16) {
     int rc = tnx_qw_sizes(d->D, d->V, d->group, nullptr, nullptr);

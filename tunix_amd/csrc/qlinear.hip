@@ -119,7 +119,7 @@ template <int MT, int NT>
 __global__ __launch_bounds__(256) void qlinear_kernel(const QLArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   uint16_t* sA = reinterpret_cast<uint16_t*>(smem);  // [16*MT][A_LD]
-  uint32_t* sLut = reinterpret_cast<uint32_t*>(smem + MT * 16 * A_LD * sizeof(uint16_t));
+  uint32_t* sLut = tile_lut(smem, MT);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t m0 = (int64_t)blockIdx.x * (MT * 16);
   const int64_t ntile0 = ((int64_t)blockIdx.y * 4 + wave) * NT;
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(256) void qlinear_kernel(const QLArgs a) {
   const uint32_t* lut_lane = sLut + (lane & (TNX_LUT_COPIES - 1));
 
   TileSrc s;
-  s.M = a.M; s.K = a.K; s.x = a.x; s.row_index = nullptr; s.row_div = 1; s.w_bf16 = nullptr;
+  s.M = a.M; s.K = a.K; s.x = a.x; s.row_index = nullptr; s.row_div = 1; s.x_rows = a.M; s.w_bf16 = nullptr;
   s.codes = a.codes; s.scales = a.scales; s.group = a.group; s.qtype = a.qtype;
   s.ntiles = a.N / 16; s.lora_rank = a.lora_rank; s.t = a.t; s.t_ld = a.t_ld;
   s.lora_b = a.lora_b; s.lora_scale = a.lora_scale;
@@ -169,7 +169,7 @@ template <int MT, int NT>
 __global__ __launch_bounds__(256) void moe_gmm_kernel(const QLArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   uint16_t* sA = reinterpret_cast<uint16_t*>(smem);
-  uint32_t* sLut = reinterpret_cast<uint32_t*>(smem + MT * 16 * A_LD * sizeof(uint16_t));
+  uint32_t* sLut = tile_lut(smem, MT);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int e = blockIdx.x;
   const int r_begin = a.offsets[e], r_end = a.offsets[e + 1];
@@ -182,7 +182,7 @@ __global__ __launch_bounds__(256) void moe_gmm_kernel(const QLArgs a) {
 
   TileSrc s;
   s.M = r_end - r_begin; s.K = a.K; s.x = a.x; s.row_index = a.sorted_route + r_begin;
-  s.row_div = a.x_div; s.w_bf16 = nullptr;
+  s.row_div = a.x_div; s.x_rows = a.M / a.x_div; s.w_bf16 = nullptr;
   s.codes = a.codes + (int64_t)e * a.codes_stride; s.scales = a.scales + (int64_t)e * a.scales_stride;
   s.group = a.group; s.qtype = a.qtype; s.ntiles = a.N / 16; s.lora_rank = 0; s.t = nullptr;
   s.t_ld = 0; s.lora_b = nullptr; s.lora_scale = 0.f;
@@ -196,6 +196,225 @@ __global__ __launch_bounds__(256) void moe_gmm_kernel(const QLArgs a) {
   const int32_t* routes = s.row_index;
   store_tile<MT, NT>(a, m0, s.M, ntile0, s.ntiles, acc,
                      [routes](int64_t r) { return (int64_t)routes[r]; });
+}
+
+// ---- the rollout-batch kernel: 65..128 rows -----------------------------------------------
+// Eight waves per work-group: waves 0-3 and 4-7 each own the 128 x 128 output tile (wave tile
+// 128 x 32) for every other k-tile, so that each SIMD holds two waves whose MFMA and
+// dequantisation streams interleave.  The two partial tiles are summed through LDS and each
+// half then finishes 64 rows (LoRA delta + epilogue).  The code-book table is replicated 64
+// times with a 256-byte entry stride, which makes the LDS address of a code byte a single
+// v_perm_b32: (byte << 8) | (lane << 2).
+constexpr int kLut64Bytes = 256 * 256;
+constexpr size_t kM128SmemBytes = kLut64Bytes + 2 * (size_t)128 * A_LD * sizeof(uint16_t);
+
+template <int BYTE>
+__device__ __forceinline__ uint32_t lut64_pair(const unsigned char* lut, uint32_t w, uint32_t lane_off) {
+  // bytes of the address: [0] = lane_off, [1] = byte BYTE of w, [2] = [3] = 0
+  const uint32_t addr = __builtin_amdgcn_perm(w, lane_off, 0x0c0c0000u | ((4u + BYTE) << 8));
+  return *reinterpret_cast<const uint32_t*>(lut + addr);
+}
+__device__ __forceinline__ u32x4 dequant8_lut64(uint32_t w, const unsigned char* lut,
+                                                uint32_t lane_off, float scale) {
+  const uint32_t p0 = lut64_pair<0>(lut, w, lane_off), p1 = lut64_pair<1>(lut, w, lane_off);
+  const uint32_t p2 = lut64_pair<2>(lut, w, lane_off), p3 = lut64_pair<3>(lut, w, lane_off);
+  u32x4 r;
+  r[0] = cvt_pk_bf16(bflo(p0) * scale, bfhi(p0) * scale);
+  r[1] = cvt_pk_bf16(bflo(p1) * scale, bfhi(p1) * scale);
+  r[2] = cvt_pk_bf16(bflo(p2) * scale, bfhi(p2) * scale);
+  r[3] = cvt_pk_bf16(bflo(p3) * scale, bfhi(p3) * scale);
+  return r;
+}
+
+__global__ __launch_bounds__(512) void qlinear_m128_kernel(const QLArgs a) {
+  constexpr int NT = 2, MT = 8, PF = 3;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int grp = wave >> 2, wn = wave & 3, gtid = tid & 255;
+  const int lm = lane & 15, lq = lane >> 4;
+  uint16_t* sA = reinterpret_cast<uint16_t*>(smem + kLut64Bytes) + grp * (128 * A_LD);
+  {  // table: thread (byte, half) writes 32 of the 64 copies of its entry, rotated over banks
+    uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
+    const int byte = tid & 255, c0 = (tid >> 8) * 32;
+    const uint32_t v = pack2bf(code_level(a.qtype, byte & 15), code_level(a.qtype, byte >> 4));
+#pragma unroll
+    for (int c = 0; c < 32; ++c) lut[byte * 64 + c0 + ((c + lane) & 31)] = v;
+  }
+  const uint32_t lane_off = (uint32_t)lane * 4u;
+  const int64_t m0 = (int64_t)blockIdx.x * 128;
+  const int64_t ntile0 = ((int64_t)blockIdx.y * 4 + wn) * NT;
+  const int64_t ntiles = a.N / 16;
+  const int ktiles = (int)(a.K / KTILE);
+  const int kt_begin = blockIdx.z * a.ktiles_per_split;
+  const int kt_end = min(ktiles, kt_begin + a.ktiles_per_split);
+  const int n_it = (kt_end - kt_begin + 1) / 2;  // group g takes k-tiles kt_begin + 2*it + g
+  const int spt = scales_per_tile(a.group);
+
+  TileSrc s;
+  s.M = a.M; s.K = a.K; s.x = a.x; s.row_index = nullptr; s.row_div = 1; s.x_rows = a.M;
+  s.w_bf16 = nullptr; s.codes = a.codes; s.scales = a.scales; s.group = a.group; s.qtype = a.qtype;
+  s.ntiles = ntiles; s.lora_rank = a.lora_rank; s.t = a.t; s.t_ld = a.t_ld; s.lora_b = a.lora_b;
+  s.lora_scale = a.lora_scale;
+  const rsrc_t rx = make_rsrc(a.x, (uint64_t)a.M * a.K * 2);
+  const uint64_t ntk = (uint64_t)ntiles * ktiles;
+  const rsrc_t rc = make_rsrc(a.codes, ntk * 1024);
+  const rsrc_t rs = make_rsrc(a.scales, ntk * 16 * spt * 2 + 16);
+
+  f32x4 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) zero_acc(acc[mt][nt]);
+
+  u32x4 a_next[MT];
+  u32x4 ring_c[PF][NT];
+  u32x2 ring_s[PF][NT];
+  auto load_w = [&](u32x4 (&c)[NT], u32x2 (&sc)[NT], int kt) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      // 32-bit offsets: the host checks that codes and scales are below 4 GiB
+      const uint32_t tile = (uint32_t)(ntile0 + nt) * (uint32_t)ktiles + (uint32_t)kt;
+      c[nt] = buf_load128(rc, tile * 1024u + (uint32_t)lane * 16u);
+      // always 8 bytes (the upper half is the next column when there are two slots): no
+      // control flow around loads, so that the waits on them can be counted exactly
+      sc[nt] = __builtin_amdgcn_raw_buffer_load_b64(rs, (tile * 16u + (uint32_t)lm) * (uint32_t)spt * 2u, 0, 0);
+    }
+  };
+  auto my_kt = [&](int it) { return kt_begin + 2 * it + grp; };
+  // Loads are never predicated: k-tiles past the end read neighbouring or out-of-range (zero)
+  // data that is never used, and the iteration count is padded to a multiple of PF.
+  load_a<MT>(s, rx, m0, my_kt(0), gtid, a_next);
+#pragma unroll
+  for (int d = 0; d < PF; ++d) load_w(ring_c[d], ring_s[d], my_kt(d));
+
+  for (int it0 = 0; it0 < n_it; it0 += PF) {
+#pragma unroll
+    for (int d = 0; d < PF; ++d) {
+      const int it = it0 + d;
+      {
+        const int kt = my_kt(it);
+        const bool active = kt < kt_end;
+        __syncthreads();  // every wave is done reading its group's activation tile
+        if (active) store_a<MT>(sA, gtid, a_next);
+        u32x4 cw[NT];
+        float sc[NT][4];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          cw[nt] = ring_c[d][nt];
+          const u32x2 p = ring_s[d][nt];
+          const float f[4] = {bflo(p[0]), bfhi(p[0]), bflo(p[1]), bfhi(p[1])};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) sc[nt][j] = spt == 2 ? f[j >> 1] : f[j];
+        }
+        __syncthreads();
+        // activations of the next k-tile first, then the weights PF tiles ahead
+        load_a<MT>(s, rx, m0, my_kt(it + 1), gtid, a_next);
+        load_w(ring_c[d], ring_s[d], my_kt(it + PF));
+        if (active) {
+          // Software pipeline over the 8 half-steps (k-step j, row half h) of the k-tile: the
+          // LDS reads of a half-step (4 A fragments; the 8 table entries of the next k-step)
+          // are issued one half-step (8 MFMAs) ahead of their use, so that the LDS latency
+          // hides behind the matrix pipe instead of stalling every MFMA.
+          auto read_a = [&](u32x4 (&dst)[4], int j, int h) {
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+              dst[m] = *reinterpret_cast<const u32x4*>(sA + ((h * 4 + m) * 16 + lm) * A_LD + j * 32 + lq * 8);
+          };
+          auto read_lut = [&](uint32_t (&dst)[NT][4], int j) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+              dst[nt][0] = lut64_pair<0>(smem, cw[nt][j], lane_off);
+              dst[nt][1] = lut64_pair<1>(smem, cw[nt][j], lane_off);
+              dst[nt][2] = lut64_pair<2>(smem, cw[nt][j], lane_off);
+              dst[nt][3] = lut64_pair<3>(smem, cw[nt][j], lane_off);
+            }
+          };
+          auto convert = [&](u32x4 (&dst)[NT], const uint32_t (&src)[NT][4], int j) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+              for (int b = 0; b < 4; ++b)
+                dst[nt][b] = cvt_pk_bf16(bflo(src[nt][b]) * sc[nt][j], bfhi(src[nt][b]) * sc[nt][j]);
+          };
+          u32x4 af0[4], af1[4], bf[NT], bf_next[NT];
+          uint32_t lp[NT][4];
+          read_lut(lp, 0);
+          read_a(af0, 0, 0);
+          convert(bf, lp, 0);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            read_a(af1, j, 1);
+            if (j < 3) read_lut(lp, j + 1);
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+#pragma unroll
+              for (int nt = 0; nt < NT; ++nt) acc[m][nt] = mfma16(af0[m], bf[nt], acc[m][nt]);
+            if (j < 3) {
+              convert(bf_next, lp, j + 1);
+              read_a(af0, j + 1, 0);
+            }
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+#pragma unroll
+              for (int nt = 0; nt < NT; ++nt) acc[4 + m][nt] = mfma16(af1[m], bf[nt], acc[4 + m][nt]);
+            if (j < 3) {
+#pragma unroll
+              for (int nt = 0; nt < NT; ++nt) bf[nt] = bf_next[nt];
+            }
+          }
+        }
+      }
+    }
+  }
+
+  // ---- sum the two k-halves: each group hands the other group's 64 rows over through LDS ----
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(smem + kLut64Bytes);  // [2][4*NT*4][256]
+  {
+    float* dst = red + (size_t)grp * (4 * NT * 4) * 256;
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float v = grp == 0 ? acc[4 + m][nt][i] : acc[m][nt][i];
+          dst[((m * NT + nt) * 4 + i) * 256 + gtid] = v;
+        }
+  }
+  __syncthreads();
+  f32x4 fin[4][NT];
+  {
+    const float* src = red + (size_t)(1 - grp) * (4 * NT * 4) * 256;
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float mine = grp == 0 ? acc[m][nt][i] : acc[4 + m][nt][i];
+          // fixed order: even k-tiles (group 0) first, then odd k-tiles (group 1)
+          const float other = src[((m * NT + nt) * 4 + i) * 256 + gtid];
+          fin[m][nt][i] = grp == 0 ? mine + other : other + mine;
+        }
+  }
+  const int64_t mh = m0 + grp * 64;  // this group finishes rows [mh, mh + 64)
+  if (a.lora_rank > 0 && blockIdx.z == 0) {
+    int toff[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int64_t col0 = (ntile0 + nt) * 16;
+      if (a.lora_nseg < 0) {
+        toff[nt] = (int)((ntile0 + nt) & 1) * a.lora_rank;
+      } else {
+        toff[nt] = a.lora_seg_toff[0];
+        for (int q = 1; q < a.lora_nseg; ++q)
+          if (col0 >= a.lora_seg_end[q - 1]) toff[nt] = a.lora_seg_toff[q];
+      }
+    }
+    tile_lora<4, NT>(s, mh, ntile0, toff, fin);
+  }
+  store_tile<4, NT>(a, mh, a.M, ntile0, ntiles, fin, [](int64_t r) { return r; });
 }
 
 // y = epi(sum of the split_k partial tiles, added in split order).  One thread per output
@@ -294,12 +513,12 @@ __global__ void quantize_pack_kernel(const void* w, int w_is_f32, int64_t K, int
   const int64_t pc = packed_col(c, N, interleave2);
   const int64_t nt = pc / 16, lm = pc % 16;
   const int64_t ktiles = K / KTILE;
-  const int spt = group >= KTILE ? 1 : KTILE / group;
-  // scales: [nt][kt][spt][16]; a group larger than a k-tile repeats its scale in every tile.
-  for (int64_t k = k0; k < k0 + group; k += (group >= KTILE ? KTILE : group)) {
+  const int spt = scales_per_tile(group), slot_w = KTILE / spt;
+  // scales: [nt][kt][16][spt]; a group wider than a slot repeats its scale in every slot.
+  for (int64_t k = k0; k < k0 + group; k += slot_w) {
     const int64_t kt = k / KTILE;
-    const int si = group >= KTILE ? 0 : (int)((k % KTILE) / group);
-    scales[((nt * ktiles + kt) * spt + si) * 16 + lm] = sbits;
+    const int si = (int)((k % KTILE) / slot_w);
+    scales[((nt * ktiles + kt) * 16 + lm) * spt + si] = sbits;
   }
   for (int i0 = 0; i0 < group; i0 += 8) {
     uint32_t word = 0;
@@ -338,12 +557,12 @@ __global__ void qw_dequant_kernel(const uint32_t* codes, const uint16_t* scales,
   if (c >= N) return;
   const int64_t pc = packed_col(c, N, interleave2);
   const int64_t nt = pc / 16, lm = pc % 16, ktiles = K / KTILE, kt = k / KTILE;
-  const int spt = group >= KTILE ? 1 : KTILE / group;
-  const int si = group >= KTILE ? 0 : (int)((k % KTILE) / group);
+  const int spt = scales_per_tile(group);
+  const int si = (int)((k % KTILE) / (KTILE / spt));
   const int j = (int)((k % KTILE) / 32), lq = (int)((k % 32) / 8), i = (int)(k % 8);
   const uint32_t word = codes[((nt * ktiles + kt) * 64 + lq * 16 + lm) * 4 + j];
-  const float s = bf2f(scales[((nt * ktiles + kt) * spt + si) * 16 + lm]);
-  out[k * N + c] = rbf(code_level(qtype, (word >> (4 * i)) & 15)) * s;
+  const float s = bf2f(scales[((nt * ktiles + kt) * 16 + lm) * spt + si]);
+  out[k * N + c] = rbf(rbf(code_level(qtype, (word >> (4 * i)) & 15)) * s);
 }
 
 QLArgs to_args(const tnx_qlinear_desc* d) {
@@ -372,6 +591,9 @@ int check_desc(const tnx_qlinear_desc* d) {
               "qlinear: unsupported group size %d for K=%lld", d->group, (long long)d->K);
   TNX_REQUIRE(d->qtype == TNX_Q_INT4 || d->qtype == TNX_Q_NF4, "qlinear: bad qtype %d", d->qtype);
   TNX_REQUIRE(d->x && d->codes && d->scales && d->y, "qlinear: null pointer");
+  TNX_REQUIRE((uint64_t)(d->M + 128) * (uint64_t)d->K * 2 < (1ull << 32) &&
+                  (uint64_t)d->K * (uint64_t)d->N / 2 < (1ull << 32),
+              "qlinear: x and the codes must stay below 4 GiB each (32-bit buffer offsets)");
   TNX_REQUIRE(d->epilogue >= TNX_EPI_STORE && d->epilogue <= TNX_EPI_F32, "qlinear: bad epilogue");
   if (d->epilogue == TNX_EPI_RESIDUAL) TNX_REQUIRE(d->residual, "qlinear: residual is null");
   if (d->epilogue == TNX_EPI_SILU_MUL || d->epilogue == TNX_EPI_GELU_MUL)
@@ -414,6 +636,17 @@ int launch_qlinear(hipStream_t st, const QLArgs& a) {
   return TNX_OK;
 }
 
+int launch_qlinear_m128(hipStream_t st, const QLArgs& a) {
+  static std::once_flag once;
+  static int attr_rc = TNX_OK;
+  std::call_once(once, [] { attr_rc = raise_lds_limit(&qlinear_m128_kernel, kM128SmemBytes); });
+  if (attr_rc) return attr_rc;
+  dim3 grid((unsigned)cdiv(a.M, 128), (unsigned)cdiv(a.N, 128), (unsigned)a.split_k);
+  hipLaunchKernelGGL(qlinear_m128_kernel, grid, dim3(512), kM128SmemBytes, st, a);
+  TNX_CHECK_LAUNCH("qlinear_m128");
+  return TNX_OK;
+}
+
 template <int MT, int NT>
 int launch_moe(hipStream_t st, const QLArgs& a, int E, int64_t max_rows) {
   static std::once_flag once;
@@ -435,9 +668,10 @@ extern "C" int tnx_qw_sizes(int64_t K, int64_t N, int group, size_t* codes_bytes
   TNX_REQUIRE(group >= 32 && group % 32 == 0 && K % group == 0 &&
                   (group <= KTILE ? KTILE % group == 0 : group % KTILE == 0),
               "qw_sizes: unsupported group %d", group);
-  const int spt = group >= KTILE ? 1 : KTILE / group;
+  const int spt = scales_per_tile(group);
   if (codes_bytes) *codes_bytes = (size_t)(K * N / 2);
-  if (scales_bytes) *scales_bytes = (size_t)((N / 16) * (K / KTILE) * spt * 16 * 2);
+  // 16 bytes of tail padding: kernels read a lane's scales as one 8-byte word
+  if (scales_bytes) *scales_bytes = (size_t)((N / 16) * (K / KTILE) * spt * 16 * 2) + 16;
   return TNX_OK;
 }
 
@@ -477,7 +711,7 @@ extern "C" int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* d) {
   if (a.M <= 16) return launch_qlinear<1, 2>(st, a);
   if (a.M <= 32) return launch_qlinear<2, 2>(st, a);
   if (a.M <= 64) return launch_qlinear<4, 2>(st, a);
-  return launch_qlinear<8, 2>(st, a);
+  return launch_qlinear_m128(st, a);
 }
 
 extern "C" int tnx_splitk_finish(void* stream, const tnx_qlinear_desc* d) {
@@ -512,6 +746,8 @@ extern "C" int tnx_moe_int4_gmm(void* stream, const tnx_moe_gmm_desc* d) {
   if (rc) return rc;
   TNX_REQUIRE(d->x && d->codes && d->scales && d->offsets && d->sorted_route && d->y, "moe_gmm: null pointer");
   TNX_REQUIRE(d->x_div >= 1, "moe_gmm: x_div must be >= 1");
+  TNX_REQUIRE((uint64_t)(d->n_routes + 128) * (uint64_t)d->K * 2 < (1ull << 32),
+              "moe_gmm: activations must stay below 4 GiB (32-bit buffer offsets)");
   TNX_REQUIRE(d->epilogue == TNX_EPI_STORE || d->epilogue == TNX_EPI_SILU_MUL, "moe_gmm: bad epilogue");
   if (d->epilogue == TNX_EPI_SILU_MUL) TNX_REQUIRE(d->N % 32 == 0, "moe_gmm: SILU_MUL needs N %% 32 == 0");
   QLArgs a;
