@@ -33,18 +33,32 @@ def log(*a):
   print(*a, file=sys.stderr, flush=True)
 
 
-def time_loop(fn, iters, warm=3):
+def time_loop(fn, iters, warm=2, per_graph=10):
+  """Mean duration (ms) of one fn() on the GPU: `per_graph` launches are captured in one HIP graph
+  (host launch overhead would otherwise floor a ~20 us kernel) and the graph is replayed between
+  two events recorded on the stream it runs on."""
   import torch
   for _ in range(warm):
     fn()
+  graph = torch.cuda.CUDAGraph()
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):
+    with torch.cuda.graph(graph, stream=side):
+      for _ in range(per_graph):
+        fn()
+  torch.cuda.current_stream().wait_stream(side)
+  torch.cuda.synchronize()
+  graph.replay()
+  reps = max(1, iters // per_graph)
   e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
   torch.cuda.synchronize()
   e0.record()
-  for _ in range(iters):
-    fn()
+  for _ in range(reps):
+    graph.replay()
   e1.record()
   torch.cuda.synchronize()
-  return e0.elapsed_time(e1) / iters  # ms
+  return e0.elapsed_time(e1) / (reps * per_graph)  # ms
 
 
 def kernel_breakdown(model, runner, st, ctx, iters):

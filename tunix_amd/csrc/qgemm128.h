@@ -1,0 +1,286 @@
+// The quantised GEMM for 65+ activation rows (rollout batch, prefill, per-token logps): one
+// work-group = 4 waves = one wave per SIMD, output tile 128 rows x (64 * NT) columns, wave tile
+// 128 x (16 * NT).  At 128 rows the op sits past the MFMA/HBM ridge of the machine (2 * 128 flop
+// per 0.53 B of weights), so the loop is built around keeping the matrix pipe fed:
+//
+//   * a k-tile (128 k) is four k-steps of 8 * NT MFMAs (16x16x32 bf16).  While the MFMAs of step
+//     g run, the same wave converts the weights of step g+1 (two v_fma_mix_f32 + one
+//     v_cvt_pk_bf16_f32 per code pair), issues the table look-ups of step g+2 and reads the
+//     activation fragments of step g+1 -- a three-deep software pipeline that runs across
+//     k-tile boundaries;
+//   * the code book is an LDS table of f16 level pairs indexed by a code byte, replicated 64
+//     times with a 256-byte entry stride, so that the LDS address of a look-up is one
+//     v_perm_b32: (byte << 8) | (lane << 2); every bf16-rounded level is exact in f16, and
+//     v_fma_mix_f32 multiplies the f16 half it selects with the fp32 scale in one instruction;
+//   * activations are double-buffered in LDS (one barrier per k-tile); packed codes and scales
+//     come through a three-deep register ring filled by buffer loads whose per-k-tile offset
+//     is a scalar, so the loop has no per-load address arithmetic.
+//
+// Included by qlinear.hip after QLArgs / store_tile.
+#pragma once
+
+namespace {
+
+typedef _Float16 h16x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) uint32_t lds_u32;
+typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+
+constexpr int kBigLutBytes = 256 * 256;
+constexpr int kBigABytes = 128 * A_LD * 2;
+constexpr size_t kBigSmemBytes = kBigLutBytes + 2 * (size_t)kBigABytes;
+
+// LDS accesses by absolute LDS byte address (the dynamic LDS block of these kernels starts at
+// address 0: they declare no static LDS).
+__device__ __forceinline__ uint32_t lds_ld32(uint32_t addr) {
+  return *reinterpret_cast<const lds_u32*>(static_cast<uintptr_t>(addr));
+}
+__device__ __forceinline__ u32x4 lds_ld128(uint32_t addr) {
+  return *reinterpret_cast<const lds_u32x4*>(static_cast<uintptr_t>(addr));
+}
+__device__ __forceinline__ void lds_st128(uint32_t addr, u32x4 v) {
+  *reinterpret_cast<lds_u32x4*>(static_cast<uintptr_t>(addr)) = v;
+}
+
+template <int V>
+using ic = std::integral_constant<int, V>;
+
+// The launch bound is a register-budget choice, not the work-group size (always 256): with
+// NT = 2 everything fits the 256 architectural VGPRs, and keeping the accumulators there
+// avoids the accumulator-register copies the compiler emits around loops whose MFMA results
+// live in AGPRs; NT = 4 needs both halves of the 512-entry file.
+template <int NT, int SPT>
+__global__ __launch_bounds__(NT == 2 ? 512 : 256)
+void qgemm128_kernel(const QLArgs a) {
+  constexpr int MT = 8, PF = 3;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wn = tid >> 6;
+  const int lm = lane & 15, lq = lane >> 4;
+  {  // table entry `tid` = f16 pair (level[tid & 15], level[tid >> 4]); copies rotated over banks
+    uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
+    const h16x2 h = {(_Float16)rbf(code_level(a.qtype, tid & 15)), (_Float16)rbf(code_level(a.qtype, tid >> 4))};
+    const uint32_t v = __builtin_bit_cast(uint32_t, h);
+#pragma unroll
+    for (int c = 0; c < 64; ++c) lut[tid * 64 + ((c + lane) & 63)] = v;
+  }
+  const uint32_t lane_off = (uint32_t)lane * 4u;
+  const int64_t m0 = (int64_t)blockIdx.x * 128;
+  const int64_t ntile0 = ((int64_t)blockIdx.y * 4 + wn) * NT;
+  const int64_t ntiles = a.N / 16;
+  const int ktiles = (int)(a.K / KTILE);
+  const int kt_begin = blockIdx.z * a.ktiles_per_split;
+  const int kt_end = min(ktiles, kt_begin + a.ktiles_per_split);
+
+  const rsrc_t rx = make_rsrc(a.x, (uint64_t)a.M * a.K * 2);
+  const uint64_t ntk = (uint64_t)ntiles * ktiles;
+  const rsrc_t rc = make_rsrc(a.codes, ntk * 1024);
+  const rsrc_t rs = make_rsrc(a.scales, ntk * 16 * SPT * 2 + 16);
+  // Per-thread offsets (32 bit: the host checks the 4 GiB limits); the k-tile enters as the
+  // scalar offset of the load.  Rows past M and column tiles past N start beyond the buffer
+  // and read zeros.
+  uint32_t xoff[MT], coff[NT], soff[NT];
+#pragma unroll
+  for (int c = 0; c < MT; ++c)
+    xoff[c] = ((uint32_t)(m0 + (tid >> 4) + 16 * c) * (uint32_t)a.K + (uint32_t)(tid & 15) * 8u) * 2u;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const uint32_t tile0 = (uint32_t)(ntile0 + nt) * (uint32_t)ktiles;
+    coff[nt] = tile0 * 1024u + (uint32_t)lane * 16u;
+    soff[nt] = (tile0 * 16u + (uint32_t)lm) * (uint32_t)(SPT * 2);
+  }
+
+  f32x4 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) zero_acc(acc[mt][nt]);
+
+  u32x4 a_next[MT];
+  u32x4 ring_c[PF][NT];
+  uint32_t ring_s[PF][NT][SPT / 2];
+  float sc[PF][NT][SPT];  // the scales of a ring stage as fp32
+  u32x4 af[2][MT / 2];    // activation fragments of one row half (4 of the 8 row tiles)
+  u32x4 bfr[2][NT];       // weight fragments of this and the next k-step
+  uint32_t lp[NT][4];     // table entries (f16 level pairs) of the k-step after the next
+
+  // k-tiles past the last one are clamped: their data is fetched but never multiplied
+  auto load_a = [&](int kt) {
+    const int s = min(kt, ktiles - 1) * (KTILE * 2);
+#pragma unroll
+    for (int c = 0; c < MT; ++c) a_next[c] = __builtin_amdgcn_raw_buffer_load_b128(rx, xoff[c], s, 0);
+  };
+  auto load_w = [&](auto Dc, int kt) {
+    constexpr int D = decltype(Dc)::value;
+    const int ktc = min(kt, ktiles - 1);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      ring_c[D][nt] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff[nt], ktc * 1024, 0);
+      if constexpr (SPT == 2) {
+        ring_s[D][nt][0] = __builtin_amdgcn_raw_buffer_load_b32(rs, soff[nt], ktc * (16 * SPT * 2), 0);
+      } else {
+        const u32x2 p = __builtin_amdgcn_raw_buffer_load_b64(rs, soff[nt], ktc * (16 * SPT * 2), 0);
+        ring_s[D][nt][0] = p[0];
+        ring_s[D][nt][1] = p[1];
+      }
+    }
+  };
+  // scales of ring stage D -> fp32 in sc[P]; a k-tile past the end gets zero scales, which
+  // turns its weights into zeros
+  auto expand_scales = [&](auto Dc, auto Pc, bool active) {
+    constexpr int D = decltype(Dc)::value, P = decltype(Pc)::value;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int i = 0; i < SPT; ++i) {
+        const float v = (i & 1) ? bfhi(ring_s[D][nt][i >> 1]) : bflo(ring_s[D][nt][i >> 1]);
+        sc[P][nt][i] = active ? v : 0.f;
+      }
+  };
+  // table look-ups of k-step J of ring stage D; the raw f16 pairs land in dst
+  auto lut_issue = [&](auto Dc, auto Jc, uint32_t (&dst)[NT][4]) {
+    constexpr int D = decltype(Dc)::value, J = decltype(Jc)::value;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const uint32_t w = ring_c[D][nt][J];
+      // address bytes: [0] = lane * 4, [1] = code byte b of w, [2] = [3] = 0
+      dst[nt][0] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0400u));
+      dst[nt][1] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0500u));
+      dst[nt][2] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0600u));
+      dst[nt][3] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0700u));
+    }
+  };
+  // f16 level pair x fp32 scale -> bf16 pair
+  auto convert = [&](auto Pc, auto Jc, u32x4 (&dst)[NT], const uint32_t (&src)[NT][4]) {
+    constexpr int P = decltype(Pc)::value, J = decltype(Jc)::value;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const float s = sc[P][nt][SPT == 2 ? (J >> 1) : J];
+      u32x4 r;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const h16x2 h = __builtin_bit_cast(h16x2, src[nt][b]);
+        r[b] = cvt_pk_bf16(__builtin_fmaf((float)h[0], s, 0.0f), __builtin_fmaf((float)h[1], s, 0.0f));
+      }
+      dst[nt] = r;
+    }
+  };
+  // LDS byte addresses of the two activation buffers as this lane reads / writes them
+  uint32_t a_rd = kBigLutBytes + (uint32_t)(lm * A_LD + lq * 8) * 2u;
+  uint32_t a_rd_nxt = a_rd + kBigABytes;
+  uint32_t a_wr = kBigLutBytes + (uint32_t)((tid >> 4) * A_LD + (tid & 15) * 8) * 2u;
+  uint32_t a_wr_nxt = a_wr + kBigABytes;
+  auto read_a = [&](u32x4 (&dst)[MT / 2], uint32_t base, auto Jc, auto Hc) {
+    constexpr int J = decltype(Jc)::value, H = decltype(Hc)::value;
+#pragma unroll
+    for (int m = 0; m < MT / 2; ++m)
+      dst[m] = lds_ld128(base + (uint32_t)(((H * 4 + m) * 16 * A_LD + J * 32) * 2));
+  };
+  auto store_a = [&](uint32_t base) {
+#pragma unroll
+    for (int c = 0; c < MT; ++c) lds_st128(base + (uint32_t)(c * 16 * A_LD * 2), a_next[c]);
+  };
+  auto mfmas = [&](auto Jc, auto Hc) {
+    constexpr int J = decltype(Jc)::value, H = decltype(Hc)::value;
+#pragma unroll
+    for (int m = 0; m < MT / 2; ++m)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        acc[H * 4 + m][nt] = mfma16(af[H][m], bfr[J & 1][nt], acc[H * 4 + m][nt]);
+  };
+
+  // One k-step of ring stage D (k-tile kt).  On entry af[0] holds row half 0 of this step,
+  // bfr[J & 1] its weights and lp the table entries of the next step.  While the MFMAs of row
+  // half 0 issue, the next step's weights are converted; during row half 1 the table look-ups
+  // of the step after that and the next activation fragments are issued.  The
+  // sched_group_barrier sequences spell the interleave out: one wave per SIMD issues in
+  // order, so whatever should overlap the matrix pipe has to sit between the MFMAs.
+  auto block = [&](auto Dc, auto Jc, int kt, bool next_active) {
+    constexpr int d = decltype(Dc)::value, j = decltype(Jc)::value;
+    constexpr int dn = (d + 1) % PF;
+    constexpr int d1 = j < 3 ? d : dn, j1 = (j + 1) & 3;   // the next k-step
+    constexpr int d2 = j < 2 ? d : dn, j2 = (j + 2) & 3;   // and the one after
+    if constexpr (j == 3) __syncthreads();  // next activation tile is in LDS; this one is read out
+    __builtin_amdgcn_sched_barrier(0);
+    read_a(af[1], a_rd, Jc, ic<1>{});
+    if constexpr (j == 0) store_a(a_wr_nxt);
+    if constexpr (j == 2) expand_scales(ic<dn>{}, ic<dn>{}, next_active);
+    convert(ic<d1>{}, ic<j1>{}, bfr[j1 & 1], lp);
+    mfmas(Jc, ic<0>{});
+    lut_issue(ic<d2>{}, ic<j2>{}, lp);
+    read_a(af[0], j < 3 ? a_rd : a_rd_nxt, ic<j1>{}, ic<0>{});
+    if constexpr (j == 1) load_a(kt + 2);
+    if constexpr (j == 3) load_w(Dc, kt + PF);
+    mfmas(Jc, ic<1>{});
+    // row half 0: 4 fragment reads up front, then 3 conversion ops behind every MFMA
+    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+    for (int i = 0; i < 4 * NT; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+      if (j == 0 && i < 8) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+    }
+    // row half 1: one address + one look-up behind every MFMA, fragment reads behind the first 4
+#pragma unroll
+    for (int i = 0; i < 4 * NT; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if (i < 4) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if ((j == 1 || j == 3) && i >= 4 && i < 12) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto tile = [&](auto Dc, int kt) {
+    const bool next_active = kt + 1 < kt_end;
+    block(Dc, ic<0>{}, kt, next_active);
+    block(Dc, ic<1>{}, kt, next_active);
+    block(Dc, ic<2>{}, kt, next_active);
+    block(Dc, ic<3>{}, kt, next_active);
+    const uint32_t r = a_rd; a_rd = a_rd_nxt; a_rd_nxt = r;
+    const uint32_t w = a_wr; a_wr = a_wr_nxt; a_wr_nxt = w;
+  };
+
+  if (kt_begin < kt_end) {
+    load_a(kt_begin);
+    load_w(ic<0>{}, kt_begin);
+    load_w(ic<1>{}, kt_begin + 1);
+    load_w(ic<2>{}, kt_begin + 2);
+    store_a(a_wr);
+    load_a(kt_begin + 1);
+    expand_scales(ic<0>{}, ic<0>{}, true);
+    __syncthreads();  // table and first activation tile
+    lut_issue(ic<0>{}, ic<0>{}, lp);
+    read_a(af[0], a_rd, ic<0>{}, ic<0>{});
+    convert(ic<0>{}, ic<0>{}, bfr[0], lp);
+    lut_issue(ic<0>{}, ic<1>{}, lp);
+    // three k-tiles (one turn of the ring) per iteration; a padded tail runs on zero scales
+    for (int kt = kt_begin; kt < kt_end; kt += PF) {
+      tile(ic<0>{}, kt);
+      tile(ic<1>{}, kt + 1);
+      tile(ic<2>{}, kt + 2);
+    }
+  }
+
+  if (a.lora_rank > 0 && blockIdx.z == 0) {
+    TileSrc s;
+    s.M = a.M; s.K = a.K; s.x = a.x; s.row_index = nullptr; s.row_div = 1; s.x_rows = a.M;
+    s.w_bf16 = nullptr; s.codes = a.codes; s.scales = a.scales; s.group = a.group; s.qtype = a.qtype;
+    s.ntiles = ntiles; s.lora_rank = a.lora_rank; s.t = a.t; s.t_ld = a.t_ld; s.lora_b = a.lora_b;
+    s.lora_scale = a.lora_scale;
+    int toff[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int64_t col0 = (ntile0 + nt) * 16;
+      if (a.lora_nseg < 0) {
+        toff[nt] = (int)((ntile0 + nt) & 1) * a.lora_rank;  // interleaved gate/up pair
+      } else {
+        toff[nt] = a.lora_seg_toff[0];
+        for (int q = 1; q < a.lora_nseg; ++q)
+          if (col0 >= a.lora_seg_end[q - 1]) toff[nt] = a.lora_seg_toff[q];
+      }
+    }
+    tile_lora<MT, NT>(s, m0, ntile0, toff, acc);
+  }
+  store_tile<MT, NT>(a, m0, a.M, ntile0, ntiles, acc, [](int64_t r) { return r; });
+}
+
+}  // namespace

@@ -198,224 +198,9 @@ __global__ __launch_bounds__(256) void moe_gmm_kernel(const QLArgs a) {
                      [routes](int64_t r) { return (int64_t)routes[r]; });
 }
 
-// ---- the rollout-batch kernel: 65..128 rows -----------------------------------------------
-// Eight waves per work-group: waves 0-3 and 4-7 each own the 128 x 128 output tile (wave tile
-// 128 x 32) for every other k-tile, so that each SIMD holds two waves whose MFMA and
-// dequantisation streams interleave.  The two partial tiles are summed through LDS and each
-// half then finishes 64 rows (LoRA delta + epilogue).  The code-book table is replicated 64
-// times with a 256-byte entry stride, which makes the LDS address of a code byte a single
-// v_perm_b32: (byte << 8) | (lane << 2).
-constexpr int kLut64Bytes = 256 * 256;
-constexpr size_t kM128SmemBytes = kLut64Bytes + 2 * (size_t)128 * A_LD * sizeof(uint16_t);
-
-template <int BYTE>
-__device__ __forceinline__ uint32_t lut64_pair(const unsigned char* lut, uint32_t w, uint32_t lane_off) {
-  // bytes of the address: [0] = lane_off, [1] = byte BYTE of w, [2] = [3] = 0
-  const uint32_t addr = __builtin_amdgcn_perm(w, lane_off, 0x0c0c0000u | ((4u + BYTE) << 8));
-  return *reinterpret_cast<const uint32_t*>(lut + addr);
-}
-__device__ __forceinline__ u32x4 dequant8_lut64(uint32_t w, const unsigned char* lut,
-                                                uint32_t lane_off, float scale) {
-  const uint32_t p0 = lut64_pair<0>(lut, w, lane_off), p1 = lut64_pair<1>(lut, w, lane_off);
-  const uint32_t p2 = lut64_pair<2>(lut, w, lane_off), p3 = lut64_pair<3>(lut, w, lane_off);
-  u32x4 r;
-  r[0] = cvt_pk_bf16(bflo(p0) * scale, bfhi(p0) * scale);
-  r[1] = cvt_pk_bf16(bflo(p1) * scale, bfhi(p1) * scale);
-  r[2] = cvt_pk_bf16(bflo(p2) * scale, bfhi(p2) * scale);
-  r[3] = cvt_pk_bf16(bflo(p3) * scale, bfhi(p3) * scale);
-  return r;
-}
-
-__global__ __launch_bounds__(512) void qlinear_m128_kernel(const QLArgs a) {
-  constexpr int NT = 2, MT = 8, PF = 3;
-  extern __shared__ __align__(16) unsigned char smem[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int grp = wave >> 2, wn = wave & 3, gtid = tid & 255;
-  const int lm = lane & 15, lq = lane >> 4;
-  uint16_t* sA = reinterpret_cast<uint16_t*>(smem + kLut64Bytes) + grp * (128 * A_LD);
-  {  // table: thread (byte, half) writes 32 of the 64 copies of its entry, rotated over banks
-    uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
-    const int byte = tid & 255, c0 = (tid >> 8) * 32;
-    const uint32_t v = pack2bf(code_level(a.qtype, byte & 15), code_level(a.qtype, byte >> 4));
-#pragma unroll
-    for (int c = 0; c < 32; ++c) lut[byte * 64 + c0 + ((c + lane) & 31)] = v;
-  }
-  const uint32_t lane_off = (uint32_t)lane * 4u;
-  const int64_t m0 = (int64_t)blockIdx.x * 128;
-  const int64_t ntile0 = ((int64_t)blockIdx.y * 4 + wn) * NT;
-  const int64_t ntiles = a.N / 16;
-  const int ktiles = (int)(a.K / KTILE);
-  const int kt_begin = blockIdx.z * a.ktiles_per_split;
-  const int kt_end = min(ktiles, kt_begin + a.ktiles_per_split);
-  const int n_it = (kt_end - kt_begin + 1) / 2;  // group g takes k-tiles kt_begin + 2*it + g
-  const int spt = scales_per_tile(a.group);
-
-  TileSrc s;
-  s.M = a.M; s.K = a.K; s.x = a.x; s.row_index = nullptr; s.row_div = 1; s.x_rows = a.M;
-  s.w_bf16 = nullptr; s.codes = a.codes; s.scales = a.scales; s.group = a.group; s.qtype = a.qtype;
-  s.ntiles = ntiles; s.lora_rank = a.lora_rank; s.t = a.t; s.t_ld = a.t_ld; s.lora_b = a.lora_b;
-  s.lora_scale = a.lora_scale;
-  const rsrc_t rx = make_rsrc(a.x, (uint64_t)a.M * a.K * 2);
-  const uint64_t ntk = (uint64_t)ntiles * ktiles;
-  const rsrc_t rc = make_rsrc(a.codes, ntk * 1024);
-  const rsrc_t rs = make_rsrc(a.scales, ntk * 16 * spt * 2 + 16);
-
-  f32x4 acc[MT][NT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) zero_acc(acc[mt][nt]);
-
-  u32x4 a_next[MT];
-  u32x4 ring_c[PF][NT];
-  u32x2 ring_s[PF][NT];
-  auto load_w = [&](u32x4 (&c)[NT], u32x2 (&sc)[NT], int kt) {
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      // 32-bit offsets: the host checks that codes and scales are below 4 GiB
-      const uint32_t tile = (uint32_t)(ntile0 + nt) * (uint32_t)ktiles + (uint32_t)kt;
-      c[nt] = buf_load128(rc, tile * 1024u + (uint32_t)lane * 16u);
-      // always 8 bytes (the upper half is the next column when there are two slots): no
-      // control flow around loads, so that the waits on them can be counted exactly
-      sc[nt] = __builtin_amdgcn_raw_buffer_load_b64(rs, (tile * 16u + (uint32_t)lm) * (uint32_t)spt * 2u, 0, 0);
-    }
-  };
-  auto my_kt = [&](int it) { return kt_begin + 2 * it + grp; };
-  // Loads are never predicated: k-tiles past the end read neighbouring or out-of-range (zero)
-  // data that is never used, and the iteration count is padded to a multiple of PF.
-  load_a<MT>(s, rx, m0, my_kt(0), gtid, a_next);
-#pragma unroll
-  for (int d = 0; d < PF; ++d) load_w(ring_c[d], ring_s[d], my_kt(d));
-
-  for (int it0 = 0; it0 < n_it; it0 += PF) {
-#pragma unroll
-    for (int d = 0; d < PF; ++d) {
-      const int it = it0 + d;
-      {
-        const int kt = my_kt(it);
-        const bool active = kt < kt_end;
-        __syncthreads();  // every wave is done reading its group's activation tile
-        if (active) store_a<MT>(sA, gtid, a_next);
-        u32x4 cw[NT];
-        float sc[NT][4];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          cw[nt] = ring_c[d][nt];
-          const u32x2 p = ring_s[d][nt];
-          const float f[4] = {bflo(p[0]), bfhi(p[0]), bflo(p[1]), bfhi(p[1])};
-#pragma unroll
-          for (int j = 0; j < 4; ++j) sc[nt][j] = spt == 2 ? f[j >> 1] : f[j];
-        }
-        __syncthreads();
-        // activations of the next k-tile first, then the weights PF tiles ahead
-        load_a<MT>(s, rx, m0, my_kt(it + 1), gtid, a_next);
-        load_w(ring_c[d], ring_s[d], my_kt(it + PF));
-        if (active) {
-          // Software pipeline over the 8 half-steps (k-step j, row half h) of the k-tile: the
-          // LDS reads of a half-step (4 A fragments; the 8 table entries of the next k-step)
-          // are issued one half-step (8 MFMAs) ahead of their use, so that the LDS latency
-          // hides behind the matrix pipe instead of stalling every MFMA.
-          auto read_a = [&](u32x4 (&dst)[4], int j, int h) {
-#pragma unroll
-            for (int m = 0; m < 4; ++m)
-              dst[m] = *reinterpret_cast<const u32x4*>(sA + ((h * 4 + m) * 16 + lm) * A_LD + j * 32 + lq * 8);
-          };
-          auto read_lut = [&](uint32_t (&dst)[NT][4], int j) {
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-              dst[nt][0] = lut64_pair<0>(smem, cw[nt][j], lane_off);
-              dst[nt][1] = lut64_pair<1>(smem, cw[nt][j], lane_off);
-              dst[nt][2] = lut64_pair<2>(smem, cw[nt][j], lane_off);
-              dst[nt][3] = lut64_pair<3>(smem, cw[nt][j], lane_off);
-            }
-          };
-          auto convert = [&](u32x4 (&dst)[NT], const uint32_t (&src)[NT][4], int j) {
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-              for (int b = 0; b < 4; ++b)
-                dst[nt][b] = cvt_pk_bf16(bflo(src[nt][b]) * sc[nt][j], bfhi(src[nt][b]) * sc[nt][j]);
-          };
-          u32x4 af0[4], af1[4], bf[NT], bf_next[NT];
-          uint32_t lp[NT][4];
-          read_lut(lp, 0);
-          read_a(af0, 0, 0);
-          convert(bf, lp, 0);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            read_a(af1, j, 1);
-            if (j < 3) read_lut(lp, j + 1);
-#pragma unroll
-            for (int m = 0; m < 4; ++m)
-#pragma unroll
-              for (int nt = 0; nt < NT; ++nt) acc[m][nt] = mfma16(af0[m], bf[nt], acc[m][nt]);
-            if (j < 3) {
-              convert(bf_next, lp, j + 1);
-              read_a(af0, j + 1, 0);
-            }
-#pragma unroll
-            for (int m = 0; m < 4; ++m)
-#pragma unroll
-              for (int nt = 0; nt < NT; ++nt) acc[4 + m][nt] = mfma16(af1[m], bf[nt], acc[4 + m][nt]);
-            if (j < 3) {
-#pragma unroll
-              for (int nt = 0; nt < NT; ++nt) bf[nt] = bf_next[nt];
-            }
-          }
-        }
-      }
-    }
-  }
-
-  // ---- sum the two k-halves: each group hands the other group's 64 rows over through LDS ----
-  __syncthreads();
-  float* red = reinterpret_cast<float*>(smem + kLut64Bytes);  // [2][4*NT*4][256]
-  {
-    float* dst = red + (size_t)grp * (4 * NT * 4) * 256;
-#pragma unroll
-    for (int m = 0; m < 4; ++m)
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float v = grp == 0 ? acc[4 + m][nt][i] : acc[m][nt][i];
-          dst[((m * NT + nt) * 4 + i) * 256 + gtid] = v;
-        }
-  }
-  __syncthreads();
-  f32x4 fin[4][NT];
-  {
-    const float* src = red + (size_t)(1 - grp) * (4 * NT * 4) * 256;
-#pragma unroll
-    for (int m = 0; m < 4; ++m)
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float mine = grp == 0 ? acc[m][nt][i] : acc[4 + m][nt][i];
-          // fixed order: even k-tiles (group 0) first, then odd k-tiles (group 1)
-          const float other = src[((m * NT + nt) * 4 + i) * 256 + gtid];
-          fin[m][nt][i] = grp == 0 ? mine + other : other + mine;
-        }
-  }
-  const int64_t mh = m0 + grp * 64;  // this group finishes rows [mh, mh + 64)
-  if (a.lora_rank > 0 && blockIdx.z == 0) {
-    int toff[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const int64_t col0 = (ntile0 + nt) * 16;
-      if (a.lora_nseg < 0) {
-        toff[nt] = (int)((ntile0 + nt) & 1) * a.lora_rank;
-      } else {
-        toff[nt] = a.lora_seg_toff[0];
-        for (int q = 1; q < a.lora_nseg; ++q)
-          if (col0 >= a.lora_seg_end[q - 1]) toff[nt] = a.lora_seg_toff[q];
-      }
-    }
-    tile_lora<4, NT>(s, mh, ntile0, toff, fin);
-  }
-  store_tile<4, NT>(a, mh, a.M, ntile0, ntiles, fin, [](int64_t r) { return r; });
-}
+}  // namespace
+#include "qgemm128.h"
+namespace {
 
 // y = epi(sum of the split_k partial tiles, added in split order).  One thread per output
 // element; the fixed summation order makes split-k results reproducible run to run.
@@ -636,14 +421,15 @@ int launch_qlinear(hipStream_t st, const QLArgs& a) {
   return TNX_OK;
 }
 
-int launch_qlinear_m128(hipStream_t st, const QLArgs& a) {
+template <int NT, int SPT>
+int launch_qgemm128(hipStream_t st, const QLArgs& a) {
   static std::once_flag once;
   static int attr_rc = TNX_OK;
-  std::call_once(once, [] { attr_rc = raise_lds_limit(&qlinear_m128_kernel, kM128SmemBytes); });
+  std::call_once(once, [] { attr_rc = raise_lds_limit(&qgemm128_kernel<NT, SPT>, kBigSmemBytes); });
   if (attr_rc) return attr_rc;
-  dim3 grid((unsigned)cdiv(a.M, 128), (unsigned)cdiv(a.N, 128), (unsigned)a.split_k);
-  hipLaunchKernelGGL(qlinear_m128_kernel, grid, dim3(512), kM128SmemBytes, st, a);
-  TNX_CHECK_LAUNCH("qlinear_m128");
+  dim3 grid((unsigned)cdiv(a.M, 128), (unsigned)cdiv(a.N, 64 * NT), (unsigned)a.split_k);
+  hipLaunchKernelGGL((qgemm128_kernel<NT, SPT>), grid, dim3(256), kBigSmemBytes, st, a);
+  TNX_CHECK_LAUNCH("qgemm128");
   return TNX_OK;
 }
 
@@ -711,7 +497,11 @@ extern "C" int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* d) {
   if (a.M <= 16) return launch_qlinear<1, 2>(st, a);
   if (a.M <= 32) return launch_qlinear<2, 2>(st, a);
   if (a.M <= 64) return launch_qlinear<4, 2>(st, a);
-  return launch_qlinear_m128(st, a);
+  // 128 x 128 work-group tiles; the 256-column variant (NT = 4) is not dispatched: its
+  // accumulators need AGPRs, and the compiler wraps loops over AGPR accumulators in register
+  // copies that cost more than the halved LDS traffic gains
+  if (scales_per_tile(a.group) == 2) return launch_qgemm128<2, 2>(st, a);
+  return launch_qgemm128<2, 4>(st, a);
 }
 
 extern "C" int tnx_splitk_finish(void* stream, const tnx_qlinear_desc* d) {
