@@ -1,0 +1,141 @@
+"""CPU checks of the boundary and the host logic: the shared library loads and exports every
+entry point include/tunix_hip.h declares (no compute call is made here), the ctypes table covers
+the same set with matching arity and struct sizes, argument checking works without a GPU where
+it happens before any launch, and the host helpers agree with the oracle / the reference's
+literal vectors."""
+import ctypes
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+from oracle import utils_ref as U
+from tunix_amd import _lib as L
+from tunix_amd import config
+from tunix_amd.generate import utils as G
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "tunix_hip.h")
+
+DECL = re.compile(r"^(?:int|int64_t|size_t|const char\*)\s+(tnx_[a-z0-9_]+)\s*\(([^;]*)\)\s*;", re.M | re.S)
+
+
+def _declared():
+  text = open(HEADER).read()
+  text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+  out = {}
+  for m in DECL.finditer(text):
+    args = m.group(2).strip()
+    n = 0 if args in ("", "void") else len([a for a in args.split(",") if a.strip()])
+    out[m.group(1)] = n
+  return out
+
+
+def test_header_declares_the_expected_entry_points():
+  d = _declared()
+  assert len(d) >= 23
+  for name in ("tnx_qlinear_lora", "tnx_gqa_attn", "tnx_qknorm_rope_kvwrite", "tnx_rmsnorm",
+               "tnx_lmhead_logp", "tnx_moe_int4_gmm", "tnx_sample_topk", "tnx_grpo_ratio"):
+    assert name in d
+
+
+def test_library_exports_every_declared_symbol():
+  assert os.path.exists(L.LIB_PATH), "libtunix_hip.so is not built (run __graft_entry__.build())"
+  handle = ctypes.CDLL(L.LIB_PATH)
+  for name in _declared():
+    assert hasattr(handle, name), f"{name} is declared in include/tunix_hip.h but not exported"
+  # and nothing beyond the declared ABI leaks out with the tnx_ prefix (tnx_set_error is the
+  # library-internal error setter shared by its translation units)
+  nm = subprocess.run(["nm", "-D", "--defined-only", L.LIB_PATH], capture_output=True, text=True).stdout
+  exported = {ln.split()[-1] for ln in nm.splitlines() if " T " in ln and ln.split()[-1].startswith("tnx_")}
+  assert exported - set(_declared()) <= {"tnx_set_error"}, exported - set(_declared())
+
+
+def test_ctypes_table_matches_header():
+  d = _declared()
+  assert set(L.SIGNATURES) == set(d)
+  for name, (_, args) in L.SIGNATURES.items():
+    assert len(args) == d[name], f"{name}: header has {d[name]} parameters, ctypes table {len(args)}"
+
+
+def test_version_and_argument_errors_without_gpu():
+  lib = L.lib()
+  assert lib.tnx_version() >= 1
+  cb, sb = ctypes.c_size_t(), ctypes.c_size_t()
+  assert lib.tnx_qw_sizes(4096, 4096, 64, ctypes.byref(cb), ctypes.byref(sb)) == 0
+  assert cb.value == 4096 * 4096 // 2
+  assert sb.value == (4096 // 16) * (4096 // 128) * 2 * 16 * 2 + 16
+  rc = lib.tnx_qw_sizes(100, 4096, 64, ctypes.byref(cb), ctypes.byref(sb))
+  assert rc == -22 and b"128" in lib.tnx_last_error()
+  with pytest.raises(ValueError, match="128"):
+    L.check(rc, "qw_sizes")
+  assert lib.tnx_qw_sizes(4096, 4096, 48, None, None) == -22
+  assert lib.tnx_lmhead_nblocks(128256) > 0
+
+
+def test_struct_layouts_are_stable():
+  # the descriptor structs cross the C ABI by pointer: their sizes are part of the contract
+  assert ctypes.sizeof(L.QLinearDesc) == 176
+  for cls in (L.RopeDesc, L.AttnDesc, L.LmHeadDesc, L.MoeGmmDesc):
+    assert ctypes.sizeof(cls) % 8 == 0
+
+
+def test_host_utils_match_oracle_and_reference_vectors():
+  assert [G.next_power_of_2(x) for x in (0, 2, 3, 4, 5)] == [1, 2, 4, 4, 8]
+  x = np.array([1, 2, 3])
+  np.testing.assert_array_equal(G.pad_to_length(x, 5, 0, left=True), U.pad_to_length(x, 5, 0, left=True))
+  for ids in ([1, 2, 3, 4, 5, 6], [0, 0, 1, 2, 3, 4], [0, 1, 2, 3, 0, 0]):
+    assert G.np_find_first_non_pad_idx(np.array(ids), 0) == U.find_first_non_pad_idx(np.array(ids), 0)
+  for ids in ([1, 2, 3, 4, 5, -1], [1, 2, -1, 4, -1, 0], [1, 2, 3, 4, 5, 6]):
+    assert G.np_find_first_eos_idx(np.array(ids), -1) == U.find_first_eos_idx(np.array(ids), -1)
+  m = np.array([[1, 1, 1, 1], [0, 1, 1, 1], [1, 1, 1, 0], [0, 1, 1, 0]])
+  np.testing.assert_array_equal(G.build_positions_from_mask(m), [[0, 1, 2, 3], [0, 0, 1, 2], [0, 1, 2, 2], [0, 0, 1, 1]])
+
+
+def test_sampling_mode_conflict_message():
+  cur = [None]
+  G.check_sampling_mode_conflict(cur, "top_p")
+  with pytest.raises(ValueError, match="Conflicts setting sampling_mode"):
+    G.check_sampling_mode_conflict(cur, "greedy")
+
+
+def test_id_tokenizer():
+  t = G.IdTokenizer(100, pad_id=0, eos_id=1, bos_id=2)
+  assert t.encode("5 6 7") == [5, 6, 7] and t.decode([5, 6]) == "5 6"
+  assert t.dedup_bos_ids([2, 2, 2, 9]) == [2, 9]
+  assert (t.pad_id(), t.eos_id(), t.bos_id()) == (0, 1, 2)
+
+
+def test_config_presets():
+  c = config.llama31_8b()
+  assert (c.num_layers, c.embed_dim, c.hidden_dim, c.num_heads, c.num_kv_heads, c.head_dim, c.vocab_size) == (
+      32, 4096, 14336, 32, 8, 128, 128256)
+  assert c.qtype == config.Q_NF4 and c.group == 64 and c.lora_rank == 64
+  g = config.gemma3_1b()
+  assert [g.is_local_layer(i) for i in range(6)] == [True] * 5 + [False]
+  assert g.rope_params(0) == (10_000.0, 1.0) and g.rope_params(5) == (1_000_000.0, 1.0)
+  m = config.qwen3_30b_a3b()
+  assert m.num_experts == 128 and m.num_experts_per_tok == 8
+  assert "l0.e_gate" in m.quantized_names() and "l0.wq" in m.lora_names() and "l0.e_gate" not in m.lora_names()
+  with pytest.raises(ValueError):
+    config.ModelConfig(family="gpt2", num_layers=1, vocab_size=8, embed_dim=8, hidden_dim=8, num_heads=1,
+                       num_kv_heads=1, head_dim=8)
+
+
+def test_product_does_not_import_the_oracle():
+  """The oracle is test infrastructure: nothing under tunix_amd/ may reference it."""
+  pkg = os.path.join(ROOT, "tunix_amd")
+  for dirpath, _, files in os.walk(pkg):
+    for f in files:
+      if f.endswith((".py", ".hip", ".h")):
+        text = open(os.path.join(dirpath, f)).read()
+        assert not re.search(r"^\s*(from|import)\s+oracle\b", text, re.M), os.path.join(dirpath, f)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+  monkeypatch.setattr(L, "_lib", None)
+  monkeypatch.setattr(L, "LIB_PATH", "/nonexistent/libtunix_hip.so")
+  with pytest.raises(ImportError, match="no CPU fallback"):
+    L.lib()

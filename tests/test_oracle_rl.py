@@ -1,0 +1,140 @@
+"""oracle/threefry.py and oracle/rl_ref.py against the golden arrays of the reference's
+tests/rl/common_test.py (their inputs are jax.random draws from PRNGKey(0), so reproducing the
+tables pins the bit stream, the uniform mapping, split and the KL / log-softmax formulas at
+once) and against closed forms."""
+import numpy as np
+import pytest
+import scipy.special
+import torch
+
+from oracle import rl_ref as R
+from oracle import threefry as T
+
+# tests/rl/common_test.py:35-77
+KL_TABLES = {
+    "kl": [[[0.38486493, 0.7469206, 0.3495195, 0.5621129], [-0.4474684, -0.13095665, 0.46064317, -0.19887352]],
+           [[0.43108296, 0.53564644, -0.25296474, 0.44137287], [-0.06834459, -0.12115264, -0.61533415, 0.15468943]]],
+    "mse_kl": [[[0.07406051, 0.27894518, 0.06108194, 0.15798548], [0.10011399, 0.00857482, 0.10609607, 0.01977534]],
+               [[0.09291626, 0.14345856, 0.03199558, 0.09740501], [0.00233549, 0.00733898, 0.18931806, 0.01196441]]],
+    "low_var_kl": [[[0.0654075, 0.220744, 0.0545462, 0.1321163], [0.1168784, 0.0089617, 0.0915209, 0.0211542]],
+                   [[0.080888, 0.1209372, 0.0348731, 0.0845257], [0.0023897, 0.0076445, 0.2349406, 0.0113707]]],
+}
+
+
+def test_threefry_known_answer():
+  """Threefry-2x32, 20 rounds: the known-answer vectors of the Random123 distribution."""
+  x0, x1 = T.threefry2x32((np.uint32(0), np.uint32(0)), np.uint32([0]), np.uint32([0]))
+  assert (int(x0[0]), int(x1[0])) == (0x6B200159, 0x99BA4EFE)
+  k = (np.uint32(0xFFFFFFFF), np.uint32(0xFFFFFFFF))
+  x0, x1 = T.threefry2x32(k, np.uint32([0xFFFFFFFF]), np.uint32([0xFFFFFFFF]))
+  assert (int(x0[0]), int(x1[0])) == (0x1CB996FC, 0xBB002BE7)
+  k = (np.uint32(0x13198A2E), np.uint32(0x03707344))
+  x0, x1 = T.threefry2x32(k, np.uint32([0x243F6A88]), np.uint32([0x85A308D3]))
+  assert (int(x0[0]), int(x1[0])) == (0xC4923A9C, 0x483DF7A0)
+
+
+@pytest.mark.parametrize("method", ["kl", "mse_kl", "low_var_kl"])
+def test_kl_tables(method):
+  key = T.prng_key(0)
+  k1, k2 = T.split(key, 2, partitionable=False)
+  logps = T.uniform(k1, (2, 2, 4), partitionable=False)
+  ref = T.uniform(k2, (2, 2, 4), partitionable=False)
+  got = R.compute_kl_divergence(logps, ref, method=method)
+  np.testing.assert_allclose(got, np.array(KL_TABLES[method]), atol=1e-5, rtol=1e-2)
+  # tighter than the reference's own tolerance: the draws themselves are reproduced
+  assert np.abs(got - np.array(KL_TABLES[method])).max() < 2e-6
+
+
+def test_kl_bad_method():
+  with pytest.raises(ValueError, match="`method` must be one of"):
+    R.compute_kl_divergence(np.zeros(2), np.zeros(2), method="nope")
+
+
+def test_selective_log_softmax_golden():
+  # tests/rl/common_test.py:92-108
+  key = T.prng_key(0)
+  logits = T.uniform(key, (2, 4, 8), partitionable=False)
+  ids = T.randint(key, (2, 4), 0, 8, partitionable=False)
+  got = R.selective_log_softmax(torch.from_numpy(logits), torch.from_numpy(ids)).numpy()
+  want = np.array([[-2.242679, -2.2733693, -2.1024966, -1.9994389],
+                   [-2.0603075, -2.4863663, -1.9176172, -2.0206313]])
+  np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
+
+
+def test_selective_log_softmax_closed_form():
+  rng = np.random.default_rng(0)
+  lg = rng.normal(size=(3, 5, 17)).astype(np.float32) * 4
+  ids = rng.integers(0, 17, size=(3, 5))
+  got = R.selective_log_softmax(torch.from_numpy(lg), torch.from_numpy(ids)).numpy()
+  want = np.take_along_axis(lg.astype(np.float64), ids[..., None], -1)[..., 0] - scipy.special.logsumexp(
+      lg.astype(np.float64), axis=-1)
+  np.testing.assert_allclose(got, want, atol=1e-5)
+  # uniform logits: -log V whatever the target
+  u = R.selective_log_softmax(torch.zeros(2, 3, 17), torch.from_numpy(ids[:2, :3]))
+  np.testing.assert_allclose(u.numpy(), -np.log(17.0), atol=1e-6)
+
+
+def test_fold_in_matches_threefry_of_zero_and_data():
+  key = T.prng_key(42)
+  a, b = T.threefry2x32(key, np.uint32([0]), np.uint32([7]))
+  assert T.fold_in(key, 7) == (np.uint32(a[0]), np.uint32(b[0]))
+
+
+def test_uniform_range_and_categorical_argmax():
+  key = T.prng_key(3)
+  u = T.uniform(key, (1000,), partitionable=False)
+  assert u.min() >= 0.0 and u.max() < 1.0 and abs(u.mean() - 0.5) < 0.05
+  # a logit far above the rest always wins the Gumbel-max draw
+  lg = np.zeros((4, 50), dtype=np.float32)
+  lg[np.arange(4), [3, 9, 0, 49]] = 100.0
+  np.testing.assert_array_equal(T.categorical(key, lg, partitionable=False), [3, 9, 0, 49])
+  # frequencies follow softmax
+  lg = np.log(np.array([0.1, 0.2, 0.7], dtype=np.float32))[None].repeat(20000, 0)
+  draws = T.categorical(T.prng_key(5), lg, partitionable=False)
+  freq = np.bincount(draws, minlength=3) / draws.size
+  np.testing.assert_allclose(freq, [0.1, 0.2, 0.7], atol=0.015)
+
+
+def test_grpo_ratio():
+  rng = np.random.default_rng(1)
+  lp = rng.normal(size=(4, 6)).astype(np.float32)
+  adv = rng.normal(size=(4,)).astype(np.float32)
+  # old logps absent: ratio 1 and loss -A (tests/rl/algo_core_test.py:51-143 on-policy case)
+  ratio, loss, clipped = R.grpo_ratio(lp, None, adv, 0.2, 0.2)
+  np.testing.assert_array_equal(ratio, 1.0)
+  np.testing.assert_allclose(loss, -adv[:, None] * np.ones_like(lp))
+  old = lp + rng.normal(size=lp.shape).astype(np.float32) * 0.3
+  ratio, loss, clipped = R.grpo_ratio(lp, old, adv, 0.2, 0.3)
+  r = np.exp(lp.astype(np.float64) - old)
+  want = np.maximum(-adv[:, None] * r, -adv[:, None] * np.clip(r, 0.8, 1.3))
+  np.testing.assert_allclose(ratio, r, rtol=1e-5)
+  np.testing.assert_allclose(loss, want, rtol=1e-5, atol=1e-6)
+
+
+def test_compute_per_token_logps_chunk_invariance():
+  """tests/rl/common_test.py:340-399: chunked == unchunked; and == direct log-softmax."""
+  from oracle import model_ref as MR
+  from tunix_amd import config, dummy_model
+  cfg = config.tiny_qwen3(num_layers=1, vocab_size=96, embed_dim=64, hidden_dim=96, num_heads=4,
+                          num_kv_heads=2, head_dim=16, group=32)
+  w = dummy_model.create_dummy_weights(cfg, seed=5, scale=0.2)
+  ref = MR.RefModel(cfg, w, bf16=False)
+  rng = np.random.default_rng(5)
+  prompt = rng.integers(1, cfg.vocab_size, size=(2, 6))
+  prompt[0, :2] = 0  # left padding
+  comp = rng.integers(1, cfg.vocab_size, size=(2, 5))
+  comp[1, 3:] = 0    # right padding
+  full = R.compute_per_token_logps(ref, prompt, comp, 0).numpy()
+  for chunk in (1, 2, 5):
+    np.testing.assert_allclose(R.compute_per_token_logps(ref, prompt, comp, 0, chunk_size=chunk).numpy(), full,
+                               atol=1e-6)
+  ids, pos, mask = R.process_ids(prompt, comp, 0)
+  lg = ref(torch.from_numpy(ids).long(), torch.from_numpy(pos).long(), ref.init_cache(2, 11),
+           torch.from_numpy(mask), 0)
+  lsm = torch.log_softmax(lg.double(), -1).numpy()
+  want = np.array([[lsm[b, 5 + t, comp[b, t]] for t in range(5)] for b in range(2)])
+  np.testing.assert_allclose(full, want, atol=1e-5)
+  t2 = R.compute_per_token_logps(ref, prompt, comp, 0, temperature=2.0).numpy()
+  lsm2 = torch.log_softmax(lg.double() / 2.0, -1).numpy()
+  want2 = np.array([[lsm2[b, 5 + t, comp[b, t]] for t in range(5)] for b in range(2)])
+  np.testing.assert_allclose(t2, want2, atol=1e-5)
