@@ -1,0 +1,208 @@
+"""GPU parity of the per-token log-probability path and the rollout engine against the oracle
+(tolerances of the path: log-probabilities <= 2e-2 absolute against the bf16-flow oracle)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import model_ref as MR
+from oracle import quant_ref as Q
+from oracle import rl_ref as R
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tiny(gpu):
+  from tunix_amd import config, dummy_model
+  from tunix_amd.model import QLoRAModel
+  cfg = config.tiny_qwen3(vocab_size=4096)
+  # N(0, 0.02) weights as in the parity configurations: logits stay below 1 in magnitude, where
+  # one bf16 ulp of a logit is far below the 2e-2 tolerance of the path
+  w = dummy_model.create_dummy_weights(cfg, seed=77)
+  return cfg, w, QLoRAModel(cfg, w, gpu)
+
+
+def _tokens(cfg, B, P, T, seed):
+  rng = np.random.default_rng(seed)
+  prompt = rng.integers(2, cfg.vocab_size, size=(B, P)).astype(np.int32)
+  comp = rng.integers(2, cfg.vocab_size, size=(B, T)).astype(np.int32)
+  prompt[0, :5] = 0          # left padding
+  prompt[2, :P - 1] = 0      # a one-token prompt
+  comp[1, T - 4:] = 0        # right padding
+  comp[3, 1:] = 0
+  return prompt, comp
+
+
+def test_per_token_logps_match_oracle(tiny, gpu):
+  from tunix_amd.rl import common
+  cfg, w, model = tiny
+  B, P, T = 4, 24, 16
+  prompt, comp = _tokens(cfg, B, P, T, 1)
+  got = common.compute_per_token_logps(model, prompt, comp, pad_id=0, eos_id=1).cpu().numpy()
+  ref = MR.RefModel(cfg, w)
+  want = R.compute_per_token_logps(ref, prompt, comp, 0).numpy()
+  valid = comp != 0
+  err = np.abs(got - want)[valid].max()
+  assert err <= 2e-2, err
+  assert np.isfinite(got).all() and (got <= 1e-6).all()
+  # temperature
+  got_t = common.compute_per_token_logps(model, prompt, comp, pad_id=0, temperature=0.7).cpu().numpy()
+  want_t = R.compute_per_token_logps(ref, prompt, comp, 0, temperature=0.7).numpy()
+  assert np.abs(got_t - want_t)[valid].max() <= 2e-2
+  assert np.abs(got_t - got)[valid].max() > 1e-3
+
+
+def test_per_token_logps_chunking_and_batching_are_invariant(tiny, gpu):
+  """tests/rl/common_test.py:340-399: the chunked computation returns the same values; here
+  bit for bit, also when the batch is split over several forward passes."""
+  from tunix_amd.rl import common
+  cfg, w, model = tiny
+  prompt, comp = _tokens(cfg, 4, 24, 16, 2)
+  full = common.compute_per_token_logps(model, prompt, comp, pad_id=0)
+  for chunk in (1, 5, 16):
+    c = common.compute_per_token_logps(model, prompt, comp, pad_id=0, chunk_size=chunk)
+    assert torch.equal(c, full), chunk
+  # one sequence per forward pass selects other GEMM tilings (fewer rows): same values up to
+  # the fp32 summation order, far inside the tolerance of the path
+  one_by_one = common.compute_per_token_logps(model, prompt, comp, pad_id=0, max_rows=40)
+  assert (one_by_one - full).abs().max().item() <= 1e-2
+
+
+def test_per_token_logps_argument_errors(tiny, gpu):
+  from tunix_amd.rl import common
+  cfg, w, model = tiny
+  with pytest.raises(ValueError):
+    common.compute_per_token_logps(model, np.zeros((2, 4), np.int32), np.zeros((3, 4), np.int32), pad_id=0)
+  with pytest.raises(NotImplementedError):
+    common.compute_per_token_logps(model, np.ones((2, 4), np.int32), np.ones((2, 4), np.int32), pad_id=0,
+                                   return_entropy=True)
+  empty = common.compute_per_token_logps(model, np.ones((2, 4), np.int32), np.ones((2, 0), np.int32), pad_id=0)
+  assert tuple(empty.shape) == (2, 0)
+
+
+def test_rollout_engine_contract_and_logprob_consistency(tiny, gpu):
+  """generate() -> RolloutOutput; the log-probabilities the sampler reports for its own greedy
+  tokens agree with get_per_token_logps over the same tokens (decode kernels vs the
+  whole-sequence pass), and update_params changes them."""
+  from tunix_amd.generate.utils import IdTokenizer
+  from tunix_amd.rl import HipRollout, RolloutConfig
+  cfg, w, model = tiny
+  tok = IdTokenizer(cfg.vocab_size, pad_id=0, eos_id=1)
+  ro = HipRollout(model, tok, 64)
+  assert ro.pad_id() == 0 and ro.eos_id() == 1 and ro.model() is model
+  rng = np.random.default_rng(3)
+  prompts = [" ".join(str(int(t)) for t in rng.integers(2, cfg.vocab_size, size=n)) for n in (7, 16, 12)]
+  rc = RolloutConfig(max_tokens_to_generate=12, temperature=0.0, top_p=None, max_prompt_length=16,
+                     eos_tokens=[-1], return_logprobs=True)
+  out = ro.generate(prompts, rc)
+  assert len(out.text) == 3 and out.left_padded_prompt_tokens.shape == (3, 16)
+  assert all(len(t) == 12 for t in out.tokens) and all(len(lp) == 12 for lp in out.logprobs)
+  comp = np.stack(out.tokens).astype(np.int32)
+  lps = ro.get_per_token_logps(out.left_padded_prompt_tokens, comp).cpu().numpy()
+  assert np.abs(lps - np.asarray(out.logprobs, dtype=np.float32)).max() <= 2e-2
+  # same tokens through the oracle
+  ref = MR.RefModel(cfg, w)
+  want = R.compute_per_token_logps(ref, out.left_padded_prompt_tokens, comp, 0).numpy()
+  assert np.abs(lps - want).max() <= 2e-2
+  # new adapter weights move the result; restoring them restores it bit for bit
+  new = {k: (v.float() * 3).to(torch.bfloat16) for k, v in w.items() if ".lora_" in k}
+  ro.update_params(new)
+  moved = ro.get_per_token_logps(out.left_padded_prompt_tokens, comp).cpu().numpy()
+  assert np.abs(moved - lps).max() > 1e-3
+  ro.update_params({k: v for k, v in w.items() if ".lora_" in k})
+  back = ro.get_per_token_logps(out.left_padded_prompt_tokens, comp).cpu().numpy()
+  np.testing.assert_array_equal(back, lps)
+  with pytest.raises(ValueError, match="same structure"):
+    ro.update_params({"l0.wq.lora_a": new["l0.wq.lora_a"]})
+
+
+def test_grpo_clipped_ratio(gpu):
+  from tunix_amd.rl import common
+  rng = np.random.default_rng(4)
+  B, T = 8, 33
+  lp = rng.normal(size=(B, T)).astype(np.float32) - 2
+  old = lp + rng.normal(size=(B, T)).astype(np.float32) * 0.3
+  adv = rng.normal(size=(B,)).astype(np.float32)
+  ratio, loss, clipped = common.grpo_clipped_ratio(torch.from_numpy(lp).to(gpu), torch.from_numpy(old).to(gpu),
+                                                   torch.from_numpy(adv).to(gpu), 0.2, 0.28)
+  r_ref, l_ref, c_ref = R.grpo_ratio(lp, old, adv, 0.2, 0.28)
+  np.testing.assert_allclose(ratio.cpu().numpy(), r_ref, rtol=2e-6)
+  np.testing.assert_allclose(loss.cpu().numpy(), l_ref, rtol=2e-6, atol=1e-7)
+  np.testing.assert_array_equal(clipped.cpu().numpy(), c_ref)
+  ratio1, loss1, _ = common.grpo_clipped_ratio(torch.from_numpy(lp).to(gpu), None, torch.from_numpy(adv).to(gpu))
+  np.testing.assert_array_equal(ratio1.cpu().numpy(), 1.0)
+  np.testing.assert_allclose(loss1.cpu().numpy(), -adv[:, None] * np.ones((B, T), np.float32))
+
+
+def test_fused_head_logps_training_scale_shapes(gpu):
+  """The standalone fused per-token-logps case: hidden N(0,1) rows x a quantized lm_head
+  (int4 g128 + LoRA r64) -> log-softmax -> gather -> GRPO ratio, logits never materialised.
+  The oracle checks it at a vocabulary the CPU handles in seconds; at the full 128256-wide
+  vocabulary the checks are properties: the fused statistics agree with the logits of a few
+  rows materialised by the same kernel, and log-probabilities are a normalised distribution."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  D, r, group = 4096, 64, 128
+
+  def run(V, rows, seed, want_logits_rows=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(rows, D, generator=g).to(torch.bfloat16)
+    w = (torch.randn(D, V, generator=g) * 0.02).to(torch.bfloat16)
+    a = (torch.randn(D, r, generator=g) * 0.02).to(torch.bfloat16)
+    b = (torch.randn(r, V, generator=g) * 0.01).to(torch.bfloat16)
+    targets = torch.randint(0, V, (rows,), generator=g, dtype=torch.int32)
+    gx, gt = x.to(gpu), targets.to(gpu)
+    c, s = ops.quantize_pack(w.to(gpu), group, Q.INT4)
+    t = torch.zeros(rows, r, dtype=torch.bfloat16, device=gpu)
+    ops.lora_down(gx, a.t().contiguous().to(gpu), t)
+    gb = b.t().contiguous().to(gpu)
+    d = L.LmHeadDesc()
+    d.M, d.D, d.V = rows, D, V
+    d.x, d.codes, d.scales, d.group, d.qtype = gx.data_ptr(), c.data_ptr(), s.data_ptr(), group, Q.INT4
+    d.lora_rank, d.t, d.t_ld, d.lora_b, d.lora_scale = r, t.data_ptr(), r, gb.data_ptr(), 1.0
+    d.temperature = 1.0
+    part = torch.empty(rows * ops.lmhead_nblocks(V) * 4, dtype=torch.float32, device=gpu)
+    tlp = torch.empty(rows, dtype=torch.float32, device=gpu)
+    lse = torch.empty(rows, dtype=torch.float32, device=gpu)
+    d.targets, d.part, d.target_logp, d.lse = gt.data_ptr(), part.data_ptr(), tlp.data_ptr(), lse.data_ptr()
+    ops.lmhead(d)
+    lg = None
+    if want_logits_rows:
+      n = want_logits_rows
+      lg = torch.empty(n, V, dtype=torch.float32, device=gpu)
+      d2 = L.LmHeadDesc.from_buffer_copy(d)
+      d2.M, d2.logits_out = n, lg.data_ptr()
+      tlp2 = torch.empty(n, dtype=torch.float32, device=gpu)
+      lse2 = torch.empty(n, dtype=torch.float32, device=gpu)
+      d2.target_logp, d2.lse = tlp2.data_ptr(), lse2.data_ptr()
+      ops.lmhead(d2)
+      assert torch.equal(tlp2, tlp[:n]) and torch.equal(lse2, lse[:n])
+    torch.cuda.synchronize()
+    return x, w, a, b, targets, tlp.cpu(), lse.cpu(), (None if lg is None else lg.cpu())
+
+  # (1) against the oracle at a reduced vocabulary
+  V = 2048
+  x, w, a, b, targets, tlp, lse, _ = run(V, 192, 11)
+  codes, scale = Q.quantize(w.float().numpy(), group, Q.INT4)
+  logits = Q.rb(Q.qlinear_lora(x.float(), codes, scale, group, Q.INT4, a.float(), b.float(), 1.0))
+  want = R.selective_log_softmax(logits, targets)
+  assert (tlp - want).abs().max().item() <= 2e-2
+  # (2) the full vocabulary: properties
+  V = 128256
+  rows = 1024
+  x, w, a, b, targets, tlp, lse, lg = run(V, rows, 12, want_logits_rows=8)
+  assert torch.isfinite(tlp).all() and (tlp <= 0).all()
+  ref_lse = torch.logsumexp(lg, -1)
+  np.testing.assert_allclose(lse[:8].numpy(), ref_lse.numpy(), atol=2e-5)
+  sel = lg[torch.arange(8), targets[:8].long()] - ref_lse
+  np.testing.assert_allclose(tlp[:8].numpy(), sel.numpy(), atol=2e-5)
+  np.testing.assert_allclose(torch.exp(lg - ref_lse[:, None]).sum(-1).numpy(), 1.0, atol=1e-4)
+  # (3) GRPO ratio against noisy reference log-probabilities (eps 0.2)
+  from tunix_amd.rl import common
+  g = torch.Generator().manual_seed(13)
+  old = tlp + torch.randn(rows, generator=g) * 0.05
+  adv = torch.randn(rows // 64, generator=g)
+  ratio, loss, _ = common.grpo_clipped_ratio(tlp.view(-1, 64).to(gpu), old.view(-1, 64).to(gpu), adv.to(gpu), 0.2)
+  r_ref, l_ref, _ = R.grpo_ratio(tlp.view(-1, 64).numpy(), old.view(-1, 64).numpy(), adv.numpy(), 0.2, 0.2)
+  np.testing.assert_allclose(ratio.cpu().numpy(), r_ref, rtol=2e-6)
+  np.testing.assert_allclose(loss.cpu().numpy(), l_ref, rtol=2e-6, atol=1e-7)

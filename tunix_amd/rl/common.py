@@ -1,0 +1,112 @@
+"""Per-token log-probabilities and the GRPO clipped ratio on the quantized model
+(mirrors tunix/rl/common.py:187-203 selective_log_softmax, :326-482 compute_per_token_logps,
+:485-571 compute_chunked_logps and the ratio of tunix/rl/algo_core.py:440-489).
+
+compute_per_token_logps runs one full forward over prompt + completion (no cache reuse, the
+reference does the same), then feeds the hidden states of the positions that predict the
+completion tokens to the fused lm_head -> log-softmax -> gather kernel: full-vocabulary logits
+are never written to HBM, so `chunk_size` only bounds the number of rows per launch.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from .. import ops
+from ..model import QLoRAModel, Runner
+
+
+def selective_log_softmax(logits: torch.Tensor, input_ids: torch.Tensor) -> torch.Tensor:
+  """log_softmax(logits)[..., input_ids] for logits that already exist as a tensor
+  (tunix/rl/common.py:187-203).  A convenience on device tensors; the rollout path itself
+  goes through the fused head kernel and never materialises logits."""
+  lg = logits.to(torch.float32)
+  tgt = torch.gather(lg, -1, input_ids.long().unsqueeze(-1)).squeeze(-1)
+  return tgt - torch.logsumexp(lg, dim=-1)
+
+
+def process_ids(prompt_tokens: torch.Tensor, completion_tokens: torch.Tensor, pad_id: int):
+  """tunix/rl/common.py:234-291 (unpacked): concatenated ids and positions counted over
+  non-pad tokens.  The attention kernels derive the causal + padding mask from the ids
+  themselves (key != pad_id and key <= query), which is make_causal_attn_mask of that mask."""
+  ids = torch.cat([prompt_tokens, completion_tokens], dim=1).to(torch.int32).contiguous()
+  mask = ids != pad_id
+  run = torch.cumsum(mask.to(torch.int32), dim=-1)
+  positions = (run - (run >= 1).to(torch.int32)).to(torch.int32).contiguous()
+  return ids, positions
+
+
+def compute_per_token_logps(model: QLoRAModel, prompt_tokens, completion_tokens, pad_id: int,
+                            eos_id: int | None = None, *, temperature: float = 1.0,
+                            chunk_size: int = 0, return_entropy: bool = False,
+                            max_rows: int = 16384) -> torch.Tensor:
+  """fp32 [B, completion_len]: log p(completion token | everything before it).
+
+  prompt_tokens [B, P] (left padded) and completion_tokens [B, T] (right padded) are integer
+  arrays or tensors.  `temperature` divides the logits as in the reference (:431-436: ignored
+  when 0 or 1).  `max_rows` bounds the token rows of one forward pass.
+  """
+  if return_entropy:
+    raise NotImplementedError("per-token entropy is not produced by the fused head kernel")
+  dev = model.device
+  pt = torch.as_tensor(np.asarray(prompt_tokens) if not isinstance(prompt_tokens, torch.Tensor)
+                       else prompt_tokens).to(dev)
+  ct = torch.as_tensor(np.asarray(completion_tokens) if not isinstance(completion_tokens, torch.Tensor)
+                       else completion_tokens).to(dev)
+  if pt.ndim != 2 or ct.ndim != 2 or pt.shape[0] != ct.shape[0]:
+    raise ValueError(f"prompt_tokens {tuple(pt.shape)} and completion_tokens {tuple(ct.shape)} "
+                     "must be [B, P] and [B, T]")
+  B, T = ct.shape
+  ids, positions = process_ids(pt, ct, pad_id)
+  Ltot = ids.shape[1]
+  if T == 0:
+    return torch.zeros(B, 0, dtype=torch.float32, device=dev)
+  if Ltot < T + 1:
+    raise ValueError("the first completion token needs at least one token before it")
+  cfg = model.cfg
+  temp = 1.0 if temperature in (0.0, 1.0) else float(temperature)
+  rows_b = max(1, min(B, max_rows // Ltot))
+  runner = Runner(model, rows_b, Ltot, Ltot, pad_id, kv_chunk=0)
+  # the cache is scratch here: every layer writes its keys / values and reads them back
+  # within the same pass, so one pair of buffers serves all layers
+  kc = torch.empty(rows_b, cfg.num_kv_heads, Ltot, cfg.head_dim, dtype=torch.bfloat16, device=dev)
+  vc = torch.empty_like(kc)
+  head_rows = rows_b * T if chunk_size <= 0 else rows_b * min(T, chunk_size)
+  head_rows = min(head_rows, 8192)
+  part = torch.empty(head_rows * runner.nvb * 4, dtype=torch.float32, device=dev)
+  runner.part = part
+  xsel = torch.empty(rows_b * T, cfg.embed_dim, dtype=torch.bfloat16, device=dev)
+  out = torch.empty(B, T, dtype=torch.float32, device=dev)
+  for b0 in range(0, B, rows_b):
+    nb = min(rows_b, B - b0)
+    xn = runner.forward_hidden(ids[b0:b0 + nb], positions[b0:b0 + nb], runner.zero,
+                               [kc[:nb]] * cfg.num_layers, [vc[:nb]] * cfg.num_layers, B=nb, T=Ltot)
+    # logits[:, -T-1:-1] predict the completion tokens (:462-467)
+    xs = xsel[: nb * T]
+    xs.view(nb, T, -1).copy_(xn[: nb * Ltot].view(nb, Ltot, -1)[:, Ltot - T - 1: Ltot - 1])
+    tg = ids[b0:b0 + nb, Ltot - T:].contiguous().view(-1)
+    lp = out[b0:b0 + nb].view(-1)
+    for r0 in range(0, nb * T, head_rows):
+      nr = min(head_rows, nb * T - r0)
+      runner.run_head(xs[r0:r0 + nr], nr, temperature=temp, targets=tg[r0:r0 + nr],
+                      target_logp=lp[r0:r0 + nr])
+  return out
+
+
+def grpo_clipped_ratio(logp: torch.Tensor, old_logp: torch.Tensor | None, advantages: torch.Tensor,
+                       epsilon: float = 0.2, epsilon_high: float | None = None):
+  """(ratio, per-token loss, clipped flag) of tunix/rl/algo_core.py:440-489:
+  ratio = exp(logp - old_logp) (old_logp None: the on-policy case, ratio 1),
+  loss = max(-A * ratio, -A * clip(ratio, 1 - eps, 1 + eps_high)); A is per sequence."""
+  B, T = logp.shape
+  eps_hi = epsilon if epsilon_high is None else epsilon_high
+  lp = logp.to(torch.float32).contiguous()
+  old = None if old_logp is None else old_logp.to(torch.float32).contiguous()
+  adv = advantages.to(torch.float32).contiguous().view(-1)
+  if adv.numel() != B:
+    raise ValueError("advantages must hold one value per sequence")
+  ratio = torch.empty_like(lp)
+  loss = torch.empty_like(lp)
+  clipped = torch.empty(B, T, dtype=torch.int32, device=lp.device)
+  ops.grpo_ratio(lp, old, adv, T, epsilon, eps_hi, ratio=ratio, loss=loss, clipped=clipped)
+  return ratio, loss, clipped.bool()
