@@ -218,6 +218,14 @@ class RefModel:
     kk = cfg.num_experts_per_tok
     # top_k: descending, lower index first among equals
     order = torch.sort(probs, dim=-1, descending=True, stable=True).indices[..., :kk]
+    # diagnostic for tests: tokens whose k-th and (k+1)-th router scores lie within two bf16
+    # ulps of each other, where a different fp32 summation order may pick the other expert
+    ss = torch.sort(scores.float(), dim=-1, descending=True).values
+    gap = ss[..., kk - 1] - ss[..., kk]
+    ulp = torch.exp2(torch.floor(torch.log2(ss[..., kk - 1].abs().clamp_min(1e-30))) - 7)
+    if not hasattr(self, "route_near_tie"):
+      self.route_near_tie = {}
+    self.route_near_tie[i] = gap <= 2 * ulp
     wts = torch.gather(probs, -1, order)
     wts = self.r(wts / wts.sum(-1, keepdim=True))
     out = torch.zeros(B, T, D, dtype=torch.float64)
