@@ -7,8 +7,9 @@ JSON line.  A "step" is one decode step of the whole batch: embedding -> 32 laye
 greedy sampling -> token commit.
 
 Extra objects on the line:
-  roofline      the kernel with the largest share of a step, timed in isolation with events on
-                the launch stream at the mean context of the timed region
+  roofline      the kernel with the largest share of a step (the quantised GEMM), timed in
+                isolation with events on its launch stream; roofline_hbm prices the same
+                launches against the HBM roof
   kernels       the same measurement for every kernel family of the step
   cpu_baseline  the CPU oracle (a port of the reference's JAX path) timed on this host on a
                 bounded sample and scaled linearly
@@ -87,13 +88,32 @@ def kernel_breakdown(model, runner, st, ctx, iters):
   out["gqa_attn"] = {"ms": time_loop(attn, iters), "bytes": kv_bytes, "flops": 0, "per_step": cfg.num_layers}
 
   def lin(key, x, y, epi=L.TNX_EPI_STORE, residual=None):
+    """One fused linear as the decode step runs it (LoRA down-projection + GEMM + split-k sum)
+    and, separately, its main GEMM launch alone (`kernel_ms`)."""
+    import ctypes
+
     f = ly[key]
     nbytes = f.codes.numel() * 4 + f.scales.numel() * 2
     if f.has_lora:
       nbytes += (f.K * f.r * len(f.names) + f.N * f.r) * 2
     nbytes += B * f.K * 2 + B * (f.N // (2 if f.interleave2 else 1)) * 2
     ms = time_loop(lambda: runner.linear(f, x, y, B, epilogue=epi, residual=residual), iters)
-    return {"ms": ms, "bytes": nbytes, "flops": 2.0 * B * f.K * f.N, "per_step": cfg.num_layers}
+    split = runner._split_k(f, B)
+    d = ops.make_qlinear_desc(
+        M=B, K=f.K, N=f.N, group=f.group, qtype=f.qtype, x=x, codes=f.codes, scales=f.scales, y=y,
+        epilogue=epi, residual=residual, lora_rank=f.rp,
+        lora_nseg=(-1 if f.interleave2 else len(f.names)), lora_seg_end=f.seg_end,
+        lora_seg_toff=f.seg_toff, t=runner.t if f.has_lora else None, t_ld=runner.t.shape[1],
+        lora_b=f.b_t if f.has_lora else None, lora_scale=f.lora_scale, split_k=split,
+        ws=runner.splitk_ws if split > 1 else None)
+    stream = torch.cuda.current_stream
+
+    def gemm_only():
+      L.check(L.lib().tnx_qlinear_lora(stream().cuda_stream, ctypes.byref(d)), "tnx_qlinear_lora")
+
+    kms = time_loop(gemm_only, iters)
+    return {"ms": ms, "kernel_ms": kms, "bytes": nbytes, "flops": 2.0 * B * f.K * f.N,
+            "per_step": cfg.num_layers, "split_k": split}
 
   out["qlinear_qkv"] = lin("qkv", runner.xn, runner.qkv)
   out["qlinear_o"] = lin("o", runner.attn, runner.tmp)
@@ -109,6 +129,28 @@ def kernel_breakdown(model, runner, st, ctx, iters):
     v["tflops"] = v["flops"] / (v["ms"] * 1e-3) / 1e12
     v["step_ms"] = v["ms"] * v["per_step"]
   return out
+
+
+def rooflines(kern):
+  """The dominant kernel of a step is the quantised GEMM (one kernel, launched for the four
+  linears of every layer).  One launch = the mean over those four shapes.  At 128 rows its
+  arithmetic intensity (2 * 128 flop per 0.53 B of packed weight = 483 flop/B) is past the
+  machine's ridge (2.5 PFLOP/s / 8 TB/s = 312 flop/B), so the bounding roof is the bf16 MFMA
+  peak; the same launches priced against the HBM roof are reported beside it."""
+  names = [k for k in kern if k.startswith("qlinear")]
+  flops = sum(kern[k]["flops"] for k in names) / len(names)
+  nbytes = sum(kern[k]["bytes"] for k in names) / len(names)
+  us = sum(kern[k]["kernel_ms"] for k in names) / len(names) * 1e3
+  tf = flops / (us * 1e-6) / 1e12
+  gbs = nbytes / (us * 1e-6) / 1e9
+  roofline = {"kernel": "qgemm128_kernel", "bound": "mfma", "achieved": round(tf, 1),
+              "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+              "traffic": None, "us_per_launch": round(us, 2), "algorithmic_flops": flops,
+              "algorithmic_bytes": nbytes,
+              "launch_shapes_us": {k: round(kern[k]["kernel_ms"] * 1e3, 2) for k in names}}
+  roofline_hbm = {"kernel": "qgemm128_kernel", "bound": "hbm", "achieved": round(gbs, 1),
+                  "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4)}
+  return roofline, roofline_hbm
 
 
 def cpu_baseline(cfg_full, B, ctx, S, threads):
@@ -167,6 +209,9 @@ def main():
   ap.add_argument("--layers", type=int, default=0, help="debug only: fewer layers (invalidates the metric)")
   ap.add_argument("--no-cpu-baseline", action="store_true")
   ap.add_argument("--kernel-iters", type=int, default=20)
+  ap.add_argument("--kernels-only", action="store_true",
+                  help="profiling aid: one layer, no prefill / decode; only the per-kernel loops at "
+                       "context prompt + gen / 2 (prints the kernel table, not the metric)")
   args = ap.parse_args()
   if args.gpus != 1:
     print("bench.py measures one GPU: this build has no multi-GPU path (the decode path shards "
@@ -189,6 +234,33 @@ def main():
     cfg = config.llama31_8b(num_layers=args.layers)
   B, P, T = args.batch, args.prompt, args.gen
   S = P + T
+  if args.kernels_only:
+    cfg = config.llama31_8b(num_layers=1)
+    model = QLoRAModel(cfg, dummy_model.create_dummy_weights(cfg, seed=20253, device=dev), dev)
+    ids = np.random.Generator(np.random.PCG64(20253)).integers(1, cfg.vocab_size, size=(B, P)).astype(np.int32)
+    st = _SamplingState(model, ids, S, S, 0, False, False)
+    st.token_buffer.fill_(5)
+    for kc, vc in zip(st.kcache, st.vcache):
+      kc.normal_()
+      vc.normal_()
+    runner = Runner(model, B, 1, S, 0)
+    for buf in (runner.xn, runner.attn, runner.act, runner.q):
+      buf.normal_()
+    kern = kernel_breakdown(model, runner, st, P + T // 2, args.kernel_iters)
+    roofline, roofline_hbm = rooflines(kern)
+    # a plain device copy of known size (256 MiB read + 256 MiB written): the yardstick that
+    # scales the FETCH_SIZE / WRITE_SIZE counters of a counter-collection run of this command
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+      dst.copy_(src)
+    torch.cuda.synchronize()
+    print(json.dumps({"kernels_only": True, "context": P + T // 2, "roofline": roofline,
+                      "roofline_hbm": roofline_hbm,
+                      "kernels": {k: {"us": round(v["ms"] * 1e3, 2),
+                                      "gemm_us": round(v.get("kernel_ms", v["ms"]) * 1e3, 2)}
+                                  for k, v in kern.items()}}), flush=True)
+    return
   W = max(1, args.warmup)
   K = args.steps
   if W + K > T - 1:
@@ -244,20 +316,7 @@ def main():
   for name, v in kern.items():
     log(f"  {name:16s} {v['ms'] * 1e3:8.1f} us/launch  {v['gbs']:7.0f} GB/s  {v['tflops']:7.1f} TFLOP/s"
         f"  x{v['per_step']} = {v['step_ms']:.3f} ms/step")
-  dom_name = max(kern, key=lambda k: kern[k]["step_ms"])
-  dom = kern[dom_name]
-  hbm_frac = dom["gbs"] / HBM_PEAK_GBS
-  roofline = {"kernel": dom_name, "bound": "hbm", "achieved": round(dom["gbs"], 1),
-              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(hbm_frac, 4), "traffic": None,
-              "us_per_launch": round(dom["ms"] * 1e3, 2), "algorithmic_bytes": dom["bytes"]}
-  lin_bytes = sum(kern[k]["bytes"] for k in kern if k.startswith("qlinear"))
-  lin_ms = sum(kern[k]["ms"] for k in kern if k.startswith("qlinear"))
-  lin_flops = sum(kern[k]["flops"] for k in kern if k.startswith("qlinear"))
-  roofline_linears = {
-      "bound": "hbm", "achieved": round(lin_bytes / (lin_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
-      "unit": "GB/s", "frac": round(lin_bytes / (lin_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-      "mfma_tflops": round(lin_flops / (lin_ms * 1e-3) / 1e12, 1),
-      "mfma_frac": round(lin_flops / (lin_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+  roofline, roofline_linears = rooflines(kern)
   wb = model.weight_bytes()
   step_bytes = (wb["quantized"] + wb["lora"] + wb["head"]
                 + B * cfg.num_kv_heads * mean_ctx * cfg.head_dim * 4 * cfg.num_layers)
@@ -271,7 +330,7 @@ def main():
                  "context_range": [step_first + 1, step_last + 1], "parallelism": "single GPU"},
       "hbm_roofline_frac_step": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
       "step_bytes": int(step_bytes), "prefill_s": round(prefill_s, 3),
-      "roofline": roofline, "roofline_linears": roofline_linears,
+      "roofline": roofline, "roofline_hbm": roofline_linears,
       "kernels": {k: {"us": round(v["ms"] * 1e3, 2), "GBps": round(v["gbs"], 1),
                       "TFLOPs": round(v["tflops"], 1), "ms_per_step": round(v["step_ms"], 4)}
                   for k, v in kern.items()},
