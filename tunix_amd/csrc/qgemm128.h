@@ -27,7 +27,7 @@ typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
 
 constexpr int kBigLutBytes = 256 * 256;
 constexpr int kBigABytes = 128 * A_LD * 2;
-constexpr size_t kBigSmemBytes = kBigLutBytes + 2 * (size_t)kBigABytes;
+constexpr size_t kBigSmemBytes = kBigLutBytes + 2 * (size_t)kBigABytes + 4 * 4096;  // + adapter fragments
 
 // LDS accesses by absolute LDS byte address (the dynamic LDS block of these kernels starts at
 // address 0: they declare no static LDS).
@@ -44,6 +44,18 @@ __device__ __forceinline__ void lds_st128(uint32_t addr, u32x4 v) {
 template <int V>
 using ic = std::integral_constant<int, V>;
 
+// Optional phase time stamps of work-group (0,0,0) for kernel tuning (off in the product build).
+#ifdef TNX_TIMING
+__device__ unsigned long long tnx_stamps[8];
+#define TNX_STAMP(i)                                                                     \
+  do {                                                                                   \
+    if (threadIdx.x == 0 && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0)       \
+      tnx_stamps[i] = __builtin_amdgcn_s_memrealtime();                                      \
+  } while (0)
+#else
+#define TNX_STAMP(i) do {} while (0)
+#endif
+
 // The launch bound is a register-budget choice, not the work-group size (always 256): with
 // NT = 2 everything fits the 256 architectural VGPRs, and keeping the accumulators there
 // avoids the accumulator-register copies the compiler emits around loops whose MFMA results
@@ -55,13 +67,13 @@ void qgemm128_kernel(const QLArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wn = tid >> 6;
   const int lm = lane & 15, lq = lane >> 4;
-  {  // table entry `tid` = f16 pair (level[tid & 15], level[tid >> 4]); copies rotated over banks
-    uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
-    const h16x2 h = {(_Float16)rbf(code_level(a.qtype, tid & 15)), (_Float16)rbf(code_level(a.qtype, tid >> 4))};
-    const uint32_t v = __builtin_bit_cast(uint32_t, h);
-#pragma unroll
-    for (int c = 0; c < 64; ++c) lut[tid * 64 + ((c + lane) & 63)] = v;
-  }
+  TNX_STAMP(0);
+  // LDS is addressed absolutely below (table at 0): bail out if the dynamic block does not
+  // start at LDS address 0, which would mean a static LDS allocation crept into this kernel
+  if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem != 0u) return;
+  // the two code-book levels of this thread's table entry, fetched before anything else so
+  // that their (constant-memory) loads are the oldest ones in flight
+  const float lvl0 = rbf(code_level(a.qtype, tid & 15)), lvl1 = rbf(code_level(a.qtype, tid >> 4));
   const uint32_t lane_off = (uint32_t)lane * 4u;
   const int64_t m0 = (int64_t)blockIdx.x * 128;
   const int64_t ntile0 = ((int64_t)blockIdx.y * 4 + wn) * NT;
@@ -77,10 +89,9 @@ void qgemm128_kernel(const QLArgs a) {
   // Per-thread offsets (32 bit: the host checks the 4 GiB limits); the k-tile enters as the
   // scalar offset of the load.  Rows past M and column tiles past N start beyond the buffer
   // and read zeros.
-  uint32_t xoff[MT], coff[NT], soff[NT];
-#pragma unroll
-  for (int c = 0; c < MT; ++c)
-    xoff[c] = ((uint32_t)(m0 + (tid >> 4) + 16 * c) * (uint32_t)a.K + (uint32_t)(tid & 15) * 8u) * 2u;
+  uint32_t coff[NT], soff[NT];
+  const uint32_t xbase = ((uint32_t)(m0 + (tid >> 4)) * (uint32_t)a.K + (uint32_t)(tid & 15) * 8u) * 2u;
+  const uint32_t xstride = 16u * (uint32_t)a.K * 2u;  // 16 rows further per chunk
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     const uint32_t tile0 = (uint32_t)(ntile0 + nt) * (uint32_t)ktiles;
@@ -102,11 +113,73 @@ void qgemm128_kernel(const QLArgs a) {
   u32x4 bfr[2][NT];       // weight fragments of this and the next k-step
   uint32_t lp[NT][4];     // table entries (f16 level pairs) of the k-step after the next
 
+  // LoRA delta through the activation pipeline: the "k-tile" after the last real one is the
+  // 128-row block of t = bf16(x . A), columns [toff_a, +64) | [toff_b, +64) (the one or two
+  // adapter segments this work-group's columns belong to), so that it is in LDS when the main
+  // loop ends; the B^T fragments of this wave's columns are fetched at kernel start.
+  int toff[NT];
+  int toff_a = 0, toff_b = 0;
+  bool lora_fast = a.lora_rank > 0 && a.lora_rank <= 64 && blockIdx.z == 0;
+  if (a.lora_rank > 0) {
+    auto seg_toff = [&](int64_t ntile) {
+      if (a.lora_nseg < 0) return (int)(ntile & 1) * a.lora_rank;  // interleaved gate / up pair
+      int o = a.lora_seg_toff[0];
+#pragma unroll
+      for (int q = 1; q < 4; ++q)  // constant bounds: the argument arrays stay in SGPRs
+        if (q < a.lora_nseg && ntile * 16 >= a.lora_seg_end[q - 1]) o = a.lora_seg_toff[q];
+      return o;
+    };
+    const int64_t wg_nt0 = (int64_t)blockIdx.y * 4 * NT;
+    toff_a = seg_toff(wg_nt0);
+    toff_b = seg_toff(min(wg_nt0 + 4 * NT - 1, ntiles - 1));
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) toff[nt] = seg_toff(min(ntile0 + nt, ntiles - 1));
+    // the tile is shared by the four waves, so the decision is taken over all column tiles of
+    // the work-group (identically in every thread; no LDS or barrier involved: this kernel
+    // addresses LDS absolutely and must not acquire a static allocation): a work-group
+    // spanning three segments falls back to fragments from global memory
+    for (int q = 0; q < 4 * NT; ++q) {
+      const int o = seg_toff(min(wg_nt0 + q, ntiles - 1));
+      lora_fast = lora_fast && (o == toff_a || o == toff_b);
+    }
+  }
+  // B^T fragments of the adapter for this wave's columns: fetched now, parked in this wave's
+  // private 4 KiB of LDS behind the activation buffers (no barrier needed) until the epilogue
+  const uint32_t lb_lds = kBigLutBytes + 2 * kBigABytes + (uint32_t)wn * 4096u + (uint32_t)lane * 16u;
+  uint32_t tbase = 0;
+  u32x4 lbv[NT][2];  // live only until the main loop starts
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) lbv[nt][j] = u32x4{0, 0, 0, 0};
+  if (lora_fast) {
+    const rsrc_t rb = make_rsrc(a.lora_b, (uint64_t)a.N * a.lora_rank * 2);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        if (j * 32 < a.lora_rank)
+          lbv[nt][j] = buf_load128(rb, (((uint32_t)(ntile0 + nt) * 16u + (uint32_t)lm) * (uint32_t)a.lora_rank +
+                                        (uint32_t)(j * 32 + lq * 8)) * 2u);
+    const int ch = tid & 15;
+    const int col = ((ch < 8) ? toff_a : toff_b) + min((ch & 7) * 8, a.lora_rank - 8);
+    tbase = (uint32_t)((m0 + (tid >> 4)) * a.t_ld + col) * 2u;
+  }
+  const rsrc_t rt = make_rsrc(lora_fast ? (const void*)a.t : (const void*)a.x,
+                              lora_fast ? (uint64_t)a.M * a.t_ld * 2 : (uint64_t)a.M * a.K * 2);
+  const uint32_t tstride = (uint32_t)(16 * a.t_ld * 2);
+
   // k-tiles past the last one are clamped: their data is fetched but never multiplied
   auto load_a = [&](int kt) {
-    const int s = min(kt, ktiles - 1) * (KTILE * 2);
+    const bool ut = lora_fast && kt >= kt_end;
+    const int s = ut ? 0 : min(kt, ktiles - 1) * (KTILE * 2);
+    const rsrc_t r = ut ? rt : rx;
+    // bit selects (not ?:, which the compiler turns into a private-memory table)
+    const uint32_t m = 0u - (uint32_t)ut;
+    const uint32_t base = xbase ^ ((xbase ^ tbase) & m), stride = xstride ^ ((xstride ^ tstride) & m);
 #pragma unroll
-    for (int c = 0; c < MT; ++c) a_next[c] = __builtin_amdgcn_raw_buffer_load_b128(rx, xoff[c], s, 0);
+    for (int c = 0; c < MT; ++c)
+      a_next[c] = __builtin_amdgcn_raw_buffer_load_b128(r, base + (uint32_t)c * stride, s, 0);
   };
   auto load_w = [&](auto Dc, int kt) {
     constexpr int D = decltype(Dc)::value;
@@ -244,6 +317,15 @@ void qgemm128_kernel(const QLArgs a) {
     load_w(ic<0>{}, kt_begin);
     load_w(ic<1>{}, kt_begin + 1);
     load_w(ic<2>{}, kt_begin + 2);
+    {  // table entry `tid` = f16 pair (level[tid & 15], level[tid >> 4]); copies rotated over
+       // banks; built while the first loads are in flight
+      uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
+      const h16x2 h = {(_Float16)lvl0, (_Float16)lvl1};
+      const uint32_t v = __builtin_bit_cast(uint32_t, h);
+#pragma unroll
+      for (int c = 0; c < 64; ++c) lut[tid * 64 + ((c + lane) & 63)] = v;
+    }
+    TNX_STAMP(1);
     store_a(a_wr);
     load_a(kt_begin + 1);
     expand_scales(ic<0>{}, ic<0>{}, true);
@@ -252,35 +334,55 @@ void qgemm128_kernel(const QLArgs a) {
     read_a(af[0], a_rd, ic<0>{}, ic<0>{});
     convert(ic<0>{}, ic<0>{}, bfr[0], lp);
     lut_issue(ic<0>{}, ic<1>{}, lp);
-    // three k-tiles (one turn of the ring) per iteration; a padded tail runs on zero scales
+    if (lora_fast) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) lds_st128(lb_lds + (uint32_t)((nt * 2 + j) * 1024), lbv[nt][j]);
+    }
+    TNX_STAMP(2);
+    // three k-tiles (one turn of the ring) per iteration
     for (int kt = kt_begin; kt < kt_end; kt += PF) {
       tile(ic<0>{}, kt);
-      tile(ic<1>{}, kt + 1);
-      tile(ic<2>{}, kt + 2);
+      if (kt + 1 < kt_end) tile(ic<1>{}, kt + 1);
+      if (kt + 2 < kt_end) tile(ic<2>{}, kt + 2);
     }
   }
+  TNX_STAMP(3);
 
-  if (a.lora_rank > 0 && blockIdx.z == 0) {
+  if (lora_fast) {
+    // the t block sits in the activation buffer the last k-tile left as "next"
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const uint32_t base = a_rd + (uint32_t)((toff[nt] == toff_a ? 0 : 64) * 2);
+      f32x4 part[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) zero_acc(part[mt]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (j * 32 < a.lora_rank) {
+          const u32x4 lbf = lds_ld128(lb_lds + (uint32_t)((nt * 2 + j) * 1024));
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            part[mt] = mfma16(lds_ld128(base + (uint32_t)((mt * 16 * A_LD + j * 32) * 2)), lbf, part[mt]);
+        }
+      }
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[mt][nt][i] += a.lora_scale * part[mt][i];
+    }
+  } else if (a.lora_rank > 0 && blockIdx.z == 0) {
     TileSrc s;
     s.M = a.M; s.K = a.K; s.x = a.x; s.row_index = nullptr; s.row_div = 1; s.x_rows = a.M;
     s.w_bf16 = nullptr; s.codes = a.codes; s.scales = a.scales; s.group = a.group; s.qtype = a.qtype;
     s.ntiles = ntiles; s.lora_rank = a.lora_rank; s.t = a.t; s.t_ld = a.t_ld; s.lora_b = a.lora_b;
     s.lora_scale = a.lora_scale;
-    int toff[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const int64_t col0 = (ntile0 + nt) * 16;
-      if (a.lora_nseg < 0) {
-        toff[nt] = (int)((ntile0 + nt) & 1) * a.lora_rank;  // interleaved gate/up pair
-      } else {
-        toff[nt] = a.lora_seg_toff[0];
-        for (int q = 1; q < a.lora_nseg; ++q)
-          if (col0 >= a.lora_seg_end[q - 1]) toff[nt] = a.lora_seg_toff[q];
-      }
-    }
     tile_lora<MT, NT>(s, m0, ntile0, toff, acc);
   }
+  TNX_STAMP(4);
   store_tile<MT, NT>(a, m0, a.M, ntile0, ntiles, acc, [](int64_t r) { return r; });
+  TNX_STAMP(5);
 }
 
 }  // namespace

@@ -555,3 +555,10 @@ extern "C" int tnx_moe_int4_gmm(void* stream, const tnx_moe_gmm_desc* d) {
   if (max_rows <= 32) return launch_moe<2, 2>(st, a, d->E, max_rows);
   return launch_moe<4, 2>(st, a, d->E, max_rows);
 }
+
+#ifdef TNX_TIMING
+// tuning aid (not part of the product build): the phase stamps of the last qgemm128 launch
+extern "C" int tnx_debug_stamps(unsigned long long* out8) {
+  return hipMemcpyFromSymbol(out8, HIP_SYMBOL(tnx_stamps), 8 * sizeof(unsigned long long)) == hipSuccess ? 0 : -1;
+}
+#endif
