@@ -70,6 +70,72 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* x, const u
   }
 }
 
+// The same op for D % 8 == 0 (every model on the path): 16-byte loads and stores, the row stays
+// in registers between the two passes (thread t owns the 8-element chunks t, t + 256, ...).
+constexpr int kNormMaxChunks = 8;  // D <= 8 * 256 * 8 = 16384
+__device__ __forceinline__ void unpack8(const u32x4& p, float (&f)[8]) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    f[2 * j] = bflo(p[j]);
+    f[2 * j + 1] = bfhi(p[j]);
+  }
+}
+__global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, const uint16_t* res_pre,
+                                                          uint16_t* h_out, const uint16_t* w,
+                                                          const uint16_t* res_post, uint16_t* y,
+                                                          int64_t D, float eps, int flavor) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const int nchunks = (int)(D / 8);
+  float h[kNormMaxChunks][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < kNormMaxChunks; ++c) {
+    const int ch = c * 256 + threadIdx.x;
+    if (ch < nchunks) {
+      const int64_t o = row * D + (int64_t)ch * 8;
+      unpack8(*reinterpret_cast<const u32x4*>(x + o), h[c]);
+      if (res_pre) {
+        float r[8];
+        unpack8(*reinterpret_cast<const u32x4*>(res_pre + o), r);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) h[c][j] = rbf(h[c][j] + r[j]);
+      }
+      if (h_out) {
+        u32x4 q;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) q[j] = pack2bf(h[c][2 * j], h[c][2 * j + 1]);
+        *reinterpret_cast<u32x4*>(h_out + o) = q;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += sq_term(h[c][j], flavor);
+    }
+  }
+  ss = block_sum(ss, red);
+  const float ms = finish_ms(ss, (float)D, flavor);
+#pragma unroll
+  for (int c = 0; c < kNormMaxChunks; ++c) {
+    const int ch = c * 256 + threadIdx.x;
+    if (ch < nchunks) {
+      const int64_t o = row * D + (int64_t)ch * 8;
+      float wv[8], v[8];
+      unpack8(*reinterpret_cast<const u32x4*>(w + (int64_t)ch * 8), wv);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = norm_elem(h[c][j], wv[j], ms, eps, flavor);
+      if (res_post) {
+        float r[8];
+        unpack8(*reinterpret_cast<const u32x4*>(res_post + o), r);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = rbf(v[j] + r[j]);
+      }
+      u32x4 q;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) q[j] = pack2bf(v[2 * j], v[2 * j + 1]);
+      *reinterpret_cast<u32x4*>(y + o) = q;
+    }
+  }
+}
+
 __global__ void embed_kernel(const uint16_t* table, int64_t V, int64_t D, const int32_t* ids,
                              int64_t ids_ld, const int32_t* col_ptr, int64_t T, float scale_bf,
                              uint16_t* out) {
@@ -198,8 +264,12 @@ extern "C" int tnx_rmsnorm(void* stream, const uint16_t* x, const uint16_t* res_
   TNX_REQUIRE(x && w && y, "rmsnorm: null pointer");
   TNX_REQUIRE(M > 0 && D > 0 && D <= 16384, "rmsnorm: D=%lld out of range (1..16384)", (long long)D);
   TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm: bad flavor %d", flavor);
-  hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)M), dim3(256), (size_t)D * sizeof(float),
-                     as_stream(stream), x, res_pre, h_out, w, res_post, y, D, eps, flavor);
+  if (D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks)
+    hipLaunchKernelGGL(rmsnorm_vec_kernel, dim3((unsigned)M), dim3(256), 0, as_stream(stream), x, res_pre,
+                       h_out, w, res_post, y, D, eps, flavor);
+  else
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)M), dim3(256), (size_t)D * sizeof(float),
+                       as_stream(stream), x, res_pre, h_out, w, res_post, y, D, eps, flavor);
   TNX_CHECK_LAUNCH("rmsnorm");
   return TNX_OK;
 }
