@@ -78,6 +78,10 @@ __global__ __launch_bounds__(64) void attn_kernel(const AttnArgs a) {
   const uint16_t* vbase = a.v + ((b * a.Hkv + hkv) * a.S) * DH;
   const int32_t* tok = a.tokens + b * a.tok_ld;
   const int vcol = (8 * lm) % (DH < 128 ? DH : 128);     // DH=64: upper lanes duplicate
+  // 16-byte token loads need 16-byte aligned rows; slots past S - 4 are clamped (keys beyond
+  // the range are masked by the range test anyway)
+  const bool tok_vec = (a.tok_ld % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.tokens) & 15) == 0) && a.S >= 4;
+  const int tok_last4 = ((int)a.S - 4) & ~3;
 
   for (int kb = k_lo & ~31; kb <= k_hi; kb += 32) {
     // ---- loads: K as A fragments (two tiles of 16 keys), V rows of this lane's 8 keys ----
@@ -99,13 +103,26 @@ __global__ __launch_bounds__(64) void attn_kernel(const AttnArgs a) {
       for (int h = 0; h < NH; ++h)
         vf[h][s] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)key * DH + h * 128 + vcol);
     }
+    // token ids of this lane's 8 keys (two runs of 4 consecutive slots), fetched unconditionally
+    // together with K and V: a predicated load per key would serialise eight memory latencies
+    int tk[8];
+    if (tok_vec) {
+      const u32x4 t0 = *reinterpret_cast<const u32x4*>(tok + min(kb + 4 * lq, tok_last4));
+      const u32x4 t1 = *reinterpret_cast<const u32x4*>(tok + min(kb + 16 + 4 * lq, tok_last4));
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        tk[s] = (int)t0[s];
+        tk[4 + s] = (int)t1[s];
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < 8; ++s) tk[s] = tok[min(keys[s], (int)a.S - 1)];
+    }
     bool kvalid[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       const int key = keys[s];
-      bool ok = qvalid && key >= max(k_lo, lo_n) && key <= min(k_hi, c_n);
-      if (ok) ok = tok[key] != a.pad_id;
-      kvalid[s] = ok;
+      kvalid[s] = qvalid && key >= max(k_lo, lo_n) && key <= min(k_hi, c_n) && tk[s] != a.pad_id;
     }
     // ---- S^T = K . q^T ----
     f32x4 st[2];
@@ -142,9 +159,18 @@ __global__ __launch_bounds__(64) void attn_kernel(const AttnArgs a) {
     pa[2] = pack2bf(p[4], p[5]);
     pa[3] = pack2bf(p[6], p[7]);
     // ---- O = O * alpha + P . V ----
-    float ar[4];
+    // the running maximum settles after a few blocks: rescale O only when some column moved
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+      float ar[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) ar[i] = __shfl(alpha, 4 * lq + i, 64);
+      for (int i = 0; i < 4; ++i) ar[i] = __shfl(alpha, 4 * lq + i, 64);
+#pragma unroll
+      for (int h = 0; h < NH; ++h)
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) O[h][jj][i] *= ar[i];
+    }
 #pragma unroll
     for (int h = 0; h < NH; ++h)
 #pragma unroll
@@ -154,10 +180,7 @@ __global__ __launch_bounds__(64) void attn_kernel(const AttnArgs a) {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
           bfrag[r] = __builtin_amdgcn_perm(vf[h][2 * r + 1][jj >> 1], vf[h][2 * r][jj >> 1], sel);
-        f32x4 o = O[h][jj];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] *= ar[i];
-        O[h][jj] = mfma16(pa, bfrag, o);
+        O[h][jj] = mfma16(pa, bfrag, O[h][jj]);
       }
   }
 
