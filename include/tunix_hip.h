@@ -152,6 +152,13 @@ int tnx_embed(void* stream, const uint16_t* table, int64_t V, int64_t D, const i
 int tnx_rmsnorm(void* stream, const uint16_t* x, const uint16_t* res_pre, uint16_t* h_out,
                 const uint16_t* w, const uint16_t* res_post, uint16_t* y, int64_t M, int64_t D,
                 float eps, int flavor);
+/* The same, with the input row taken from the fp32 partial planes ws[split_k][M][D] that
+ * tnx_qlinear_lora leaves when split_k > 1 (N == D): x = bf16(sum_z ws[z]) in split order.  It
+ * replaces tnx_splitk_finish + tnx_rmsnorm for a linear whose output feeds a residual add and a
+ * norm (o_proj / down_proj: llama3/model.py:560-563).  D % 8 == 0. */
+int tnx_rmsnorm_splitk(void* stream, const float* ws, int split_k, const uint16_t* res_pre,
+                       uint16_t* h_out, const uint16_t* w, const uint16_t* res_post, uint16_t* y,
+                       int64_t M, int64_t D, float eps, int flavor);
 
 /* ---------------------------------------------------------------------------------------
  * Per-head q/k RMSNorm (optional) + RoPE + KV-cache write for T tokens per row.

@@ -566,3 +566,32 @@ def test_argument_errors_raise(gpu):
   x = torch.zeros(4, 128, dtype=torch.bfloat16, device=gpu)
   with pytest.raises(ValueError):
     ops.quantize_pack(x.t().contiguous(), 48, 0)
+
+
+@pytest.mark.parametrize("family", ["llama3", "qwen3"])
+def test_rmsnorm_splitk_equals_finish_then_norm(gpu, family):
+  """The folded pass (sum of split-k planes + residual + norm) against the two separate
+  kernels it replaces: bit for bit."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  from tunix_amd.model import _NORM
+  M, K, D, g, split = 128, 1024, 512, 64, 4
+  x, res = rnd((M, K), 80), rnd((M, D), 81)
+  w = rnd((K, D), 82, 0.02)
+  nw = bf(rnd((D,), 83, 0.3) + 1.0).to(gpu)
+  c, s = ops.quantize_pack(bf(w).to(gpu), g, Q.NF4)
+  gx, gres = bf(x).to(gpu), bf(res).to(gpu)
+  ws = torch.empty(split * M * D, dtype=torch.float32, device=gpu)
+  h1 = torch.empty(M, D, dtype=torch.bfloat16, device=gpu)
+  d = ops.make_qlinear_desc(M=M, K=K, N=D, group=g, qtype=Q.NF4, x=gx, codes=c, scales=s, y=h1,
+                            epilogue=L.TNX_EPI_RESIDUAL, residual=gres, split_k=split, ws=ws)
+  ops.qlinear(d)                                   # partial planes + finishing pass
+  y1 = torch.empty_like(h1)
+  ops.rmsnorm(h1, nw, y1, 1e-5, _NORM[family])
+  ops.qlinear(d, finish=False)                     # planes only
+  h2 = gres.clone()
+  y2 = torch.empty_like(h1)
+  ops.rmsnorm_splitk(ws, split, nw, y2, 1e-5, _NORM[family], M, D, res_pre=h2, h_out=h2)
+  torch.cuda.synchronize()
+  assert torch.equal(h1, h2)
+  assert torch.equal(y1, y2)

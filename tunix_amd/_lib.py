@@ -91,6 +91,7 @@ SIGNATURES = {
     "tnx_lora_down": (_i32, [_p, _p, _i64, _i64, _p, _i32, _p, _i64]),
     "tnx_embed": (_i32, [_p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _f32, _p]),
     "tnx_rmsnorm": (_i32, [_p, _p, _p, _p, _p, _p, _p, _i64, _i64, _f32, _i32]),
+    "tnx_rmsnorm_splitk": (_i32, [_p, _p, _i32, _p, _p, _p, _p, _p, _i64, _i64, _f32, _i32]),
     "tnx_qknorm_rope_kvwrite": (_i32, [_p, C.POINTER(RopeDesc)]),
     "tnx_attn_ws_bytes": (C.c_size_t, [_i64, _i64, _i64, _i32, _i32, _i32]),
     "tnx_gqa_attn": (_i32, [_p, C.POINTER(AttnDesc)]),

@@ -80,10 +80,13 @@ __device__ __forceinline__ void unpack8(const u32x4& p, float (&f)[8]) {
     f[2 * j + 1] = bfhi(p[j]);
   }
 }
+// With `ws` the input row is bf16(sum of the split_k fp32 partial planes ws[z][row][:]) of a
+// split-k linear, added in split order: the linear's own finishing pass folded into the norm.
 __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, const uint16_t* res_pre,
                                                           uint16_t* h_out, const uint16_t* w,
                                                           const uint16_t* res_post, uint16_t* y,
-                                                          int64_t D, float eps, int flavor) {
+                                                          int64_t D, float eps, int flavor,
+                                                          const float* ws, int split_k, int64_t plane) {
   __shared__ float red[4];
   const int64_t row = blockIdx.x;
   const int nchunks = (int)(D / 8);
@@ -94,7 +97,23 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
     const int ch = c * 256 + threadIdx.x;
     if (ch < nchunks) {
       const int64_t o = row * D + (int64_t)ch * 8;
-      unpack8(*reinterpret_cast<const u32x4*>(x + o), h[c]);
+      if (ws) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) h[c][j] = 0.f;
+        for (int z = 0; z < split_k; ++z) {
+          const f32x4 p0 = *reinterpret_cast<const f32x4*>(ws + z * plane + o);
+          const f32x4 p1 = *reinterpret_cast<const f32x4*>(ws + z * plane + o + 4);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            h[c][j] += p0[j];
+            h[c][4 + j] += p1[j];
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) h[c][j] = rbf(h[c][j]);
+      } else {
+        unpack8(*reinterpret_cast<const u32x4*>(x + o), h[c]);
+      }
       if (res_pre) {
         float r[8];
         unpack8(*reinterpret_cast<const u32x4*>(res_pre + o), r);
@@ -266,11 +285,26 @@ extern "C" int tnx_rmsnorm(void* stream, const uint16_t* x, const uint16_t* res_
   TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm: bad flavor %d", flavor);
   if (D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks)
     hipLaunchKernelGGL(rmsnorm_vec_kernel, dim3((unsigned)M), dim3(256), 0, as_stream(stream), x, res_pre,
-                       h_out, w, res_post, y, D, eps, flavor);
+                       h_out, w, res_post, y, D, eps, flavor, (const float*)nullptr, 0, (int64_t)0);
   else
     hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)M), dim3(256), (size_t)D * sizeof(float),
                        as_stream(stream), x, res_pre, h_out, w, res_post, y, D, eps, flavor);
   TNX_CHECK_LAUNCH("rmsnorm");
+  return TNX_OK;
+}
+
+extern "C" int tnx_rmsnorm_splitk(void* stream, const float* ws, int split_k, const uint16_t* res_pre,
+                                  uint16_t* h_out, const uint16_t* w, const uint16_t* res_post,
+                                  uint16_t* y, int64_t M, int64_t D, float eps, int flavor) {
+  TNX_REQUIRE(ws && w && y, "rmsnorm_splitk: null pointer");
+  TNX_REQUIRE(split_k >= 1, "rmsnorm_splitk: split_k must be >= 1");
+  TNX_REQUIRE(M > 0 && D > 0 && D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks,
+              "rmsnorm_splitk: D=%lld must be a multiple of 8 and <= 16384", (long long)D);
+  TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm_splitk: bad flavor %d", flavor);
+  hipLaunchKernelGGL(rmsnorm_vec_kernel, dim3((unsigned)M), dim3(256), 0, as_stream(stream),
+                     (const uint16_t*)nullptr, res_pre, h_out, w, res_post, y, D, eps, flavor, ws, split_k,
+                     (int64_t)(M * D));
+  TNX_CHECK_LAUNCH("rmsnorm_splitk");
   return TNX_OK;
 }
 

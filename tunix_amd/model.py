@@ -279,7 +279,10 @@ class Runner:
       return 1
     return int(max(1, min(8, ktiles, 256 // blocks)))
 
-  def linear(self, f: FusedLinear, x, y, M, epilogue=L.TNX_EPI_STORE, residual=None):
+  def linear(self, f: FusedLinear, x, y, M, epilogue=L.TNX_EPI_STORE, residual=None, defer=False):
+    """Runs one fused linear.  With defer=True a split-k RESIDUAL linear whose output width is
+    the model width skips its finishing pass and returns split_k (> 1): the caller hands the
+    partial planes in self.splitk_ws to `norm_after`; otherwise returns 1 with y complete."""
     if f.has_lora:
       ops.lora_down(x, f.a_t, self.t, M=M)
     split = self._split_k(f, M)
@@ -290,7 +293,21 @@ class Runner:
         lora_seg_toff=f.seg_toff, t=self.t if f.has_lora else None, t_ld=self.t.shape[1],
         lora_b=f.b_t if f.has_lora else None, lora_scale=f.lora_scale, split_k=split,
         ws=self.splitk_ws if split > 1 else None)
-    ops.qlinear(d)
+    deferred = (defer and split > 1 and epilogue == L.TNX_EPI_RESIDUAL and f.N == self.cfg.embed_dim
+                and f.N % 8 == 0)
+    ops.qlinear(d, finish=not deferred)
+    return split if deferred else 1
+
+  def norm_after(self, pending: int, w, M):
+    """self.xn = norm(self.h) -- or, with the partial planes of a deferred linear pending,
+    self.h += bf16(sum of planes) first (the linear's residual epilogue) in the same kernel."""
+    cfg = self.cfg
+    flavor = _NORM[cfg.family]
+    if pending > 1:
+      ops.rmsnorm_splitk(self.splitk_ws, pending, w, self.xn, cfg.norm_eps, flavor, M, cfg.embed_dim,
+                         res_pre=self.h, h_out=self.h)
+    else:
+      ops.rmsnorm(self.h, w, self.xn, cfg.norm_eps, flavor, M=M)
 
   def forward_hidden(self, tokens, positions, col_ptr, kcache, vcache, B=None, T=None):
     """Runs all layers for tokens[b, col .. col+T) of each row; leaves the final-normed hidden
@@ -302,8 +319,10 @@ class Runner:
     flavor = _NORM[cfg.family]
     emb_scale = math.sqrt(cfg.embed_dim) if cfg.family == "gemma3" else 1.0
     ops.embed(m.embed, tokens, col_ptr, B, T, emb_scale, self.h)
+    pending = 1  # split count of a down-projection whose partial planes still await their sum
     for i, ly in enumerate(m.layers):
-      ops.rmsnorm(self.h, ly["attn_norm"], self.xn, cfg.norm_eps, flavor, M=M)
+      self.norm_after(pending, ly["attn_norm"], M)
+      pending = 1
       self.linear(ly["qkv"], self.xn, self.qkv, M)
       rd = L.RopeDesc()
       rd.B, rd.T, rd.S = B, T, self.S
@@ -336,9 +355,11 @@ class Runner:
         self.linear(ly["o"], self.attn, self.tmp, M)
         ops.rmsnorm(self.tmp, ly["post_attn_norm"], self.h, cfg.norm_eps, flavor, M=M,
                     res_post=self.h)
+        ops.rmsnorm(self.h, ly["mlp_norm"], self.xn, cfg.norm_eps, flavor, M=M)
       else:
-        self.linear(ly["o"], self.attn, self.h, M, epilogue=L.TNX_EPI_RESIDUAL, residual=self.h)
-      ops.rmsnorm(self.h, ly["mlp_norm"], self.xn, cfg.norm_eps, flavor, M=M)
+        po = self.linear(ly["o"], self.attn, self.h, M, epilogue=L.TNX_EPI_RESIDUAL, residual=self.h,
+                         defer=True)
+        self.norm_after(po, ly["mlp_norm"], M)
       if cfg.num_experts:
         self._moe(ly["experts"], M)
       elif cfg.family == "gemma3":
@@ -348,8 +369,9 @@ class Runner:
                     res_post=self.h)
       else:
         self.linear(ly["gu"], self.xn, self.act, M, epilogue=L.TNX_EPI_SILU_MUL)
-        self.linear(ly["down"], self.act, self.h, M, epilogue=L.TNX_EPI_RESIDUAL, residual=self.h)
-    ops.rmsnorm(self.h, m.final_norm, self.xn, cfg.norm_eps, flavor, M=M)
+        pending = self.linear(ly["down"], self.act, self.h, M, epilogue=L.TNX_EPI_RESIDUAL,
+                              residual=self.h, defer=True)
+    self.norm_after(pending, m.final_norm, M)
     return self.xn
 
   def _moe(self, ex: ExpertBank, M: int):

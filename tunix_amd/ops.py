@@ -75,9 +75,11 @@ def make_qlinear_desc(*, M, K, N, group, qtype, x, codes, scales, y, epilogue=L.
   return d
 
 
-def qlinear(desc: L.QLinearDesc):
+def qlinear(desc: L.QLinearDesc, finish: bool = True):
+  """finish=False leaves the split-k partial planes in desc.ws for a consumer that sums them
+  itself (rmsnorm_splitk)."""
   L.check(L.lib().tnx_qlinear_lora(_stream(), C.byref(desc)), "tnx_qlinear_lora")
-  if desc.split_k > 1:
+  if desc.split_k > 1 and finish:
     L.check(L.lib().tnx_splitk_finish(_stream(), C.byref(desc)), "tnx_splitk_finish")
 
 
@@ -101,6 +103,14 @@ def rmsnorm(x, w, y, eps, flavor, M=None, res_pre=None, h_out=None, res_post=Non
   D = x.shape[1]
   L.check(L.lib().tnx_rmsnorm(_stream(), _ptr(x), _ptr(res_pre), _ptr(h_out), _ptr(w),
                               _ptr(res_post), _ptr(y), M, D, float(eps), flavor), "tnx_rmsnorm")
+
+
+def rmsnorm_splitk(ws, split_k, w, y, eps, flavor, M, D, res_pre=None, h_out=None, res_post=None):
+  """y = norm(h), h = bf16(bf16(sum_z ws[z]) + res_pre): the finishing pass of a split-k linear
+  (N == D) folded into the residual add + norm that consumes it."""
+  L.check(L.lib().tnx_rmsnorm_splitk(_stream(), _ptr(ws), split_k, _ptr(res_pre), _ptr(h_out), _ptr(w),
+                                     _ptr(res_post), _ptr(y), M, D, float(eps), flavor),
+          "tnx_rmsnorm_splitk")
 
 
 def rope_kvwrite(desc: L.RopeDesc):
