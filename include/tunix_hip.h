@@ -123,11 +123,24 @@ typedef struct tnx_qlinear_desc {
   float* ws;                /* fp32 [split_k, M, N] workspace (need not be initialised);
                                required when split_k > 1; tnx_splitk_finish adds the
                                partial tiles in split order and applies the epilogue        */
+  /* Optional (next_tpart != NULL), *_MUL epilogues with split_k == 1 and M > 64 only: the LoRA
+   * down-projection of the NEXT linear -- the one that consumes y, e.g. down_proj after
+   * gate|up -- fused into this epilogue.  Each 128-row x 128-column work-group tile leaves its
+   * share of y . A_next as one fp32 fragment plane; tnx_lora_reduce adds the planes in a fixed
+   * order and writes t_next = bf16(y . A_next), which tnx_lora_down would have produced.    */
+  const uint16_t* next_a_t; /* bf16 [next_rank, N/2]: A_next transposed                     */
+  int next_rank;            /* multiple of 16, <= 64                                        */
+  float* next_tpart;        /* fp32 [ceil(M/128) * ceil(N/128)][8192]                       */
 } tnx_qlinear_desc;
 
 int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* h_desc);
 /* Epilogue for split_k > 1 (same desc): y = epi(sum_z ws[z]). */
 int tnx_splitk_finish(void* stream, const tnx_qlinear_desc* h_desc);
+
+/* t[M, :R] = bf16(sum over the n_col_blocks fragment planes that tnx_qlinear_lora left in
+ * tpart through next_tpart), planes added in column-block order. */
+int tnx_lora_reduce(void* stream, const float* tpart, int64_t M, int64_t n_col_blocks, int R,
+                    uint16_t* t, int64_t t_ld);
 
 /* t[M, R] = bf16( x[M,K] . A ), a_t = A transposed: bf16 [R, K].  R multiple of 16.
  * The LoRA "down" half of qwix's x @ lora_a @ lora_b (shapes at

@@ -595,3 +595,35 @@ def test_rmsnorm_splitk_equals_finish_then_norm(gpu, family):
   torch.cuda.synchronize()
   assert torch.equal(h1, h2)
   assert torch.equal(y1, y2)
+
+
+@pytest.mark.parametrize("M,F,r", [(128, 1024, 64), (200, 192, 32)])
+def test_mul_epilogue_fuses_next_adapter_projection(gpu, M, F, r):
+  """A gate|up linear with next_tpart: y equals the plain launch bit for bit, and
+  tnx_lora_reduce over the planes equals bf16(y . A_next) (what tnx_lora_down gives)."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  K, g = 512, 64
+  x = rnd((M, K), 90)
+  wg, wu = rnd((K, F), 91, 0.05), rnd((K, F), 92, 0.05)
+  a_next = rnd((F, r), 93, 0.02)
+  c, s = ops.quantize_pack(bf(torch.cat([wg, wu], 1)).to(gpu), g, Q.NF4, True)
+  gx = bf(x).to(gpu)
+  y0 = torch.empty(M, F, dtype=torch.bfloat16, device=gpu)
+  y1 = torch.full((M, F), 3.0, dtype=torch.bfloat16, device=gpu)
+  base = dict(M=M, K=K, N=2 * F, group=g, qtype=Q.NF4, x=gx, codes=c, scales=s, epilogue=L.TNX_EPI_SILU_MUL)
+  ops.qlinear(ops.make_qlinear_desc(y=y0, **base))
+  ncb = math.ceil(2 * F / 128)
+  tpart = torch.full((math.ceil(M / 128) * ncb * 8192,), float("nan"), dtype=torch.float32, device=gpu)
+  a_t = bf(a_next).t().contiguous().to(gpu)
+  ops.qlinear(ops.make_qlinear_desc(y=y1, next_a_t=a_t, next_rank=r, next_tpart=tpart, **base))
+  t = torch.full((M, r + 16), 5.0, dtype=torch.bfloat16, device=gpu)
+  ops.lora_reduce(tpart, M, ncb, r, t)
+  torch.cuda.synchronize()
+  assert torch.equal(y0, y1)
+  want = Q.rb((y1.float().cpu().double() @ a_next.double()).float())
+  assert_bf16_close(t[:, :r], want, what="fused next-adapter projection")
+  assert (t[:, r:] == 5.0).all()
+  t2 = torch.zeros(M, r, dtype=torch.bfloat16, device=gpu)
+  ops.lora_down(y1, a_t, t2)
+  assert (t[:, :r].float() - t2.float()).abs().max().item() <= 2.0 ** -7 * max(1e-3, t2.float().abs().max().item())

@@ -32,6 +32,7 @@ class QLinearDesc(C.Structure):
       ("t_ld", _i64), ("t", _p), ("lora_b", _p), ("lora_scale", _f32),
       ("epilogue", _i32), ("residual", _p), ("y", _p),
       ("split_k", _i32), ("ws", _p),
+      ("next_a_t", _p), ("next_rank", _i32), ("next_tpart", _p),
   ]
 
 
@@ -88,6 +89,7 @@ SIGNATURES = {
     "tnx_qw_dequant": (_i32, [_p, _p, _p, _i64, _i64, _i32, _i32, _i32, _p]),
     "tnx_qlinear_lora": (_i32, [_p, C.POINTER(QLinearDesc)]),
     "tnx_splitk_finish": (_i32, [_p, C.POINTER(QLinearDesc)]),
+    "tnx_lora_reduce": (_i32, [_p, _p, _i64, _i64, _i32, _p, _i64]),
     "tnx_lora_down": (_i32, [_p, _p, _i64, _i64, _p, _i32, _p, _i64]),
     "tnx_embed": (_i32, [_p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _f32, _p]),
     "tnx_rmsnorm": (_i32, [_p, _p, _p, _p, _p, _p, _p, _i64, _i64, _f32, _i32]),

@@ -381,7 +381,69 @@ void qgemm128_kernel(const QLArgs a) {
     tile_lora<MT, NT>(s, m0, ntile0, toff, acc);
   }
   TNX_STAMP(4);
-  store_tile<MT, NT>(a, m0, a.M, ntile0, ntiles, acc, [](int64_t r) { return r; });
+  const bool mul = a.epilogue == TNX_EPI_SILU_MUL || a.epilogue == TNX_EPI_GELU_MUL;
+  if (NT == 2 && mul && a.split_k <= 1) {
+    // act = f(gate) * up goes through LDS (the activation buffer the adapter block is not in):
+    // rows leave the work-group as 128-byte runs instead of 2-byte scatters, and, when asked,
+    // the tile is multiplied with the NEXT linear's adapter A (its LoRA down-projection, whose
+    // K axis is this kernel's output axis), one fp32 fragment plane per work-group.
+    constexpr int ACT_LD = 72;  // 64 act columns + 8 pad (bf16 elements)
+    const uint32_t act_lds = a_rd_nxt - (uint32_t)(lm * A_LD + lq * 8) * 2u;
+    const int64_t ldy = a.N / 2;
+    const int64_t wgcol0 = (int64_t)blockIdx.y * 64;      // first act column of the work-group
+    const bool fuse_next = a.next_tpart != nullptr;
+    u32x4 bn[4][2];
+    if (fuse_next) {
+      const rsrc_t rn = make_rsrc(a.next_a_t, (uint64_t)a.next_rank * ldy * 2);
+#pragma unroll
+      for (int n = 0; n < 4; ++n)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int64_t k = wgcol0 + j * 32 + lq * 8;
+          const bool ok = n * 16 < a.next_rank && k + 8 <= ldy;
+          bn[n][j] = buf_load128(rn, ok ? (uint32_t)(((int64_t)(n * 16 + lm) * ldy + k) * 2) : 0xfffffff0u);
+        }
+    }
+    uint16_t* act_s = reinterpret_cast<uint16_t*>(smem + act_lds);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float g = rbf(acc[mt][0][i]);
+        const float u = rbf(acc[mt][1][i]);
+        const float act = a.epilogue == TNX_EPI_SILU_MUL ? silu_bf16(g) : gelu_tanh_bf16(g);
+        act_s[(mt * 16 + lq * 4 + i) * ACT_LD + wn * 16 + lm] = f2bf(rbf(act) * u);
+      }
+    __syncthreads();
+    uint16_t* y = reinterpret_cast<uint16_t*>(a.y);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int idx = tid + 256 * c, row = idx >> 3, ch = idx & 7;
+      const u32x4 v = lds_ld128(act_lds + (uint32_t)((row * ACT_LD + ch * 8) * 2));
+      if (m0 + row < a.M && wgcol0 + ch * 8 + 8 <= ldy)
+        *reinterpret_cast<u32x4*>(y + (m0 + row) * ldy + wgcol0 + ch * 8) = v;
+    }
+    if (fuse_next) {
+      float* plane = a.next_tpart + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * 8192;
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const int mt = wn * 2 + q;
+        u32x4 af2[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          af2[j] = lds_ld128(act_lds + (uint32_t)(((mt * 16 + lm) * ACT_LD + j * 32 + lq * 8) * 2));
+#pragma unroll
+        for (int n = 0; n < 4; ++n) {
+          f32x4 pacc = f32x4{0.f, 0.f, 0.f, 0.f};
+          pacc = mfma16(af2[0], bn[n][0], pacc);
+          pacc = mfma16(af2[1], bn[n][1], pacc);
+          *reinterpret_cast<f32x4*>(plane + ((mt * 4 + n) * 64 + lane) * 4) = pacc;
+        }
+      }
+    }
+  } else {
+    store_tile<MT, NT>(a, m0, a.M, ntile0, ntiles, acc, [](int64_t r) { return r; });
+  }
   TNX_STAMP(5);
 }
 

@@ -33,6 +33,10 @@ struct QLArgs {
   const int32_t* sorted_route;
   int x_div;
   int64_t codes_stride, scales_stride;  // per-expert strides in elements
+  // fused down-projection of the next linear's adapter (*_MUL epilogue of qgemm128)
+  const uint16_t* next_a_t;
+  int next_rank;
+  float* next_tpart;
 };
 
 __device__ __forceinline__ float silu_bf16(float g) {
@@ -271,6 +275,31 @@ __global__ __launch_bounds__(512) void lora_down_kernel(const uint16_t* x, int64
   }
 }
 
+// t[M, :R] = bf16(sum of fragment planes).  One thread per (row block, row tile, column tile,
+// lane): it owns the four rows 4*(lane/16)+i of column lane%16 of that 16 x 16 tile, exactly
+// as the MFMA that produced the plane laid them out.
+__global__ void lora_reduce_kernel(const float* tpart, int64_t M, int64_t ncb, int R, uint16_t* t,
+                                   int64_t t_ld) {
+  const int ntile = R / 16;
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int lane = (int)(gid & 63);
+  int64_t q = gid >> 6;
+  const int n = (int)(q % ntile);
+  q /= ntile;
+  const int mt = (int)(q & 7);
+  const int64_t mb = q >> 3;
+  if (mb * 128 >= M) return;
+  const float* p = tpart + mb * ncb * 8192 + ((mt * 4 + n) * 64 + lane) * 4;
+  f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+  for (int64_t cb = 0; cb < ncb; ++cb) s += *reinterpret_cast<const f32x4*>(p + cb * 8192);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t row = mb * 128 + mt * 16 + (lane >> 4) * 4 + i;
+    if (row < M) t[row * t_ld + n * 16 + (lane & 15)] = f2bf(s[i]);
+  }
+}
+
 // ---- QW packer ---------------------------------------------------------------------------
 __device__ __forceinline__ int64_t packed_col(int64_t c, int64_t N, int interleave2) {
   if (!interleave2) return c;
@@ -362,6 +391,7 @@ QLArgs to_args(const tnx_qlinear_desc* d) {
   const int ktiles = (int)(d->K / KTILE);
   a.ktiles_per_split = (ktiles + a.split_k - 1) / a.split_k;
   a.offsets = nullptr; a.sorted_route = nullptr; a.x_div = 1; a.codes_stride = 0; a.scales_stride = 0;
+  a.next_a_t = d->next_a_t; a.next_rank = d->next_rank; a.next_tpart = d->next_tpart;
   return a;
 }
 
@@ -395,6 +425,14 @@ int check_desc(const tnx_qlinear_desc* d) {
                   "qlinear: LoRA segment %d misaligned", s);
   }
   if (d->split_k > 1) TNX_REQUIRE(d->ws, "qlinear: split_k > 1 needs a workspace");
+  if (d->next_tpart) {
+    TNX_REQUIRE(d->epilogue == TNX_EPI_SILU_MUL || d->epilogue == TNX_EPI_GELU_MUL,
+                "qlinear: next_tpart needs a *_MUL epilogue");
+    TNX_REQUIRE(d->split_k <= 1 && d->M > 64, "qlinear: next_tpart needs split_k == 1 and M > 64");
+    TNX_REQUIRE(d->next_a_t && d->next_rank > 0 && d->next_rank % 16 == 0 && d->next_rank <= 64,
+                "qlinear: next_rank must be a multiple of 16 and <= 64 (got %d)", d->next_rank);
+    TNX_REQUIRE((d->N / 2) % 8 == 0, "qlinear: next_tpart needs N/2 %% 8 == 0");
+  }
   return TNX_OK;
 }
 
@@ -514,6 +552,18 @@ extern "C" int tnx_splitk_finish(void* stream, const tnx_qlinear_desc* d) {
   hipLaunchKernelGGL(splitk_finish_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0,
                      as_stream(stream), a);
   TNX_CHECK_LAUNCH("splitk_finish");
+  return TNX_OK;
+}
+
+extern "C" int tnx_lora_reduce(void* stream, const float* tpart, int64_t M, int64_t n_col_blocks, int R,
+                               uint16_t* t, int64_t t_ld) {
+  TNX_REQUIRE(tpart && t, "lora_reduce: null pointer");
+  TNX_REQUIRE(M > 0 && n_col_blocks > 0, "lora_reduce: bad shape");
+  TNX_REQUIRE(R > 0 && R % 16 == 0 && R <= 64 && t_ld >= R, "lora_reduce: R=%d must be a multiple of 16, <= 64 and <= t_ld", R);
+  const int64_t threads = cdiv(M, 128) * 8 * (R / 16) * 64;
+  hipLaunchKernelGGL(lora_reduce_kernel, dim3((unsigned)cdiv(threads, 256)), dim3(256), 0, as_stream(stream),
+                     tpart, M, n_col_blocks, R, t, t_ld);
+  TNX_CHECK_LAUNCH("lora_reduce");
   return TNX_OK;
 }
 

@@ -242,6 +242,10 @@ class Runner:
     else:
       self.act = torch.empty(M, F, dtype=bf, device=dev)
     self.split_k_override = {}
+    self.next_tpart = None
+    if 64 < M <= 1024 and not cfg.num_experts and model.layers and "gu" in model.layers[0]:
+      n_planes = math.ceil(M / 128) * math.ceil(model.layers[0]["gu"].N / 128)
+      self.next_tpart = torch.empty(n_planes * 8192, dtype=torch.float32, device=dev)
     need = 1
     for ly in model.layers:
       for key in ("qkv", "o", "gu", "down"):
@@ -279,24 +283,39 @@ class Runner:
       return 1
     return int(max(1, min(8, ktiles, 256 // blocks)))
 
-  def linear(self, f: FusedLinear, x, y, M, epilogue=L.TNX_EPI_STORE, residual=None, defer=False):
+  def linear(self, f: FusedLinear, x, y, M, epilogue=L.TNX_EPI_STORE, residual=None, defer=False,
+             next_f: FusedLinear | None = None, t_ready: bool = False):
     """Runs one fused linear.  With defer=True a split-k RESIDUAL linear whose output width is
     the model width skips its finishing pass and returns split_k (> 1): the caller hands the
     partial planes in self.splitk_ws to `norm_after`; otherwise returns 1 with y complete."""
-    if f.has_lora:
+    if f.has_lora and not t_ready:
       ops.lora_down(x, f.a_t, self.t, M=M)
     split = self._split_k(f, M)
+    # a gate|up linear can leave the down-projection of the next linear's adapter behind
+    # (`fuses_next`): then that linear is called with t_ready=True
+    kw = {}
+    if next_f is not None and self.fuses_next(f, next_f, M, epilogue):
+      kw = dict(next_a_t=next_f.a_t, next_rank=next_f.rp, next_tpart=self.next_tpart)
     d = ops.make_qlinear_desc(
         M=M, K=f.K, N=f.N, group=f.group, qtype=f.qtype, x=x, codes=f.codes, scales=f.scales, y=y,
         epilogue=epilogue, residual=residual, lora_rank=f.rp,
         lora_nseg=(-1 if f.interleave2 else len(f.names)), lora_seg_end=f.seg_end,
         lora_seg_toff=f.seg_toff, t=self.t if f.has_lora else None, t_ld=self.t.shape[1],
         lora_b=f.b_t if f.has_lora else None, lora_scale=f.lora_scale, split_k=split,
-        ws=self.splitk_ws if split > 1 else None)
+        ws=self.splitk_ws if split > 1 else None, **kw)
+    if kw:
+      ops.qlinear(d)
+      ops.lora_reduce(self.next_tpart, M, math.ceil(f.N / 128), next_f.rp, self.t)
+      return 1
     deferred = (defer and split > 1 and epilogue == L.TNX_EPI_RESIDUAL and f.N == self.cfg.embed_dim
                 and f.N % 8 == 0)
     ops.qlinear(d, finish=not deferred)
     return split if deferred else 1
+
+  def fuses_next(self, f: FusedLinear, next_f: FusedLinear, M: int, epilogue: int) -> bool:
+    return (next_f.has_lora and next_f.rp <= 64 and 64 < M <= 1024 and self._split_k(f, M) == 1
+            and epilogue in (L.TNX_EPI_SILU_MUL, L.TNX_EPI_GELU_MUL) and (f.N // 2) % 8 == 0
+            and self.next_tpart is not None)
 
   def norm_after(self, pending: int, w, M):
     """self.xn = norm(self.h) -- or, with the partial planes of a deferred linear pending,
@@ -363,14 +382,16 @@ class Runner:
       if cfg.num_experts:
         self._moe(ly["experts"], M)
       elif cfg.family == "gemma3":
-        self.linear(ly["gu"], self.xn, self.act, M, epilogue=L.TNX_EPI_GELU_MUL)
-        self.linear(ly["down"], self.act, self.tmp, M)
+        fused = self.fuses_next(ly["gu"], ly["down"], M, L.TNX_EPI_GELU_MUL)
+        self.linear(ly["gu"], self.xn, self.act, M, epilogue=L.TNX_EPI_GELU_MUL, next_f=ly["down"])
+        self.linear(ly["down"], self.act, self.tmp, M, t_ready=fused)
         ops.rmsnorm(self.tmp, ly["post_ffw_norm"], self.h, cfg.norm_eps, flavor, M=M,
                     res_post=self.h)
       else:
-        self.linear(ly["gu"], self.xn, self.act, M, epilogue=L.TNX_EPI_SILU_MUL)
+        fused = self.fuses_next(ly["gu"], ly["down"], M, L.TNX_EPI_SILU_MUL)
+        self.linear(ly["gu"], self.xn, self.act, M, epilogue=L.TNX_EPI_SILU_MUL, next_f=ly["down"])
         pending = self.linear(ly["down"], self.act, self.h, M, epilogue=L.TNX_EPI_RESIDUAL,
-                              residual=self.h, defer=True)
+                              residual=self.h, defer=True, t_ready=fused)
     self.norm_after(pending, m.final_norm, M)
     return self.xn
 

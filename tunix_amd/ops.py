@@ -60,7 +60,8 @@ def qw_dequant(codes, scales, K, N, group, qtype, interleave2=False) -> torch.Te
 
 def make_qlinear_desc(*, M, K, N, group, qtype, x, codes, scales, y, epilogue=L.TNX_EPI_STORE,
                       residual=None, lora_rank=0, lora_nseg=1, lora_seg_end=(), lora_seg_toff=(),
-                      t=None, t_ld=0, lora_b=None, lora_scale=0.0, split_k=1, ws=None):
+                      t=None, t_ld=0, lora_b=None, lora_scale=0.0, split_k=1, ws=None,
+                      next_a_t=None, next_rank=0, next_tpart=None):
   d = L.QLinearDesc()
   d.M, d.K, d.N, d.group, d.qtype = M, K, N, group, qtype
   d.x, d.codes, d.scales, d.y = _ptr(x), _ptr(codes), _ptr(scales), _ptr(y)
@@ -72,6 +73,7 @@ def make_qlinear_desc(*, M, K, N, group, qtype, x, codes, scales, y, epilogue=L.
     d.lora_seg_toff[i] = v
   d.t, d.t_ld, d.lora_b, d.lora_scale = _ptr(t), t_ld, _ptr(lora_b), lora_scale
   d.split_k, d.ws = split_k, _ptr(ws)
+  d.next_a_t, d.next_rank, d.next_tpart = _ptr(next_a_t), next_rank, _ptr(next_tpart)
   return d
 
 
@@ -81,6 +83,12 @@ def qlinear(desc: L.QLinearDesc, finish: bool = True):
   L.check(L.lib().tnx_qlinear_lora(_stream(), C.byref(desc)), "tnx_qlinear_lora")
   if desc.split_k > 1 and finish:
     L.check(L.lib().tnx_splitk_finish(_stream(), C.byref(desc)), "tnx_splitk_finish")
+
+
+def lora_reduce(tpart, M, n_col_blocks, R, t):
+  """t[M, :R] = bf16(sum of the fragment planes a *_MUL linear left in tpart)."""
+  L.check(L.lib().tnx_lora_reduce(_stream(), _ptr(tpart), M, n_col_blocks, R, _ptr(t), t.shape[1]),
+          "tnx_lora_reduce")
 
 
 def lora_down(x, a_t, t, M=None):
