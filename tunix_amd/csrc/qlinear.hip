@@ -239,26 +239,42 @@ __global__ void splitk_finish_kernel(const QLArgs a) {
     reinterpret_cast<uint16_t*>(a.y)[idx] = f2bf(v);
 }
 
-// t[M,R] = bf16(x . A): one 16x16 output tile per work-group, K split over 8 waves.
+// t[M,R] = bf16(x . A): one tm x tn output tile (tm, tn <= 16) per work-group, K split over
+// 8 waves.  A compute unit draws only a few tens of GB/s from L2, so the op is bound by the
+// bytes one work-group must read, (tm + tn) rows of K elements: for decode-sized M the host
+// picks tiles smaller than the 16 x 16 MFMA shape (unused rows and columns are zero operands)
+// to spread the reads over every compute unit.
+// The contraction may visit k in any order as long as both operands agree, so each lane takes
+// 16 consecutive elements per 64-wide step (two MFMAs): the four lanes of a row cover one whole
+// 128-byte line.
 __global__ __launch_bounds__(512) void lora_down_kernel(const uint16_t* x, int64_t M, int64_t K,
                                                         const uint16_t* a_t, int R, uint16_t* t,
-                                                        int64_t t_ld) {
+                                                        int64_t t_ld, int tm, int tn) {
   __shared__ float red[8][64][4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int lm = lane & 15, lq = lane >> 4;
-  const int64_t m0 = (int64_t)blockIdx.x * 16;
-  const int n0 = blockIdx.y * 16;
+  const int64_t m0 = (int64_t)blockIdx.x * tm;
+  const int n0 = blockIdx.y * tn;
   const int64_t row = m0 + lm;
-  const uint16_t* xr = x + row * K + lq * 8;
-  const uint16_t* ar = a_t + (int64_t)(n0 + lm) * K + lq * 8;
+  const bool a_on = lm < tm && row < M, b_on = lm < tn && n0 + lm < R;
+  const uint16_t* xr = x + (a_on ? row : 0) * K + lq * 16;
+  const uint16_t* ar = a_t + (int64_t)(b_on ? n0 + lm : 0) * K + lq * 16;
   f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int ksteps = (int)(K / 32);
+  const int ksteps = (int)((K + 63) / 64);
 #pragma unroll 4
   for (int ks = wave; ks < ksteps; ks += 8) {
-    u32x4 af = u32x4{0, 0, 0, 0};
-    if (row < M) af = *reinterpret_cast<const u32x4*>(xr + (int64_t)ks * 32);
-    const u32x4 bf = *reinterpret_cast<const u32x4*>(ar + (int64_t)ks * 32);
-    acc = mfma16(af, bf, acc);
+    u32x4 a0 = u32x4{0, 0, 0, 0}, a1 = a0, b0 = a0, b1 = a0;
+    const bool k_on = (int64_t)ks * 64 + lq * 16 < K;
+    if (a_on && k_on) {
+      a0 = *reinterpret_cast<const u32x4*>(xr + (int64_t)ks * 64);
+      a1 = *reinterpret_cast<const u32x4*>(xr + (int64_t)ks * 64 + 8);
+    }
+    if (b_on && k_on) {
+      b0 = *reinterpret_cast<const u32x4*>(ar + (int64_t)ks * 64);
+      b1 = *reinterpret_cast<const u32x4*>(ar + (int64_t)ks * 64 + 8);
+    }
+    acc = mfma16(a0, b0, acc);
+    acc = mfma16(a1, b1, acc);
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) red[wave][lane][i] = acc[i];
@@ -269,8 +285,8 @@ __global__ __launch_bounds__(512) void lora_down_kernel(const uint16_t* x, int64
       float s = 0.f;
 #pragma unroll
       for (int w = 0; w < 8; ++w) s += red[w][lane][i];
-      const int64_t r = m0 + lq * 4 + i;
-      if (r < M) t[r * t_ld + n0 + lm] = f2bf(s);
+      const int mi = lq * 4 + i;
+      if (mi < tm && m0 + mi < M && b_on) t[(m0 + mi) * t_ld + n0 + lm] = f2bf(s);
     }
   }
 }
@@ -572,8 +588,21 @@ extern "C" int tnx_lora_down(void* stream, const uint16_t* x, int64_t M, int64_t
   TNX_REQUIRE(x && a_t && t, "lora_down: null pointer");
   TNX_REQUIRE(M > 0 && K > 0 && K % 32 == 0, "lora_down: K=%lld must be a multiple of 32", (long long)K);
   TNX_REQUIRE(R > 0 && R % 16 == 0 && t_ld >= R, "lora_down: R=%d must be a multiple of 16 and <= t_ld", R);
-  dim3 grid((unsigned)cdiv(M, 16), (unsigned)(R / 16));
-  hipLaunchKernelGGL(lora_down_kernel, grid, dim3(512), 0, as_stream(stream), x, M, K, a_t, R, t, t_ld);
+  // smallest tm + tn whose grid still fits the device once; 16 x 16 when nothing does
+  int tm = 16, tn = 16;
+  {
+    static const int kTm[] = {4, 8, 16}, kTn[] = {4, 8, 12, 16};
+    int best = 33;
+    for (int a : kTm)
+      for (int b : kTn)
+        if (cdiv(M, a) * cdiv(R, b) <= 256 && a + b < best) {
+          best = a + b;
+          tm = a;
+          tn = b;
+        }
+  }
+  dim3 grid((unsigned)cdiv(M, tm), (unsigned)cdiv(R, tn));
+  hipLaunchKernelGGL(lora_down_kernel, grid, dim3(512), 0, as_stream(stream), x, M, K, a_t, R, t, t_ld, tm, tn);
   TNX_CHECK_LAUNCH("lora_down");
   return TNX_OK;
 }
