@@ -201,6 +201,11 @@ typedef struct tnx_rope_desc {
   uint16_t* q_out;
   uint16_t* kcache;
   uint16_t* vcache;
+  const float* qkv_ws;       /* optional: split_k fp32 partial planes [split_k][B*T][(Hq+2Hkv)*dh]
+                                of the qkv linear (tnx_qlinear_lora with finish skipped); the
+                                input is then bf16(sum of the planes, in split order) and qkv
+                                may be NULL                                                   */
+  int split_k;
 } tnx_rope_desc;
 int tnx_qknorm_rope_kvwrite(void* stream, const tnx_rope_desc* h_desc);
 

@@ -597,6 +597,54 @@ def test_rmsnorm_splitk_equals_finish_then_norm(gpu, family):
   assert torch.equal(y1, y2)
 
 
+@pytest.mark.parametrize("family", ["llama3", "qwen3"])
+def test_rope_from_splitk_planes_equals_finish_then_rope(gpu, family):
+  """The rope / cache-write kernel fed with the partial planes of a split-k qkv linear against
+  the finishing pass followed by the same kernel on its output: bit for bit."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  from tunix_amd.model import _NORM, _ROPE, rope_timescale
+  B, T, S, Hq, Hkv, dh, K, g, split, col = 128, 1, 16, 4, 2, 64, 1024, 64, 4, 7
+  N = (Hq + 2 * Hkv) * dh
+  x, w = rnd((B, K), 84), rnd((K, N), 85, 0.02)
+  c, s = ops.quantize_pack(bf(w).to(gpu), g, Q.NF4)
+  gx = bf(x).to(gpu)
+  ws = torch.empty(split * B * N, dtype=torch.float32, device=gpu)
+  qkv = torch.empty(B, N, dtype=torch.bfloat16, device=gpu)
+  ld = ops.make_qlinear_desc(M=B, K=K, N=N, group=g, qtype=Q.NF4, x=gx, codes=c, scales=s, y=qkv,
+                             split_k=split, ws=ws)
+  ops.qlinear(ld)                                  # planes + finishing pass -> qkv
+  pos = torch.randint(0, 900, (B, S), generator=torch.Generator().manual_seed(86), dtype=torch.int32).to(gpu)
+  ts = torch.from_numpy(rope_timescale(dh, 1e6)).to(gpu)
+  qn, kn = bf(rnd((dh,), 87, 0.3) + 1).to(gpu), bf(rnd((dh,), 88, 0.3) + 1).to(gpu)
+  colp = torch.tensor([col], dtype=torch.int32, device=gpu)
+  outs = []
+  for planes in (False, True):
+    d = L.RopeDesc()
+    d.B, d.T, d.S, d.Hq, d.Hkv, d.dh = B, T, S, Hq, Hkv, dh
+    d.rope_flavor, d.rope_scale, d.timescale = _ROPE[family], 1.0, ts.data_ptr()
+    if family != "llama3":
+      d.qk_norm, d.norm_eps, d.q_norm_w, d.k_norm_w = _NORM[family], 1e-6, qn.data_ptr(), kn.data_ptr()
+    else:
+      d.qk_norm = -1
+    qo = torch.zeros(B * T, Hq * dh, dtype=torch.bfloat16, device=gpu)
+    kc = torch.zeros(B, Hkv, S, dh, dtype=torch.bfloat16, device=gpu)
+    vc = torch.zeros_like(kc)
+    d.positions, d.pos_ld, d.col_ptr = pos.data_ptr(), S, colp.data_ptr()
+    d.q_out, d.kcache, d.vcache = qo.data_ptr(), kc.data_ptr(), vc.data_ptr()
+    if planes:
+      ops.qlinear(ld, finish=False)
+      d.qkv_ws, d.split_k = ws.data_ptr(), split
+    else:
+      d.qkv = qkv.data_ptr()
+    ops.rope_kvwrite(d)
+    torch.cuda.synchronize()
+    outs.append((qo, kc, vc))
+  assert outs[0][0].float().abs().max() > 0
+  for a, b in zip(*outs):
+    assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("M,F,r", [(128, 1024, 64), (200, 192, 32)])
 def test_mul_epilogue_fuses_next_adapter_projection(gpu, M, F, r):
   """A gate|up linear with next_tpart: y equals the plain launch bit for bit, and

@@ -45,6 +45,7 @@ class RopeDesc(C.Structure):
       ("q_norm_w", _p), ("k_norm_w", _p), ("q_prescale", _f32),
       ("qkv", _p), ("positions", _p), ("pos_ld", _i64), ("col_ptr", _p),
       ("q_out", _p), ("kcache", _p), ("vcache", _p),
+      ("qkv_ws", _p), ("split_k", _i32),
   ]
 
 

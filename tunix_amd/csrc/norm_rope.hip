@@ -189,6 +189,8 @@ struct RopeArgs {
   uint16_t* q_out;
   uint16_t* kcache;
   uint16_t* vcache;
+  const float* ws;   // split-k partial planes of the qkv linear instead of qkv, or null
+  int split_k;
 };
 
 // grid (B*T, Hq + 2*Hkv); max(64, dh/2) threads: thread i < dh/2 owns elements i and i + dh/2
@@ -202,19 +204,28 @@ __global__ void rope_kernel(const RopeArgs a) {
   const bool live = i < half;
   const int col = *a.col_ptr;
   const int ld = (a.Hq + 2 * a.Hkv) * a.dh;
-  const uint16_t* src = a.qkv + row * ld + (int64_t)head * a.dh;
+  const int64_t src_off = row * ld + (int64_t)head * a.dh;
+  // element e of this head: from the finished linear output, or as the linear's own finishing
+  // pass would produce it, bf16(sum of the split-k planes in split order)
+  auto src_at = [&](int e) -> float {
+    if (a.ws == nullptr) return bf2f(a.qkv[src_off + e]);
+    const int64_t plane = a.B * a.T * (int64_t)ld;
+    float v = 0.f;
+    for (int z = 0; z < a.split_k; ++z) v += a.ws[z * plane + src_off + e];
+    return rbf(v);
+  };
   const int slot = (int)((col + t) % a.S);
   if (head >= a.Hq + a.Hkv) {  // V: plain copy into the cache slot
     const int hk = head - a.Hq - a.Hkv;
     uint16_t* dst = a.vcache + (((b * a.Hkv + hk) * a.S) + slot) * a.dh;
     if (live) {
-      dst[i] = src[i];
-      dst[i + half] = src[i + half];
+      dst[i] = f2bf(src_at(i));
+      dst[i + half] = f2bf(src_at(i + half));
     }
     return;
   }
   const bool is_q = head < a.Hq;
-  float x1 = live ? bf2f(src[i]) : 0.f, x2 = live ? bf2f(src[i + half]) : 0.f;
+  float x1 = live ? src_at(i) : 0.f, x2 = live ? src_at(i + half) : 0.f;
   if (a.qk_norm >= 0) {
     const float ss = block_sum(sq_term(x1, a.qk_norm) + sq_term(x2, a.qk_norm), red);
     const float ms = finish_ms(ss, (float)a.dh, a.qk_norm);
@@ -312,9 +323,10 @@ extern "C" int tnx_qknorm_rope_kvwrite(void* stream, const tnx_rope_desc* d) {
   TNX_REQUIRE(d, "rope: null descriptor");
   TNX_REQUIRE(d->B > 0 && d->T > 0 && d->S > 0, "rope: bad shape");
   TNX_REQUIRE(d->dh % 2 == 0 && d->dh >= 2 && d->dh <= 512, "rope: bad head_dim %d", d->dh);
-  TNX_REQUIRE(d->qkv && d->positions && d->col_ptr && d->timescale && d->q_out && d->kcache &&
-                  d->vcache,
+  TNX_REQUIRE((d->qkv || d->qkv_ws) && d->positions && d->col_ptr && d->timescale && d->q_out &&
+                  d->kcache && d->vcache,
               "rope: null pointer");
+  if (d->qkv_ws) TNX_REQUIRE(d->split_k >= 1 && d->split_k <= 64, "rope: split_k=%d out of range", d->split_k);
   TNX_REQUIRE(d->rope_flavor >= TNX_ROPE_LLAMA && d->rope_flavor <= TNX_ROPE_GEMMA3, "rope: bad flavor");
   TNX_REQUIRE(d->qk_norm >= -1 && d->qk_norm <= TNX_NORM_GEMMA3, "rope: bad qk_norm");
   if (d->qk_norm >= 0) TNX_REQUIRE(d->q_norm_w && d->k_norm_w, "rope: qk_norm weights are null");
@@ -327,6 +339,7 @@ extern "C" int tnx_qknorm_rope_kvwrite(void* stream, const tnx_rope_desc* d) {
   a.q_prescale_bf = d->q_prescale != 0.f ? host_round_bf16(d->q_prescale) : 0.f;
   a.qkv = d->qkv; a.positions = d->positions; a.pos_ld = d->pos_ld; a.col_ptr = d->col_ptr;
   a.timescale = d->timescale; a.q_out = d->q_out; a.kcache = d->kcache; a.vcache = d->vcache;
+  a.ws = d->qkv_ws; a.split_k = d->split_k;
   dim3 grid((unsigned)(d->B * d->T), (unsigned)(d->Hq + 2 * d->Hkv));
   hipLaunchKernelGGL(rope_kernel, grid, dim3(d->dh / 2 < 64 ? 64 : d->dh / 2), 0, as_stream(stream), a);
   TNX_CHECK_LAUNCH("qknorm_rope_kvwrite");

@@ -1,6 +1,6 @@
 // The quantised GEMM for 65+ activation rows (rollout batch, prefill, per-token logps): one
-// work-group = 4 waves = one wave per SIMD, output tile 128 rows x (64 * NT) columns, wave tile
-// 128 x (16 * NT).  At 128 rows the op sits past the MFMA/HBM ridge of the machine (2 * 128 flop
+// work-group = 8 waves = two per SIMD, output tile 128 rows x (64 * NT) columns; a wave covers
+// 128 rows x (16 * NT) columns over one half of every k-tile.  At 128 rows the op sits past the MFMA/HBM ridge of the machine (2 * 128 flop
 // per 0.53 B of weights), so the loop is built around keeping the matrix pipe fed:
 //
 //   * a k-tile (128 k) is four k-steps of 8 * NT MFMAs (16x16x32 bf16).  While the MFMAs of step
@@ -56,16 +56,15 @@ __device__ unsigned long long tnx_stamps[8];
 #define TNX_STAMP(i) do {} while (0)
 #endif
 
-// The launch bound is a register-budget choice, not the work-group size (always 256): with
-// NT = 2 everything fits the 256 architectural VGPRs, and keeping the accumulators there
-// avoids the accumulator-register copies the compiler emits around loops whose MFMA results
-// live in AGPRs; NT = 4 needs both halves of the 512-entry file.
+// 512 threads: waves 0-3 and 4-7 share the four column groups and split every k-tile between
+// them (k-steps 0,1 | 2,3), which puts two waves on each SIMD at 256 registers each.
 template <int NT, int SPT>
-__global__ __launch_bounds__(NT == 2 ? 512 : 256)
+__global__ __launch_bounds__(512)
 void qgemm128_kernel(const QLArgs a) {
-  constexpr int MT = 8, PF = 3;
+  constexpr int MT = 8, HM = 4, PF = 3;
+  constexpr int SW = SPT / 2;  // scales of one wave's two k-steps
   extern __shared__ __align__(16) unsigned char smem[];
-  const int tid = threadIdx.x, lane = tid & 63, wn = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, wn = wv & 3, kh = wv >> 2;
   const int lm = lane & 15, lq = lane >> 4;
   TNX_STAMP(0);
   // LDS is addressed absolutely below (table at 0): bail out if the dynamic block does not
@@ -73,7 +72,7 @@ void qgemm128_kernel(const QLArgs a) {
   if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem != 0u) return;
   // the two code-book levels of this thread's table entry, fetched before anything else so
   // that their (constant-memory) loads are the oldest ones in flight
-  const float lvl0 = rbf(code_level(a.qtype, tid & 15)), lvl1 = rbf(code_level(a.qtype, tid >> 4));
+  const float lvl0 = rbf(code_level(a.qtype, tid & 15)), lvl1 = rbf(code_level(a.qtype, (tid >> 4) & 15));
   const uint32_t lane_off = (uint32_t)lane * 4u;
   const int64_t m0 = (int64_t)blockIdx.x * 128;
   const int64_t ntile0 = ((int64_t)blockIdx.y * 4 + wn) * NT;
@@ -88,15 +87,15 @@ void qgemm128_kernel(const QLArgs a) {
   const rsrc_t rs = make_rsrc(a.scales, ntk * 16 * SPT * 2 + 16);
   // Per-thread offsets (32 bit: the host checks the 4 GiB limits); the k-tile enters as the
   // scalar offset of the load.  Rows past M and column tiles past N start beyond the buffer
-  // and read zeros.
+  // and read zeros.  A lane's 16 bytes of codes are four k-steps: this wave takes its half.
   uint32_t coff[NT], soff[NT];
   const uint32_t xbase = ((uint32_t)(m0 + (tid >> 4)) * (uint32_t)a.K + (uint32_t)(tid & 15) * 8u) * 2u;
-  const uint32_t xstride = 16u * (uint32_t)a.K * 2u;  // 16 rows further per chunk
+  const uint32_t xstride = 32u * (uint32_t)a.K * 2u;  // 32 rows further per chunk
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     const uint32_t tile0 = (uint32_t)(ntile0 + nt) * (uint32_t)ktiles;
-    coff[nt] = tile0 * 1024u + (uint32_t)lane * 16u;
-    soff[nt] = (tile0 * 16u + (uint32_t)lm) * (uint32_t)(SPT * 2);
+    coff[nt] = tile0 * 1024u + (uint32_t)lane * 16u + (uint32_t)kh * 8u;
+    soff[nt] = (tile0 * 16u + (uint32_t)lm) * (uint32_t)(SPT * 2) + (SPT == 4 ? (uint32_t)kh * 4u : 0u);
   }
 
   f32x4 acc[MT][NT];
@@ -105,12 +104,12 @@ void qgemm128_kernel(const QLArgs a) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) zero_acc(acc[mt][nt]);
 
-  u32x4 a_next[MT];
-  u32x4 ring_c[PF][NT];
-  uint32_t ring_s[PF][NT][SPT / 2];
-  float sc[PF][NT][SPT];  // the scales of a ring stage as fp32
-  u32x4 af[2][MT / 2];    // activation fragments of one row half (4 of the 8 row tiles)
-  u32x4 bfr[2][NT];       // weight fragments of this and the next k-step
+  u32x4 a_next[HM];
+  u32x2 ring_c[PF][NT];
+  uint32_t ring_s[PF][NT];
+  float sc[PF][NT][SW];   // the scales of a ring stage as fp32
+  u32x4 af[2][2][HM];     // activation fragments of this wave's two k-steps, both row halves
+  u32x4 bfr[2][NT];       // weight fragments of the two k-steps
   uint32_t lp[NT][4];     // table entries (f16 level pairs) of the k-step after the next
 
   // LoRA delta through the activation pipeline: the "k-tile" after the last real one is the
@@ -134,7 +133,7 @@ void qgemm128_kernel(const QLArgs a) {
     toff_b = seg_toff(min(wg_nt0 + 4 * NT - 1, ntiles - 1));
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) toff[nt] = seg_toff(min(ntile0 + nt, ntiles - 1));
-    // the tile is shared by the four waves, so the decision is taken over all column tiles of
+    // the tile is shared by all waves, so the decision is taken over all column tiles of
     // the work-group (identically in every thread; no LDS or barrier involved: this kernel
     // addresses LDS absolutely and must not acquire a static allocation): a work-group
     // spanning three segments falls back to fragments from global memory
@@ -143,8 +142,9 @@ void qgemm128_kernel(const QLArgs a) {
       lora_fast = lora_fast && (o == toff_a || o == toff_b);
     }
   }
-  // B^T fragments of the adapter for this wave's columns: fetched now, parked in this wave's
-  // private 4 KiB of LDS behind the activation buffers (no barrier needed) until the epilogue
+  // B^T fragments of the adapter for this column group: fetched now, parked in the group's
+  // 4 KiB of LDS behind the activation buffers until the epilogue (both waves of the group
+  // write the same values; the barriers of the main loop order them before the reads)
   const uint32_t lb_lds = kBigLutBytes + 2 * kBigABytes + (uint32_t)wn * 4096u + (uint32_t)lane * 16u;
   uint32_t tbase = 0;
   u32x4 lbv[NT][2];  // live only until the main loop starts
@@ -167,7 +167,7 @@ void qgemm128_kernel(const QLArgs a) {
   }
   const rsrc_t rt = make_rsrc(lora_fast ? (const void*)a.t : (const void*)a.x,
                               lora_fast ? (uint64_t)a.M * a.t_ld * 2 : (uint64_t)a.M * a.K * 2);
-  const uint32_t tstride = (uint32_t)(16 * a.t_ld * 2);
+  const uint32_t tstride = (uint32_t)(32 * a.t_ld * 2);
 
   // k-tiles past the last one are clamped: their data is fetched but never multiplied
   auto load_a = [&](int kt) {
@@ -178,7 +178,7 @@ void qgemm128_kernel(const QLArgs a) {
     const uint32_t m = 0u - (uint32_t)ut;
     const uint32_t base = xbase ^ ((xbase ^ tbase) & m), stride = xstride ^ ((xstride ^ tstride) & m);
 #pragma unroll
-    for (int c = 0; c < MT; ++c)
+    for (int c = 0; c < HM; ++c)
       a_next[c] = __builtin_amdgcn_raw_buffer_load_b128(r, base + (uint32_t)c * stride, s, 0);
   };
   auto load_w = [&](auto Dc, int kt) {
@@ -186,29 +186,27 @@ void qgemm128_kernel(const QLArgs a) {
     const int ktc = min(kt, ktiles - 1);
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      ring_c[D][nt] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff[nt], ktc * 1024, 0);
-      if constexpr (SPT == 2) {
-        ring_s[D][nt][0] = __builtin_amdgcn_raw_buffer_load_b32(rs, soff[nt], ktc * (16 * SPT * 2), 0);
+      ring_c[D][nt] = __builtin_amdgcn_raw_buffer_load_b64(rc, coff[nt], ktc * 1024, 0);
+      ring_s[D][nt] = __builtin_amdgcn_raw_buffer_load_b32(rs, soff[nt], ktc * (16 * SPT * 2), 0);
+    }
+  };
+  // scales of ring stage D -> fp32; a k-tile past the end gets zero scales, which turns its
+  // weights into zeros
+  auto expand_scales = [&](auto Dc, bool active) {
+    constexpr int D = decltype(Dc)::value;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const uint32_t w = ring_s[D][nt];
+      if constexpr (SPT == 2) {  // one group per two k-steps: this wave's half of the pair
+        const uint32_t bits = kh ? (w & 0xffff0000u) : (w << 16);
+        sc[D][nt][0] = active ? __builtin_bit_cast(float, bits) : 0.f;
       } else {
-        const u32x2 p = __builtin_amdgcn_raw_buffer_load_b64(rs, soff[nt], ktc * (16 * SPT * 2), 0);
-        ring_s[D][nt][0] = p[0];
-        ring_s[D][nt][1] = p[1];
+        sc[D][nt][0] = active ? bflo(w) : 0.f;
+        sc[D][nt][1] = active ? bfhi(w) : 0.f;
       }
     }
   };
-  // scales of ring stage D -> fp32 in sc[P]; a k-tile past the end gets zero scales, which
-  // turns its weights into zeros
-  auto expand_scales = [&](auto Dc, auto Pc, bool active) {
-    constexpr int D = decltype(Dc)::value, P = decltype(Pc)::value;
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-      for (int i = 0; i < SPT; ++i) {
-        const float v = (i & 1) ? bfhi(ring_s[D][nt][i >> 1]) : bflo(ring_s[D][nt][i >> 1]);
-        sc[P][nt][i] = active ? v : 0.f;
-      }
-  };
-  // table look-ups of k-step J of ring stage D; the raw f16 pairs land in dst
+  // table look-ups of this wave's k-step J (0 | 1) of ring stage D; the raw f16 pairs land in dst
   auto lut_issue = [&](auto Dc, auto Jc, uint32_t (&dst)[NT][4]) {
     constexpr int D = decltype(Dc)::value, J = decltype(Jc)::value;
 #pragma unroll
@@ -222,11 +220,11 @@ void qgemm128_kernel(const QLArgs a) {
     }
   };
   // f16 level pair x fp32 scale -> bf16 pair
-  auto convert = [&](auto Pc, auto Jc, u32x4 (&dst)[NT], const uint32_t (&src)[NT][4]) {
-    constexpr int P = decltype(Pc)::value, J = decltype(Jc)::value;
+  auto convert = [&](auto Dc, auto Jc, u32x4 (&dst)[NT], const uint32_t (&src)[NT][4]) {
+    constexpr int D = decltype(Dc)::value, J = decltype(Jc)::value;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const float s = sc[P][nt][SPT == 2 ? (J >> 1) : J];
+      const float s = sc[D][nt][SPT == 2 ? 0 : J];
       u32x4 r;
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
@@ -236,78 +234,81 @@ void qgemm128_kernel(const QLArgs a) {
       dst[nt] = r;
     }
   };
-  // LDS byte addresses of the two activation buffers as this lane reads / writes them
-  uint32_t a_rd = kBigLutBytes + (uint32_t)(lm * A_LD + lq * 8) * 2u;
+  // LDS byte addresses of the two activation buffers as this lane reads (its k half) / writes them
+  uint32_t a_rd = kBigLutBytes + (uint32_t)(lm * A_LD + lq * 8 + kh * 64) * 2u;
   uint32_t a_rd_nxt = a_rd + kBigABytes;
   uint32_t a_wr = kBigLutBytes + (uint32_t)((tid >> 4) * A_LD + (tid & 15) * 8) * 2u;
   uint32_t a_wr_nxt = a_wr + kBigABytes;
-  auto read_a = [&](u32x4 (&dst)[MT / 2], uint32_t base, auto Jc, auto Hc) {
-    constexpr int J = decltype(Jc)::value, H = decltype(Hc)::value;
+  auto read_a = [&](u32x4 (&dst)[2][HM], uint32_t base, auto Jc) {
+    constexpr int J = decltype(Jc)::value;
 #pragma unroll
-    for (int m = 0; m < MT / 2; ++m)
-      dst[m] = lds_ld128(base + (uint32_t)(((H * 4 + m) * 16 * A_LD + J * 32) * 2));
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int m = 0; m < HM; ++m)
+        dst[h][m] = lds_ld128(base + (uint32_t)(((h * 4 + m) * 16 * A_LD + J * 32) * 2));
   };
   auto store_a = [&](uint32_t base) {
 #pragma unroll
-    for (int c = 0; c < MT; ++c) lds_st128(base + (uint32_t)(c * 16 * A_LD * 2), a_next[c]);
+    for (int c = 0; c < HM; ++c) lds_st128(base + (uint32_t)(c * 32 * A_LD * 2), a_next[c]);
   };
-  auto mfmas = [&](auto Jc, auto Hc) {
-    constexpr int J = decltype(Jc)::value, H = decltype(Hc)::value;
+  auto mfmas = [&](auto Jc) {
+    constexpr int J = decltype(Jc)::value;
 #pragma unroll
-    for (int m = 0; m < MT / 2; ++m)
+    for (int h = 0; h < 2; ++h)
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-        acc[H * 4 + m][nt] = mfma16(af[H][m], bfr[J & 1][nt], acc[H * 4 + m][nt]);
+      for (int m = 0; m < HM; ++m)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          acc[h * 4 + m][nt] = mfma16(af[J][h][m], bfr[J][nt], acc[h * 4 + m][nt]);
   };
 
-  // One k-step of ring stage D (k-tile kt).  On entry af[0] holds row half 0 of this step,
-  // bfr[J & 1] its weights and lp the table entries of the next step.  While the MFMAs of row
-  // half 0 issue, the next step's weights are converted; during row half 1 the table look-ups
-  // of the step after that and the next activation fragments are issued.  The
-  // sched_group_barrier sequences spell the interleave out: one wave per SIMD issues in
-  // order, so whatever should overlap the matrix pipe has to sit between the MFMAs.
-  auto block = [&](auto Dc, auto Jc, int kt, bool next_active) {
-    constexpr int d = decltype(Dc)::value, j = decltype(Jc)::value;
-    constexpr int dn = (d + 1) % PF;
-    constexpr int d1 = j < 3 ? d : dn, j1 = (j + 1) & 3;   // the next k-step
-    constexpr int d2 = j < 2 ? d : dn, j2 = (j + 2) & 3;   // and the one after
-    if constexpr (j == 3) __syncthreads();  // next activation tile is in LDS; this one is read out
-    __builtin_amdgcn_sched_barrier(0);
-    read_a(af[1], a_rd, Jc, ic<1>{});
-    if constexpr (j == 0) store_a(a_wr_nxt);
-    if constexpr (j == 2) expand_scales(ic<dn>{}, ic<dn>{}, next_active);
-    convert(ic<d1>{}, ic<j1>{}, bfr[j1 & 1], lp);
-    mfmas(Jc, ic<0>{});
-    lut_issue(ic<d2>{}, ic<j2>{}, lp);
-    read_a(af[0], j < 3 ? a_rd : a_rd_nxt, ic<j1>{}, ic<0>{});
-    if constexpr (j == 1) load_a(kt + 2);
-    if constexpr (j == 3) load_w(Dc, kt + PF);
-    mfmas(Jc, ic<1>{});
-    // row half 0: 4 fragment reads up front, then 3 conversion ops behind every MFMA
-    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-    for (int i = 0; i < 4 * NT; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
-      if (j == 0 && i < 8) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-    }
-    // row half 1: one address + one look-up behind every MFMA, fragment reads behind the first 4
-#pragma unroll
-    for (int i = 0; i < 4 * NT; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      if (i < 4) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      if ((j == 1 || j == 3) && i >= 4 && i < 12) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  };
+  // One k-tile of ring stage D = this wave's two k-steps.  On entry af[0] holds the activation
+  // fragments of the first step, bfr[0] its weights and lp the table entries of the second.
+  // Step 0 converts the weights of step 1, issues the look-ups of the next k-tile's first step,
+  // reads the fragments of step 1 and stores the next activation tile; step 1, behind the one
+  // barrier of the k-tile (every wave has finished reading this tile and stored the next),
+  // does the same one step further and issues the global loads.  Two waves share a SIMD, so
+  // one's conversions overlap the other's MFMAs; the group barriers only keep the memory
+  // operations spread between the MFMAs.
   auto tile = [&](auto Dc, int kt) {
+    constexpr int d = decltype(Dc)::value, dn = (d + 1) % PF;
     const bool next_active = kt + 1 < kt_end;
-    block(Dc, ic<0>{}, kt, next_active);
-    block(Dc, ic<1>{}, kt, next_active);
-    block(Dc, ic<2>{}, kt, next_active);
-    block(Dc, ic<3>{}, kt, next_active);
+    __builtin_amdgcn_sched_barrier(0);
+    expand_scales(ic<dn>{}, next_active);
+    convert(Dc, ic<1>{}, bfr[1], lp);
+    mfmas(ic<0>{});
+    lut_issue(ic<dn>{}, ic<0>{}, lp);
+    read_a(af[1], a_rd, ic<1>{});
+    store_a(a_wr_nxt);
+#ifndef TNX_NO_SGB
+#pragma unroll
+    for (int i = 0; i < 8 * NT; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+      if (i < 4) __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if (i >= 8 && i < 8 + HM) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+    }
+#endif
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    convert(ic<dn>{}, ic<0>{}, bfr[0], lp);
+    mfmas(ic<1>{});
+    lut_issue(ic<dn>{}, ic<1>{}, lp);
+    read_a(af[0], a_rd_nxt, ic<0>{});
+    load_a(kt + 2);
+    load_w(Dc, kt + PF);
+#ifndef TNX_NO_SGB
+#pragma unroll
+    for (int i = 0; i < 8 * NT; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if (i >= 4 && i < 4 + HM + 2 * NT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+#endif
+    __builtin_amdgcn_sched_barrier(0);
     const uint32_t r = a_rd; a_rd = a_rd_nxt; a_rd_nxt = r;
     const uint32_t w = a_wr; a_wr = a_wr_nxt; a_wr_nxt = w;
   };
@@ -317,21 +318,22 @@ void qgemm128_kernel(const QLArgs a) {
     load_w(ic<0>{}, kt_begin);
     load_w(ic<1>{}, kt_begin + 1);
     load_w(ic<2>{}, kt_begin + 2);
-    {  // table entry `tid` = f16 pair (level[tid & 15], level[tid >> 4]); copies rotated over
-       // banks; built while the first loads are in flight
+    {  // table entry e = f16 pair (level[e & 15], level[e >> 4]); copies rotated over banks,
+       // half of them per thread; built while the first loads are in flight
       uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
       const h16x2 h = {(_Float16)lvl0, (_Float16)lvl1};
       const uint32_t v = __builtin_bit_cast(uint32_t, h);
+      const int e = tid & 255, c0 = (tid >> 8) * 32;
 #pragma unroll
-      for (int c = 0; c < 64; ++c) lut[tid * 64 + ((c + lane) & 63)] = v;
+      for (int c = 0; c < 32; ++c) lut[e * 64 + ((c0 + c + lane) & 63)] = v;
     }
     TNX_STAMP(1);
     store_a(a_wr);
     load_a(kt_begin + 1);
-    expand_scales(ic<0>{}, ic<0>{}, true);
+    expand_scales(ic<0>{}, true);
     __syncthreads();  // table and first activation tile
     lut_issue(ic<0>{}, ic<0>{}, lp);
-    read_a(af[0], a_rd, ic<0>{}, ic<0>{});
+    read_a(af[0], a_rd, ic<0>{});
     convert(ic<0>{}, ic<0>{}, bfr[0], lp);
     lut_issue(ic<0>{}, ic<1>{}, lp);
     if (lora_fast) {
@@ -350,27 +352,55 @@ void qgemm128_kernel(const QLArgs a) {
   }
   TNX_STAMP(3);
 
+  // The two k halves meet: each wave keeps the row half kh of its column group, hands the other
+  // half to its partner through the (now idle) table area and adds what the partner hands over.
+  f32x4 out[HM][NT];
+  {
+    __syncthreads();  // every wave is done with the table
+    const uint32_t xw = (uint32_t)wv * 8192u + (uint32_t)lane * 16u;
+    const uint32_t xr = (uint32_t)(wv ^ 4) * 8192u + (uint32_t)lane * 16u;
+#pragma unroll
+    for (int m = 0; m < HM; ++m)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const f32x4 v = kh ? acc[m][nt] : acc[HM + m][nt];
+        lds_st128(xw + (uint32_t)((m * NT + nt) * 1024), __builtin_bit_cast(u32x4, v));
+      }
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < HM; ++m)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const f32x4 own = kh ? acc[HM + m][nt] : acc[m][nt];
+        const f32x4 got = __builtin_bit_cast(f32x4, lds_ld128(xr + (uint32_t)((m * NT + nt) * 1024)));
+        out[m][nt] = own + got;
+      }
+  }
+  const int64_t m0w = m0 + kh * 64;   // first row of this wave's tile
+  const uint32_t row_lds = (uint32_t)(kh * 64 * A_LD * 2);
+
   if (lora_fast) {
     // the t block sits in the activation buffer the last k-tile left as "next"
+    const uint32_t tb = a_rd - (uint32_t)(kh * 64 * 2) + row_lds;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const uint32_t base = a_rd + (uint32_t)((toff[nt] == toff_a ? 0 : 64) * 2);
-      f32x4 part[MT];
+      const uint32_t base = tb + (uint32_t)((toff[nt] == toff_a ? 0 : 64) * 2);
+      f32x4 part[HM];
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) zero_acc(part[mt]);
+      for (int mt = 0; mt < HM; ++mt) zero_acc(part[mt]);
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         if (j * 32 < a.lora_rank) {
           const u32x4 lbf = lds_ld128(lb_lds + (uint32_t)((nt * 2 + j) * 1024));
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
+          for (int mt = 0; mt < HM; ++mt)
             part[mt] = mfma16(lds_ld128(base + (uint32_t)((mt * 16 * A_LD + j * 32) * 2)), lbf, part[mt]);
         }
       }
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+      for (int mt = 0; mt < HM; ++mt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[mt][nt][i] += a.lora_scale * part[mt][i];
+        for (int i = 0; i < 4; ++i) out[mt][nt][i] += a.lora_scale * part[mt][i];
     }
   } else if (a.lora_rank > 0 && blockIdx.z == 0) {
     TileSrc s;
@@ -378,7 +408,7 @@ void qgemm128_kernel(const QLArgs a) {
     s.w_bf16 = nullptr; s.codes = a.codes; s.scales = a.scales; s.group = a.group; s.qtype = a.qtype;
     s.ntiles = ntiles; s.lora_rank = a.lora_rank; s.t = a.t; s.t_ld = a.t_ld; s.lora_b = a.lora_b;
     s.lora_scale = a.lora_scale;
-    tile_lora<MT, NT>(s, m0, ntile0, toff, acc);
+    tile_lora<HM, NT>(s, m0w, ntile0, toff, out);
   }
   TNX_STAMP(4);
   const bool mul = a.epilogue == TNX_EPI_SILU_MUL || a.epilogue == TNX_EPI_GELU_MUL;
@@ -388,7 +418,7 @@ void qgemm128_kernel(const QLArgs a) {
     // the tile is multiplied with the NEXT linear's adapter A (its LoRA down-projection, whose
     // K axis is this kernel's output axis), one fp32 fragment plane per work-group.
     constexpr int ACT_LD = 72;  // 64 act columns + 8 pad (bf16 elements)
-    const uint32_t act_lds = a_rd_nxt - (uint32_t)(lm * A_LD + lq * 8) * 2u;
+    const uint32_t act_lds = a_rd_nxt - (uint32_t)(lm * A_LD + lq * 8 + kh * 64) * 2u;
     const int64_t ldy = a.N / 2;
     const int64_t wgcol0 = (int64_t)blockIdx.y * 64;      // first act column of the work-group
     const bool fuse_next = a.next_tpart != nullptr;
@@ -406,28 +436,27 @@ void qgemm128_kernel(const QLArgs a) {
     }
     uint16_t* act_s = reinterpret_cast<uint16_t*>(smem + act_lds);
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int mt = 0; mt < HM; ++mt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float g = rbf(acc[mt][0][i]);
-        const float u = rbf(acc[mt][1][i]);
+        const float g = rbf(out[mt][0][i]);
+        const float u = rbf(out[mt][1][i]);
         const float act = a.epilogue == TNX_EPI_SILU_MUL ? silu_bf16(g) : gelu_tanh_bf16(g);
-        act_s[(mt * 16 + lq * 4 + i) * ACT_LD + wn * 16 + lm] = f2bf(rbf(act) * u);
+        act_s[(kh * 64 + mt * 16 + lq * 4 + i) * ACT_LD + wn * 16 + lm] = f2bf(rbf(act) * u);
       }
     __syncthreads();
     uint16_t* y = reinterpret_cast<uint16_t*>(a.y);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const int idx = tid + 256 * c, row = idx >> 3, ch = idx & 7;
+    for (int c = 0; c < 2; ++c) {
+      const int idx = tid + 512 * c, row = idx >> 3, ch = idx & 7;
       const u32x4 v = lds_ld128(act_lds + (uint32_t)((row * ACT_LD + ch * 8) * 2));
       if (m0 + row < a.M && wgcol0 + ch * 8 + 8 <= ldy)
         *reinterpret_cast<u32x4*>(y + (m0 + row) * ldy + wgcol0 + ch * 8) = v;
     }
     if (fuse_next) {
       float* plane = a.next_tpart + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * 8192;
-#pragma unroll
-      for (int q = 0; q < 2; ++q) {
-        const int mt = wn * 2 + q;
+      {
+        const int mt = wv;
         u32x4 af2[2];
 #pragma unroll
         for (int j = 0; j < 2; ++j)
@@ -442,7 +471,7 @@ void qgemm128_kernel(const QLArgs a) {
       }
     }
   } else {
-    store_tile<MT, NT>(a, m0, a.M, ntile0, ntiles, acc, [](int64_t r) { return r; });
+    store_tile<HM, NT>(a, m0w, a.M, ntile0, ntiles, out, [](int64_t r) { return r; });
   }
   TNX_STAMP(5);
 }

@@ -482,7 +482,7 @@ int launch_qgemm128(hipStream_t st, const QLArgs& a) {
   std::call_once(once, [] { attr_rc = raise_lds_limit(&qgemm128_kernel<NT, SPT>, kBigSmemBytes); });
   if (attr_rc) return attr_rc;
   dim3 grid((unsigned)cdiv(a.M, 128), (unsigned)cdiv(a.N, 64 * NT), (unsigned)a.split_k);
-  hipLaunchKernelGGL((qgemm128_kernel<NT, SPT>), grid, dim3(256), kBigSmemBytes, st, a);
+  hipLaunchKernelGGL((qgemm128_kernel<NT, SPT>), grid, dim3(512), kBigSmemBytes, st, a);
   TNX_CHECK_LAUNCH("qgemm128");
   return TNX_OK;
 }

@@ -285,9 +285,10 @@ class Runner:
 
   def linear(self, f: FusedLinear, x, y, M, epilogue=L.TNX_EPI_STORE, residual=None, defer=False,
              next_f: FusedLinear | None = None, t_ready: bool = False):
-    """Runs one fused linear.  With defer=True a split-k RESIDUAL linear whose output width is
-    the model width skips its finishing pass and returns split_k (> 1): the caller hands the
-    partial planes in self.splitk_ws to `norm_after`; otherwise returns 1 with y complete."""
+    """Runs one fused linear.  With defer=True a split-k linear skips its finishing pass and
+    returns split_k (> 1): the caller hands the partial planes in self.splitk_ws to the kernel
+    that consumes them (`norm_after` for a RESIDUAL linear of model width, the rope / cache
+    write for a plain STORE); otherwise returns 1 with y complete."""
     if f.has_lora and not t_ready:
       ops.lora_down(x, f.a_t, self.t, M=M)
     split = self._split_k(f, M)
@@ -307,8 +308,9 @@ class Runner:
       ops.qlinear(d)
       ops.lora_reduce(self.next_tpart, M, math.ceil(f.N / 128), next_f.rp, self.t)
       return 1
-    deferred = (defer and split > 1 and epilogue == L.TNX_EPI_RESIDUAL and f.N == self.cfg.embed_dim
-                and f.N % 8 == 0)
+    deferred = defer and split > 1 and (
+        epilogue == L.TNX_EPI_STORE
+        or (epilogue == L.TNX_EPI_RESIDUAL and f.N == self.cfg.embed_dim and f.N % 8 == 0))
     ops.qlinear(d, finish=not deferred)
     return split if deferred else 1
 
@@ -342,7 +344,7 @@ class Runner:
     for i, ly in enumerate(m.layers):
       self.norm_after(pending, ly["attn_norm"], M)
       pending = 1
-      self.linear(ly["qkv"], self.xn, self.qkv, M)
+      qkv_split = self.linear(ly["qkv"], self.xn, self.qkv, M, defer=True)
       rd = L.RopeDesc()
       rd.B, rd.T, rd.S = B, T, self.S
       rd.Hq, rd.Hkv, rd.dh = cfg.num_heads, cfg.num_kv_heads, cfg.head_dim
@@ -356,6 +358,8 @@ class Runner:
         rd.qk_norm = -1
       rd.q_prescale = cfg.query_pre_attn_scalar if cfg.family == "gemma3" else 0.0
       rd.qkv, rd.positions, rd.pos_ld = self.qkv.data_ptr(), positions.data_ptr(), positions.shape[1]
+      if qkv_split > 1:  # the rope kernel sums the partial planes itself
+        rd.qkv_ws, rd.split_k = self.splitk_ws.data_ptr(), qkv_split
       rd.col_ptr = col_ptr.data_ptr()
       rd.q_out, rd.kcache, rd.vcache = self.q.data_ptr(), kcache[i].data_ptr(), vcache[i].data_ptr()
       ops.rope_kvwrite(rd)
