@@ -291,24 +291,27 @@ __global__ __launch_bounds__(512) void lora_down_kernel(const uint16_t* x, int64
   }
 }
 
-// t[M, :R] = bf16(sum of fragment planes).  One thread per (row block, row tile, column tile,
-// lane): it owns the four rows 4*(lane/16)+i of column lane%16 of that 16 x 16 tile, exactly
-// as the MFMA that produced the plane laid them out.
-__global__ void lora_reduce_kernel(const float* tpart, int64_t M, int64_t ncb, int R, uint16_t* t,
-                                   int64_t t_ld) {
-  const int ntile = R / 16;
-  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int lane = (int)(gid & 63);
-  int64_t q = gid >> 6;
-  const int n = (int)(q % ntile);
-  q /= ntile;
-  const int mt = (int)(q & 7);
-  const int64_t mb = q >> 3;
-  if (mb * 128 >= M) return;
-  const float* p = tpart + mb * ncb * 8192 + ((mt * 4 + n) * 64 + lane) * 4;
+// t[M, :R] = bf16(sum of fragment planes).  A plane holds, per (row tile, column tile, lane), the
+// four rows 4*(lane/16)+i of column lane%16 of a 16 x 16 tile, exactly as the MFMA that produced
+// it laid them out.  One work-group sums 8 consecutive lanes' values (128 bytes of every plane):
+// 32 thread groups take every 32nd plane each, then the 32 partial sums are added in order.
+__global__ __launch_bounds__(256) void lora_reduce_kernel(const float* tpart, int64_t M, int64_t ncb, int R,
+                                                          uint16_t* t, int64_t t_ld) {
+  __shared__ f32x4 red[32][8];
+  const int g = threadIdx.x & 7, sl = threadIdx.x >> 3;
+  const int q = blockIdx.x * 8 + g;           // (row tile * 4 + column tile) * 64 + lane
+  const int lane = q & 63, n = (q >> 6) & 3, mt = q >> 8;
+  const int64_t mb = blockIdx.y;
+  if (n * 16 >= R) return;                     // same for the whole work-group
+  const float* p = tpart + mb * ncb * 8192 + (int64_t)q * 4;
   f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int64_t cb = sl; cb < ncb; cb += 32) s += *reinterpret_cast<const f32x4*>(p + cb * 8192);
+  red[sl][g] = s;
+  __syncthreads();
+  if (sl != 0) return;
 #pragma unroll 8
-  for (int64_t cb = 0; cb < ncb; ++cb) s += *reinterpret_cast<const f32x4*>(p + cb * 8192);
+  for (int k = 1; k < 32; ++k) s += red[k][g];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int64_t row = mb * 128 + mt * 16 + (lane >> 4) * 4 + i;
@@ -576,8 +579,7 @@ extern "C" int tnx_lora_reduce(void* stream, const float* tpart, int64_t M, int6
   TNX_REQUIRE(tpart && t, "lora_reduce: null pointer");
   TNX_REQUIRE(M > 0 && n_col_blocks > 0, "lora_reduce: bad shape");
   TNX_REQUIRE(R > 0 && R % 16 == 0 && R <= 64 && t_ld >= R, "lora_reduce: R=%d must be a multiple of 16, <= 64 and <= t_ld", R);
-  const int64_t threads = cdiv(M, 128) * 8 * (R / 16) * 64;
-  hipLaunchKernelGGL(lora_reduce_kernel, dim3((unsigned)cdiv(threads, 256)), dim3(256), 0, as_stream(stream),
+  hipLaunchKernelGGL(lora_reduce_kernel, dim3(256, (unsigned)cdiv(M, 128)), dim3(256), 0, as_stream(stream),
                      tpart, M, n_col_blocks, R, t, t_ld);
   TNX_CHECK_LAUNCH("lora_reduce");
   return TNX_OK;
