@@ -33,9 +33,10 @@ struct AttnArgs {
 constexpr float kNegBig = -1.0e30f;
 
 template <int DH>
-__global__ __launch_bounds__(64) void attn_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2 : 1, DH > 128 ? 2 : 1))) void attn_kernel(const AttnArgs a) {
   constexpr int KS = DH / 32;                 // k-steps of the QK product
   constexpr int NH = DH > 128 ? DH / 128 : 1; // 128-column halves of V / O
+  constexpr int NS = DH > 128 ? 1 : 3;        // register stages of the key-block pipeline
   const int lane = threadIdx.x, lm = lane & 15, lq = lane >> 4;
   const int chunk = blockIdx.x, hkv = blockIdx.y;
   const int PT = 16 / a.Gp;                              // positions per query tile
@@ -78,51 +79,68 @@ __global__ __launch_bounds__(64) void attn_kernel(const AttnArgs a) {
   const uint16_t* vbase = a.v + ((b * a.Hkv + hkv) * a.S) * DH;
   const int32_t* tok = a.tokens + b * a.tok_ld;
   const int vcol = (8 * lm) % (DH < 128 ? DH : 128);     // DH=64: upper lanes duplicate
-  // 16-byte token loads need 16-byte aligned rows; slots past S - 4 are clamped (keys beyond
+  // 16-byte token loads need 16-byte aligned rows and whole groups of four slots (keys beyond
   // the range are masked by the range test anyway)
-  const bool tok_vec = (a.tok_ld % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.tokens) & 15) == 0) && a.S >= 4;
-  const int tok_last4 = ((int)a.S - 4) & ~3;
+  const bool tok_vec = (a.tok_ld % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.tokens) & 15) == 0) && a.S % 4 == 0;
 
-  for (int kb = k_lo & ~31; kb <= k_hi; kb += 32) {
-    // ---- loads: K as A fragments (two tiles of 16 keys), V rows of this lane's 8 keys ----
+  // A ring of NS register stages: the loads of the next NS-1 key blocks are in flight while a
+  // block is computed, so the memory system is never left idle behind a wave's softmax and
+  // MFMAs.  One wave per SIMD owns the whole register file for this (nothing else hides the
+  // latency: a wave has no second wave to alternate with).  Prefetches past the last block are
+  // redirected to the last block (cache hits) rather than skipped: with every load issued
+  // unconditionally the number of loads in flight is static, and the wait for a stage's data
+  // does not have to drain the younger stages.
+  struct Stage {
     u32x4 kf[2][KS];
+    u32x4 vf[NH][8];
+    int tk[8];
+  };
+  // K / V of this (row, kv head) and the row's token ids as buffer resources: a lane's byte
+  // offset is a per-kernel constant plus the block's first key, so a block costs a handful of
+  // address instructions, and keys past the cache (S not a multiple of 32, or a prefetch past
+  // the end) read zeros; they are masked by the range test anyway.
+  const uint32_t slab_bytes = (uint32_t)a.S * DH * 2u;
+  const rsrc_t rk = make_rsrc(kbase, slab_bytes), rv = make_rsrc(vbase, slab_bytes);
+  const rsrc_t rtok = make_rsrc(tok, (uint64_t)a.S * 4);
+  const uint32_t koff = (uint32_t)(lm * DH + lq * 8) * 2u;           // + tt * 16 keys, + j * 64 B
+  const uint32_t voff = (uint32_t)(4 * lq * DH + vcol) * 2u;         // + s keys, + 16 keys, + h * 256 B
+  auto load_block = [&](int kb, Stage& sg) {
+    const uint32_t kb_bytes = (uint32_t)kb * (DH * 2u);
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
-      const int key = min(kb + 16 * tt + lm, (int)a.S - 1);
+      const uint32_t o = koff + kb_bytes + (uint32_t)(tt * 16 * DH * 2);
 #pragma unroll
-      for (int j = 0; j < KS; ++j)
-        kf[tt][j] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)key * DH + j * 32 + lq * 8);
+      for (int j = 0; j < KS; ++j) sg.kf[tt][j] = __builtin_amdgcn_raw_buffer_load_b128(rk, o + (uint32_t)(j * 64), 0, 0);
     }
-    u32x4 vf[NH][8];
-    int keys[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-      keys[s] = kb + (s < 4 ? 4 * lq + s : 16 + 4 * lq + (s - 4));
-      const int key = min(keys[s], (int)a.S - 1);
+      const uint32_t o = voff + kb_bytes + (uint32_t)(((s < 4 ? s : 12 + s)) * DH * 2);
 #pragma unroll
-      for (int h = 0; h < NH; ++h)
-        vf[h][s] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)key * DH + h * 128 + vcol);
+      for (int h = 0; h < NH; ++h) sg.vf[h][s] = __builtin_amdgcn_raw_buffer_load_b128(rv, o + (uint32_t)(h * 256), 0, 0);
     }
     // token ids of this lane's 8 keys (two runs of 4 consecutive slots), fetched unconditionally
     // together with K and V: a predicated load per key would serialise eight memory latencies
-    int tk[8];
     if (tok_vec) {
-      const u32x4 t0 = *reinterpret_cast<const u32x4*>(tok + min(kb + 4 * lq, tok_last4));
-      const u32x4 t1 = *reinterpret_cast<const u32x4*>(tok + min(kb + 16 + 4 * lq, tok_last4));
+      const u32x4 t0 = __builtin_amdgcn_raw_buffer_load_b128(rtok, (uint32_t)(kb + 4 * lq) * 4u, 0, 0);
+      const u32x4 t1 = __builtin_amdgcn_raw_buffer_load_b128(rtok, (uint32_t)(kb + 16 + 4 * lq) * 4u, 0, 0);
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        tk[s] = (int)t0[s];
-        tk[4 + s] = (int)t1[s];
+        sg.tk[s] = (int)t0[s];
+        sg.tk[4 + s] = (int)t1[s];
       }
     } else {
 #pragma unroll
-      for (int s = 0; s < 8; ++s) tk[s] = tok[min(keys[s], (int)a.S - 1)];
+      for (int s = 0; s < 8; ++s)
+        sg.tk[s] = (int)__builtin_amdgcn_raw_buffer_load_b32(
+            rtok, (uint32_t)(kb + (s < 4 ? 4 * lq + s : 16 + 4 * lq + (s - 4))) * 4u, 0, 0);
     }
+  };
+  auto compute_block = [&](int kb, const Stage& sg) {
     bool kvalid[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-      const int key = keys[s];
-      kvalid[s] = qvalid && key >= max(k_lo, lo_n) && key <= min(k_hi, c_n) && tk[s] != a.pad_id;
+      const int key = kb + (s < 4 ? 4 * lq + s : 16 + 4 * lq + (s - 4));
+      kvalid[s] = qvalid && key >= max(k_lo, lo_n) && key <= min(k_hi, c_n) && sg.tk[s] != a.pad_id;
     }
     // ---- S^T = K . q^T ----
     f32x4 st[2];
@@ -130,7 +148,7 @@ __global__ __launch_bounds__(64) void attn_kernel(const AttnArgs a) {
     for (int tt = 0; tt < 2; ++tt) {
       st[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int j = 0; j < KS; ++j) st[tt] = mfma16(kf[tt][j], qf[j], st[tt]);
+      for (int j = 0; j < KS; ++j) st[tt] = mfma16(sg.kf[tt][j], qf[j], st[tt]);
     }
     float sv[8];
     float bmax = kNegBig;
@@ -179,9 +197,28 @@ __global__ __launch_bounds__(64) void attn_kernel(const AttnArgs a) {
         u32x4 bfrag;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-          bfrag[r] = __builtin_amdgcn_perm(vf[h][2 * r + 1][jj >> 1], vf[h][2 * r][jj >> 1], sel);
+          bfrag[r] = __builtin_amdgcn_perm(sg.vf[h][2 * r + 1][jj >> 1], sg.vf[h][2 * r][jj >> 1], sel);
         O[h][jj] = mfma16(pa, bfrag, O[h][jj]);
       }
+  };
+  {
+    Stage sg[NS];
+    const int kb0 = k_lo & ~31;
+    const int kb_last = k_hi & ~31;
+    if (kb0 <= k_hi) {
+#pragma unroll
+      for (int u = 0; u < NS - 1; ++u) load_block(min(kb0 + 32 * u, kb_last), sg[u]);
+      for (int kb = kb0; kb <= k_hi; kb += 32 * NS) {
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+          const int kbu = kb + 32 * u;
+          if (kbu > k_hi) break;
+          load_block(min(kbu + 32 * (NS - 1), kb_last), sg[(u + NS - 1) % NS]);
+          __builtin_amdgcn_sched_barrier(0);
+          compute_block(kbu, sg[u]);
+        }
+      }
+    }
   }
 
   l_run += __shfl_xor(l_run, 16, 64);

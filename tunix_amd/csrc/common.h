@@ -116,3 +116,15 @@ __device__ __forceinline__ float wave_max(float v) {
 
 static inline hipStream_t as_stream(void* s) { return (hipStream_t)s; }
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Raw buffer resources: 32-bit byte offsets, and loads whose vector offset (plus the
+// immediate) lies past the size return zeros instead of faulting.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint64_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0,
+                                           (uint32_t)(bytes > 0xffffffffull ? 0xffffffffull : bytes),
+                                           0x00020000);
+}
+__device__ __forceinline__ u32x4 buf_load128(rsrc_t r, uint32_t byte_off) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
+}

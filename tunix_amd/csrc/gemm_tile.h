@@ -25,16 +25,6 @@ __device__ __forceinline__ uint32_t* tile_lut(unsigned char* smem, int mt) {
   return reinterpret_cast<uint32_t*>(smem + 2 * (size_t)mt * 16 * A_LD * sizeof(uint16_t));
 }
 
-typedef __amdgpu_buffer_rsrc_t rsrc_t;
-__device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint64_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0,
-                                           (uint32_t)(bytes > 0xffffffffull ? 0xffffffffull : bytes),
-                                           0x00020000);
-}
-__device__ __forceinline__ u32x4 buf_load128(rsrc_t r, uint32_t byte_off) {
-  return __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
-}
-
 struct TileSrc {
   int64_t M, K;
   const uint16_t* x;         // bf16 [M,K] (or gathered through row_index)

@@ -8,7 +8,9 @@ kernel.  LoRA A/B stay separate buffers so that `update_lora` can swap them betw
 """
 from __future__ import annotations
 
+import json
 import math
+import os
 
 import numpy as np
 import torch
@@ -241,7 +243,8 @@ class Runner:
       self.y_route = torch.empty(M * k, D, dtype=bf, device=dev)
     else:
       self.act = torch.empty(M, F, dtype=bf, device=dev)
-    self.split_k_override = {}
+    # tuning knob: TUNIX_SPLIT_K='{"o": 4}' pins the k split of the linears with that name
+    self.split_k_override = json.loads(os.environ.get("TUNIX_SPLIT_K", "{}"))
     self.next_tpart = None
     if 64 < M <= 1024 and not cfg.num_experts and model.layers and "gu" in model.layers[0]:
       n_planes = math.ceil(M / 128) * math.ceil(model.layers[0]["gu"].N / 128)
@@ -255,7 +258,15 @@ class Runner:
             need = max(need, sk * M * ly[key].N)
     self.splitk_ws = torch.empty(need, dtype=torch.float32, device=dev)
     if kv_chunk is None:
-      kv_chunk = 256 if (T == 1 and S > 256) else 0
+      # decode: one wave streams the keys of one (row, kv head); the key range is split only as
+      # far as needed to put about a thousand waves (one per SIMD) on the device
+      kv_chunk = 0
+      waves = B * cfg.num_kv_heads
+      if T == 1 and waves < 1024 and S > 64:
+        n_chunks = min(math.ceil(1024 / waves), S // 32)
+        kv_chunk = max(32, math.ceil(S / n_chunks / 32) * 32)
+        if kv_chunk >= S:
+          kv_chunk = 0
     self.kv_chunk = kv_chunk
     nb = ops.attn_ws_bytes(B, T, S, cfg.num_heads, cfg.head_dim, kv_chunk)
     self.attn_ws = torch.empty(max(nb // 4, 1), dtype=torch.float32, device=dev)
