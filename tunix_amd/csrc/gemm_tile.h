@@ -128,7 +128,7 @@ __device__ __forceinline__ void tile_mainloop(const TileSrc& s, int64_t m0, int6
       }
     }
   } else {
-    constexpr int PF = 4;  // weight k-tiles in flight
+    constexpr int PF = 2;  // weight k-tiles in flight
     const int spt = scales_per_tile(s.group);  // scale slots per tile and column (2 or 4)
     const uint64_t ntk = (uint64_t)s.ntiles * ktiles;
     const rsrc_t rc = make_rsrc(s.codes, ntk * 1024);

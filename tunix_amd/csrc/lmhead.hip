@@ -52,8 +52,11 @@ __device__ __forceinline__ Stat merge(const Stat& a, const Stat& b) {
   return r;
 }
 
+// The dense (bf16 weight) flavour is latency bound on its weight stream: it needs no code-book
+// table, so its LDS footprint lets two work-groups share a compute unit, and the launch bound
+// (a register budget, the work-group size is always 256) keeps it within half the register file.
 template <int MT, bool DENSE>
-__global__ __launch_bounds__(256) void lmhead_kernel(const LHArgs a) {
+__global__ __launch_bounds__(DENSE ? 512 : 256) void lmhead_kernel(const LHArgs a) {
   constexpr int NT = 2;
   extern __shared__ __align__(16) unsigned char smem[];
   uint16_t* sA = reinterpret_cast<uint16_t*>(smem);
@@ -201,10 +204,11 @@ template <int MT, bool DENSE>
 int launch_lmhead(hipStream_t st, const LHArgs& a) {
   static std::once_flag once;
   static int attr_rc = TNX_OK;
-  std::call_once(once, [] { attr_rc = raise_lds_limit(&lmhead_kernel<MT, DENSE>, tile_smem_bytes(MT)); });
+  constexpr size_t kLds = DENSE ? 2 * (size_t)MT * 16 * A_LD * sizeof(uint16_t) : tile_smem_bytes(MT);
+  std::call_once(once, [] { attr_rc = raise_lds_limit(&lmhead_kernel<MT, DENSE>, kLds); });
   if (attr_rc) return attr_rc;
   dim3 grid((unsigned)a.nvb, (unsigned)cdiv(a.M, MT * 16));
-  hipLaunchKernelGGL((lmhead_kernel<MT, DENSE>), grid, dim3(256), tile_smem_bytes(MT), st, a);
+  hipLaunchKernelGGL((lmhead_kernel<MT, DENSE>), grid, dim3(256), kLds, st, a);
   TNX_CHECK_LAUNCH("lmhead");
   return TNX_OK;
 }
