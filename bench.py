@@ -131,7 +131,13 @@ def kernel_breakdown(model, runner, st, ctx, iters):
   return out
 
 
-def rooflines(kern):
+# HBM bytes of one qgemm128 launch on the default workload (batch 128, Llama-3.1-8B shapes, mean
+# over the four linears): rocprofv3 FETCH_SIZE + WRITE_SIZE, (22843 + 12949) KiB, both counters
+# scaled by 1.000 against a plain copy of known size (profiles/qgemm128_kernel_llama8b_decode_b128.md).
+QGEMM128_TRAFFIC_BYTES_B128 = 36_651_008
+
+
+def rooflines(kern, default_workload=False):
   """The dominant kernel of a step is the quantised GEMM (one kernel, launched for the four
   linears of every layer).  One launch = the mean over those four shapes.  At 128 rows its
   arithmetic intensity (2 * 128 flop per 0.53 B of packed weight = 483 flop/B) is past the
@@ -145,7 +151,8 @@ def rooflines(kern):
   gbs = nbytes / (us * 1e-6) / 1e9
   roofline = {"kernel": "qgemm128_kernel", "bound": "mfma", "achieved": round(tf, 1),
               "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-              "traffic": None, "us_per_launch": round(us, 2), "algorithmic_flops": flops,
+              "traffic": QGEMM128_TRAFFIC_BYTES_B128 if default_workload else None,
+              "us_per_launch": round(us, 2), "algorithmic_flops": flops,
               "algorithmic_bytes": nbytes,
               "launch_shapes_us": {k: round(kern[k]["kernel_ms"] * 1e3, 2) for k in names}}
   roofline_hbm = {"kernel": "qgemm128_kernel", "bound": "hbm", "achieved": round(gbs, 1),
@@ -247,7 +254,7 @@ def main():
     for buf in (runner.xn, runner.attn, runner.act, runner.q):
       buf.normal_()
     kern = kernel_breakdown(model, runner, st, P + T // 2, args.kernel_iters)
-    roofline, roofline_hbm = rooflines(kern)
+    roofline, roofline_hbm = rooflines(kern, default_workload=(B == 128))
     # a plain device copy of known size (256 MiB read + 256 MiB written): the yardstick that
     # scales the FETCH_SIZE / WRITE_SIZE counters of a counter-collection run of this command
     src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
@@ -316,7 +323,7 @@ def main():
   for name, v in kern.items():
     log(f"  {name:16s} {v['ms'] * 1e3:8.1f} us/launch  {v['gbs']:7.0f} GB/s  {v['tflops']:7.1f} TFLOP/s"
         f"  x{v['per_step']} = {v['step_ms']:.3f} ms/step")
-  roofline, roofline_linears = rooflines(kern)
+  roofline, roofline_linears = rooflines(kern, default_workload=(B == 128 and not args.layers))
   wb = model.weight_bytes()
   step_bytes = (wb["quantized"] + wb["lora"] + wb["head"]
                 + B * cfg.num_kv_heads * mean_ctx * cfg.head_dim * 4 * cfg.num_layers)
