@@ -60,6 +60,19 @@ __device__ __constant__ const float kNf4Levels[16] = {
 __device__ __forceinline__ float code_level(int qtype, int code) {
   return qtype == TNX_Q_NF4 ? kNf4Levels[code] : (float)(code - 8);
 }
+// The same value from literals (a select tree over the code's bits): no memory access, for
+// kernels whose first instructions would otherwise wait on the table.
+__device__ __forceinline__ float code_level_imm(int qtype, int code) {
+  const bool b0 = code & 1, b1 = code & 2, b2 = code & 4, b3 = code & 8;
+  const float p0 = b0 ? -0.6961928f : -1.0f, p1 = b0 ? -0.39491749f : -0.52507305f;
+  const float p2 = b0 ? -0.18477343f : -0.28444138f, p3 = b0 ? 0.0f : -0.09105004f;
+  const float p4 = b0 ? 0.1609302f : 0.0795803f, p5 = b0 ? 0.33791524f : 0.2461123f;
+  const float p6 = b0 ? 0.562617f : 0.44070983f, p7 = b0 ? 1.0f : 0.72295684f;
+  const float q0 = b1 ? p1 : p0, q1 = b1 ? p3 : p2, q2 = b1 ? p5 : p4, q3 = b1 ? p7 : p6;
+  const float r0 = b2 ? q1 : q0, r1 = b2 ? q3 : q2;
+  const float nf4 = b3 ? r1 : r0;
+  return qtype == TNX_Q_NF4 ? nf4 : (float)(code - 8);
+}
 
 // Scales stored per (k-tile of 128, column): S = max(2, 128 / group) slots of 128 / S k each
 // (a group of 128 or more repeats its scale), so that a lane's scales are one aligned 4- or 8-byte word.

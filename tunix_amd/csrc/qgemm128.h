@@ -64,15 +64,26 @@ void qgemm128_kernel(const QLArgs a) {
   constexpr int MT = 8, HM = 4, PF = 3;
   constexpr int SW = SPT / 2;  // scales of one wave's two k-steps
   extern __shared__ __align__(16) unsigned char smem[];
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, wn = wv & 3, kh = wv >> 2;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6), wn = wv & 3, kh = wv >> 2;  // wave-uniform
   const int lm = lane & 15, lq = lane >> 4;
   TNX_STAMP(0);
   // LDS is addressed absolutely below (table at 0): bail out if the dynamic block does not
   // start at LDS address 0, which would mean a static LDS allocation crept into this kernel
   if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem != 0u) return;
-  // the two code-book levels of this thread's table entry, fetched before anything else so
-  // that their (constant-memory) loads are the oldest ones in flight
-  const float lvl0 = rbf(code_level(a.qtype, tid & 15)), lvl1 = rbf(code_level(a.qtype, (tid >> 4) & 15));
+  // Pull the whole argument block into SGPRs with one batch of scalar loads: left alone, the
+  // compiler sinks each field's load next to its first use, and the prologue pays one scalar
+  // memory round trip after the other.
+  asm volatile("" ::"s"(a.M), "s"(a.K), "s"(a.N), "s"(a.qtype), "s"(a.x), "s"(a.codes), "s"(a.scales),
+               "s"(a.lora_rank), "s"(a.lora_nseg), "s"(a.lora_seg_end[0]), "s"(a.lora_seg_end[1]),
+               "s"(a.lora_seg_end[2]), "s"(a.lora_seg_toff[0]), "s"(a.lora_seg_toff[1]),
+               "s"(a.lora_seg_toff[2]), "s"(a.lora_seg_toff[3]));
+  asm volatile("" ::"s"(a.t_ld), "s"(a.t), "s"(a.lora_b), "s"(a.lora_scale), "s"(a.epilogue), "s"(a.y),
+               "s"(a.split_k), "s"(a.ws), "s"(a.ktiles_per_split), "s"(a.next_a_t), "s"(a.next_rank),
+               "s"(a.next_tpart));
+  // the two code-book levels of this thread's table entry, from literals: nothing at the start
+  // of the kernel waits on memory except the loads of the first tiles
+  const float lvl0 = rbf(code_level_imm(a.qtype, tid & 15)), lvl1 = rbf(code_level_imm(a.qtype, (tid >> 4) & 15));
   const uint32_t lane_off = (uint32_t)lane * 4u;
   const int64_t m0 = (int64_t)blockIdx.x * 128;
   const int64_t ntile0 = ((int64_t)blockIdx.y * 4 + wn) * NT;
@@ -98,6 +109,7 @@ void qgemm128_kernel(const QLArgs a) {
     soff[nt] = (tile0 * 16u + (uint32_t)lm) * (uint32_t)(SPT * 2) + (SPT == 4 ? (uint32_t)kh * 4u : 0u);
   }
 
+  TNX_STAMP(6);
   f32x4 acc[MT][NT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
@@ -120,26 +132,39 @@ void qgemm128_kernel(const QLArgs a) {
   int toff_a = 0, toff_b = 0;
   bool lora_fast = a.lora_rank > 0 && a.lora_rank <= 64 && blockIdx.z == 0;
   if (a.lora_rank > 0) {
-    auto seg_toff = [&](int64_t ntile) {
-      if (a.lora_nseg < 0) return (int)(ntile & 1) * a.lora_rank;  // interleaved gate / up pair
-      int o = a.lora_seg_toff[0];
+    if (a.lora_nseg < 0) {  // interleaved gate / up pair: even tiles segment 0, odd tiles segment 1
+      toff_a = 0;
+      toff_b = a.lora_rank;
 #pragma unroll
-      for (int q = 1; q < 4; ++q)  // constant bounds: the argument arrays stay in SGPRs
-        if (q < a.lora_nseg && ntile * 16 >= a.lora_seg_end[q - 1]) o = a.lora_seg_toff[q];
-      return o;
-    };
-    const int64_t wg_nt0 = (int64_t)blockIdx.y * 4 * NT;
-    toff_a = seg_toff(wg_nt0);
-    toff_b = seg_toff(min(wg_nt0 + 4 * NT - 1, ntiles - 1));
+      for (int nt = 0; nt < NT; ++nt) toff[nt] = (int)((ntile0 + nt) & 1) * a.lora_rank;
+    } else {
+      // segments are contiguous column ranges: index and offset by straight selects (no
+      // branches, the argument arrays stay in SGPRs); N < 2^31, the host checks the 4 GiB limits
+      int e0 = (int)a.lora_seg_end[0], e1 = (int)a.lora_seg_end[1], e2 = (int)a.lora_seg_end[2];
+      int t0 = a.lora_seg_toff[0], t1 = a.lora_seg_toff[1], t2 = a.lora_seg_toff[2], t3 = a.lora_seg_toff[3];
+      // opaque copies: otherwise the selects below are folded back into indexed loads from the
+      // argument block, one more scalar memory round trip each
+      asm volatile("" : "+s"(e0), "+s"(e1), "+s"(e2), "+s"(t0), "+s"(t1), "+s"(t2), "+s"(t3));
+      auto seg_idx = [&](int ntile) {
+        const int col = ntile * 16;
+        return (int)(a.lora_nseg > 1 && col >= e0) + (int)(a.lora_nseg > 2 && col >= e1) +
+               (int)(a.lora_nseg > 3 && col >= e2);
+      };
+      auto idx_toff = [&](int i) {
+        // bit selects (a chain of ?: over an index becomes a table in private memory)
+        auto pick = [](int cur, int cand, bool c) { return cur ^ ((cur ^ cand) & (0 - (int)c)); };
+        return pick(pick(pick(t0, t1, i == 1), t2, i == 2), t3, i == 3);
+      };
+      const int last = (int)ntiles - 1;
+      const int wg_nt0 = (int)blockIdx.y * 4 * NT;
+      const int ia = seg_idx(wg_nt0), ib = seg_idx(min(wg_nt0 + 4 * NT - 1, last));
+      toff_a = idx_toff(ia);
+      toff_b = idx_toff(ib);
+      // the tile is shared by all waves: a work-group spanning three segments falls back to
+      // fragments from global memory (decided identically in every thread, no LDS involved)
+      lora_fast = lora_fast && ib - ia <= 1;
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) toff[nt] = seg_toff(min(ntile0 + nt, ntiles - 1));
-    // the tile is shared by all waves, so the decision is taken over all column tiles of
-    // the work-group (identically in every thread; no LDS or barrier involved: this kernel
-    // addresses LDS absolutely and must not acquire a static allocation): a work-group
-    // spanning three segments falls back to fragments from global memory
-    for (int q = 0; q < 4 * NT; ++q) {
-      const int o = seg_toff(min(wg_nt0 + q, ntiles - 1));
-      lora_fast = lora_fast && (o == toff_a || o == toff_b);
+      for (int nt = 0; nt < NT; ++nt) toff[nt] = idx_toff(seg_idx(min((int)ntile0 + nt, last)));
     }
   }
   // B^T fragments of the adapter for this column group: fetched now, parked in the group's
@@ -152,7 +177,9 @@ void qgemm128_kernel(const QLArgs a) {
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
     for (int j = 0; j < 2; ++j) lbv[nt][j] = u32x4{0, 0, 0, 0};
-  if (lora_fast) {
+  // (issued behind the first weight and activation loads: at kernel start every buffer is a
+  // fresh page, address translation misses are served in order, and these are needed last)
+  auto load_adapter_b = [&]() {
     const rsrc_t rb = make_rsrc(a.lora_b, (uint64_t)a.N * a.lora_rank * 2);
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
@@ -161,6 +188,8 @@ void qgemm128_kernel(const QLArgs a) {
         if (j * 32 < a.lora_rank)
           lbv[nt][j] = buf_load128(rb, (((uint32_t)(ntile0 + nt) * 16u + (uint32_t)lm) * (uint32_t)a.lora_rank +
                                         (uint32_t)(j * 32 + lq * 8)) * 2u);
+  };
+  if (lora_fast) {
     const int ch = tid & 15;
     const int col = ((ch < 8) ? toff_a : toff_b) + min((ch & 7) * 8, a.lora_rank - 8);
     tbase = (uint32_t)((m0 + (tid >> 4)) * a.t_ld + col) * 2u;
@@ -318,6 +347,8 @@ void qgemm128_kernel(const QLArgs a) {
     load_w(ic<0>{}, kt_begin);
     load_w(ic<1>{}, kt_begin + 1);
     load_w(ic<2>{}, kt_begin + 2);
+    if (lora_fast) load_adapter_b();
+    TNX_STAMP(7);
     {  // table entry e = f16 pair (level[e & 15], level[e >> 4]); copies rotated over banks,
        // half of them per thread; built while the first loads are in flight
       uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
