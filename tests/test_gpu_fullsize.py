@@ -84,3 +84,38 @@ def test_full_size_decode_agrees_with_whole_sequence_pass(gpu):
         f"mean {err.mean():.3e}, median {np.median(err / ulp):.2f} ulp")
   assert np.median(err / ulp) <= 2.0
   assert (err <= 8.0 * ulp + 2e-2).all()
+
+
+def test_gemma3_1b_full_size_decode_agrees_with_whole_sequence_pass(gpu):
+  """The Gemma3-1B workload at its real sizes (26 layers, head_dim 256, one KV head, sliding
+  window 512, 262144-entry tied head, int4 g128, LoRA r16, batch 64, prompt 256): greedy decode
+  log-probabilities against compute_per_token_logps, graph replay against eager."""
+  from tunix_amd import config, dummy_model
+  from tunix_amd.generate import CacheConfig, Sampler
+  from tunix_amd.generate.utils import IdTokenizer
+  from tunix_amd.model import QLoRAModel
+  from tunix_amd.rl.common import compute_per_token_logps
+  cfg = config.gemma3_1b()
+  model = QLoRAModel(cfg, dummy_model.create_dummy_weights(cfg, seed=20258, device=gpu), gpu)
+  B, P, T = 64, 256, 6
+  tok = IdTokenizer(cfg.vocab_size, pad_id=0, eos_id=1)
+  cc = CacheConfig(512, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim)
+  prompts = _prompts(B, P, cfg.vocab_size, 20258)
+  a = Sampler(model, tok, cc, use_graph=True)(prompts, T, max_prompt_length=P, return_logprobs=True, eos_tokens=[-1])
+  b = Sampler(model, tok, cc, use_graph=False)(prompts, T, max_prompt_length=P, return_logprobs=True,
+                                               return_logits=True, eos_tokens=[-1])
+  for x, y in zip(a.tokens, b.tokens):
+    np.testing.assert_array_equal(x, y)
+  np.testing.assert_array_equal(np.asarray(a.logprobs), np.asarray(b.logprobs))
+  comp = np.stack(a.tokens).astype(np.int32)
+  lps = compute_per_token_logps(model, a.padded_prompt_tokens, comp, 0, max_rows=16 * (P + T)).cpu().numpy()
+  got = np.asarray(a.logprobs, dtype=np.float32)
+  lg = np.asarray(b.logits)
+  chosen = np.take_along_axis(lg, comp[:, :, None].astype(np.int64), -1)[..., 0]
+  ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(chosen), 2.0 ** -20))) - 7)
+  err = np.abs(lps - got)
+  print(f"gemma3-1b full size: max {err.max():.3e} ({(err / ulp).max():.1f} ulp), mean {err.mean():.3e}, "
+        f"median {np.median(err / ulp):.2f} ulp")
+  assert np.isfinite(got).all() and np.isfinite(lps).all()
+  assert np.median(err / ulp) <= 2.0
+  assert (err <= 8.0 * ulp + 2e-2).all()
