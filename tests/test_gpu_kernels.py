@@ -413,13 +413,21 @@ def test_lmhead_forbidden_and_ties(gpu):
   assert best.cpu().tolist() == [511] * M
 
 
+@pytest.mark.parametrize("V", [3000, 40001])
+@pytest.mark.parametrize("segmented", [False, True])
 @pytest.mark.parametrize("k,top_p,variant", [(50, 1.0, 0), (50, 0.7, 0), (8, 0.9, 1), (0, 1.0, 0)])
-def test_sample_topk_matches_oracle(gpu, k, top_p, variant):
+def test_sample_topk_matches_oracle(gpu, k, top_p, variant, segmented, V):
+  """Both flavours of the kernel (one work-group per row; row segments + merge, chosen by passing
+  a workspace) against the oracle's sample_top_p: ids exactly, log-probabilities to 2e-5.
+  V = 40001 spans three segments, with ties that straddle them."""
   from tunix_amd import ops
-  M, V = 16, 3000
+  M = 16
   g = torch.Generator().manual_seed(60)
   logits = (torch.randn(M, V, generator=g) * 2).float()
   logits[:, 17] = logits[:, 29]                      # ties inside the top-k
+  top = torch.topk(logits, 3, dim=1).values
+  logits[:, V - 7] = top[:, 1]                       # ... and across segments, at the far end
+  logits[:, V // 2] = top[:, 2]
   key = TF.prng_key(1234)
   step = 77
   temp = 0.7
@@ -429,7 +437,11 @@ def test_sample_topk_matches_oracle(gpu, k, top_p, variant):
   ids = torch.empty(M, dtype=torch.int32, device=gpu)
   lp = torch.empty(M, dtype=torch.float32, device=gpu)
   stp = torch.tensor([step], dtype=torch.int32, device=gpu)
-  ws = torch.empty(8, dtype=torch.float32, device=gpu)
+  ws = None
+  if segmented:
+    nb = ops.sample_topk_ws_bytes(M, V, k)
+    assert (nb > 0) == (k > 0)
+    ws = torch.empty(max(nb // 4, 1), dtype=torch.float32, device=gpu)
   ops.sample_topk(logits.to(gpu), k, top_p, temp, (int(key[0]), int(key[1])), variant, stp, ws, ids, lp)
   torch.cuda.synchronize()
   assert ids.cpu().long().tolist() == tok_ref.tolist()
@@ -444,6 +456,28 @@ def test_sample_topk_matches_oracle(gpu, k, top_p, variant):
                   forbidden=fb)
   assert ids.cpu().long().tolist() == tok_ref2.tolist()
   np.testing.assert_allclose(lp.cpu().numpy(), lp_ref2.numpy(), atol=2e-5)
+
+
+@pytest.mark.parametrize("segmented", [False, True])
+def test_sample_topk_with_massive_ties(gpu, segmented):
+  """Logits with only a handful of distinct values: thousands of elements tie at the k-th value,
+  the k lowest indices among them must be taken (jax.lax.top_k order); in the segmented kernel
+  this is the exact radix-select path behind the pivot shortcut."""
+  from tunix_amd import ops
+  M, V, k, top_p, temp, step = 8, 50000, 50, 0.95, 1.0, 3
+  g = torch.Generator().manual_seed(61)
+  logits = torch.round(torch.randn(M, V, generator=g)).float()     # values in {-4 .. 4}
+  logits[0] = 1.0                                                   # a constant row
+  key = TF.prng_key(99)
+  tok_ref, lp_ref = SR.sample_top_p(logits, TF.fold_in(key, step), temp, top_p, k)
+  ids = torch.empty(M, dtype=torch.int32, device=gpu)
+  lp = torch.empty(M, dtype=torch.float32, device=gpu)
+  stp = torch.tensor([step], dtype=torch.int32, device=gpu)
+  ws = torch.empty(ops.sample_topk_ws_bytes(M, V, k) // 4, dtype=torch.float32, device=gpu) if segmented else None
+  ops.sample_topk(logits.to(gpu), k, top_p, temp, (int(key[0]), int(key[1])), 0, stp, ws, ids, lp)
+  torch.cuda.synchronize()
+  assert ids.cpu().long().tolist() == tok_ref.tolist()
+  np.testing.assert_allclose(lp.cpu().numpy(), lp_ref.numpy(), atol=2e-5)
 
 
 def test_sample_commit_and_fill(gpu):

@@ -1,5 +1,7 @@
 // Top-k / top-p sampling from materialised fp32 logits with the threefry2x32 bit stream of
 // jax.random (fold_in -> random_bits -> uniform -> gumbel -> argmax), one work-group per row.
+#include <mutex>
+
 #include "common.h"
 
 namespace {
@@ -276,14 +278,320 @@ __global__ __launch_bounds__(NTH) void sample_topk_kernel(const float* logits, i
   }
 }
 
+
+// ---- top-k in two launches ---------------------------------------------------------------
+// One work-group per row makes nine passes over half a megabyte through a single compute
+// unit.  With a workspace the row is cut into segments of at most kSegElems logits, one
+// work-group each: the segment is read from HBM once into LDS, reduced to (max, sum of
+// exponentials) and to its own k best candidates (same order: larger value, then lower index),
+// and a second kernel merges the segments' candidates and statistics and draws the token.  The
+// k best of the row are among the k best of the segments, ties included, so the result is the
+// one of the single-launch kernel.
+constexpr int kSegElems = 16384;   // 64 KiB of LDS
+constexpr int kSegThreads = 512;
+constexpr int kListMax = 2048;     // candidates at or above the pivot kept for the exact sort
+
+__global__ __launch_bounds__(kSegThreads) void topk_segment_kernel(
+    const float* logits, int64_t V, int k, int seg_len, float temperature, const int32_t* forbidden,
+    int n_forbidden, float* ws) {
+  extern __shared__ __align__(16) float seg[];   // [seg_len]
+  __shared__ uint32_t hist[256];
+  __shared__ float red_f[kSegThreads / 64];
+  __shared__ uint32_t wave_cnt[kSegThreads / 64];
+  __shared__ uint32_t s_sel, s_rem, s_cnt, s_base;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int nseg = gridDim.x, sidx = blockIdx.x;
+  const int64_t row = blockIdx.y;
+  const int64_t v0 = (int64_t)sidx * seg_len;
+  const int n = (int)max((int64_t)0, min((int64_t)seg_len, V - v0));
+  const float* lr = logits + row * V + v0;
+  float* stats = ws + (row * nseg + sidx) * (2 + 2 * (int64_t)k);
+  float* cand_v = stats + 2;
+  int* cand_i = reinterpret_cast<int*>(stats + 2 + k);
+
+  // the segment, scaled and masked, into LDS (16-byte loads where the row allows them)
+  float mx = kNegInf;
+  const bool vec = ((reinterpret_cast<uintptr_t>(lr) & 15) == 0);
+  for (int i = tid * 4; i < n; i += kSegThreads * 4) {
+    float x[4];
+    if (vec && i + 4 <= n) {
+      const f32x4 q = *reinterpret_cast<const f32x4*>(lr + i);
+      x[0] = q[0]; x[1] = q[1]; x[2] = q[2]; x[3] = q[3];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) x[j] = i + j < n ? lr[i + j] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (i + j >= n) break;
+      float y = __fdiv_rn(x[j], temperature);
+      for (int f = 0; f < n_forbidden; ++f)
+        if (forbidden[f] == (int32_t)(v0 + i + j)) y = kNegInf;
+      seg[i + j] = y;
+      mx = fmaxf(mx, y);
+    }
+  }
+  // maximum and sum of exponentials of the segment
+  mx = wave_max(mx);
+  __syncthreads();
+  if (lane == 0) red_f[wave] = mx;
+  __syncthreads();
+  mx = red_f[0];
+  for (int w = 1; w < kSegThreads / 64; ++w) mx = fmaxf(mx, red_f[w]);
+  __syncthreads();
+  float se = 0.f;
+  if (mx != kNegInf)
+    for (int i = tid; i < n; i += kSegThreads) se += expf(seg[i] - mx);
+  se = wave_sum(se);
+  if (lane == 0) red_f[wave] = se;
+  __syncthreads();
+  if (tid == 0) {
+    float t = 0.f;
+    for (int w = 0; w < kSegThreads / 64; ++w) t += red_f[w];
+    stats[0] = mx;
+    stats[1] = t;
+  }
+  for (int i = tid; i < k; i += kSegThreads) {   // fewer than k elements: the rest never wins
+    cand_v[i] = kNegInf;
+    cand_i[i] = 0x7fffffff;
+  }
+  if (n <= k) {
+    for (int i = tid; i < n; i += kSegThreads) {
+      cand_v[i] = seg[i];
+      cand_i[i] = (int)(v0 + i);
+    }
+    return;
+  }
+  // Pivot: the k-th largest of the per-thread maxima (each over a strided subset) is a lower
+  // bound of the k-th largest element, so {x >= pivot} contains the k best including every tie at
+  // the k-th value; for all but adversarial data it holds between k and a few k elements, which
+  // are compacted and sorted.  (A histogram of the key bytes in LDS, the textbook radix select,
+  // serialises here: almost all logits share their exponent byte.)
+  {
+    __shared__ float pmax[kSegThreads];
+    __shared__ float lst_v[kListMax];
+    __shared__ int lst_i[kListMax];
+    float lm = kNegInf;
+    for (int i = tid; i < n; i += kSegThreads) lm = fmaxf(lm, seg[i]);
+    pmax[tid] = lm;
+    __syncthreads();
+    for (int size = 2; size <= kSegThreads; size <<= 1)      // bitonic, descending
+      for (int st = size >> 1; st > 0; st >>= 1) {
+        const int partner = tid ^ st;
+        if (partner > tid) {
+          const float x = pmax[tid], y = pmax[partner];
+          const bool up = (tid & size) == 0;
+          if (up != (x >= y)) {
+            pmax[tid] = y;
+            pmax[partner] = x;
+          }
+        }
+        __syncthreads();
+      }
+    const float pivot = pmax[k - 1];   // k <= kSegThreads is checked by the host
+    if (tid == 0) s_cnt = 0;
+    __syncthreads();
+    for (int i = tid; i < n; i += kSegThreads) {
+      const float x = seg[i];
+      if (x >= pivot) {
+        const uint32_t p = atomicAdd(&s_cnt, 1u);
+        if (p < kListMax) {
+          lst_v[p] = x;
+          lst_i[p] = (int)(v0 + i);
+        }
+      }
+    }
+    __syncthreads();
+    const int c = (int)s_cnt;
+    if (c <= kListMax) {
+      int m2 = 64;
+      while (m2 < c) m2 <<= 1;
+      for (int i = c + tid; i < m2; i += kSegThreads) {
+        lst_v[i] = kNegInf;
+        lst_i[i] = 0x7fffffff;
+      }
+      __syncthreads();
+      for (int size = 2; size <= m2; size <<= 1)             // larger value, then lower index
+        for (int st = size >> 1; st > 0; st >>= 1) {
+          for (int t = tid; t < m2; t += kSegThreads) {
+            const int partner = t ^ st;
+            if (partner > t) {
+              ArgMax x{lst_v[t], lst_i[t]}, y{lst_v[partner], lst_i[partner]};
+              const bool x_first = (x.v > y.v) || (x.v == y.v && x.i < y.i);
+              const bool up = (t & size) == 0;
+              if (up != x_first) {
+                lst_v[t] = y.v; lst_i[t] = y.i;
+                lst_v[partner] = x.v; lst_i[partner] = x.i;
+              }
+            }
+          }
+          __syncthreads();
+        }
+      for (int i = tid; i < k; i += kSegThreads) {
+        cand_v[i] = lst_v[i];
+        cand_i[i] = lst_i[i];
+      }
+      return;
+    }
+  }
+  // more than kListMax elements at or above the pivot (many equal values): exact radix select
+  uint32_t prefix = 0, mask = 0;
+  if (tid == 0) s_rem = (uint32_t)k;
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    if (tid < 256) hist[tid] = 0;
+    __syncthreads();
+    for (int i = tid; i < n; i += kSegThreads) {
+      const uint32_t kk = order_key(seg[i]);
+      if ((kk & mask) == prefix) atomicAdd(&hist[(kk >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    if (tid == 0) {
+      uint32_t cum = 0, rem = s_rem;
+      int b = 255;
+      for (; b > 0; --b) {
+        if (cum + hist[b] >= rem) break;
+        cum += hist[b];
+      }
+      s_sel = (uint32_t)b;
+      s_rem = rem - cum;
+    }
+    __syncthreads();
+    prefix |= s_sel << shift;
+    mask |= 0xffu << shift;
+  }
+  const uint32_t thr = prefix;
+  const uint32_t r_eq = s_rem;  // how many elements equal to the threshold are taken
+  if (tid == 0) {
+    s_cnt = 0;
+    s_base = 0;
+  }
+  __syncthreads();
+  for (int i = tid; i < n; i += kSegThreads) {   // above the threshold: any order
+    const float x = seg[i];
+    if (order_key(x) > thr) {
+      const uint32_t p = atomicAdd(&s_cnt, 1u);
+      cand_v[p] = x;
+      cand_i[p] = (int)(v0 + i);
+    }
+  }
+  __syncthreads();
+  const uint32_t n_gt = s_cnt;
+  for (int i0 = 0; i0 < n; i0 += kSegThreads) {   // equal to it: the r_eq lowest indices
+    if (s_base >= r_eq) break;
+    const int i = i0 + tid;
+    const bool eq = i < n && order_key(seg[i]) == thr;
+    const uint64_t bal = __ballot(eq);
+    const uint32_t before = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_cnt[wave] = (uint32_t)__popcll(bal);
+    __syncthreads();
+    uint32_t woff = 0, tot = 0;
+    for (int w = 0; w < kSegThreads / 64; ++w) {
+      if (w < wave) woff += wave_cnt[w];
+      tot += wave_cnt[w];
+    }
+    const uint32_t pos = s_base + woff + before;
+    if (eq && pos < r_eq) {
+      cand_v[n_gt + pos] = seg[i];
+      cand_i[n_gt + pos] = (int)(v0 + i);
+    }
+    __syncthreads();
+    if (tid == 0) s_base += tot;
+    __syncthreads();
+  }
+}
+
+__global__ __launch_bounds__(NTH) void topk_merge_sample_kernel(
+    const float* ws, int nseg, int k, float top_p, uint32_t key0, uint32_t key1, int variant,
+    const int32_t* step_ptr, int64_t M, int32_t* ids_out, float* logp_out) {
+  __shared__ float cval[NTH];
+  __shared__ int cidx[NTH];
+  __shared__ ArgMax red_am[NTH / 64];
+  __shared__ float red_f[NTH / 64];
+  __shared__ float prob[NTH];
+  __shared__ float excl[NTH];
+  const int tid = threadIdx.x;
+  const int64_t row = blockIdx.x;
+  const int64_t stride = 2 + 2 * (int64_t)k;
+  const float* rw = ws + row * nseg * stride;
+  uint32_t ks0 = 0u, ks1 = (uint32_t)(*step_ptr);
+  threefry2x32(key0, key1, ks0, ks1);
+  // log-sum-exp of the row from the segments' (max, sum)
+  float gm = kNegInf;
+  for (int sg = 0; sg < nseg; ++sg) gm = fmaxf(gm, rw[sg * stride]);
+  float se = 0.f;
+  for (int sg = 0; sg < nseg; ++sg) {
+    const float m = rw[sg * stride];
+    if (m != kNegInf) se += rw[sg * stride + 1] * expf(m - gm);
+  }
+  const float lse = gm + logf(se);
+  // all candidates, best first
+  cval[tid] = kNegInf;
+  cidx[tid] = 0x7fffffff;
+  if (tid < nseg * k) {
+    const int sg = tid / k, j = tid % k;
+    cval[tid] = rw[sg * stride + 2 + j];
+    cidx[tid] = reinterpret_cast<const int*>(rw + sg * stride + 2 + k)[j];
+  }
+  __syncthreads();
+  int m2 = 64;   // sort only as many slots as there are candidates (the rest is -inf padding)
+  while (m2 < nseg * k) m2 <<= 1;
+  for (int size = 2; size <= m2; size <<= 1) {
+    for (int st = size >> 1; st > 0; st >>= 1) {
+      const int partner = tid ^ st;
+      if (tid < m2 && partner > tid) {
+        ArgMax a{cval[tid], cidx[tid]}, b{cval[partner], cidx[partner]};
+        const bool a_first = (a.v > b.v) || (a.v == b.v && a.i < b.i);
+        const bool up = (tid & size) == 0;
+        if (up != a_first) {
+          cval[tid] = b.v; cidx[tid] = b.i;
+          cval[partner] = a.v; cidx[partner] = a.i;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  // softmax over the k sorted logits, top-p cut, gumbel arg-max (as in sample_topk_kernel)
+  const float mx = cval[0];
+  float e = tid < k ? expf(cval[tid] - mx) : 0.f;
+  const float tot = block_sum_f(e, red_f);
+  prob[tid] = e / tot;
+  __syncthreads();
+  if (tid == 0) {
+    float c = 0.f;
+    for (int j = 0; j < k; ++j) {
+      c += prob[j];
+      excl[j] = c - prob[j];
+    }
+  }
+  __syncthreads();
+  ArgMax g;
+  g.v = kNegInf;
+  g.i = 0x7fffffff;
+  if (tid < k) {
+    const float lgt = excl[tid] > top_p ? kNegInf : cval[tid];
+    g.v = lgt + gumbel_from_bits(random_bits(ks0, ks1, (uint64_t)(row * k + tid), (uint64_t)(M * k), variant));
+    g.i = tid;
+  }
+  g = block_argmax(g, red_am);
+  if (tid == 0) {
+    ids_out[row] = cidx[g.i];
+    if (logp_out) logp_out[row] = cval[g.i] - lse;
+  }
+}
+
 }  // namespace
+
+extern "C" size_t tnx_sample_topk_ws_bytes(int64_t M, int64_t V, int k) {
+  if (M <= 0 || V <= 0 || k <= 0) return 0;
+  return (size_t)(M * cdiv(V, kSegElems) * (2 + 2 * (int64_t)k)) * sizeof(float);
+}
 
 extern "C" int tnx_sample_topk(void* stream, const float* logits, int64_t M, int64_t V, int k,
                                float top_p, float temperature, uint32_t key0, uint32_t key1,
                                int rng_variant, const int32_t* forbidden, int n_forbidden,
                                const int32_t* step_ptr, float* ws, int32_t* ids_out,
                                float* logp_out) {
-  (void)ws;
   TNX_REQUIRE(logits && step_ptr && ids_out, "sample_topk: null pointer");
   TNX_REQUIRE(M > 0 && V > 0 && V < (1ll << 31), "sample_topk: bad shape");
   TNX_REQUIRE(rng_variant == 0 || rng_variant == 1, "sample_topk: rng_variant must be 0 or 1");
@@ -296,6 +604,26 @@ extern "C" int tnx_sample_topk(void* stream, const float* logits, int64_t M, int
     k = 0;
   }
   TNX_REQUIRE(k <= NTH, "sample_topk: top_k=%d exceeds %d", k, NTH);
+  const int nseg = (int)cdiv(V, kSegElems);
+  if (ws && k > 0 && k <= kSegThreads && (int64_t)nseg * k <= NTH) {
+    // segments of equal length, a multiple of 4 so that aligned rows stay aligned
+    const int seg_len = (int)(cdiv(cdiv(V, nseg), 4) * 4);
+    static std::once_flag once;
+    static hipError_t attr_rc = hipSuccess;
+    std::call_once(once, [] {
+      attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(topk_segment_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, kSegElems * 4);
+    });
+    TNX_REQUIRE(attr_rc == hipSuccess, "sample_topk: cannot raise the dynamic LDS limit");
+    hipLaunchKernelGGL(topk_segment_kernel, dim3((unsigned)nseg, (unsigned)M), dim3(kSegThreads),
+                       (size_t)seg_len * 4, as_stream(stream), logits, V, k, seg_len, temperature, forbidden,
+                       forbidden ? n_forbidden : 0, ws);
+    TNX_CHECK_LAUNCH("sample_topk (segments)");
+    hipLaunchKernelGGL(topk_merge_sample_kernel, dim3((unsigned)M), dim3(NTH), 0, as_stream(stream), ws, nseg,
+                       k, top_p, key0, key1, rng_variant, step_ptr, M, ids_out, logp_out);
+    TNX_CHECK_LAUNCH("sample_topk (merge)");
+    return TNX_OK;
+  }
   hipLaunchKernelGGL(sample_topk_kernel, dim3((unsigned)M), dim3(NTH), 0, as_stream(stream), logits,
                      V, k, top_p, key0, key1, rng_variant, step_ptr, M, temperature, forbidden,
                      forbidden ? n_forbidden : 0, ids_out, logp_out);

@@ -216,7 +216,9 @@ class Sampler:
       no_topk = top_k is None or top_k <= 0
       k = 0 if no_topk else int(min(top_k, cfg.vocab_size))
       mode.update(name="top_p", temperature=float(temperature), top_p=float(top_p), top_k=k,
-                  key=key, ws=torch.empty(B * 2 * max(k, 1), dtype=torch.float32, device=dev),
+                  key=key,
+                  ws=torch.empty(max(ops.sample_topk_ws_bytes(B, model.cfg.vocab_size, k) // 4, 1),
+                                 dtype=torch.float32, device=dev),
                   ids=torch.empty(B, dtype=torch.int32, device=dev),
                   logp=torch.empty(B, dtype=torch.float32, device=dev))
     need_logits = return_logits or mode["name"] == "top_p"
