@@ -291,7 +291,7 @@ int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* h_desc);
  * 0 = original (counter array split in halves).  k <= 0 or k >= V with top_p >= 1 draws from
  * the whole vocabulary.  logp_out = full-vocabulary log-softmax at the drawn id (:141-144).
  * k <= 1024.  With a workspace `ws` of tnx_sample_topk_ws_bytes(M, V, k) bytes (and
- * ceil(V / 16384) * k <= 1024) the row is processed in segments by many work-groups and a merging
+ * ceil(V / 8192) * k <= 4096, k <= 512) the row is processed in segments by many work-groups and a merging
  * launch; with ws = NULL one work-group per row does everything.  Both give the same result. */
 size_t tnx_sample_topk_ws_bytes(int64_t M, int64_t V, int k);
 int tnx_sample_topk(void* stream, const float* logits, int64_t M, int64_t V, int k, float top_p,

@@ -440,7 +440,7 @@ def test_sample_topk_matches_oracle(gpu, k, top_p, variant, segmented, V):
   ws = None
   if segmented:
     nb = ops.sample_topk_ws_bytes(M, V, k)
-    assert (nb > 0) == (k > 0)
+    assert nb > 0
     ws = torch.empty(max(nb // 4, 1), dtype=torch.float32, device=gpu)
   ops.sample_topk(logits.to(gpu), k, top_p, temp, (int(key[0]), int(key[1])), variant, stp, ws, ids, lp)
   torch.cuda.synchronize()

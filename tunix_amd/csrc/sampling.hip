@@ -287,13 +287,15 @@ __global__ __launch_bounds__(NTH) void sample_topk_kernel(const float* logits, i
 // and a second kernel merges the segments' candidates and statistics and draws the token.  The
 // k best of the row are among the k best of the segments, ties included, so the result is the
 // one of the single-launch kernel.
-constexpr int kSegElems = 16384;   // 64 KiB of LDS
+constexpr int kSegElems = 8192;    // 32 KiB of LDS: three work-groups per compute unit
 constexpr int kSegThreads = 512;
-constexpr int kListMax = 2048;     // candidates at or above the pivot kept for the exact sort
+constexpr int kListMax = 2048;     // candidates at or above the pivot kept for the exact ranking
+constexpr int kMergeMax = 4096;    // candidates (segments x k) the merging launch can rank
 
 __global__ __launch_bounds__(kSegThreads) void topk_segment_kernel(
     const float* logits, int64_t V, int k, int seg_len, float temperature, const int32_t* forbidden,
-    int n_forbidden, float* ws) {
+    int n_forbidden, float* ws, uint32_t key0, uint32_t key1, int variant, const int32_t* step_ptr,
+    int64_t M) {
   extern __shared__ __align__(16) float seg[];   // [seg_len]
   __shared__ uint32_t hist[256];
   __shared__ float red_f[kSegThreads / 64];
@@ -305,7 +307,7 @@ __global__ __launch_bounds__(kSegThreads) void topk_segment_kernel(
   const int64_t v0 = (int64_t)sidx * seg_len;
   const int n = (int)max((int64_t)0, min((int64_t)seg_len, V - v0));
   const float* lr = logits + row * V + v0;
-  float* stats = ws + (row * nseg + sidx) * (2 + 2 * (int64_t)k);
+  float* stats = ws + (row * nseg + sidx) * (k > 0 ? 2 + 2 * (int64_t)k : 5);
   float* cand_v = stats + 2;
   int* cand_i = reinterpret_cast<int*>(stats + 2 + k);
 
@@ -351,6 +353,38 @@ __global__ __launch_bounds__(kSegThreads) void topk_segment_kernel(
     stats[0] = mx;
     stats[1] = t;
   }
+  if (k <= 0) {
+    // categorical over the whole vocabulary: this segment's arg-max of logit + gumbel noise
+    // (noise of element v of the row: counter row * V + v of M * V, as one draw over [M, V])
+    __shared__ ArgMax red_g[kSegThreads / 64];
+    uint32_t ks0 = 0u, ks1 = (uint32_t)(*step_ptr);
+    threefry2x32(key0, key1, ks0, ks1);
+    ArgMax g;
+    g.v = kNegInf;
+    g.i = 0x7fffffff;
+    for (int i = tid; i < n; i += kSegThreads) {
+      ArgMax c;
+      c.v = seg[i] + gumbel_from_bits(random_bits(ks0, ks1, (uint64_t)(row * V + v0 + i), (uint64_t)(M * V), variant));
+      c.i = (int)(v0 + i);
+      g = better(g, c);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      ArgMax y;
+      y.v = __shfl_xor(g.v, o, 64);
+      y.i = __shfl_xor(g.i, o, 64);
+      g = better(g, y);
+    }
+    if (lane == 0) red_g[wave] = g;
+    __syncthreads();
+    if (tid == 0) {
+      for (int w = 1; w < kSegThreads / 64; ++w) g = better(g, red_g[w]);
+      stats[2] = g.v;
+      reinterpret_cast<int*>(stats)[3] = g.i;
+      stats[4] = g.i == 0x7fffffff ? kNegInf : seg[g.i - (int)v0];
+    }
+    return;
+  }
   for (int i = tid; i < k; i += kSegThreads) {   // fewer than k elements: the rest never wins
     cand_v[i] = kNegInf;
     cand_i[i] = 0x7fffffff;
@@ -362,35 +396,34 @@ __global__ __launch_bounds__(kSegThreads) void topk_segment_kernel(
     }
     return;
   }
-  // Pivot: the k-th largest of the per-thread maxima (each over a strided subset) is a lower
-  // bound of the k-th largest element, so {x >= pivot} contains the k best including every tie at
-  // the k-th value; for all but adversarial data it holds between k and a few k elements, which
-  // are compacted and sorted.  (A histogram of the key bytes in LDS, the textbook radix select,
+  // Pivot: every wave sorts its 64 per-thread maxima (each over a strided subset) and offers its
+  // j-th largest, j = ceil(k / waves); at least waves * j >= k elements lie at or above the
+  // smallest offer, so {x >= pivot} contains the k best including every tie at the k-th value.
+  // For all but adversarial data that set holds a few k elements, which are compacted and
+  // ranked by counting.  (A histogram of the key bytes in LDS, the textbook radix select,
   // serialises here: almost all logits share their exponent byte.)
   {
-    __shared__ float pmax[kSegThreads];
     __shared__ float lst_v[kListMax];
     __shared__ int lst_i[kListMax];
+    constexpr int kWaves = kSegThreads / 64;
     float lm = kNegInf;
     for (int i = tid; i < n; i += kSegThreads) lm = fmaxf(lm, seg[i]);
-    pmax[tid] = lm;
-    __syncthreads();
-    for (int size = 2; size <= kSegThreads; size <<= 1)      // bitonic, descending
+#pragma unroll
+    for (int size = 2; size <= 64; size <<= 1)               // bitonic in the wave, descending
+#pragma unroll
       for (int st = size >> 1; st > 0; st >>= 1) {
-        const int partner = tid ^ st;
-        if (partner > tid) {
-          const float x = pmax[tid], y = pmax[partner];
-          const bool up = (tid & size) == 0;
-          if (up != (x >= y)) {
-            pmax[tid] = y;
-            pmax[partner] = x;
-          }
-        }
-        __syncthreads();
+        const float y = __shfl_xor(lm, st, 64);
+        const bool up = (lane & size) == 0, low = (lane & st) == 0;
+        lm = (up == low) ? fmaxf(lm, y) : fminf(lm, y);
       }
-    const float pivot = pmax[k - 1];   // k <= kSegThreads is checked by the host
+    const int j = (k + kWaves - 1) / kWaves;                 // <= 64: k <= kSegThreads
+    const float offer = __shfl(lm, j - 1, 64);
+    __syncthreads();
+    if (lane == 0) red_f[wave] = offer;
     if (tid == 0) s_cnt = 0;
     __syncthreads();
+    float pivot = red_f[0];
+    for (int w = 1; w < kWaves; ++w) pivot = fminf(pivot, red_f[w]);
     for (int i = tid; i < n; i += kSegThreads) {
       const float x = seg[i];
       if (x >= pivot) {
@@ -404,32 +437,18 @@ __global__ __launch_bounds__(kSegThreads) void topk_segment_kernel(
     __syncthreads();
     const int c = (int)s_cnt;
     if (c <= kListMax) {
-      int m2 = 64;
-      while (m2 < c) m2 <<= 1;
-      for (int i = c + tid; i < m2; i += kSegThreads) {
-        lst_v[i] = kNegInf;
-        lst_i[i] = 0x7fffffff;
-      }
-      __syncthreads();
-      for (int size = 2; size <= m2; size <<= 1)             // larger value, then lower index
-        for (int st = size >> 1; st > 0; st >>= 1) {
-          for (int t = tid; t < m2; t += kSegThreads) {
-            const int partner = t ^ st;
-            if (partner > t) {
-              ArgMax x{lst_v[t], lst_i[t]}, y{lst_v[partner], lst_i[partner]};
-              const bool x_first = (x.v > y.v) || (x.v == y.v && x.i < y.i);
-              const bool up = (t & size) == 0;
-              if (up != x_first) {
-                lst_v[t] = y.v; lst_i[t] = y.i;
-                lst_v[partner] = x.v; lst_i[partner] = x.i;
-              }
-            }
-          }
-          __syncthreads();
+      // rank = number of better candidates (larger value, then lower index): a strict order
+      for (int t = tid; t < c; t += kSegThreads) {
+        const ArgMax me{lst_v[t], lst_i[t]};
+        int r = 0;
+        for (int q = 0; q < c; ++q) {
+          const float v = lst_v[q];
+          r += (v > me.v || (v == me.v && lst_i[q] < me.i)) ? 1 : 0;
         }
-      for (int i = tid; i < k; i += kSegThreads) {
-        cand_v[i] = lst_v[i];
-        cand_i[i] = lst_i[i];
+        if (r < k) {
+          cand_v[r] = me.v;
+          cand_i[r] = me.i;
+        }
       }
       return;
     }
@@ -506,13 +525,15 @@ __global__ __launch_bounds__(NTH) void topk_merge_sample_kernel(
     const int32_t* step_ptr, int64_t M, int32_t* ids_out, float* logp_out) {
   __shared__ float cval[NTH];
   __shared__ int cidx[NTH];
+  __shared__ float mval[kMergeMax];
+  __shared__ int midx[kMergeMax];
   __shared__ ArgMax red_am[NTH / 64];
   __shared__ float red_f[NTH / 64];
   __shared__ float prob[NTH];
   __shared__ float excl[NTH];
   const int tid = threadIdx.x;
   const int64_t row = blockIdx.x;
-  const int64_t stride = 2 + 2 * (int64_t)k;
+  const int64_t stride = k > 0 ? 2 + 2 * (int64_t)k : 5;
   const float* rw = ws + row * nseg * stride;
   uint32_t ks0 = 0u, ks1 = (uint32_t)(*step_ptr);
   threefry2x32(key0, key1, ks0, ks1);
@@ -525,32 +546,56 @@ __global__ __launch_bounds__(NTH) void topk_merge_sample_kernel(
     if (m != kNegInf) se += rw[sg * stride + 1] * expf(m - gm);
   }
   const float lse = gm + logf(se);
-  // all candidates, best first
-  cval[tid] = kNegInf;
-  cidx[tid] = 0x7fffffff;
-  if (tid < nseg * k) {
-    const int sg = tid / k, j = tid % k;
-    cval[tid] = rw[sg * stride + 2 + j];
-    cidx[tid] = reinterpret_cast<const int*>(rw + sg * stride + 2 + k)[j];
+  if (k <= 0) {  // whole-vocabulary draw: best (logit + noise) over the segments
+    if (tid == 0) {
+      ArgMax g;
+      g.v = kNegInf;
+      g.i = 0x7fffffff;
+      float lgt = kNegInf;
+      for (int sg = 0; sg < nseg; ++sg) {
+        ArgMax c;
+        c.v = rw[sg * stride + 2];
+        c.i = reinterpret_cast<const int*>(rw + sg * stride)[3];
+        const ArgMax w = better(g, c);
+        if (w.i != g.i) lgt = rw[sg * stride + 4];
+        g = w;
+      }
+      ids_out[row] = g.i;
+      if (logp_out) logp_out[row] = lgt - lse;
+    }
+    return;
+  }
+  // all candidates into LDS, bitonic sort (best first: larger value, then lower index); only as
+  // many slots as there are candidates take part, padded to a power of two with -inf
+  const int nc = nseg * k;
+  int m2 = 64;
+  while (m2 < nc) m2 <<= 1;
+  for (int t = tid; t < m2; t += NTH) {
+    const int sg = t / k, j = t % k;
+    mval[t] = t < nc ? rw[sg * stride + 2 + j] : kNegInf;
+    midx[t] = t < nc ? reinterpret_cast<const int*>(rw + sg * stride + 2 + k)[j] : 0x7fffffff;
   }
   __syncthreads();
-  int m2 = 64;   // sort only as many slots as there are candidates (the rest is -inf padding)
-  while (m2 < nseg * k) m2 <<= 1;
   for (int size = 2; size <= m2; size <<= 1) {
     for (int st = size >> 1; st > 0; st >>= 1) {
-      const int partner = tid ^ st;
-      if (tid < m2 && partner > tid) {
-        ArgMax a{cval[tid], cidx[tid]}, b{cval[partner], cidx[partner]};
-        const bool a_first = (a.v > b.v) || (a.v == b.v && a.i < b.i);
-        const bool up = (tid & size) == 0;
-        if (up != a_first) {
-          cval[tid] = b.v; cidx[tid] = b.i;
-          cval[partner] = a.v; cidx[partner] = a.i;
+      for (int t = tid; t < m2; t += NTH) {
+        const int partner = t ^ st;
+        if (partner > t) {
+          ArgMax x{mval[t], midx[t]}, y{mval[partner], midx[partner]};
+          const bool x_first = (x.v > y.v) || (x.v == y.v && x.i < y.i);
+          const bool up = (t & size) == 0;
+          if (up != x_first) {
+            mval[t] = y.v; midx[t] = y.i;
+            mval[partner] = x.v; midx[partner] = x.i;
+          }
         }
       }
       __syncthreads();
     }
   }
+  cval[tid] = tid < m2 ? mval[tid] : kNegInf;
+  cidx[tid] = tid < m2 ? midx[tid] : 0x7fffffff;
+  __syncthreads();
   // softmax over the k sorted logits, top-p cut, gumbel arg-max (as in sample_topk_kernel)
   const float mx = cval[0];
   float e = tid < k ? expf(cval[tid] - mx) : 0.f;
@@ -583,8 +628,9 @@ __global__ __launch_bounds__(NTH) void topk_merge_sample_kernel(
 }  // namespace
 
 extern "C" size_t tnx_sample_topk_ws_bytes(int64_t M, int64_t V, int k) {
-  if (M <= 0 || V <= 0 || k <= 0) return 0;
-  return (size_t)(M * cdiv(V, kSegElems) * (2 + 2 * (int64_t)k)) * sizeof(float);
+  if (M <= 0 || V <= 0) return 0;
+  if (k <= 0 || k >= V) k = 0;  // whole-vocabulary draw: (max, sum, noisy best, its id, its logit)
+  return (size_t)(M * cdiv(V, kSegElems) * (k > 0 ? 2 + 2 * (int64_t)k : 5)) * sizeof(float);
 }
 
 extern "C" int tnx_sample_topk(void* stream, const float* logits, int64_t M, int64_t V, int k,
@@ -605,7 +651,7 @@ extern "C" int tnx_sample_topk(void* stream, const float* logits, int64_t M, int
   }
   TNX_REQUIRE(k <= NTH, "sample_topk: top_k=%d exceeds %d", k, NTH);
   const int nseg = (int)cdiv(V, kSegElems);
-  if (ws && k > 0 && k <= kSegThreads && (int64_t)nseg * k <= NTH) {
+  if (ws && (k == 0 || (k <= kSegThreads && (int64_t)nseg * k <= kMergeMax))) {
     // segments of equal length, a multiple of 4 so that aligned rows stay aligned
     const int seg_len = (int)(cdiv(cdiv(V, nseg), 4) * 4);
     static std::once_flag once;
@@ -617,7 +663,7 @@ extern "C" int tnx_sample_topk(void* stream, const float* logits, int64_t M, int
     TNX_REQUIRE(attr_rc == hipSuccess, "sample_topk: cannot raise the dynamic LDS limit");
     hipLaunchKernelGGL(topk_segment_kernel, dim3((unsigned)nseg, (unsigned)M), dim3(kSegThreads),
                        (size_t)seg_len * 4, as_stream(stream), logits, V, k, seg_len, temperature, forbidden,
-                       forbidden ? n_forbidden : 0, ws);
+                       forbidden ? n_forbidden : 0, ws, key0, key1, rng_variant, step_ptr, M);
     TNX_CHECK_LAUNCH("sample_topk (segments)");
     hipLaunchKernelGGL(topk_merge_sample_kernel, dim3((unsigned)M), dim3(NTH), 0, as_stream(stream), ws, nseg,
                        k, top_p, key0, key1, rng_variant, step_ptr, M, ids_out, logp_out);
