@@ -292,8 +292,12 @@ int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* h_desc);
  * the whole vocabulary.  logp_out = full-vocabulary log-softmax at the drawn id (:141-144).
  * k <= 1024.  With a workspace `ws` of tnx_sample_topk_ws_bytes(M, V, k) bytes (and
  * ceil(V / 8192) * k <= 4096, k <= 512) the row is processed in segments by many work-groups and a merging
- * launch; with ws = NULL one work-group per row does everything.  Both give the same result. */
+ * launch; with ws = NULL one work-group per row does everything.  Both give the same result.
+ * top_p < 1 without top_k (k <= 0) sorts every row completely, as the reference does with
+ * jax.lax.top_k(k = V) (:126-127), and needs ws of tnx_sample_fullsort_ws_bytes(M, V) bytes
+ * (four [M,V] arrays plus the sort's scratch; M * V < 2^31). */
 size_t tnx_sample_topk_ws_bytes(int64_t M, int64_t V, int k);
+size_t tnx_sample_fullsort_ws_bytes(int64_t M, int64_t V);
 int tnx_sample_topk(void* stream, const float* logits, int64_t M, int64_t V, int k, float top_p,
                     float temperature, uint32_t key0, uint32_t key1, int rng_variant,
                     const int32_t* forbidden, int n_forbidden, const int32_t* step_ptr, float* ws,

@@ -480,6 +480,32 @@ def test_sample_topk_with_massive_ties(gpu, segmented):
   np.testing.assert_allclose(lp.cpu().numpy(), lp_ref.numpy(), atol=2e-5)
 
 
+@pytest.mark.parametrize("V,top_p,variant", [(3000, 0.7, 0), (40001, 0.9, 0), (40001, 0.3, 1)])
+def test_sample_top_p_over_the_whole_vocabulary(gpu, V, top_p, variant):
+  """top_p < 1 with top_k absent: the reference sorts the whole row (sampler.py:126-127); ids
+  against the oracle exactly, log-probabilities to 2e-5; without a workspace the call is refused."""
+  from tunix_amd import ops
+  from tunix_amd._lib import TnxError
+  M, temp, step = 16, 0.8, 11
+  g = torch.Generator().manual_seed(62)
+  logits = (torch.randn(M, V, generator=g) * 3).float()
+  logits[:, 17] = logits[:, 29]
+  key = TF.prng_key(4321)
+  tok_ref, lp_ref = SR.sample_top_p(logits, TF.fold_in(key, step), temp, top_p, None, partitionable=bool(variant))
+  ids = torch.empty(M, dtype=torch.int32, device=gpu)
+  lp = torch.empty(M, dtype=torch.float32, device=gpu)
+  stp = torch.tensor([step], dtype=torch.int32, device=gpu)
+  nb = ops.sample_fullsort_ws_bytes(M, V)
+  assert nb >= 4 * M * V * 4
+  ws = torch.empty(nb // 4, dtype=torch.float32, device=gpu)
+  ops.sample_topk(logits.to(gpu), 0, top_p, temp, (int(key[0]), int(key[1])), variant, stp, ws, ids, lp)
+  torch.cuda.synchronize()
+  assert ids.cpu().long().tolist() == tok_ref.tolist()
+  np.testing.assert_allclose(lp.cpu().numpy(), lp_ref.numpy(), atol=2e-5)
+  with pytest.raises((TnxError, ValueError), match="workspace"):
+    ops.sample_topk(logits.to(gpu), 0, top_p, temp, (int(key[0]), int(key[1])), variant, stp, None, ids, lp)
+
+
 def test_sample_commit_and_fill(gpu):
   from tunix_amd import ops
   B, Ld = 5, 12

@@ -159,8 +159,10 @@ def test_sampler_contract(tiny, gpu):
     sampler(["5"], 2, beam_size=2)
 
 
-def test_top_p_sampling_against_oracle(tiny, gpu):
-  """temperature / top-k / top-p.  The draw depends on the RANK of every candidate (the noise is
+@pytest.mark.parametrize("top_k,top_p", [(50, 0.95), (None, 0.9), (None, 1.0)])
+def test_top_p_sampling_against_oracle(tiny, gpu, top_k, top_p):
+  """temperature / top-k / top-p, top-p over the whole vocabulary (no top-k) and the plain
+  categorical draw (the reference's default rollout configuration: top_p 1.0, no top-k).  The draw depends on the RANK of every candidate (the noise is
   indexed by sorted position), so one bf16 ulp in one logit re-deals the noise: ids are checked
   exactly against the oracle's draw from the logits the GPU itself produced, and those logits
   against the teacher-forced oracle within bf16 resolution."""
@@ -172,7 +174,7 @@ def test_top_p_sampling_against_oracle(tiny, gpu):
   tok = IdTokenizer(cfg.vocab_size, pad_id=0, eos_id=1)
   sampler = Sampler(model, tok, CacheConfig(P + T, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim))
   prompts = _prompts(B, P, cfg.vocab_size, 99, ragged=False)
-  temp, top_k, top_p = 0.8, 50, 0.95
+  temp = 0.8
   out = sampler(prompts, T, max_prompt_length=P, temperature=temp, top_p=top_p, top_k=top_k, seed=42,
                 return_logprobs=True, return_logits=True, eos_tokens=[-1])
   tb = sampler._last_state.token_buffer.cpu().numpy()

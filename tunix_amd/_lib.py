@@ -101,6 +101,7 @@ SIGNATURES = {
     "tnx_lmhead_nblocks": (_i64, [_i64]),
     "tnx_lmhead_logp": (_i32, [_p, C.POINTER(LmHeadDesc)]),
     "tnx_sample_topk_ws_bytes": (C.c_size_t, [_i64, _i64, _i32]),
+    "tnx_sample_fullsort_ws_bytes": (C.c_size_t, [_i64, _i64]),
     "tnx_sample_topk": (_i32, [_p, _p, _i64, _i64, _i32, _f32, _f32, C.c_uint32, C.c_uint32, _i32,
                                _p, _i32, _p, _p, _p, _p]),
     "tnx_sample_commit": (_i32, [_p, _p, _p, _i64, _p, _i64, _p, _p, _p, _i32, _p]),

@@ -2,6 +2,8 @@
 // jax.random (fold_in -> random_bits -> uniform -> gumbel -> argmax), one work-group per row.
 #include <mutex>
 
+#include <rocprim/device/device_segmented_radix_sort.hpp>
+
 #include "common.h"
 
 namespace {
@@ -625,7 +627,101 @@ __global__ __launch_bounds__(NTH) void topk_merge_sample_kernel(
   }
 }
 
+
+// ---- top-p over the whole vocabulary (top_k absent, top_p < 1) ------------------------------
+// sample_top_p then sorts the full row (jax.lax.top_k with k = V): a stable segmented radix sort
+// (rocPRIM) of (scaled logit, id) pairs per row, then one work-group per row that soft-maxes the
+// sorted row, keeps the entries whose exclusive cumulative probability is <= top_p and draws
+// by Gumbel-max with the noise of the SORTED position, as jax.random.categorical over the
+// sorted logits does.
+__global__ void fullsort_prepare_kernel(const float* logits, int64_t M, int64_t V, float temperature,
+                                        const int32_t* forbidden, int n_forbidden, float* keys,
+                                        int* ids, int* offsets) {
+  const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (n <= M) offsets[n] = (int)(n * V);
+  if (n >= M * V) return;
+  const int v = (int)(n % V);
+  float y = __fdiv_rn(logits[n], temperature);
+  for (int f = 0; f < n_forbidden; ++f)
+    if (forbidden[f] == v) y = kNegInf;
+  keys[n] = y;
+  ids[n] = v;
+}
+
+__global__ __launch_bounds__(NTH) void fullsort_sample_kernel(const float* skeys, const int* sids, int64_t V,
+                                                              float top_p, uint32_t key0, uint32_t key1,
+                                                              int variant, const int32_t* step_ptr, int64_t M,
+                                                              int32_t* ids_out, float* logp_out) {
+  __shared__ ArgMax red_am[NTH / 64];
+  __shared__ float red_f[NTH / 64];
+  __shared__ float chunk_sum[NTH];
+  const int tid = threadIdx.x;
+  const int64_t row = blockIdx.x;
+  const float* sk = skeys + row * V;
+  uint32_t ks0 = 0u, ks1 = (uint32_t)(*step_ptr);
+  threefry2x32(key0, key1, ks0, ks1);
+  const float mx = sk[0];
+  // every thread owns a contiguous chunk of the sorted row
+  const int64_t per = (V + NTH - 1) / NTH;
+  const int64_t j0 = min(V, tid * per), j1 = min(V, j0 + per);
+  float se = 0.f;
+  for (int64_t j = j0; j < j1; ++j) se += expf(sk[j] - mx);
+  chunk_sum[tid] = se;
+  const float tot = block_sum_f(se, red_f);
+  // exclusive prefix of the chunk sums (in probability units), then the scan inside the chunk
+  __syncthreads();
+  float before = 0.f;
+  for (int t = 0; t < tid; ++t) before += chunk_sum[t];
+  float c = before / tot;
+  ArgMax g;
+  g.v = kNegInf;
+  g.i = 0x7fffffff;
+  for (int64_t j = j0; j < j1; ++j) {
+    const float pj = expf(sk[j] - mx) / tot;
+    const float lg = c > top_p ? kNegInf : sk[j];          // cumsum - p > top_p is dropped
+    c += pj;
+    ArgMax x;
+    x.v = lg + gumbel_from_bits(random_bits(ks0, ks1, (uint64_t)(row * V + j), (uint64_t)(M * V), variant));
+    x.i = (int)j;
+    g = better(g, x);
+  }
+  g = block_argmax(g, red_am);
+  if (tid == 0) {
+    ids_out[row] = sids[row * V + g.i];
+    if (logp_out) logp_out[row] = sk[g.i] - (mx + logf(tot));
+  }
+}
+
+struct FullSortWs {
+  size_t keys_in, keys_out, ids_in, ids_out, offsets, temp, temp_bytes, total;
+};
+int fullsort_layout(int64_t M, int64_t V, FullSortWs* w) {
+  const size_t n = (size_t)(M * V);
+  auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
+  size_t temp_bytes = 0;
+  const hipError_t e = rocprim::segmented_radix_sort_pairs_desc(
+      nullptr, temp_bytes, (const float*)nullptr, (float*)nullptr, (const int*)nullptr, (int*)nullptr,
+      (unsigned)n, (unsigned)M, (const int*)nullptr, (const int*)nullptr, 0, 32, (hipStream_t)0);
+  if (e != hipSuccess) return -1;
+  size_t o = 0;
+  w->keys_in = o; o += up(n * 4);
+  w->keys_out = o; o += up(n * 4);
+  w->ids_in = o; o += up(n * 4);
+  w->ids_out = o; o += up(n * 4);
+  w->offsets = o; o += up((size_t)(M + 1) * 4);
+  w->temp = o; o += up(temp_bytes);
+  w->temp_bytes = temp_bytes;
+  w->total = o;
+  return 0;
+}
+
 }  // namespace
+
+extern "C" size_t tnx_sample_fullsort_ws_bytes(int64_t M, int64_t V) {
+  FullSortWs w;
+  if (M <= 0 || V <= 0 || M * V >= (1ll << 31) || fullsort_layout(M, V, &w) != 0) return 0;
+  return w.total;
+}
 
 extern "C" size_t tnx_sample_topk_ws_bytes(int64_t M, int64_t V, int k) {
   if (M <= 0 || V <= 0) return 0;
@@ -644,8 +740,30 @@ extern "C" int tnx_sample_topk(void* stream, const float* logits, int64_t M, int
   TNX_REQUIRE(temperature > 0.f, "sample_topk: temperature must be positive, got %f", temperature);
   if (k <= 0 || k >= V) {
     if (top_p < 1.0f) {
-      tnx_set_error("sample_topk: top_p < 1 without top_k needs a full-vocabulary sort (not built)");
-      return TNX_ENOSYS;
+      TNX_REQUIRE(ws, "sample_topk: top_p < 1 without top_k sorts the whole row and needs a workspace of "
+                      "tnx_sample_fullsort_ws_bytes(M, V) bytes");
+      TNX_REQUIRE(M * V < (1ll << 31), "sample_topk: M * V too large for the full-row sort");
+      FullSortWs w;
+      TNX_REQUIRE(fullsort_layout(M, V, &w) == 0, "sample_topk: rocPRIM refused the sort configuration");
+      unsigned char* base = reinterpret_cast<unsigned char*>(ws);
+      float* kin = reinterpret_cast<float*>(base + w.keys_in);
+      float* kout = reinterpret_cast<float*>(base + w.keys_out);
+      int* iin = reinterpret_cast<int*>(base + w.ids_in);
+      int* iout = reinterpret_cast<int*>(base + w.ids_out);
+      int* off = reinterpret_cast<int*>(base + w.offsets);
+      const int64_t n = M * V;
+      hipLaunchKernelGGL(fullsort_prepare_kernel, dim3((unsigned)cdiv(n + 1, 256)), dim3(256), 0, as_stream(stream),
+                         logits, M, V, temperature, forbidden, forbidden ? n_forbidden : 0, kin, iin, off);
+      TNX_CHECK_LAUNCH("sample_topk (sort keys)");
+      size_t tb = w.temp_bytes;
+      const hipError_t e = rocprim::segmented_radix_sort_pairs_desc(
+          base + w.temp, tb, (const float*)kin, kout, (const int*)iin, iout, (unsigned)n, (unsigned)M,
+          (const int*)off, (const int*)(off + 1), 0, 32, as_stream(stream));
+      TNX_REQUIRE(e == hipSuccess, "sample_topk: segmented sort failed: %s", hipGetErrorString(e));
+      hipLaunchKernelGGL(fullsort_sample_kernel, dim3((unsigned)M), dim3(NTH), 0, as_stream(stream), kout, iout, V,
+                         top_p, key0, key1, rng_variant, step_ptr, M, ids_out, logp_out);
+      TNX_CHECK_LAUNCH("sample_topk (sorted draw)");
+      return TNX_OK;
     }
     k = 0;
   }

@@ -217,7 +217,8 @@ class Sampler:
       k = 0 if no_topk else int(min(top_k, cfg.vocab_size))
       mode.update(name="top_p", temperature=float(temperature), top_p=float(top_p), top_k=k,
                   key=key,
-                  ws=torch.empty(max(ops.sample_topk_ws_bytes(B, model.cfg.vocab_size, k) // 4, 1),
+                  ws=torch.empty(max((ops.sample_fullsort_ws_bytes(B, cfg.vocab_size) if (no_topk and top_p < 1.0)
+                                      else ops.sample_topk_ws_bytes(B, cfg.vocab_size, k)) // 4, 1),
                                  dtype=torch.float32, device=dev),
                   ids=torch.empty(B, dtype=torch.int32, device=dev),
                   logp=torch.empty(B, dtype=torch.float32, device=dev))

@@ -145,6 +145,10 @@ def sample_topk_ws_bytes(M, V, k) -> int:
   return int(L.lib().tnx_sample_topk_ws_bytes(M, V, 0 if k is None else int(k)))
 
 
+def sample_fullsort_ws_bytes(M, V) -> int:
+  return int(L.lib().tnx_sample_fullsort_ws_bytes(M, V))
+
+
 def sample_topk(logits, k, top_p, temperature, key, rng_variant, step_ptr, ws, ids_out, logp_out,
                 forbidden=None):
   """logits: raw fp32 [M,V]; they are divided by `temperature` inside the kernel."""
