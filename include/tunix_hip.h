@@ -277,6 +277,10 @@ typedef struct tnx_lmhead_desc {
   float* lse;                 /* fp32 [M] or NULL                                            */
   float* logits_out;          /* fp32 [M,V] or NULL: materialise logits (return_logits /
                                  top-k sampling path)                                       */
+  float* part_entropy;        /* fp32 workspace [M, n_vblocks], needed when entropy != NULL  */
+  float* entropy;             /* fp32 [M] or NULL: -sum_v p_v log p_v of the (temperature-
+                                 scaled) distribution, compute_entropy_from_logits
+                                 tunix/rl/common.py:1136-1148                                */
 } tnx_lmhead_desc;
 int64_t tnx_lmhead_nblocks(int64_t V);
 int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* h_desc);

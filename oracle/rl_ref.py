@@ -45,8 +45,16 @@ def process_ids(prompt_tokens: np.ndarray, completion_tokens: np.ndarray, pad_id
   return ids, positions, attn_mask
 
 
+def compute_entropy_from_logits(logits: torch.Tensor) -> torch.Tensor:
+  """tunix/rl/common.py:1136-1148: log_probs = log_softmax(logits); probs = softmax(log_probs);
+  entropy = -sum(probs * log_probs) over the last axis."""
+  lp = torch.log_softmax(logits.to(torch.float32), dim=-1)
+  pr = torch.softmax(lp, dim=-1)
+  return -(pr * lp).sum(-1)
+
+
 def compute_per_token_logps(ref_model, prompt_tokens, completion_tokens, pad_id,
-                            temperature: float = 1.0, chunk_size: int = 0):
+                            temperature: float = 1.0, chunk_size: int = 0, return_entropy: bool = False):
   """tunix/rl/common.py:326-482: one full forward without cache, logits[:, -T-1:-1],
   optional temperature, gather - logsumexp.  chunk_size > 0 follows compute_chunked_logps
   (:485-571): the head is applied per sequence chunk."""
@@ -72,6 +80,9 @@ def compute_per_token_logps(ref_model, prompt_tokens, completion_tokens, pad_id,
     for s in range(0, T, chunk_size):
       outs.append(selective_log_softmax(head(hk[:, s:s + chunk_size]), targets[:, s:s + chunk_size]))
     return torch.cat(outs, dim=1)
+  if return_entropy:  # :479-481, on the same (temperature-scaled) logits
+    lg = head(hk)
+    return selective_log_softmax(lg, targets), compute_entropy_from_logits(lg)
   return selective_log_softmax(head(hk), targets)
 
 

@@ -52,6 +52,26 @@ def test_per_token_logps_match_oracle(tiny, gpu):
   assert np.abs(got_t - got)[valid].max() > 1e-3
 
 
+def test_per_token_entropy_matches_oracle(tiny, gpu):
+  """return_entropy: -sum p log p of the (temperature-scaled) next-token distribution at every
+  completion position (tunix/rl/common.py:479-481, :1136-1148), from the fused head kernel."""
+  from tunix_amd.rl import common
+  cfg, w, model = tiny
+  prompt, comp = _tokens(cfg, 4, 24, 16, 3)
+  ref = MR.RefModel(cfg, w)
+  for temp in (1.0, 0.6):
+    lp, ent = common.compute_per_token_logps(model, prompt, comp, pad_id=0, temperature=temp, return_entropy=True)
+    want_lp, want_ent = R.compute_per_token_logps(ref, prompt, comp, 0, temperature=temp, return_entropy=True)
+    valid = comp != 0
+    tol = 2e-2 / temp   # the bf16 resolution of a logit, divided by the temperature with it
+    assert np.abs(lp.cpu().numpy() - want_lp.numpy())[valid].max() <= tol
+    got = ent.cpu().numpy()
+    assert np.isfinite(got).all() and (got >= 0).all() and (got <= np.log(cfg.vocab_size) + 1e-4).all()
+    assert np.abs(got - want_ent.numpy())[valid].max() <= tol
+    # the plain call returns the same log-probabilities bit for bit
+    assert torch.equal(lp, common.compute_per_token_logps(model, prompt, comp, pad_id=0, temperature=temp))
+
+
 def test_per_token_logps_chunking_and_batching_are_invariant(tiny, gpu):
   """tests/rl/common_test.py:340-399: the chunked computation returns the same values; here
   bit for bit, also when the batch is split over several forward passes."""
@@ -73,9 +93,6 @@ def test_per_token_logps_argument_errors(tiny, gpu):
   cfg, w, model = tiny
   with pytest.raises(ValueError):
     common.compute_per_token_logps(model, np.zeros((2, 4), np.int32), np.zeros((3, 4), np.int32), pad_id=0)
-  with pytest.raises(NotImplementedError):
-    common.compute_per_token_logps(model, np.ones((2, 4), np.int32), np.ones((2, 4), np.int32), pad_id=0,
-                                   return_entropy=True)
   empty = common.compute_per_token_logps(model, np.ones((2, 4), np.int32), np.ones((2, 0), np.int32), pad_id=0)
   assert tuple(empty.shape) == (2, 0)
 

@@ -138,3 +138,26 @@ def test_compute_per_token_logps_chunk_invariance():
   lsm2 = torch.log_softmax(lg.double() / 2.0, -1).numpy()
   want2 = np.array([[lsm2[b, 5 + t, comp[b, t]] for t in range(5)] for b in range(2)])
   np.testing.assert_allclose(t2, want2, atol=1e-5)
+
+
+def test_entropy_from_logits_closed_forms():
+  """Pins oracle.rl_ref.compute_entropy_from_logits: a uniform row has entropy log V whatever the
+  common offset, a one-hot row 0, a two-point distribution the binary entropy, and the value
+  agrees with scipy's definition on random rows."""
+  import scipy.stats
+  from oracle import rl_ref
+  V = 37
+  uni = torch.full((2, V), 3.25)
+  np.testing.assert_allclose(rl_ref.compute_entropy_from_logits(uni).numpy(), np.log(V), rtol=1e-6)
+  hot = torch.full((1, V), -1e4)
+  hot[0, 5] = 0.0
+  assert abs(float(rl_ref.compute_entropy_from_logits(hot)[0])) < 1e-6
+  p = 0.3
+  two = torch.full((1, V), -1e4)
+  two[0, 1], two[0, 2] = np.log(p), np.log(1 - p)
+  np.testing.assert_allclose(float(rl_ref.compute_entropy_from_logits(two)[0]),
+                             -(p * np.log(p) + (1 - p) * np.log(1 - p)), rtol=1e-5)
+  g = torch.Generator().manual_seed(5)
+  lg = torch.randn(6, 101, generator=g) * 3
+  want = scipy.stats.entropy(torch.softmax(lg.double(), -1).numpy(), axis=-1)
+  np.testing.assert_allclose(rl_ref.compute_entropy_from_logits(lg).numpy(), want, rtol=1e-5)

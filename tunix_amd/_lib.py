@@ -69,6 +69,7 @@ class LmHeadDesc(C.Structure):
       ("temperature", _f32), ("forbidden", _p), ("n_forbidden", _i32),
       ("targets", _p), ("part", _p), ("best_id", _p), ("best_logp", _p),
       ("target_logp", _p), ("lse", _p), ("logits_out", _p),
+      ("part_entropy", _p), ("entropy", _p),
   ]
 
 

@@ -30,6 +30,7 @@ struct LHArgs {
   float* part;
   int64_t nvb;
   float* logits_out;
+  float* part_ent;   // optional [M, nvb]: sum of exp(l - max) * l per block, for the entropy
 };
 
 constexpr float kNegInf = -__builtin_inff();
@@ -39,6 +40,7 @@ struct Stat {
   int idx;
   float sum;
   float tgt;
+  float wsum;  // sum of exp(l - mx) * l  (entropy = logsumexp - wsum / sum)
 };
 // Merge two statistics; `a` covers lower column indices than `b`.
 __device__ __forceinline__ Stat merge(const Stat& a, const Stat& b) {
@@ -48,6 +50,7 @@ __device__ __forceinline__ Stat merge(const Stat& a, const Stat& b) {
   const float wa = a.mx == kNegInf ? 0.f : __expf(a.mx - r.mx);
   const float wb = b.mx == kNegInf ? 0.f : __expf(b.mx - r.mx);
   r.sum = a.sum * wa + b.sum * wb;
+  r.wsum = a.wsum * wa + b.wsum * wb;
   r.tgt = fmaxf(a.tgt, b.tgt);
   return r;
 }
@@ -132,13 +135,20 @@ __global__ __launch_bounds__(DENSE ? 512 : 256) void lmhead_kernel(const LHArgs 
         }
         st.tgt = fmaxf(st.tgt, __shfl_xor(st.tgt, o, 64));
       }
-      float se = 0.f;
-      if (mx != kNegInf) se = (la == kNegInf ? 0.f : __expf(la - mx)) + (lb == kNegInf ? 0.f : __expf(lb - mx));
+      float se = 0.f, we = 0.f;
+      if (mx != kNegInf) {
+        const float ea = la == kNegInf ? 0.f : __expf(la - mx), eb = lb == kNegInf ? 0.f : __expf(lb - mx);
+        se = ea + eb;
+        we = (la == kNegInf ? 0.f : ea * la) + (lb == kNegInf ? 0.f : eb * lb);
+      }
 #pragma unroll
-      for (int o = 1; o < 16; o <<= 1) se += __shfl_xor(se, o, 64);
+      for (int o = 1; o < 16; o <<= 1) {
+        se += __shfl_xor(se, o, 64);
+        we += __shfl_xor(we, o, 64);
+      }
       if (lm == 0) {
         Stat r;
-        r.mx = mx; r.idx = idx; r.sum = se; r.tgt = st.tgt;
+        r.mx = mx; r.idx = idx; r.sum = se; r.tgt = st.tgt; r.wsum = we;
         sRed[wave * (MT * 16) + rl] = r;
       }
     }
@@ -152,23 +162,26 @@ __global__ __launch_bounds__(DENSE ? 512 : 256) void lmhead_kernel(const LHArgs 
     p[1] = __int_as_float(r.idx);
     p[2] = r.sum;
     p[3] = r.tgt;
+    if (a.part_ent) a.part_ent[(m0 + tid) * a.nvb + vb] = r.wsum;
   }
 }
 
 // One wave per row merges the per-block statistics in column order.
 __global__ __launch_bounds__(64) void lmhead_finish_kernel(const float* part, int64_t nvb,
                                                            int32_t* best_id, float* best_logp,
-                                                           float* target_logp, float* lse_out) {
+                                                           float* target_logp, float* lse_out,
+                                                           const float* part_ent, float* entropy_out) {
   const int64_t row = blockIdx.x;
   const int lane = threadIdx.x;
   const float* p = part + row * nvb * 4;
   // lane l owns the contiguous block range [l*per, (l+1)*per): merges stay in column order
   const int64_t per = (nvb + 63) / 64;
   Stat r;
-  r.mx = kNegInf; r.idx = 0x7fffffff; r.sum = 0.f; r.tgt = kNegInf;
+  r.mx = kNegInf; r.idx = 0x7fffffff; r.sum = 0.f; r.tgt = kNegInf; r.wsum = 0.f;
   for (int64_t c = lane * per; c < min(nvb, (lane + 1) * per); ++c) {
     Stat b;
     b.mx = p[c * 4]; b.idx = __float_as_int(p[c * 4 + 1]); b.sum = p[c * 4 + 2]; b.tgt = p[c * 4 + 3];
+    b.wsum = part_ent ? part_ent[row * nvb + c] : 0.f;
     r = merge(r, b);
   }
 #pragma unroll
@@ -178,6 +191,7 @@ __global__ __launch_bounds__(64) void lmhead_finish_kernel(const float* part, in
     b.idx = __shfl_xor(r.idx, o, 64);
     b.sum = __shfl_xor(r.sum, o, 64);
     b.tgt = __shfl_xor(r.tgt, o, 64);
+    b.wsum = __shfl_xor(r.wsum, o, 64);
     r = (lane & o) ? merge(b, r) : merge(r, b);  // the lower lane holds the lower columns
   }
   if (lane == 0) {
@@ -186,6 +200,7 @@ __global__ __launch_bounds__(64) void lmhead_finish_kernel(const float* part, in
     if (best_logp) best_logp[row] = r.mx - lse;
     if (target_logp) target_logp[row] = r.tgt - lse;
     if (lse_out) lse_out[row] = lse;
+    if (entropy_out) entropy_out[row] = lse - r.wsum / r.sum;  // -sum p log p
   }
 }
 
@@ -243,6 +258,8 @@ extern "C" int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* d) {
   a.forbidden = d->forbidden; a.n_forbidden = d->forbidden ? d->n_forbidden : 0;
   a.targets = d->targets; a.part = d->part; a.nvb = tnx_lmhead_nblocks(d->V);
   a.logits_out = d->logits_out;
+  TNX_REQUIRE(!d->entropy || d->part_entropy, "lmhead: entropy needs the part_entropy workspace [M, n_vblocks]");
+  a.part_ent = d->entropy ? d->part_entropy : nullptr;
   hipStream_t st = as_stream(stream);
   int rc;
   const bool dense = d->w_bf16 != nullptr;
@@ -252,7 +269,7 @@ extern "C" int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* d) {
   else rc = dense ? launch_lmhead<8, true>(st, a) : launch_lmhead<8, false>(st, a);
   if (rc) return rc;
   hipLaunchKernelGGL(lmhead_finish_kernel, dim3((unsigned)d->M), dim3(64), 0, st, a.part, a.nvb,
-                     d->best_id, d->best_logp, d->target_logp, d->lse);
+                     d->best_id, d->best_logp, d->target_logp, d->lse, a.part_ent, d->entropy);
   TNX_CHECK_LAUNCH("lmhead_finish");
   return TNX_OK;
 }

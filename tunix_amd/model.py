@@ -435,7 +435,8 @@ class Runner:
     ops.moe_combine(self.y_route, self.topk_w, M, k, cfg.embed_dim, self.h, self.h)
 
   def head_desc(self, x, rows, part, temperature=1.0, targets=None, best_id=None, best_logp=None,
-                target_logp=None, lse=None, logits_out=None, forbidden=None) -> L.LmHeadDesc:
+                target_logp=None, lse=None, logits_out=None, forbidden=None, entropy=None,
+                part_entropy=None) -> L.LmHeadDesc:
     cfg, m = self.cfg, self.model
     d = L.LmHeadDesc()
     d.M, d.D, d.V = rows, cfg.embed_dim, cfg.vocab_size
@@ -452,7 +453,8 @@ class Runner:
     if forbidden is not None:
       d.forbidden, d.n_forbidden = forbidden.data_ptr(), forbidden.numel()
     for name, tns in (("targets", targets), ("best_id", best_id), ("best_logp", best_logp),
-                      ("target_logp", target_logp), ("lse", lse), ("logits_out", logits_out)):
+                      ("target_logp", target_logp), ("lse", lse), ("logits_out", logits_out),
+                      ("entropy", entropy), ("part_entropy", part_entropy)):
       if tns is not None:
         setattr(d, name, tns.data_ptr())
     d.part = part.data_ptr()

@@ -44,10 +44,10 @@ def compute_per_token_logps(model: QLoRAModel, prompt_tokens, completion_tokens,
 
   prompt_tokens [B, P] (left padded) and completion_tokens [B, T] (right padded) are integer
   arrays or tensors.  `temperature` divides the logits as in the reference (:431-436: ignored
-  when 0 or 1).  `max_rows` bounds the token rows of one forward pass.
+  when 0 or 1).  `max_rows` bounds the token rows of one forward pass.  With return_entropy the
+  result is (logps, entropy), entropy = -sum p log p of the same (temperature-scaled) logits
+  (compute_entropy_from_logits, :1136-1148), also from the fused head kernel.
   """
-  if return_entropy:
-    raise NotImplementedError("per-token entropy is not produced by the fused head kernel")
   dev = model.device
   pt = torch.as_tensor(np.asarray(prompt_tokens) if not isinstance(prompt_tokens, torch.Tensor)
                        else prompt_tokens).to(dev)
@@ -77,6 +77,8 @@ def compute_per_token_logps(model: QLoRAModel, prompt_tokens, completion_tokens,
   runner.part = part
   xsel = torch.empty(rows_b * T, cfg.embed_dim, dtype=torch.bfloat16, device=dev)
   out = torch.empty(B, T, dtype=torch.float32, device=dev)
+  ent = torch.empty(B, T, dtype=torch.float32, device=dev) if return_entropy else None
+  part_ent = torch.empty(head_rows * runner.nvb, dtype=torch.float32, device=dev) if return_entropy else None
   for b0 in range(0, B, rows_b):
     nb = min(rows_b, B - b0)
     xn = runner.forward_hidden(ids[b0:b0 + nb], positions[b0:b0 + nb], runner.zero,
@@ -88,9 +90,12 @@ def compute_per_token_logps(model: QLoRAModel, prompt_tokens, completion_tokens,
     lp = out[b0:b0 + nb].view(-1)
     for r0 in range(0, nb * T, head_rows):
       nr = min(head_rows, nb * T - r0)
+      kw = {}
+      if return_entropy:  # entropy of the temperature-scaled distribution (:479-481)
+        kw = dict(entropy=ent[b0:b0 + nb].view(-1)[r0:r0 + nr], part_entropy=part_ent)
       runner.run_head(xs[r0:r0 + nr], nr, temperature=temp, targets=tg[r0:r0 + nr],
-                      target_logp=lp[r0:r0 + nr])
-  return out
+                      target_logp=lp[r0:r0 + nr], **kw)
+  return (out, ent) if return_entropy else out
 
 
 def grpo_clipped_ratio(logp: torch.Tensor, old_logp: torch.Tensor | None, advantages: torch.Tensor,
