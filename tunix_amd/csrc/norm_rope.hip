@@ -100,14 +100,25 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
       if (ws) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) h[c][j] = 0.f;
-        for (int z = 0; z < split_k; ++z) {
-          const f32x4 p0 = *reinterpret_cast<const f32x4*>(ws + z * plane + o);
-          const f32x4 p1 = *reinterpret_cast<const f32x4*>(ws + z * plane + o + 4);
+        // four planes' loads in flight at a time (planes past the last are clamped and not
+        // added); the sum itself stays in split order
+        for (int z0 = 0; z0 < split_k; z0 += 4) {
+          f32x4 p0[4], p1[4];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            h[c][j] += p0[j];
-            h[c][4 + j] += p1[j];
+          for (int u = 0; u < 4; ++u) {
+            const int64_t zo = (int64_t)min(z0 + u, split_k - 1) * plane + o;
+            p0[u] = *reinterpret_cast<const f32x4*>(ws + zo);
+            p1[u] = *reinterpret_cast<const f32x4*>(ws + zo + 4);
           }
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            if (z0 + u < split_k) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                h[c][j] += p0[u][j];
+                h[c][4 + j] += p1[u][j];
+              }
+            }
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) h[c][j] = rbf(h[c][j]);
