@@ -222,7 +222,14 @@ __global__ void rope_kernel(const RopeArgs a) {
     if (a.ws == nullptr) return bf2f(a.qkv[src_off + e]);
     const int64_t plane = a.B * a.T * (int64_t)ld;
     float v = 0.f;
-    for (int z = 0; z < a.split_k; ++z) v += a.ws[z * plane + src_off + e];
+    for (int z0 = 0; z0 < a.split_k; z0 += 8) {  // eight planes' loads in flight; sum in split order
+      float p[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) p[u] = a.ws[(int64_t)min(z0 + u, a.split_k - 1) * plane + src_off + e];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (z0 + u < a.split_k) v += p[u];
+    }
     return rbf(v);
   };
   const int slot = (int)((col + t) % a.S);
