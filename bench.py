@@ -205,6 +205,34 @@ def cpu_baseline(cfg_full, B, ctx, S, threads):
           "layer_s": t_layer, "head_s": t_head}
 
 
+def summarize_step_trace(path):
+  """Prints the kernels of the last complete decode step found in a `rocprofv3 --kernel-trace`
+  csv of this script (a step = the dispatches between two sample_commit kernels): count, total
+  and mean duration per kernel, start-to-start time included (the dependent-launch gaps)."""
+  import collections
+  import csv
+  rows = sorted(csv.DictReader(open(path)), key=lambda r: int(r["Start_Timestamp"]))
+  commits = [i for i, r in enumerate(rows) if "sample_commit" in r["Kernel_Name"]]
+  if len(commits) < 3:
+    raise SystemExit("the trace holds fewer than two decode steps")
+  step = rows[commits[-3] + 1: commits[-2] + 1]
+  t0, t1 = int(step[0]["Start_Timestamp"]), int(step[-1]["End_Timestamp"])
+  agg = collections.OrderedDict()
+  for r, nxt in zip(step, step[1:] + [None]):
+    name = r["Kernel_Name"].replace("(anonymous namespace)::", "").replace("void ", "").split("(")[0]
+    busy = int(r["End_Timestamp"]) - int(r["Start_Timestamp"])
+    span = (int(nxt["Start_Timestamp"]) if nxt else t1) - int(r["Start_Timestamp"])
+    e = agg.setdefault(name, [0, 0, 0])
+    e[0] += 1
+    e[1] += busy
+    e[2] += span
+  print(f"one decode step: {(t1 - t0) / 1e3:.1f} us, {len(step)} kernels")
+  print(f"| {'kernel':34s} | calls | total us | mean us | mean start-to-start us |")
+  print(f"|{'-' * 36}|-------|----------|---------|------------------------|")
+  for name, (n, busy, span) in agg.items():
+    print(f"| {name:34s} | {n:5d} | {busy / 1e3:8.1f} | {busy / n / 1e3:7.2f} | {span / n / 1e3:22.2f} |")
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -219,7 +247,12 @@ def main():
   ap.add_argument("--kernels-only", action="store_true",
                   help="profiling aid: one layer, no prefill / decode; only the per-kernel loops at "
                        "context prompt + gen / 2 (prints the kernel table, not the metric)")
+  ap.add_argument("--summarize-trace", metavar="CSV", default=None,
+                  help="no GPU work: tabulate one decode step of a rocprofv3 kernel-trace csv of this script")
   args = ap.parse_args()
+  if args.summarize_trace:
+    summarize_step_trace(args.summarize_trace)
+    return
   if args.gpus != 1:
     print("bench.py measures one GPU: this build has no multi-GPU path (the decode path shards "
           "by batch rows with no exchange); run with --gpus 1", file=sys.stderr)
