@@ -208,6 +208,11 @@ typedef struct tnx_rope_desc {
   int split_k;
 } tnx_rope_desc;
 int tnx_qknorm_rope_kvwrite(void* stream, const tnx_rope_desc* h_desc);
+/* sin / cos of positions[b, *col_ptr] / timescale[i], fp32 [B, dh/2] each: the angles of the
+ * Llama rotation above for one decode step, shared by all layers (input of the fused mode of
+ * tnx_gqa_attn). */
+int tnx_rope_table(void* stream, const int32_t* positions, int64_t pos_ld, const int32_t* col_ptr,
+                   int64_t B, const float* timescale, int dh, float* sin_out, float* cos_out);
 
 /* ---------------------------------------------------------------------------------------
  * GQA attention over the KV cache for T query tokens per row (T = 1: decode).
@@ -238,6 +243,18 @@ typedef struct tnx_attn_desc {
   int kv_chunk;              /* keys per work-group when splitting (multiple of 32); 0: no split */
   float* ws;
   uint16_t* out;
+  /* Optional fused RoPE + cache write for decode (rope_sin != NULL; needs T == 1,
+   * dh == 128, a model without q/k norm and the Llama rotation): the kernel takes the step's
+   * q, k and v from the qkv linear's output (finished bf16 `qkv` [B, (Hq+2Hkv)*dh], or its
+   * `qkv_split` fp32 partial planes `qkv_ws`), rotates q and k exactly as
+   * tnx_qknorm_rope_kvwrite does (with the step's sines / cosines from tnx_rope_table), writes k
+   * and v into cache slot *col_ptr and attends them from registers; `q` is not read and that
+   * separate launch is not needed. */
+  const float* qkv_ws;
+  const uint16_t* qkv;
+  int qkv_split;
+  const float* rope_sin;     /* fp32 [B, dh/2] from tnx_rope_table                           */
+  const float* rope_cos;
 } tnx_attn_desc;
 size_t tnx_attn_ws_bytes(int64_t B, int64_t T, int64_t S, int Hq, int dh, int kv_chunk);
 int tnx_gqa_attn(void* stream, const tnx_attn_desc* h_desc);

@@ -657,6 +657,80 @@ def test_rmsnorm_splitk_equals_finish_then_norm(gpu, family):
   assert torch.equal(y1, y2)
 
 
+@pytest.mark.parametrize("kv_chunk,window,planes", [(0, 0, False), (32, 0, True), (0, 40, True), (64, 0, False)])
+def test_attention_with_fused_rope_equals_rope_then_attention(gpu, kv_chunk, window, planes):
+  """Decode attention that rotates q / k and writes the step's key / value itself (from the qkv
+  linear's bf16 output or its split-k planes) against the two launches it replaces: the cache
+  ends up bit-identical, the output agrees to a bf16 ulp (the step's own key enters the online
+  softmax as a block of its own instead of inside the last 32-key block)."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  from tunix_amd.model import rope_timescale
+  B, S, Hq, Hkv, dh, col, split = 6, 96, 8, 2, 128, 70, 3
+  ld = (Hq + 2 * Hkv) * dh
+  g = torch.Generator().manual_seed(95)
+  pl = torch.randn(split, B, ld, generator=g).float()
+  qkv = pl.sum(0).to(torch.bfloat16)
+  ws = pl.to(gpu).contiguous() if planes else None
+  if planes:   # the reference path sees bf16(sum of planes in split order)
+    acc = torch.zeros(B, ld)
+    for z in range(split):
+      acc = acc + pl[z]
+    qkv = acc.to(torch.bfloat16)
+  gq = qkv.to(gpu)
+  pos = torch.randint(0, 900, (B, S), generator=g, dtype=torch.int32).to(gpu)
+  ts = torch.from_numpy(rope_timescale(dh, 5e5)).to(gpu)
+  tokens = torch.randint(1, 50, (B, S), generator=g, dtype=torch.int32)
+  tokens[1, :9] = 0                                                # a left-padded row
+  tokens = tokens.to(gpu)
+  colp = torch.tensor([col], dtype=torch.int32, device=gpu)
+  kc0 = torch.randn(B, Hkv, S, dh, generator=g).to(torch.bfloat16).to(gpu)
+  vc0 = torch.randn(B, Hkv, S, dh, generator=g).to(torch.bfloat16).to(gpu)
+
+  def attn(q, kc, vc, fused):
+    d = L.AttnDesc()
+    d.B, d.T, d.S, d.Hq, d.Hkv, d.dh = B, 1, S, Hq, Hkv, dh
+    d.scale, d.window, d.pad_id = dh ** -0.5, window, 0
+    d.kcache, d.vcache = kc.data_ptr(), vc.data_ptr()
+    d.tokens, d.tok_ld, d.col_ptr = tokens.data_ptr(), S, colp.data_ptr()
+    d.kv_chunk = kv_chunk
+    wsa = torch.empty(max(ops.attn_ws_bytes(B, 1, S, Hq, dh, kv_chunk) // 4, 1), dtype=torch.float32, device=gpu)
+    out = torch.empty(B, Hq * dh, dtype=torch.bfloat16, device=gpu)
+    d.ws, d.out = wsa.data_ptr(), out.data_ptr()
+    if fused:
+      if planes:
+        d.qkv_ws, d.qkv_split = ws.data_ptr(), split
+      else:
+        d.qkv = gq.data_ptr()
+      sn = torch.empty(B, dh // 2, dtype=torch.float32, device=gpu)
+      cs = torch.empty_like(sn)
+      ops.rope_table(pos, colp, B, ts, dh, sn, cs)
+      d.rope_sin, d.rope_cos = sn.data_ptr(), cs.data_ptr()
+    else:
+      d.q = q.data_ptr()
+    ops.gqa_attn(d)
+    torch.cuda.synchronize()
+    return out
+
+  # the two launches
+  kc1, vc1 = kc0.clone(), vc0.clone()
+  rd = L.RopeDesc()
+  rd.B, rd.T, rd.S, rd.Hq, rd.Hkv, rd.dh = B, 1, S, Hq, Hkv, dh
+  rd.rope_flavor, rd.rope_scale, rd.timescale, rd.qk_norm = L.TNX_ROPE_LLAMA, 1.0, ts.data_ptr(), -1
+  q1 = torch.empty(B, Hq * dh, dtype=torch.bfloat16, device=gpu)
+  rd.qkv, rd.positions, rd.pos_ld, rd.col_ptr = gq.data_ptr(), pos.data_ptr(), S, colp.data_ptr()
+  rd.q_out, rd.kcache, rd.vcache = q1.data_ptr(), kc1.data_ptr(), vc1.data_ptr()
+  ops.rope_kvwrite(rd)
+  out1 = attn(q1, kc1, vc1, False)
+  # the fused launch
+  kc2, vc2 = kc0.clone(), vc0.clone()
+  out2 = attn(None, kc2, vc2, True)
+  assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+  assert not torch.equal(kc2, kc0)
+  assert out1.float().abs().max() > 0.05
+  assert (out1.float() - out2.float()).abs().max().item() <= 4e-3
+
+
 @pytest.mark.parametrize("family", ["llama3", "qwen3"])
 def test_rope_from_splitk_planes_equals_finish_then_rope(gpu, family):
   """The rope / cache-write kernel fed with the partial planes of a split-k qkv linear against

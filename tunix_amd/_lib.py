@@ -57,6 +57,7 @@ class AttnDesc(C.Structure):
       ("q", _p), ("kcache", _p), ("vcache", _p),
       ("tokens", _p), ("tok_ld", _i64), ("col_ptr", _p),
       ("kv_chunk", _i32), ("ws", _p), ("out", _p),
+      ("qkv_ws", _p), ("qkv", _p), ("qkv_split", _i32), ("rope_sin", _p), ("rope_cos", _p),
   ]
 
 
@@ -97,6 +98,7 @@ SIGNATURES = {
     "tnx_rmsnorm": (_i32, [_p, _p, _p, _p, _p, _p, _p, _i64, _i64, _f32, _i32]),
     "tnx_rmsnorm_splitk": (_i32, [_p, _p, _i32, _p, _p, _p, _p, _p, _i64, _i64, _f32, _i32]),
     "tnx_qknorm_rope_kvwrite": (_i32, [_p, C.POINTER(RopeDesc)]),
+    "tnx_rope_table": (_i32, [_p, _p, _i64, _p, _i64, _p, _i32, _p, _p]),
     "tnx_attn_ws_bytes": (C.c_size_t, [_i64, _i64, _i64, _i32, _i32, _i32]),
     "tnx_gqa_attn": (_i32, [_p, C.POINTER(AttnDesc)]),
     "tnx_lmhead_nblocks": (_i64, [_i64]),

@@ -28,11 +28,18 @@ struct AttnArgs {
   int kv_chunk, n_chunks;
   float* ws;
   uint16_t* out;
+  // fused RoPE + cache write of the step's own token (decode, T == 1, no q/k norm, Llama
+  // rotation): the query, key and value come from the qkv linear's output instead of q / the cache
+  const float* qkv_ws;        // split-k partial planes [qkv_split][B][(Hq + 2 Hkv) * dh], or null
+  const uint16_t* qkv;        // ... or the finished bf16 output
+  int qkv_split;
+  const float* rope_sin;      // fp32 [B, dh/2] of this step's positions; non-null switches the mode on
+  const float* rope_cos;
 };
 
 constexpr float kNegBig = -1.0e30f;
 
-template <int DH>
+template <int DH, bool FUSE>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2 : 1, DH > 128 ? 2 : 1))) void attn_kernel(const AttnArgs a) {
   constexpr int KS = DH / 32;                 // k-steps of the QK product
   constexpr int NH = DH > 128 ? DH / 128 : 1; // 128-column halves of V / O
@@ -61,12 +68,18 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
     k_hi = min(k_hi, chunk * a.kv_chunk + a.kv_chunk - 1);
   }
 
+  constexpr bool fused = FUSE;                           // T == 1: c_n = col0 for every lane
   u32x4 qf[KS];
 #pragma unroll
   for (int j = 0; j < KS; ++j) {
     qf[j] = u32x4{0, 0, 0, 0};
-    if (qvalid) qf[j] = *reinterpret_cast<const u32x4*>(a.q + qvec * DH + j * 32 + lq * 8);
+    if (qvalid && !fused) qf[j] = *reinterpret_cast<const u32x4*>(a.q + qvec * DH + j * 32 + lq * 8);
   }
+  // in fused mode the step's own key / value never come from the cache: the loop stops one key
+  // short and they are added from registers at the end
+  int key_hi = fused ? c_n - 1 : c_n;
+  const bool writer = fused && col0 >= k_lo && col0 <= k_hi;   // the chunk that owns the new token
+  if (fused) k_hi = min(k_hi, col0 - 1);
 
   f32x4 O[NH][8];
 #pragma unroll
@@ -140,7 +153,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       const int key = kb + (s < 4 ? 4 * lq + s : 16 + 4 * lq + (s - 4));
-      kvalid[s] = qvalid && key >= max(k_lo, lo_n) && key <= min(k_hi, c_n) && sg.tk[s] != a.pad_id;
+      kvalid[s] = qvalid && key >= max(k_lo, lo_n) && key <= min(k_hi, key_hi) && sg.tk[s] != a.pad_id;
     }
     // ---- S^T = K . q^T ----
     f32x4 st[2];
@@ -205,9 +218,124 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
     Stage sg[NS];
     const int kb0 = k_lo & ~31;
     const int kb_last = k_hi & ~31;
-    if (kb0 <= k_hi) {
+    const bool any = kb0 <= k_hi;
+    if (any) {
 #pragma unroll
       for (int u = 0; u < NS - 1; ++u) load_block(min(kb0 + 32 * u, kb_last), sg[u]);
+    }
+    // the step's own key / value wait in LDS while the cached keys stream through the registers
+    __shared__ u32x4 park[FUSE ? KS + NH : 1][64];
+    if constexpr (fused) {
+      u32x4 kn[KS], vn[NH];
+      // ---- this step's q (G heads), k and v of the kv head from the qkv linear's output, RoPE
+      // applied as the stand-alone kernel does; the first key blocks are already in flight ----
+      const int ld = (a.Hq + 2 * a.Hkv) * DH;
+      const int64_t plane = a.B * (int64_t)ld;
+      const int64_t rowoff = b * (int64_t)ld;
+      // The G query heads, the key head and the value head of this (row, kv head), (G + 2) * DH
+      // values, are fetched once by the whole wave (16 bytes per lane and plane, all planes of
+      // a group in flight together), summed in split order, rounded to bf16 and staged in LDS,
+      // from where every lane picks the elements of its fragments.
+      __shared__ float xs[18 * DH];
+      {
+        const int n4 = (a.G + 2) * (DH / 4);
+        for (int i4 = lane; i4 < n4; i4 += 64) {
+          const int hsel = i4 / (DH / 4), d = (i4 % (DH / 4)) * 4;
+          const int head = hsel < a.G ? hkv * a.G + hsel : (hsel == a.G ? a.Hq + hkv : a.Hq + a.Hkv + hkv);
+          const int64_t o = rowoff + (int64_t)head * DH + d;
+          f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+          if (a.qkv_ws) {
+            for (int z0 = 0; z0 < a.qkv_split; z0 += 8) {
+              f32x4 p[8];
+#pragma unroll
+              for (int u = 0; u < 8; ++u)
+                p[u] = *reinterpret_cast<const f32x4*>(a.qkv_ws + (int64_t)min(z0 + u, a.qkv_split - 1) * plane + o);
+#pragma unroll
+              for (int u = 0; u < 8; ++u)
+                if (z0 + u < a.qkv_split) acc += p[u];
+            }
+          } else {
+            const u32x2 q = *reinterpret_cast<const u32x2*>(a.qkv + o);
+            acc = f32x4{bflo(q[0]), bfhi(q[0]), bflo(q[1]), bfhi(q[1])};
+          }
+          *reinterpret_cast<f32x4*>(&xs[i4 * 4]) = f32x4{rbf(acc[0]), rbf(acc[1]), rbf(acc[2]), rbf(acc[3])};
+        }
+        __syncthreads();
+      }
+      auto fetch8 = [&](int hsel, int d, float (&x)[8]) {
+        const f32x4 v0 = *reinterpret_cast<const f32x4*>(&xs[hsel * DH + d]);
+        const f32x4 v1 = *reinterpret_cast<const f32x4*>(&xs[hsel * DH + d + 4]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          x[e] = v0[e];
+          x[4 + e] = v1[e];
+        }
+      };
+      // sine / cosine of this row's position: a per-step table (tnx_rope_table), computed with
+      // the arithmetic of the stand-alone kernel
+      float sn[KS / 2][8], cs[KS / 2][8];
+#pragma unroll
+      for (int j = 0; j < KS / 2; ++j) {
+        const int64_t o = b * (DH / 2) + j * 32 + lq * 8;
+        const f32x4 s0 = *reinterpret_cast<const f32x4*>(a.rope_sin + o), s1 = *reinterpret_cast<const f32x4*>(a.rope_sin + o + 4);
+        const f32x4 c0 = *reinterpret_cast<const f32x4*>(a.rope_cos + o), c1 = *reinterpret_cast<const f32x4*>(a.rope_cos + o + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          sn[j][e] = s0[e]; sn[j][4 + e] = s1[e];
+          cs[j][e] = c0[e]; cs[j][4 + e] = c1[e];
+        }
+      }
+      // rotate the head whose first column is `col`: pairs (d, d + DH/2) sit in k-steps j, j + KS/2
+      auto rotated = [&](int hsel, u32x4 (&dst)[KS]) {
+        float x[KS][8];
+#pragma unroll
+        for (int j = 0; j < KS; ++j) fetch8(hsel, j * 32 + lq * 8, x[j]);
+#pragma unroll
+        for (int j = 0; j < KS / 2; ++j) {
+          float o1[8], o2[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float x1 = x[j][e], x2 = x[j + KS / 2][e];
+            o1[e] = rbf(__fsub_rn(__fmul_rn(x1, cs[j][e]), __fmul_rn(x2, sn[j][e])));
+            o2[e] = rbf(__fadd_rn(__fmul_rn(x2, cs[j][e]), __fmul_rn(x1, sn[j][e])));
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            dst[j][e] = pack2bf(o1[2 * e], o1[2 * e + 1]);
+            dst[j + KS / 2][e] = pack2bf(o2[2 * e], o2[2 * e + 1]);
+          }
+        }
+      };
+      if (qvalid) rotated(g, qf);
+#pragma unroll
+      for (int j = 0; j < KS; ++j) kn[j] = u32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int h = 0; h < NH; ++h) vn[h] = u32x4{0, 0, 0, 0};
+      if (writer) {
+        const int64_t slot = ((b * a.Hkv + hkv) * a.S + (col0 % (int)a.S)) * DH;
+        if (lm == 0) {   // lanes (0, lq) hold the key as row 0 of an A fragment
+          rotated(a.G, kn);
+#pragma unroll
+          for (int j = 0; j < KS; ++j)
+            *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(a.k) + slot + j * 32 + lq * 8) = kn[j];
+        }
+        if (lq == 0 && 8 * lm < (DH < 128 ? DH : 128)) {   // lanes (lm, 0) hold the value row of key 0
+#pragma unroll
+          for (int h = 0; h < NH; ++h) {
+            float x[8];
+            fetch8(a.G + 1, h * 128 + 8 * lm, x);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) vn[h][e] = pack2bf(x[2 * e], x[2 * e + 1]);
+            *reinterpret_cast<u32x4*>(const_cast<uint16_t*>(a.v) + slot + h * 128 + 8 * lm) = vn[h];
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < KS; ++j) park[j][lane] = kn[j];
+#pragma unroll
+      for (int h = 0; h < NH; ++h) park[KS + h][lane] = vn[h];
+    }
+    if (any) {
       for (int kb = kb0; kb <= k_hi; kb += 32 * NS) {
 #pragma unroll
         for (int u = 0; u < NS; ++u) {
@@ -218,6 +346,25 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
           compute_block(kbu, sg[u]);
         }
       }
+    }
+    if (writer) {
+      // the step's own key / value as a block of one key (at position col0) from registers
+      Stage& one = sg[0];
+#pragma unroll
+      for (int j = 0; j < KS; ++j) {
+        one.kf[0][j] = park[j][lane];
+        one.kf[1][j] = u32x4{0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int h = 0; h < NH; ++h)
+#pragma unroll
+        for (int sidx = 0; sidx < 8; ++sidx) one.vf[h][sidx] = sidx == 0 ? park[KS + h][lane] : u32x4{0, 0, 0, 0};
+      const int own_tok = tok[col0];
+#pragma unroll
+      for (int sidx = 0; sidx < 8; ++sidx) one.tk[sidx] = own_tok;
+      k_hi = col0;
+      key_hi = col0;
+      compute_block(col0, one);
     }
   }
 
@@ -311,7 +458,7 @@ extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
   TNX_REQUIRE(d->Hkv > 0 && d->Hq % d->Hkv == 0, "attn: Hq=%d not a multiple of Hkv=%d", d->Hq, d->Hkv);
   const int G = d->Hq / d->Hkv;
   TNX_REQUIRE(G <= 16, "attn: group size %d > 16 not supported", G);
-  TNX_REQUIRE(d->q && d->kcache && d->vcache && d->tokens && d->col_ptr && d->out, "attn: null pointer");
+  TNX_REQUIRE(d->kcache && d->vcache && d->tokens && d->col_ptr && d->out, "attn: null pointer");
   TNX_REQUIRE(d->kv_chunk >= 0 && d->kv_chunk % 32 == 0, "attn: kv_chunk must be a multiple of 32");
   TNX_REQUIRE(d->tok_ld >= d->S || d->tok_ld > 0, "attn: bad tok_ld");
   AttnArgs a;
@@ -330,6 +477,16 @@ extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
   a.col_ptr = d->col_ptr; a.kv_chunk = d->kv_chunk;
   a.n_chunks = d->kv_chunk > 0 ? (int)cdiv(d->S, d->kv_chunk) : 1;
   a.ws = d->ws; a.out = d->out;
+  a.qkv_ws = nullptr; a.qkv = nullptr; a.qkv_split = 0; a.rope_sin = nullptr; a.rope_cos = nullptr;
+  if (d->rope_sin) {
+    TNX_REQUIRE(d->T == 1 && d->dh == 128, "attn: the fused RoPE / cache write needs T == 1 and head_dim 128");
+    TNX_REQUIRE(d->rope_cos && (d->qkv || d->qkv_ws), "attn: fused RoPE needs the sine / cosine table and the qkv output");
+    if (d->qkv_ws) TNX_REQUIRE(d->qkv_split >= 1 && d->qkv_split <= 64, "attn: qkv_split=%d out of range", d->qkv_split);
+    a.qkv_ws = d->qkv_ws; a.qkv = d->qkv; a.qkv_split = d->qkv_split;
+    a.rope_sin = d->rope_sin; a.rope_cos = d->rope_cos;
+  } else {
+    TNX_REQUIRE(d->q, "attn: null pointer");
+  }
   if (a.n_chunks > 1) TNX_REQUIRE(d->ws, "attn: split key range needs a workspace");
   const int PT = 16 / a.Gp;
   const int64_t QT = cdiv(d->T, PT);
@@ -337,9 +494,12 @@ extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
   dim3 grid((unsigned)a.n_chunks, (unsigned)d->Hkv, (unsigned)(d->B * QT));
   hipStream_t st = as_stream(stream);
   switch (d->dh) {
-    case 64: hipLaunchKernelGGL(attn_kernel<64>, grid, dim3(64), 0, st, a); break;
-    case 128: hipLaunchKernelGGL(attn_kernel<128>, grid, dim3(64), 0, st, a); break;
-    default: hipLaunchKernelGGL(attn_kernel<256>, grid, dim3(64), 0, st, a); break;
+    case 64: hipLaunchKernelGGL((attn_kernel<64, false>), grid, dim3(64), 0, st, a); break;
+    case 128:
+      if (a.rope_sin) hipLaunchKernelGGL((attn_kernel<128, true>), grid, dim3(64), 0, st, a);
+      else hipLaunchKernelGGL((attn_kernel<128, false>), grid, dim3(64), 0, st, a);
+      break;
+    default: hipLaunchKernelGGL((attn_kernel<256, false>), grid, dim3(64), 0, st, a); break;
   }
   TNX_CHECK_LAUNCH("gqa_attn");
   if (a.n_chunks > 1) {

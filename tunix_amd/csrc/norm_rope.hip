@@ -285,6 +285,19 @@ __global__ void rope_kernel(const RopeArgs a) {
   }
 }
 
+// sin / cos of angle = position / timescale[i] for the token in column *col_ptr of every row: the
+// values rope_kernel computes for the Llama rotation, once per decode step instead of per layer.
+__global__ void rope_table_kernel(const int32_t* positions, int64_t pos_ld, const int32_t* col_ptr,
+                                  const float* timescale, int half, float* sin_out, float* cos_out) {
+  const int64_t b = blockIdx.x;
+  const int i = threadIdx.x;
+  if (i >= half) return;
+  const float pos = (float)positions[b * pos_ld + *col_ptr];
+  const float ang = __fdiv_rn(pos, timescale[i]);
+  sin_out[b * half + i] = sinf(ang);
+  cos_out[b * half + i] = cosf(ang);
+}
+
 float host_round_bf16(float f) {
   uint32_t u;
   memcpy(&u, &f, 4);
@@ -334,6 +347,16 @@ extern "C" int tnx_rmsnorm_splitk(void* stream, const float* ws, int split_k, co
                      (const uint16_t*)nullptr, res_pre, h_out, w, res_post, y, D, eps, flavor, ws, split_k,
                      (int64_t)(M * D));
   TNX_CHECK_LAUNCH("rmsnorm_splitk");
+  return TNX_OK;
+}
+
+extern "C" int tnx_rope_table(void* stream, const int32_t* positions, int64_t pos_ld, const int32_t* col_ptr,
+                              int64_t B, const float* timescale, int dh, float* sin_out, float* cos_out) {
+  TNX_REQUIRE(positions && col_ptr && timescale && sin_out && cos_out, "rope_table: null pointer");
+  TNX_REQUIRE(B > 0 && dh % 2 == 0 && dh >= 2 && dh <= 2048, "rope_table: bad shape");
+  hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)B), dim3((unsigned)(dh / 2 < 64 ? 64 : dh / 2)), 0,
+                     as_stream(stream), positions, pos_ld, col_ptr, timescale, dh / 2, sin_out, cos_out);
+  TNX_CHECK_LAUNCH("rope_table");
   return TNX_OK;
 }
 

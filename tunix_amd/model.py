@@ -245,6 +245,9 @@ class Runner:
       self.act = torch.empty(M, F, dtype=bf, device=dev)
     # tuning knob: TUNIX_SPLIT_K='{"o": 4}' pins the k split of the linears with that name
     self.split_k_override = json.loads(os.environ.get("TUNIX_SPLIT_K", "{}"))
+    self.fuse_rope = True   # decode: RoPE + cache write inside the attention kernel where it can
+    self.rope_sin = torch.empty(B, max(cfg.head_dim // 2, 1), dtype=torch.float32, device=dev)
+    self.rope_cos = torch.empty_like(self.rope_sin)
     self.next_tpart = None
     if 64 < M <= 1024 and not cfg.num_experts and model.layers and "gu" in model.layers[0]:
       n_planes = math.ceil(M / 128) * math.ceil(model.layers[0]["gu"].N / 128)
@@ -352,28 +355,37 @@ class Runner:
     emb_scale = math.sqrt(cfg.embed_dim) if cfg.family == "gemma3" else 1.0
     ops.embed(m.embed, tokens, col_ptr, B, T, emb_scale, self.h)
     pending = 1  # split count of a down-projection whose partial planes still await their sum
+    if (T == 1 and self.fuse_rope and m.layers and "q_norm" not in m.layers[0]
+        and _ROPE[cfg.family] == L.TNX_ROPE_LLAMA and cfg.head_dim == 128):
+      # one table of this step's sines / cosines for all layers (they share theta)
+      ops.rope_table(positions, col_ptr, B, m.layers[0]["timescale"], cfg.head_dim, self.rope_sin, self.rope_cos)
     for i, ly in enumerate(m.layers):
       self.norm_after(pending, ly["attn_norm"], M)
       pending = 1
       qkv_split = self.linear(ly["qkv"], self.xn, self.qkv, M, defer=True)
-      rd = L.RopeDesc()
-      rd.B, rd.T, rd.S = B, T, self.S
-      rd.Hq, rd.Hkv, rd.dh = cfg.num_heads, cfg.num_kv_heads, cfg.head_dim
-      rd.rope_flavor, rd.rope_scale = _ROPE[cfg.family], ly["rope_scale"]
-      rd.timescale = ly["timescale"].data_ptr()
-      if "q_norm" in ly:
-        rd.qk_norm = flavor
-        rd.norm_eps = cfg.norm_eps if cfg.family == "qwen3" else 1e-6
-        rd.q_norm_w, rd.k_norm_w = ly["q_norm"].data_ptr(), ly["k_norm"].data_ptr()
-      else:
-        rd.qk_norm = -1
-      rd.q_prescale = cfg.query_pre_attn_scalar if cfg.family == "gemma3" else 0.0
-      rd.qkv, rd.positions, rd.pos_ld = self.qkv.data_ptr(), positions.data_ptr(), positions.shape[1]
-      if qkv_split > 1:  # the rope kernel sums the partial planes itself
-        rd.qkv_ws, rd.split_k = self.splitk_ws.data_ptr(), qkv_split
-      rd.col_ptr = col_ptr.data_ptr()
-      rd.q_out, rd.kcache, rd.vcache = self.q.data_ptr(), kcache[i].data_ptr(), vcache[i].data_ptr()
-      ops.rope_kvwrite(rd)
+      # decode step of a model without q/k norm and with the Llama rotation: the attention kernel
+      # rotates q / k and writes the cache itself, and the stand-alone launch is dropped
+      fuse_rope = (T == 1 and "q_norm" not in ly and _ROPE[cfg.family] == L.TNX_ROPE_LLAMA
+                   and cfg.head_dim == 128 and self.fuse_rope)
+      if not fuse_rope:
+        rd = L.RopeDesc()
+        rd.B, rd.T, rd.S = B, T, self.S
+        rd.Hq, rd.Hkv, rd.dh = cfg.num_heads, cfg.num_kv_heads, cfg.head_dim
+        rd.rope_flavor, rd.rope_scale = _ROPE[cfg.family], ly["rope_scale"]
+        rd.timescale = ly["timescale"].data_ptr()
+        if "q_norm" in ly:
+          rd.qk_norm = flavor
+          rd.norm_eps = cfg.norm_eps if cfg.family == "qwen3" else 1e-6
+          rd.q_norm_w, rd.k_norm_w = ly["q_norm"].data_ptr(), ly["k_norm"].data_ptr()
+        else:
+          rd.qk_norm = -1
+        rd.q_prescale = cfg.query_pre_attn_scalar if cfg.family == "gemma3" else 0.0
+        rd.qkv, rd.positions, rd.pos_ld = self.qkv.data_ptr(), positions.data_ptr(), positions.shape[1]
+        if qkv_split > 1:  # the rope kernel sums the partial planes itself
+          rd.qkv_ws, rd.split_k = self.splitk_ws.data_ptr(), qkv_split
+        rd.col_ptr = col_ptr.data_ptr()
+        rd.q_out, rd.kcache, rd.vcache = self.q.data_ptr(), kcache[i].data_ptr(), vcache[i].data_ptr()
+        ops.rope_kvwrite(rd)
       ad = L.AttnDesc()
       ad.B, ad.T, ad.S = B, T, self.S
       ad.Hq, ad.Hkv, ad.dh = cfg.num_heads, cfg.num_kv_heads, cfg.head_dim
@@ -384,6 +396,12 @@ class Runner:
       ad.tokens, ad.tok_ld, ad.col_ptr = tokens.data_ptr(), tokens.shape[1], col_ptr.data_ptr()
       ad.kv_chunk = self.kv_chunk if T == 1 else 0
       ad.ws, ad.out = self.attn_ws.data_ptr(), self.attn.data_ptr()
+      if fuse_rope:
+        if qkv_split > 1:
+          ad.qkv_ws, ad.qkv_split = self.splitk_ws.data_ptr(), qkv_split
+        else:
+          ad.qkv = self.qkv.data_ptr()
+        ad.rope_sin, ad.rope_cos = self.rope_sin.data_ptr(), self.rope_cos.data_ptr()
       ops.gqa_attn(ad)
       if cfg.family == "gemma3":
         self.linear(ly["o"], self.attn, self.tmp, M)

@@ -125,6 +125,11 @@ def rope_kvwrite(desc: L.RopeDesc):
   L.check(L.lib().tnx_qknorm_rope_kvwrite(_stream(), C.byref(desc)), "tnx_qknorm_rope_kvwrite")
 
 
+def rope_table(positions, col_ptr, B, timescale, dh, sin_out, cos_out):
+  L.check(L.lib().tnx_rope_table(_stream(), _ptr(positions), positions.shape[1], _ptr(col_ptr), B,
+                                 _ptr(timescale), dh, _ptr(sin_out), _ptr(cos_out)), "tnx_rope_table")
+
+
 def attn_ws_bytes(B, T, S, Hq, dh, kv_chunk) -> int:
   return int(L.lib().tnx_attn_ws_bytes(B, T, S, Hq, dh, kv_chunk))
 
