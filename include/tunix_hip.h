@@ -298,6 +298,16 @@ typedef struct tnx_lmhead_desc {
   float* entropy;             /* fp32 [M] or NULL: -sum_v p_v log p_v of the (temperature-
                                  scaled) distribution, compute_entropy_from_logits
                                  tunix/rl/common.py:1136-1148                                */
+  /* Optional whole-vocabulary categorical draw inside the head (draw_id != NULL): what
+   * tnx_sample_topk does for top_p >= 1 without top_k (sample_top_p, sampler.py:119-121),
+   * jax.random.categorical over logits / temperature with the noise of fold_in(key, *step),
+   * without materialising the logits. */
+  float* part_draw;           /* fp32 workspace [M, n_vblocks, 3]                            */
+  uint32_t draw_key0, draw_key1;
+  int draw_rng_variant;       /* as rng_variant of tnx_sample_topk                           */
+  const int32_t* draw_step_ptr;
+  int32_t* draw_id;           /* int32 [M]                                                   */
+  float* draw_logp;           /* fp32 [M]: log-softmax at the drawn id, or NULL              */
 } tnx_lmhead_desc;
 int64_t tnx_lmhead_nblocks(int64_t V);
 int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* h_desc);

@@ -413,6 +413,49 @@ def test_lmhead_forbidden_and_ties(gpu):
   assert best.cpu().tolist() == [511] * M
 
 
+@pytest.mark.parametrize("M,V,variant", [(128, 4096, 0), (40, 1040, 1), (7, 512, 0)])
+def test_lmhead_categorical_draw_matches_oracle(gpu, M, V, variant):
+  """The whole-vocabulary draw inside the head: ids equal jax.random.categorical (restated by the
+  oracle) over the logits the kernel itself produced, divided by the temperature, with a
+  forbidden id; the log-probabilities agree to 2e-5; tnx_sample_topk on the materialised logits
+  draws the same ids."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  D, temp, step = 256, 0.9, 41
+  x, w = rnd((M, D), 54), rnd((D, V), 55, 0.3)
+  gx, gw = bf(x).to(gpu), bf(w).t().contiguous().to(gpu)
+  key = TF.prng_key(777)
+  nvb = ops.lmhead_nblocks(V)
+  d = L.LmHeadDesc()
+  d.M, d.D, d.V, d.x, d.w_bf16, d.temperature = M, D, V, gx.data_ptr(), gw.data_ptr(), temp
+  part = torch.empty(M * nvb * 4, dtype=torch.float32, device=gpu)
+  pdraw = torch.empty(M * nvb * 3, dtype=torch.float32, device=gpu)
+  lg_out = torch.empty(M, V, dtype=torch.float32, device=gpu)
+  ids = torch.empty(M, dtype=torch.int32, device=gpu)
+  lp = torch.empty(M, dtype=torch.float32, device=gpu)
+  stp = torch.tensor([step], dtype=torch.int32, device=gpu)
+  fb = torch.tensor([3], dtype=torch.int32, device=gpu)
+  d.part, d.logits_out, d.forbidden, d.n_forbidden = part.data_ptr(), lg_out.data_ptr(), fb.data_ptr(), 1
+  d.part_draw, d.draw_key0, d.draw_key1, d.draw_rng_variant = pdraw.data_ptr(), int(key[0]), int(key[1]), variant
+  d.draw_step_ptr, d.draw_id, d.draw_logp = stp.data_ptr(), ids.data_ptr(), lp.data_ptr()
+  ops.lmhead(d)
+  torch.cuda.synchronize()
+  raw = lg_out.cpu()
+  masked = raw.clone()
+  masked[:, 3] = -np.inf
+  tok_ref, lp_ref = SR.sample_top_p(masked, TF.fold_in(key, step), temp, 1.0, None, partitionable=bool(variant))
+  assert ids.cpu().long().tolist() == tok_ref.tolist()
+  np.testing.assert_allclose(lp.cpu().numpy(), lp_ref.numpy(), atol=2e-5)
+  assert len(set(ids.cpu().tolist())) > 1 or M < 4
+  ids2 = torch.empty_like(ids)
+  lp2 = torch.empty_like(lp)
+  ws = torch.empty(ops.sample_topk_ws_bytes(M, V, 0) // 4, dtype=torch.float32, device=gpu)
+  ops.sample_topk(lg_out, 0, 1.0, temp, (int(key[0]), int(key[1])), variant, stp, ws, ids2, lp2, forbidden=fb)
+  torch.cuda.synchronize()
+  assert torch.equal(ids, ids2)
+  np.testing.assert_allclose(lp.cpu().numpy(), lp2.cpu().numpy(), atol=2e-5)
+
+
 @pytest.mark.parametrize("V", [3000, 40001])
 @pytest.mark.parametrize("segmented", [False, True])
 @pytest.mark.parametrize("k,top_p,variant", [(50, 1.0, 0), (50, 0.7, 0), (8, 0.9, 1), (0, 1.0, 0)])

@@ -8,6 +8,7 @@
 #include <mutex>
 
 #include "gemm_tile.h"
+#include "rng.h"
 
 namespace {
 
@@ -31,6 +32,11 @@ struct LHArgs {
   int64_t nvb;
   float* logits_out;
   float* part_ent;   // optional [M, nvb]: sum of exp(l - max) * l per block, for the entropy
+  // optional whole-vocabulary categorical draw (Gumbel-max with jax's threefry stream)
+  float* part_draw;  // [M, nvb, 3]: best (logit + noise), its id, its logit
+  uint32_t key0, key1;
+  int variant;
+  const int32_t* step_ptr;
 };
 
 constexpr float kNegInf = -__builtin_inff();
@@ -41,6 +47,9 @@ struct Stat {
   float sum;
   float tgt;
   float wsum;  // sum of exp(l - mx) * l  (entropy = logsumexp - wsum / sum)
+  float gv;    // best logit + gumbel noise, its column and its logit (the categorical draw)
+  int gi;
+  float gl;
 };
 // Merge two statistics; `a` covers lower column indices than `b`.
 __device__ __forceinline__ Stat merge(const Stat& a, const Stat& b) {
@@ -52,6 +61,10 @@ __device__ __forceinline__ Stat merge(const Stat& a, const Stat& b) {
   r.sum = a.sum * wa + b.sum * wb;
   r.wsum = a.wsum * wa + b.wsum * wb;
   r.tgt = fmaxf(a.tgt, b.tgt);
+  const bool tb = b.gv > a.gv || (b.gv == a.gv && b.gi < a.gi);  // larger value, then lower index
+  r.gv = tb ? b.gv : a.gv;
+  r.gi = tb ? b.gi : a.gi;
+  r.gl = tb ? b.gl : a.gl;
   return r;
 }
 
@@ -102,6 +115,12 @@ __global__ __launch_bounds__(DENSE ? 512 : 256) void lmhead_kernel(const LHArgs 
     if (fid == colA) okA = false;
     if (fid == colB) okB = false;
   }
+  // fold_in(key, step) for the draw: threefry of the key over the counter pair (0, step)
+  uint32_t ks0 = 0u, ks1 = 0u;
+  if (a.part_draw) {
+    ks1 = (uint32_t)(*a.step_ptr);
+    threefry2x32(a.key0, a.key1, ks0, ks1);
+  }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -146,9 +165,35 @@ __global__ __launch_bounds__(DENSE ? 512 : 256) void lmhead_kernel(const LHArgs 
         se += __shfl_xor(se, o, 64);
         we += __shfl_xor(we, o, 64);
       }
+      // the draw: arg-max of logit + gumbel noise over the 32 columns of this row in the wave
+      // (noise of element (row, v): counter row * V + v of M * V, one draw over [M, V])
+      float gv = kNegInf, gl = kNegInf;
+      int gi = 0x7fffffff;
+      if (a.part_draw && rok) {
+        const uint64_t tot = (uint64_t)a.M * (uint64_t)a.V;
+        const float na = la == kNegInf ? kNegInf
+            : la + gumbel_from_bits(random_bits(ks0, ks1, (uint64_t)row * a.V + colA, tot, a.variant));
+        const float nb = lb == kNegInf ? kNegInf
+            : lb + gumbel_from_bits(random_bits(ks0, ks1, (uint64_t)row * a.V + colB, tot, a.variant));
+        const bool tb = nb > na;   // colA < colB: ties keep the lower column
+        gv = tb ? nb : na;
+        gi = tb ? (int)colB : (int)colA;
+        gl = tb ? lb : la;
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) {
+          const float ov = __shfl_xor(gv, o, 64), ol = __shfl_xor(gl, o, 64);
+          const int oi = __shfl_xor(gi, o, 64);
+          if (ov > gv || (ov == gv && oi < gi)) {
+            gv = ov;
+            gi = oi;
+            gl = ol;
+          }
+        }
+      }
       if (lm == 0) {
         Stat r;
         r.mx = mx; r.idx = idx; r.sum = se; r.tgt = st.tgt; r.wsum = we;
+        r.gv = gv; r.gi = gi; r.gl = gl;
         sRed[wave * (MT * 16) + rl] = r;
       }
     }
@@ -163,6 +208,12 @@ __global__ __launch_bounds__(DENSE ? 512 : 256) void lmhead_kernel(const LHArgs 
     p[2] = r.sum;
     p[3] = r.tgt;
     if (a.part_ent) a.part_ent[(m0 + tid) * a.nvb + vb] = r.wsum;
+    if (a.part_draw) {
+      float* q = a.part_draw + ((m0 + tid) * a.nvb + vb) * 3;
+      q[0] = r.gv;
+      q[1] = __int_as_float(r.gi);
+      q[2] = r.gl;
+    }
   }
 }
 
@@ -170,7 +221,9 @@ __global__ __launch_bounds__(DENSE ? 512 : 256) void lmhead_kernel(const LHArgs 
 __global__ __launch_bounds__(64) void lmhead_finish_kernel(const float* part, int64_t nvb,
                                                            int32_t* best_id, float* best_logp,
                                                            float* target_logp, float* lse_out,
-                                                           const float* part_ent, float* entropy_out) {
+                                                           const float* part_ent, float* entropy_out,
+                                                           const float* part_draw, int32_t* draw_id,
+                                                           float* draw_logp) {
   const int64_t row = blockIdx.x;
   const int lane = threadIdx.x;
   const float* p = part + row * nvb * 4;
@@ -178,10 +231,16 @@ __global__ __launch_bounds__(64) void lmhead_finish_kernel(const float* part, in
   const int64_t per = (nvb + 63) / 64;
   Stat r;
   r.mx = kNegInf; r.idx = 0x7fffffff; r.sum = 0.f; r.tgt = kNegInf; r.wsum = 0.f;
+  r.gv = kNegInf; r.gi = 0x7fffffff; r.gl = kNegInf;
   for (int64_t c = lane * per; c < min(nvb, (lane + 1) * per); ++c) {
     Stat b;
     b.mx = p[c * 4]; b.idx = __float_as_int(p[c * 4 + 1]); b.sum = p[c * 4 + 2]; b.tgt = p[c * 4 + 3];
     b.wsum = part_ent ? part_ent[row * nvb + c] : 0.f;
+    b.gv = kNegInf; b.gi = 0x7fffffff; b.gl = kNegInf;
+    if (part_draw) {
+      const float* q = part_draw + (row * nvb + c) * 3;
+      b.gv = q[0]; b.gi = __float_as_int(q[1]); b.gl = q[2];
+    }
     r = merge(r, b);
   }
 #pragma unroll
@@ -192,6 +251,9 @@ __global__ __launch_bounds__(64) void lmhead_finish_kernel(const float* part, in
     b.sum = __shfl_xor(r.sum, o, 64);
     b.tgt = __shfl_xor(r.tgt, o, 64);
     b.wsum = __shfl_xor(r.wsum, o, 64);
+    b.gv = __shfl_xor(r.gv, o, 64);
+    b.gi = __shfl_xor(r.gi, o, 64);
+    b.gl = __shfl_xor(r.gl, o, 64);
     r = (lane & o) ? merge(b, r) : merge(r, b);  // the lower lane holds the lower columns
   }
   if (lane == 0) {
@@ -201,6 +263,8 @@ __global__ __launch_bounds__(64) void lmhead_finish_kernel(const float* part, in
     if (target_logp) target_logp[row] = r.tgt - lse;
     if (lse_out) lse_out[row] = lse;
     if (entropy_out) entropy_out[row] = lse - r.wsum / r.sum;  // -sum p log p
+    if (draw_id) draw_id[row] = r.gi;
+    if (draw_logp) draw_logp[row] = r.gl - lse;
   }
 }
 
@@ -260,6 +324,14 @@ extern "C" int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* d) {
   a.logits_out = d->logits_out;
   TNX_REQUIRE(!d->entropy || d->part_entropy, "lmhead: entropy needs the part_entropy workspace [M, n_vblocks]");
   a.part_ent = d->entropy ? d->part_entropy : nullptr;
+  a.part_draw = nullptr; a.key0 = a.key1 = 0; a.variant = 0; a.step_ptr = nullptr;
+  if (d->draw_id) {
+    TNX_REQUIRE(d->part_draw && d->draw_step_ptr, "lmhead: the draw needs the part_draw workspace [M, n_vblocks, 3] and a step pointer");
+    TNX_REQUIRE(d->draw_rng_variant == 0 || d->draw_rng_variant == 1, "lmhead: rng_variant must be 0 or 1");
+    TNX_REQUIRE(d->temperature > 0.f, "lmhead: the draw needs a positive temperature");
+    a.part_draw = d->part_draw; a.key0 = d->draw_key0; a.key1 = d->draw_key1; a.variant = d->draw_rng_variant;
+    a.step_ptr = d->draw_step_ptr;
+  }
   hipStream_t st = as_stream(stream);
   int rc;
   const bool dense = d->w_bf16 != nullptr;
@@ -269,7 +341,8 @@ extern "C" int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* d) {
   else rc = dense ? launch_lmhead<8, true>(st, a) : launch_lmhead<8, false>(st, a);
   if (rc) return rc;
   hipLaunchKernelGGL(lmhead_finish_kernel, dim3((unsigned)d->M), dim3(64), 0, st, a.part, a.nvb,
-                     d->best_id, d->best_logp, d->target_logp, d->lse, a.part_ent, d->entropy);
+                     d->best_id, d->best_logp, d->target_logp, d->lse, a.part_ent, d->entropy, a.part_draw,
+                     d->draw_id, d->draw_logp);
   TNX_CHECK_LAUNCH("lmhead_finish");
   return TNX_OK;
 }

@@ -114,6 +114,14 @@ class Sampler:
       runner.run_head(x, runner.B, best_id=runner.best_id, best_logp=runner.best_logp,
                       forbidden=mode["forbidden"], logits_out=runner.logits)
       ids, lp = runner.best_id, (runner.best_logp if want_lp else None)
+    elif mode["top_k"] == 0 and mode["top_p"] >= 1.0:
+      # the plain categorical draw (the reference's default rollout configuration) happens inside
+      # the head kernel: no logits in HBM, no sampling launch
+      runner.run_head(x, runner.B, temperature=mode["temperature"], forbidden=mode["forbidden"],
+                      logits_out=runner.logits,
+                      draw=dict(part=mode["part_draw"], key=mode["key"], variant=self.rng_variant,
+                                step=st.step, ids=mode["ids"], logp=mode["logp"]))
+      ids, lp = mode["ids"], (mode["logp"] if want_lp else None)
     else:
       runner.run_head(x, runner.B, best_id=runner.best_id, logits_out=runner.logits)
       ops.sample_topk(runner.logits, mode["top_k"], mode["top_p"], mode["temperature"], mode["key"],
@@ -222,7 +230,11 @@ class Sampler:
                                  dtype=torch.float32, device=dev),
                   ids=torch.empty(B, dtype=torch.int32, device=dev),
                   logp=torch.empty(B, dtype=torch.float32, device=dev))
-    need_logits = return_logits or mode["name"] == "top_p"
+      if k == 0 and top_p >= 1.0:
+        mode["part_draw"] = torch.empty(B * ops.lmhead_nblocks(cfg.vocab_size) * 3, dtype=torch.float32,
+                                        device=dev)
+    in_head_draw = mode["name"] == "top_p" and mode["top_k"] == 0 and mode["top_p"] >= 1.0
+    need_logits = return_logits or (mode["name"] == "top_p" and not in_head_draw)
     runner = Runner(model, B, 1, S, pad, want_logits=need_logits)
 
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]

@@ -454,7 +454,7 @@ class Runner:
 
   def head_desc(self, x, rows, part, temperature=1.0, targets=None, best_id=None, best_logp=None,
                 target_logp=None, lse=None, logits_out=None, forbidden=None, entropy=None,
-                part_entropy=None) -> L.LmHeadDesc:
+                part_entropy=None, draw=None) -> L.LmHeadDesc:
     cfg, m = self.cfg, self.model
     d = L.LmHeadDesc()
     d.M, d.D, d.V = rows, cfg.embed_dim, cfg.vocab_size
@@ -476,6 +476,13 @@ class Runner:
       if tns is not None:
         setattr(d, name, tns.data_ptr())
     d.part = part.data_ptr()
+    if draw is not None:  # whole-vocabulary categorical draw inside the head
+      d.part_draw = draw["part"].data_ptr()
+      d.draw_key0, d.draw_key1 = int(draw["key"][0]), int(draw["key"][1])
+      d.draw_rng_variant, d.draw_step_ptr = int(draw["variant"]), draw["step"].data_ptr()
+      d.draw_id = draw["ids"].data_ptr()
+      if draw.get("logp") is not None:
+        d.draw_logp = draw["logp"].data_ptr()
     return d
 
   def run_head(self, x, rows, **kw):
