@@ -244,6 +244,8 @@ def main():
   ap.add_argument("--layers", type=int, default=0, help="debug only: fewer layers (invalidates the metric)")
   ap.add_argument("--no-cpu-baseline", action="store_true")
   ap.add_argument("--kernel-iters", type=int, default=20)
+  ap.add_argument("--sampling-steps", type=int, default=64,
+                  help="decode steps of the extra temperature-1.0 measurement (0: skip it)")
   ap.add_argument("--kernels-only", action="store_true",
                   help="profiling aid: one layer, no prefill / decode; only the per-kernel loops at "
                        "context prompt + gen / 2 (prints the kernel table, not the metric)")
@@ -352,6 +354,27 @@ def main():
   mean_ctx = (step_first + 1 + step_last) / 2.0 + 0.5
   log(f"decode: {K} steps, {ms_per_step:.3f} ms/step, {value:.0f} tokens/s, mean context {mean_ctx:.1f}")
 
+  # The workload's other variant: temperature 1.0, top_p 1.0, no top-k (the reference's default
+  # rollout sampling: one categorical draw over the whole vocabulary per row and step), through
+  # the public Sampler call; two rollouts of different length, so that prefill, graph capture
+  # and host work cancel.  Reported beside the headline (greedy) number, never instead of it.
+  sampling = None
+  if args.sampling_steps > 0:
+    prompts = [ids[b] for b in range(B)]
+    times = []
+    for n in (4, 4 + args.sampling_steps):
+      torch.cuda.synchronize()
+      t0 = time.perf_counter()
+      sampler(prompts, n, max_prompt_length=P, temperature=1.0, top_p=1.0, top_k=None, seed=7,
+              return_logprobs=True, eos_tokens=[-1])
+      torch.cuda.synchronize()
+      times.append(time.perf_counter() - t0)
+    s_ms = (times[1] - times[0]) / args.sampling_steps * 1e3
+    sampling = {"mode": "temperature 1.0, top_p 1.0, no top-k (categorical over the vocabulary)",
+                "steps": args.sampling_steps, "ms_per_step": round(s_ms, 4),
+                "tokens_per_s": round(B / (s_ms * 1e-3), 1), "context_range": [P + 4, P + 4 + args.sampling_steps]}
+    log(f"sampling variant: {s_ms:.3f} ms/step over {args.sampling_steps} steps from context {P + 4}")
+
   kern = kernel_breakdown(model, runner, st, int(round(mean_ctx)), args.kernel_iters)
   for name, v in kern.items():
     log(f"  {name:16s} {v['ms'] * 1e3:8.1f} us/launch  {v['gbs']:7.0f} GB/s  {v['tflops']:7.1f} TFLOP/s"
@@ -375,6 +398,8 @@ def main():
                       "TFLOPs": round(v["tflops"], 1), "ms_per_step": round(v["step_ms"], 4)}
                   for k, v in kern.items()},
   }
+  if sampling is not None:
+    result["sampling_variant"] = sampling
   if not args.no_cpu_baseline:
     threads = min(16, os.cpu_count() or 1)
     t0 = time.time()
