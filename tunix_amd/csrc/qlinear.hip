@@ -447,7 +447,7 @@ int check_desc(const tnx_qlinear_desc* d) {
   if (d->next_tpart) {
     TNX_REQUIRE(d->epilogue == TNX_EPI_SILU_MUL || d->epilogue == TNX_EPI_GELU_MUL,
                 "qlinear: next_tpart needs a *_MUL epilogue");
-    TNX_REQUIRE(d->split_k <= 1 && d->M > 64, "qlinear: next_tpart needs split_k == 1 and M > 64");
+    TNX_REQUIRE(d->split_k <= 1 && d->M > 32, "qlinear: next_tpart needs split_k == 1 and M > 32");
     TNX_REQUIRE(d->next_a_t && d->next_rank > 0 && d->next_rank % 16 == 0 && d->next_rank <= 64,
                 "qlinear: next_rank must be a multiple of 16 and <= 64 (got %d)", d->next_rank);
     TNX_REQUIRE((d->N / 2) % 8 == 0, "qlinear: next_tpart needs N/2 %% 8 == 0");
@@ -553,8 +553,9 @@ extern "C" int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* d) {
   hipStream_t st = as_stream(stream);
   if (a.M <= 16) return launch_qlinear<1, 2>(st, a);
   if (a.M <= 32) return launch_qlinear<2, 2>(st, a);
-  if (a.M <= 64) return launch_qlinear<4, 2>(st, a);
-  // 128 x 128 work-group tiles; the 256-column variant (NT = 4) is not dispatched: its
+  // 33+ rows: 128 x 128 work-group tiles (rows past M cost no fetches: they are read as zeros
+  // through the buffer bounds); the row tile of the small-batch kernel would re-read the weights
+  // no less and runs a slower loop; the 256-column variant (NT = 4) is not dispatched: its
   // accumulators need AGPRs, and the compiler wraps loops over AGPR accumulators in register
   // copies that cost more than the halved LDS traffic gains
   if (scales_per_tile(a.group) == 2) return launch_qgemm128<2, 2>(st, a);
