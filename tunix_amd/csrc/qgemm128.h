@@ -1,6 +1,7 @@
-// The quantised GEMM for 65+ activation rows (rollout batch, prefill, per-token logps): one
-// work-group = 8 waves = two per SIMD, output tile 128 rows x (64 * NT) columns; a wave covers
-// 128 rows x (16 * NT) columns over one half of every k-tile.  At 128 rows the op sits past the MFMA/HBM ridge of the machine (2 * 128 flop
+// The quantised GEMM (rollout batch, prefill, per-token logps): one work-group = 8 waves = two
+// per SIMD, output tile 16 * MT rows x (64 * NT) columns (MT = 8: 128 rows; 1, 2, 4 for decode
+// batches of up to 16, 32, 64 rows); a wave covers all rows x (16 * NT) columns over one half
+// of every k-tile.  At 128 rows the op sits past the MFMA/HBM ridge of the machine (2 * 128 flop
 // per 0.53 B of weights), so the loop is built around keeping the matrix pipe fed:
 //
 //   * a k-tile (128 k) is four k-steps of 8 * NT MFMAs (16x16x32 bf16).  While the MFMAs of step
@@ -58,10 +59,15 @@ __device__ unsigned long long tnx_stamps[8];
 
 // 512 threads: waves 0-3 and 4-7 share the four column groups and split every k-tile between
 // them (k-steps 0,1 | 2,3), which puts two waves on each SIMD at 256 registers each.
-template <int NT, int SPT>
+// MT = row tiles of 16 (8 for 65+ rows; 1, 2, 4 for decode batches of up to 16, 32, 64 rows: the
+// weight stream and its dequantisation are the same, the MFMA, fragment and activation work
+// shrink with the rows).
+template <int NT, int SPT, int MT>
 __global__ __launch_bounds__(512)
 void qgemm128_kernel(const QLArgs a) {
-  constexpr int MT = 8, HM = 4, PF = 3;
+  constexpr int HM = (MT + 1) / 2, PF = 3;   // HM: row tiles a wave finishes after the k halves meet
+  constexpr int ROWS = 16 * MT;
+  constexpr int AP = (ROWS + 31) / 32;       // passes of the activation copy (512 threads x 16 B = 32 rows)
   constexpr int SW = SPT / 2;  // scales of one wave's two k-steps
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -85,7 +91,7 @@ void qgemm128_kernel(const QLArgs a) {
   // of the kernel waits on memory except the loads of the first tiles
   const float lvl0 = rbf(code_level_imm(a.qtype, tid & 15)), lvl1 = rbf(code_level_imm(a.qtype, (tid >> 4) & 15));
   const uint32_t lane_off = (uint32_t)lane * 4u;
-  const int64_t m0 = (int64_t)blockIdx.x * 128;
+  const int64_t m0 = (int64_t)blockIdx.x * ROWS;
   const int64_t ntile0 = ((int64_t)blockIdx.y * 4 + wn) * NT;
   const int64_t ntiles = a.N / 16;
   const int ktiles = (int)(a.K / KTILE);
@@ -116,11 +122,11 @@ void qgemm128_kernel(const QLArgs a) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) zero_acc(acc[mt][nt]);
 
-  u32x4 a_next[HM];
+  u32x4 a_next[AP];
   u32x2 ring_c[PF][NT];
   uint32_t ring_s[PF][NT];
   float sc[PF][NT][SW];   // the scales of a ring stage as fp32
-  u32x4 af[2][2][HM];     // activation fragments of this wave's two k-steps, both row halves
+  u32x4 af[2][MT];        // activation fragments of this wave's two k-steps
   u32x4 bfr[2][NT];       // weight fragments of the two k-steps
   uint32_t lp[NT][4];     // table entries (f16 level pairs) of the k-step after the next
 
@@ -207,7 +213,7 @@ void qgemm128_kernel(const QLArgs a) {
     const uint32_t m = 0u - (uint32_t)ut;
     const uint32_t base = xbase ^ ((xbase ^ tbase) & m), stride = xstride ^ ((xstride ^ tstride) & m);
 #pragma unroll
-    for (int c = 0; c < HM; ++c)
+    for (int c = 0; c < AP; ++c)
       a_next[c] = __builtin_amdgcn_raw_buffer_load_b128(r, base + (uint32_t)c * stride, s, 0);
   };
   auto load_w = [&](auto Dc, int kt) {
@@ -268,27 +274,23 @@ void qgemm128_kernel(const QLArgs a) {
   uint32_t a_rd_nxt = a_rd + kBigABytes;
   uint32_t a_wr = kBigLutBytes + (uint32_t)((tid >> 4) * A_LD + (tid & 15) * 8) * 2u;
   uint32_t a_wr_nxt = a_wr + kBigABytes;
-  auto read_a = [&](u32x4 (&dst)[2][HM], uint32_t base, auto Jc) {
+  auto read_a = [&](u32x4 (&dst)[MT], uint32_t base, auto Jc) {
     constexpr int J = decltype(Jc)::value;
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int m = 0; m < HM; ++m)
-        dst[h][m] = lds_ld128(base + (uint32_t)(((h * 4 + m) * 16 * A_LD + J * 32) * 2));
+    for (int m = 0; m < MT; ++m) dst[m] = lds_ld128(base + (uint32_t)((m * 16 * A_LD + J * 32) * 2));
   };
+  // (with fewer than 32 rows the copy still moves 32: the extra rows are zeros or rows of
+  // nobody's tile, and land in LDS rows no fragment reads)
   auto store_a = [&](uint32_t base) {
 #pragma unroll
-    for (int c = 0; c < HM; ++c) lds_st128(base + (uint32_t)(c * 32 * A_LD * 2), a_next[c]);
+    for (int c = 0; c < AP; ++c) lds_st128(base + (uint32_t)(c * 32 * A_LD * 2), a_next[c]);
   };
   auto mfmas = [&](auto Jc) {
     constexpr int J = decltype(Jc)::value;
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int m = 0; m < MT; ++m)
 #pragma unroll
-      for (int m = 0; m < HM; ++m)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          acc[h * 4 + m][nt] = mfma16(af[J][h][m], bfr[J][nt], acc[h * 4 + m][nt]);
+      for (int nt = 0; nt < NT; ++nt) acc[m][nt] = mfma16(af[J][m], bfr[J][nt], acc[m][nt]);
   };
 
   // One k-tile of ring stage D = this wave's two k-steps.  On entry af[0] holds the activation
@@ -309,16 +311,16 @@ void qgemm128_kernel(const QLArgs a) {
     lut_issue(ic<dn>{}, ic<0>{}, lp);
     read_a(af[1], a_rd, ic<1>{});
     store_a(a_wr_nxt);
-#ifndef TNX_NO_SGB
+    if constexpr (MT == 8) {
 #pragma unroll
-    for (int i = 0; i < 8 * NT; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-      if (i < 4) __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      if (i >= 8 && i < 8 + HM) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      for (int i = 0; i < 8 * NT; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+        if (i < 4) __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (i >= 8 && i < 8 + AP) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      }
     }
-#endif
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
@@ -328,15 +330,15 @@ void qgemm128_kernel(const QLArgs a) {
     read_a(af[0], a_rd_nxt, ic<0>{});
     load_a(kt + 2);
     load_w(Dc, kt + PF);
-#ifndef TNX_NO_SGB
+    if constexpr (MT == 8) {
 #pragma unroll
-    for (int i = 0; i < 8 * NT; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      if (i >= 4 && i < 4 + HM + 2 * NT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      for (int i = 0; i < 8 * NT; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (i >= 4 && i < 4 + AP + 2 * NT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
     }
-#endif
     __builtin_amdgcn_sched_barrier(0);
     const uint32_t r = a_rd; a_rd = a_rd_nxt; a_rd_nxt = r;
     const uint32_t w = a_wr; a_wr = a_wr_nxt; a_wr_nxt = w;
@@ -383,8 +385,11 @@ void qgemm128_kernel(const QLArgs a) {
   }
   TNX_STAMP(3);
 
-  // The two k halves meet: each wave keeps the row half kh of its column group, hands the other
-  // half to its partner through the (now idle) table area and adds what the partner hands over.
+  // The two k halves meet: each wave keeps the row half kh of its column group (row tiles
+  // [kh * HM, ...); with a single row tile the first wave keeps it and the second keeps none),
+  // hands the other tiles to its partner through the (now idle) table area and adds what the
+  // partner hands over.
+  const bool has_rows = MT > 1 || kh == 0;
   f32x4 out[HM][NT];
   {
     __syncthreads();  // every wave is done with the table
@@ -394,7 +399,7 @@ void qgemm128_kernel(const QLArgs a) {
     for (int m = 0; m < HM; ++m)
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        const f32x4 v = kh ? acc[m][nt] : acc[HM + m][nt];
+        const f32x4 v = kh ? acc[m][nt] : acc[HM + m < MT ? HM + m : 0][nt];
         lds_st128(xw + (uint32_t)((m * NT + nt) * 1024), __builtin_bit_cast(u32x4, v));
       }
     __syncthreads();
@@ -402,15 +407,15 @@ void qgemm128_kernel(const QLArgs a) {
     for (int m = 0; m < HM; ++m)
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        const f32x4 own = kh ? acc[HM + m][nt] : acc[m][nt];
+        const f32x4 own = kh ? acc[HM + m < MT ? HM + m : 0][nt] : acc[m][nt];
         const f32x4 got = __builtin_bit_cast(f32x4, lds_ld128(xr + (uint32_t)((m * NT + nt) * 1024)));
         out[m][nt] = own + got;
       }
   }
-  const int64_t m0w = m0 + kh * 64;   // first row of this wave's tile
-  const uint32_t row_lds = (uint32_t)(kh * 64 * A_LD * 2);
+  const int64_t m0w = m0 + kh * (HM * 16);   // first row of this wave's tile
+  const uint32_t row_lds = (uint32_t)(kh * (HM * 16) * A_LD * 2);
 
-  if (lora_fast) {
+  if (lora_fast && has_rows) {
     // the t block sits in the activation buffer the last k-tile left as "next"
     const uint32_t tb = a_rd - (uint32_t)(kh * 64 * 2) + row_lds;
 #pragma unroll
@@ -433,7 +438,7 @@ void qgemm128_kernel(const QLArgs a) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) out[mt][nt][i] += a.lora_scale * part[mt][i];
     }
-  } else if (a.lora_rank > 0 && blockIdx.z == 0) {
+  } else if (a.lora_rank > 0 && blockIdx.z == 0 && !lora_fast && has_rows) {
     TileSrc s;
     s.M = a.M; s.K = a.K; s.x = a.x; s.row_index = nullptr; s.row_div = 1; s.x_rows = a.M;
     s.w_bf16 = nullptr; s.codes = a.codes; s.scales = a.scales; s.group = a.group; s.qtype = a.qtype;
@@ -466,25 +471,28 @@ void qgemm128_kernel(const QLArgs a) {
         }
     }
     uint16_t* act_s = reinterpret_cast<uint16_t*>(smem + act_lds);
+    if (has_rows) {
 #pragma unroll
-    for (int mt = 0; mt < HM; ++mt)
+      for (int mt = 0; mt < HM; ++mt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float g = rbf(out[mt][0][i]);
-        const float u = rbf(out[mt][1][i]);
-        const float act = a.epilogue == TNX_EPI_SILU_MUL ? silu_bf16(g) : gelu_tanh_bf16(g);
-        act_s[(kh * 64 + mt * 16 + lq * 4 + i) * ACT_LD + wn * 16 + lm] = f2bf(rbf(act) * u);
-      }
+        for (int i = 0; i < 4; ++i) {
+          const float g = rbf(out[mt][0][i]);
+          const float u = rbf(out[mt][1][i]);
+          const float act = a.epilogue == TNX_EPI_SILU_MUL ? silu_bf16(g) : gelu_tanh_bf16(g);
+          act_s[(kh * (HM * 16) + mt * 16 + lq * 4 + i) * ACT_LD + wn * 16 + lm] = f2bf(rbf(act) * u);
+        }
+    }
     __syncthreads();
     uint16_t* y = reinterpret_cast<uint16_t*>(a.y);
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
+    for (int c = 0; c < (ROWS * 8 + 511) / 512; ++c) {
       const int idx = tid + 512 * c, row = idx >> 3, ch = idx & 7;
+      if (row >= ROWS) break;
       const u32x4 v = lds_ld128(act_lds + (uint32_t)((row * ACT_LD + ch * 8) * 2));
       if (m0 + row < a.M && wgcol0 + ch * 8 + 8 <= ldy)
         *reinterpret_cast<u32x4*>(y + (m0 + row) * ldy + wgcol0 + ch * 8) = v;
     }
-    if (fuse_next) {
+    if (fuse_next && wv < MT) {   // one row tile per wave; fewer rows leave plane slots unwritten
       float* plane = a.next_tpart + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * 8192;
       {
         const int mt = wv;
@@ -502,7 +510,7 @@ void qgemm128_kernel(const QLArgs a) {
       }
     }
   } else {
-    store_tile<HM, NT>(a, m0w, a.M, ntile0, ntiles, out, [](int64_t r) { return r; });
+    if (has_rows) store_tile<HM, NT>(a, m0w, a.M, ntile0, ntiles, out, [](int64_t r) { return r; });
   }
   TNX_STAMP(5);
 }

@@ -119,53 +119,6 @@ __device__ __forceinline__ void store_tile(const QLArgs& a, int64_t m0, int64_t 
   }
 }
 
-template <int MT, int NT>
-__global__ __launch_bounds__(256) void qlinear_kernel(const QLArgs a) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  uint16_t* sA = reinterpret_cast<uint16_t*>(smem);  // [16*MT][A_LD]
-  uint32_t* sLut = tile_lut(smem, MT);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int64_t m0 = (int64_t)blockIdx.x * (MT * 16);
-  const int64_t ntile0 = ((int64_t)blockIdx.y * 4 + wave) * NT;
-  const int ktiles = (int)(a.K / KTILE);
-  const int kt_begin = blockIdx.z * a.ktiles_per_split;
-  const int kt_end = min(ktiles, kt_begin + a.ktiles_per_split);
-
-  build_lut(sLut, a.qtype, tid, 256);
-  const uint32_t* lut_lane = sLut + (lane & (TNX_LUT_COPIES - 1));
-
-  TileSrc s;
-  s.M = a.M; s.K = a.K; s.x = a.x; s.row_index = nullptr; s.row_div = 1; s.x_rows = a.M; s.w_bf16 = nullptr;
-  s.codes = a.codes; s.scales = a.scales; s.group = a.group; s.qtype = a.qtype;
-  s.ntiles = a.N / 16; s.lora_rank = a.lora_rank; s.t = a.t; s.t_ld = a.t_ld;
-  s.lora_b = a.lora_b; s.lora_scale = a.lora_scale;
-
-  f32x4 acc[MT][NT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) zero_acc(acc[mt][nt]);
-
-  tile_mainloop<MT, NT, false>(s, m0, ntile0, kt_begin, kt_end, sA, lut_lane, acc);
-
-  if (a.lora_rank > 0 && blockIdx.z == 0) {
-    int toff[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const int64_t col0 = (ntile0 + nt) * 16;
-      if (a.lora_nseg < 0) {
-        toff[nt] = (int)((ntile0 + nt) & 1) * a.lora_rank;  // interleaved gate/up pair
-      } else {
-        toff[nt] = a.lora_seg_toff[0];
-        for (int q = 1; q < a.lora_nseg; ++q)
-          if (col0 >= a.lora_seg_end[q - 1]) toff[nt] = a.lora_seg_toff[q];
-      }
-    }
-    tile_lora<MT, NT>(s, m0, ntile0, toff, acc);
-  }
-  store_tile<MT, NT>(a, m0, a.M, ntile0, s.ntiles, acc, [](int64_t r) { return r; });
-}
-
 // Grouped GEMM over routed tokens: blockIdx.x = expert, blockIdx.z = 16*MT-row block inside
 // the expert's route list.  Rows are gathered through sorted_route; outputs are indexed by
 // route.
@@ -447,7 +400,7 @@ int check_desc(const tnx_qlinear_desc* d) {
   if (d->next_tpart) {
     TNX_REQUIRE(d->epilogue == TNX_EPI_SILU_MUL || d->epilogue == TNX_EPI_GELU_MUL,
                 "qlinear: next_tpart needs a *_MUL epilogue");
-    TNX_REQUIRE(d->split_k <= 1 && d->M > 32, "qlinear: next_tpart needs split_k == 1 and M > 32");
+    TNX_REQUIRE(d->split_k <= 1, "qlinear: next_tpart needs split_k == 1");
     TNX_REQUIRE(d->next_a_t && d->next_rank > 0 && d->next_rank % 16 == 0 && d->next_rank <= 64,
                 "qlinear: next_rank must be a multiple of 16 and <= 64 (got %d)", d->next_rank);
     TNX_REQUIRE((d->N / 2) % 8 == 0, "qlinear: next_tpart needs N/2 %% 8 == 0");
@@ -466,26 +419,14 @@ int raise_lds_limit(Kern kern, size_t bytes) {
   return TNX_OK;
 }
 
-template <int MT, int NT>
-int launch_qlinear(hipStream_t st, const QLArgs& a) {
-  static std::once_flag once;
-  static int attr_rc = TNX_OK;
-  std::call_once(once, [] { attr_rc = raise_lds_limit(&qlinear_kernel<MT, NT>, tile_smem_bytes(MT)); });
-  if (attr_rc) return attr_rc;
-  dim3 grid((unsigned)cdiv(a.M, MT * 16), (unsigned)cdiv(a.N, 64 * NT), (unsigned)a.split_k);
-  hipLaunchKernelGGL((qlinear_kernel<MT, NT>), grid, dim3(256), tile_smem_bytes(MT), st, a);
-  TNX_CHECK_LAUNCH("qlinear");
-  return TNX_OK;
-}
-
-template <int NT, int SPT>
+template <int NT, int SPT, int MT>
 int launch_qgemm128(hipStream_t st, const QLArgs& a) {
   static std::once_flag once;
   static int attr_rc = TNX_OK;
-  std::call_once(once, [] { attr_rc = raise_lds_limit(&qgemm128_kernel<NT, SPT>, kBigSmemBytes); });
+  std::call_once(once, [] { attr_rc = raise_lds_limit(&qgemm128_kernel<NT, SPT, MT>, kBigSmemBytes); });
   if (attr_rc) return attr_rc;
-  dim3 grid((unsigned)cdiv(a.M, 128), (unsigned)cdiv(a.N, 64 * NT), (unsigned)a.split_k);
-  hipLaunchKernelGGL((qgemm128_kernel<NT, SPT>), grid, dim3(512), kBigSmemBytes, st, a);
+  dim3 grid((unsigned)cdiv(a.M, 16 * MT), (unsigned)cdiv(a.N, 64 * NT), (unsigned)a.split_k);
+  hipLaunchKernelGGL((qgemm128_kernel<NT, SPT, MT>), grid, dim3(512), kBigSmemBytes, st, a);
   TNX_CHECK_LAUNCH("qgemm128");
   return TNX_OK;
 }
@@ -551,15 +492,16 @@ extern "C" int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* d) {
   if (rc) return rc;
   const QLArgs a = to_args(d);
   hipStream_t st = as_stream(stream);
-  if (a.M <= 16) return launch_qlinear<1, 2>(st, a);
-  if (a.M <= 32) return launch_qlinear<2, 2>(st, a);
-  // 33+ rows: 128 x 128 work-group tiles (rows past M cost no fetches: they are read as zeros
-  // through the buffer bounds); the row tile of the small-batch kernel would re-read the weights
-  // no less and runs a slower loop; the 256-column variant (NT = 4) is not dispatched: its
-  // accumulators need AGPRs, and the compiler wraps loops over AGPR accumulators in register
-  // copies that cost more than the halved LDS traffic gains
-  if (scales_per_tile(a.group) == 2) return launch_qgemm128<2, 2>(st, a);
-  return launch_qgemm128<2, 4>(st, a);
+  // One kernel for every row count: 128 x 128 work-group tiles at 65+ rows, 16 / 32 / 64 rows for
+  // decode batches that small (the weight stream and its dequantisation are the same; MFMA,
+  // fragment and activation work shrink with the rows).  The 256-column variant (NT = 4) is not
+  // dispatched: its accumulators need AGPRs, and the compiler wraps loops over AGPR accumulators
+  // in register copies that cost more than the halved LDS traffic gains.
+  const bool s2 = scales_per_tile(a.group) == 2;
+  if (a.M <= 16) return s2 ? launch_qgemm128<2, 2, 1>(st, a) : launch_qgemm128<2, 4, 1>(st, a);
+  if (a.M <= 32) return s2 ? launch_qgemm128<2, 2, 2>(st, a) : launch_qgemm128<2, 4, 2>(st, a);
+  if (a.M <= 64) return s2 ? launch_qgemm128<2, 2, 4>(st, a) : launch_qgemm128<2, 4, 4>(st, a);
+  return s2 ? launch_qgemm128<2, 2, 8>(st, a) : launch_qgemm128<2, 4, 8>(st, a);
 }
 
 extern "C" int tnx_splitk_finish(void* stream, const tnx_qlinear_desc* d) {

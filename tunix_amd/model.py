@@ -249,7 +249,7 @@ class Runner:
     self.rope_sin = torch.empty(B, max(cfg.head_dim // 2, 1), dtype=torch.float32, device=dev)
     self.rope_cos = torch.empty_like(self.rope_sin)
     self.next_tpart = None
-    if 32 < M <= 1024 and not cfg.num_experts and model.layers and "gu" in model.layers[0]:
+    if M <= 1024 and not cfg.num_experts and model.layers and "gu" in model.layers[0]:
       n_planes = math.ceil(M / 128) * math.ceil(model.layers[0]["gu"].N / 128)
       self.next_tpart = torch.empty(n_planes * 8192, dtype=torch.float32, device=dev)
     need = 1
@@ -329,7 +329,7 @@ class Runner:
     return split if deferred else 1
 
   def fuses_next(self, f: FusedLinear, next_f: FusedLinear, M: int, epilogue: int) -> bool:
-    return (next_f.has_lora and next_f.rp <= 64 and 32 < M <= 1024 and self._split_k(f, M) == 1
+    return (next_f.has_lora and next_f.rp <= 64 and M <= 1024 and self._split_k(f, M) == 1
             and epilogue in (L.TNX_EPI_SILU_MUL, L.TNX_EPI_GELU_MUL) and (f.N // 2) % 8 == 0
             and self.next_tpart is not None)
 
