@@ -28,10 +28,13 @@ def rnd(shape, seed, scale=1.0):
   return (torch.randn(*shape, generator=g) * scale).to(torch.bfloat16).float()
 
 
-def assert_bf16_close(got, ref, atol=1e-6, min_equal=0.97, what=""):
+def assert_bf16_close(got, ref, atol=1e-6, min_equal=0.97, what="", mag=None, ulps=1):
+  """mag: magnitude the one-ulp allowance is taken from when it is not the result itself (a sum
+  with a residual can cancel: the ulp that matters is the one of the larger operand).  ulps: for
+  results computed from several rounded intermediates, each of which may be one ulp off."""
   got, ref = got.float().cpu(), ref.float().cpu()
   diff = (got - ref).abs()
-  tol = ref.abs() * 2.0 ** -7 + atol
+  tol = (ref.abs() if mag is None else torch.maximum(ref.abs(), mag.float().cpu().abs())) * (ulps * 2.0 ** -7) + atol
   bad = (diff > tol).sum().item()
   eq = (got == ref).float().mean().item()
   assert bad == 0, f"{what}: {bad} elements beyond one bf16 ulp, max diff {diff.max().item()}"
@@ -107,6 +110,74 @@ def test_qlinear_lora_matches_oracle(gpu, M, K, N, group, qtype, r, split):
   ops.qlinear(d)
   torch.cuda.synchronize()
   assert_bf16_close(y, ref, what="qlinear")
+
+
+@pytest.mark.parametrize("M,K,N,group,qtype,r,seg_widths,epi", [
+    (1100, 256, 7424, 64, Q.NF4, 64, None, "store"),             # ragged rows, one adapter
+    (640, 384, 13312, 128, Q.INT4, 16, [8192, 2560, 2560], "store"),  # three adapter segments, 3 k-tiles
+    (520, 128, 13440, 32, Q.NF4, 0, None, "residual"),           # ragged last column tile, group 32, one k-tile
+    (1024, 512, 8448, 64, Q.INT4, 32, None, "silu"),             # gate|up pair with its two adapters
+    (515, 640, 16896, 64, Q.NF4, 0, None, "gelu"),
+])
+def test_qlinear_many_rows_matches_oracle(gpu, M, K, N, group, qtype, r, seg_widths, epi):
+  """Row counts that go to the 128 x 256-tile kernel (prefill, per-token logps): every epilogue,
+  adapter segments, ragged row and column tiles, against the oracle."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  x = rnd((M, K), 21)
+  w = rnd((K, N), 22, 0.02)
+  codes, scale = Q.quantize(w.numpy(), group, qtype)
+  mul = epi in ("silu", "gelu")
+  widths = seg_widths or ([N // 2, N // 2] if mul else [N])
+  rp = (r + 31) // 32 * 32 if r else 0
+  ref = torch.empty(M, N)
+  a_t = torch.zeros(len(widths) * max(rp, 1), K)
+  b_full = torch.zeros(N, max(rp, 1))
+  off = 0
+  for i, wd in enumerate(widths):
+    a = b = None
+    if r:
+      a, b = _lora(K, wd, r, 30 + 2 * i)
+      a_t[i * rp: i * rp + r] = a.t()
+      b_full[off: off + wd, :r] = b.t()
+    ref[:, off: off + wd] = Q.qlinear_lora(x, codes[:, off: off + wd], scale[:, off: off + wd], group, qtype,
+                                           a, b, lora_scale=0.5)
+    off += wd
+  ref = Q.rb(ref)
+  res = mag = None
+  if epi == "residual":
+    res = rnd((M, N), 23)
+    mag = ref
+    ref = Q.rb(ref + res)
+  elif mul:
+    gte, up = ref[:, : N // 2], ref[:, N // 2:]
+    act = Q.rb(gte * Q.rb(torch.sigmoid(gte))) if epi == "silu" else \
+        Q.rb(torch.nn.functional.gelu(gte, approximate="tanh"))
+    ref = Q.rb(act * up)
+  gx = bf(x).to(gpu)
+  c, s = ops.quantize_pack(bf(w).to(gpu), group, qtype, mul)
+  y = torch.empty(M, N // 2 if mul else N, dtype=torch.bfloat16, device=gpu)
+  kw = {}
+  if r:
+    t = torch.zeros(M, len(widths) * rp, dtype=torch.bfloat16, device=gpu)
+    ops.lora_down(gx, bf(a_t).to(gpu), t)
+    b_t = b_full
+    if mul:
+      b_t = torch.zeros_like(b_full)
+      b_t[torch.from_numpy(Q.packed_col(np.arange(N), N, True))] = b_full
+    ends = list(np.cumsum(widths))
+    kw = dict(lora_rank=rp, lora_nseg=-1 if mul else len(widths), lora_seg_end=[int(e) for e in ends],
+              lora_seg_toff=[i * rp for i in range(len(widths))], t=t, t_ld=len(widths) * rp,
+              lora_b=bf(b_t).to(gpu), lora_scale=0.5)
+  e = {"store": L.TNX_EPI_STORE, "residual": L.TNX_EPI_RESIDUAL, "silu": L.TNX_EPI_SILU_MUL,
+       "gelu": L.TNX_EPI_GELU_MUL}[epi]
+  if res is not None:
+    kw["residual"] = bf(res).to(gpu)
+  ops.qlinear(ops.make_qlinear_desc(M=M, K=K, N=N, group=group, qtype=qtype, x=gx, codes=c, scales=s, y=y,
+                                    epilogue=e, **kw))
+  torch.cuda.synchronize()
+  assert_bf16_close(y, ref, atol=1e-5 if mul else 1e-6, min_equal=0.9 if mul else 0.97, what=f"wide {epi}", mag=mag,
+                    ulps=3 if mul else 1)   # act(gate) * up: gate and up may each be one ulp off
 
 
 def test_qlinear_invariants(gpu):

@@ -27,8 +27,9 @@ typedef __attribute__((address_space(3))) uint32_t lds_u32;
 typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
 
 constexpr int kBigLutBytes = 256 * 256;
-constexpr int kBigABytes = 128 * A_LD * 2;
-constexpr size_t kBigSmemBytes = kBigLutBytes + 2 * (size_t)kBigABytes + 4 * 4096;  // + adapter fragments
+// table, two activation buffers of max(32, rows) rows, adapter fragments (2 KiB per column tile)
+constexpr size_t big_abytes(int mt) { return (size_t)(mt < 2 ? 32 : 16 * mt) * A_LD * 2; }
+constexpr size_t big_smem_bytes(int nt, int mt) { return kBigLutBytes + 2 * big_abytes(mt) + 4 * (size_t)nt * 2048; }
 
 // LDS accesses by absolute LDS byte address (the dynamic LDS block of these kernels starts at
 // address 0: they declare no static LDS).
@@ -69,6 +70,7 @@ void qgemm128_kernel(const QLArgs a) {
   constexpr int ROWS = 16 * MT;
   constexpr int AP = (ROWS + 31) / 32;       // passes of the activation copy (512 threads x 16 B = 32 rows)
   constexpr int SW = SPT / 2;  // scales of one wave's two k-steps
+  constexpr uint32_t ABYTES = (uint32_t)big_abytes(MT);
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6), wn = wv & 3, kh = wv >> 2;  // wave-uniform
@@ -176,7 +178,7 @@ void qgemm128_kernel(const QLArgs a) {
   // B^T fragments of the adapter for this column group: fetched now, parked in the group's
   // 4 KiB of LDS behind the activation buffers until the epilogue (both waves of the group
   // write the same values; the barriers of the main loop order them before the reads)
-  const uint32_t lb_lds = kBigLutBytes + 2 * kBigABytes + (uint32_t)wn * 4096u + (uint32_t)lane * 16u;
+  const uint32_t lb_lds = kBigLutBytes + 2 * ABYTES + (uint32_t)wn * (uint32_t)(NT * 2048) + (uint32_t)lane * 16u;
   uint32_t tbase = 0;
   u32x4 lbv[NT][2];  // live only until the main loop starts
 #pragma unroll
@@ -271,9 +273,9 @@ void qgemm128_kernel(const QLArgs a) {
   };
   // LDS byte addresses of the two activation buffers as this lane reads (its k half) / writes them
   uint32_t a_rd = kBigLutBytes + (uint32_t)(lm * A_LD + lq * 8 + kh * 64) * 2u;
-  uint32_t a_rd_nxt = a_rd + kBigABytes;
+  uint32_t a_rd_nxt = a_rd + ABYTES;
   uint32_t a_wr = kBigLutBytes + (uint32_t)((tid >> 4) * A_LD + (tid & 15) * 8) * 2u;
-  uint32_t a_wr_nxt = a_wr + kBigABytes;
+  uint32_t a_wr_nxt = a_wr + ABYTES;
   auto read_a = [&](u32x4 (&dst)[MT], uint32_t base, auto Jc) {
     constexpr int J = decltype(Jc)::value;
 #pragma unroll
@@ -345,9 +347,17 @@ void qgemm128_kernel(const QLArgs a) {
   };
 
   if (kt_begin < kt_end) {
+    // Order of the first loads: each is followed by at least as many later loads as it will be
+    // in the steady state of the loop, so the counted waits of the loop body need not fall back
+    // to "everything outstanding" for the sake of the path that enters from here.  The first
+    // activation tile has registers of its own for that (live only up to its store).
+    u32x4 a_first[AP];
     load_a(kt_begin);
+#pragma unroll
+    for (int c = 0; c < AP; ++c) a_first[c] = a_next[c];
     load_w(ic<0>{}, kt_begin);
     load_w(ic<1>{}, kt_begin + 1);
+    load_a(kt_begin + 1);
     load_w(ic<2>{}, kt_begin + 2);
     if (lora_fast) load_adapter_b();
     TNX_STAMP(7);
@@ -361,8 +371,8 @@ void qgemm128_kernel(const QLArgs a) {
       for (int c = 0; c < 32; ++c) lut[e * 64 + ((c0 + c + lane) & 63)] = v;
     }
     TNX_STAMP(1);
-    store_a(a_wr);
-    load_a(kt_begin + 1);
+#pragma unroll
+    for (int c = 0; c < AP; ++c) lds_st128(a_wr + (uint32_t)(c * 32 * A_LD * 2), a_first[c]);
     expand_scales(ic<0>{}, true);
     __syncthreads();  // table and first activation tile
     lut_issue(ic<0>{}, ic<0>{}, lp);
@@ -376,11 +386,18 @@ void qgemm128_kernel(const QLArgs a) {
         for (int j = 0; j < 2; ++j) lds_st128(lb_lds + (uint32_t)((nt * 2 + j) * 1024), lbv[nt][j]);
     }
     TNX_STAMP(2);
-    // three k-tiles (one turn of the ring) per iteration
-    for (int kt = kt_begin; kt < kt_end; kt += PF) {
+    // whole turns of the ring (three k-tiles) without a branch inside -- a conditional tile
+    // would make the waits of the tile after it assume that its loads never happened -- then
+    // the one or two tiles left
+    int kt = kt_begin;
+    for (; kt + PF <= kt_end; kt += PF) {
+      tile(ic<0>{}, kt);
+      tile(ic<1>{}, kt + 1);
+      tile(ic<2>{}, kt + 2);
+    }
+    if (kt < kt_end) {
       tile(ic<0>{}, kt);
       if (kt + 1 < kt_end) tile(ic<1>{}, kt + 1);
-      if (kt + 2 < kt_end) tile(ic<2>{}, kt + 2);
     }
   }
   TNX_STAMP(3);

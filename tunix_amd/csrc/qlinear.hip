@@ -157,6 +157,7 @@ __global__ __launch_bounds__(256) void moe_gmm_kernel(const QLArgs a) {
 
 }  // namespace
 #include "qgemm128.h"
+#include "qgemm_wide.h"
 namespace {
 
 // y = epi(sum of the split_k partial tiles, added in split order).  One thread per output
@@ -423,12 +424,52 @@ template <int NT, int SPT, int MT>
 int launch_qgemm128(hipStream_t st, const QLArgs& a) {
   static std::once_flag once;
   static int attr_rc = TNX_OK;
-  std::call_once(once, [] { attr_rc = raise_lds_limit(&qgemm128_kernel<NT, SPT, MT>, kBigSmemBytes); });
+  constexpr size_t kSmem = big_smem_bytes(NT, MT);
+  std::call_once(once, [] { attr_rc = raise_lds_limit(&qgemm128_kernel<NT, SPT, MT>, kSmem); });
   if (attr_rc) return attr_rc;
   dim3 grid((unsigned)cdiv(a.M, 16 * MT), (unsigned)cdiv(a.N, 64 * NT), (unsigned)a.split_k);
-  hipLaunchKernelGGL((qgemm128_kernel<NT, SPT, MT>), grid, dim3(512), kBigSmemBytes, st, a);
+  hipLaunchKernelGGL((qgemm128_kernel<NT, SPT, MT>), grid, dim3(512), kSmem, st, a);
   TNX_CHECK_LAUNCH("qgemm128");
   return TNX_OK;
+}
+
+template <int SPT>
+int launch_qgemm_wide(hipStream_t st, const QLArgs& a) {
+  static std::once_flag once;
+  static int attr_rc = TNX_OK;
+  std::call_once(once, [] { attr_rc = raise_lds_limit(&qgemm_wide_kernel<SPT>, kWideSmemBytes); });
+  if (attr_rc) return attr_rc;
+  const unsigned wgs = (unsigned)(cdiv(a.M, kWideRows) * cdiv(a.N, kWideCols));
+  hipLaunchKernelGGL((qgemm_wide_kernel<SPT>), dim3(wgs), dim3(256), kWideSmemBytes, st, a);
+  TNX_CHECK_LAUNCH("qgemm_wide");
+  return TNX_OK;
+}
+
+// Shapes the 128 x 256 kernel takes: enough rows to fill the device with its tiles, no k split,
+// a bf16 output whose rows can be written in 16-byte chunks, and an adapter (if any) of rank
+// <= 64 none of whose 256-column windows touches more than two segments.
+bool wide_shape(const QLArgs& a) {
+  if (a.split_k > 1 || a.next_tpart || a.M < 512) return false;
+  if (cdiv(a.M, kWideRows) * cdiv(a.N, kWideCols) < 256) return false;
+  const bool mul = a.epilogue == TNX_EPI_SILU_MUL || a.epilogue == TNX_EPI_GELU_MUL;
+  if (!mul && a.epilogue != TNX_EPI_STORE && a.epilogue != TNX_EPI_RESIDUAL) return false;
+  if ((mul ? a.N / 2 : a.N) % 8 != 0 || ((uintptr_t)a.y & 15) != 0) return false;
+  if (a.epilogue == TNX_EPI_RESIDUAL && ((uintptr_t)a.residual & 15) != 0) return false;
+  if (a.lora_rank > 0) {
+    if (a.lora_rank > 64 || a.lora_rank % 8 != 0) return false;
+    if (a.lora_nseg > 2) {
+      for (int64_t c0 = 0; c0 < a.N; c0 += kWideCols) {
+        const int64_t c1 = std::min<int64_t>(c0 + kWideCols, a.N) - 1;
+        int first = 0, last = 0;
+        for (int i = 0; i < a.lora_nseg - 1; ++i) {
+          first += c0 >= a.lora_seg_end[i];
+          last += c1 >= a.lora_seg_end[i];
+        }
+        if (last - first > 1) return false;
+      }
+    }
+  }
+  return true;
 }
 
 template <int MT, int NT>
@@ -498,6 +539,7 @@ extern "C" int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* d) {
   // dispatched: its accumulators need AGPRs, and the compiler wraps loops over AGPR accumulators
   // in register copies that cost more than the halved LDS traffic gains.
   const bool s2 = scales_per_tile(a.group) == 2;
+  if (wide_shape(a)) return s2 ? launch_qgemm_wide<2>(st, a) : launch_qgemm_wide<4>(st, a);
   if (a.M <= 16) return s2 ? launch_qgemm128<2, 2, 1>(st, a) : launch_qgemm128<2, 4, 1>(st, a);
   if (a.M <= 32) return s2 ? launch_qgemm128<2, 2, 2>(st, a) : launch_qgemm128<2, 4, 2>(st, a);
   if (a.M <= 64) return s2 ? launch_qgemm128<2, 2, 4>(st, a) : launch_qgemm128<2, 4, 4>(st, a);
