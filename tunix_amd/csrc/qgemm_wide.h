@@ -1,14 +1,22 @@
 // The quantised GEMM for many rows (prefill, per-token logps): output tile 128 rows x 256
 // columns per work-group of four waves, one per SIMD with the whole register file (the 128
-// accumulator registers of a wave's 128 x 64 block next to the operand pipeline).  Past a few
-// hundred rows the op is bound by the matrix pipe, and what keeps the pipe waiting is the
-// traffic between L2 and the compute unit: a 128 x 256 tile fetches 32 KB of activations and
-// 17 KB of packed weights per k-tile for twice the MFMA work a 128 x 128 tile gets from
-// 32 + 8.5 KB.  Same weight format, table look-up, conversion and software pipeline as
-// qgemm128_kernel, but every wave walks all four k-steps of a k-tile (no k split inside the
-// work-group, so no exchange of accumulators) and the products are formed transposed
-// (weights as the MFMA's A operand): a lane then owns four consecutive output columns of one
-// row, and the tile leaves through LDS as whole 16-byte row chunks.
+// accumulator registers of a wave's 128 x 64 block next to the operand pipeline).  Same weight
+// format, table look-up and conversion as qgemm128_kernel; what differs follows from what a
+// wave that has its SIMD to itself can issue:
+//
+//   * 32x32x16 MFMAs.  One wave issues independent 16x16x32 MFMAs at half the rate of the
+//     matrix pipe and serialises every vector instruction behind them; a 32x32x16 MFMA keeps
+//     the pipe busy for 32 clocks and leaves room for the four conversion instructions, the
+//     look-up and the fragment read that go with it.  The packed weight tiles (16 columns x
+//     128 k, built for the 16x16x32 operand layout) are read with another lane -> chunk map for
+//     that: lane l takes column l % 32 of a 32-column group and, per k-tile, the two 16-byte
+//     chunks that hold its k-groups 8 (l / 32) + 16 u of that column.
+//   * every wave walks all eight 16-deep slabs of a k-tile (no k split inside the work-group,
+//     no exchange of accumulators); products are formed transposed (weights as the MFMA's A
+//     operand), so that a lane owns runs of four consecutive output columns of one row and the
+//     tile leaves through LDS as whole 16-byte row chunks.
+//   * a slab is written as eight slots in issue order, one MFMA each with its share of the
+//     work for the following slabs; group barriers restate the slots for the scheduler.
 //
 // Work-groups are numbered so that the eight XCDs (consecutive work-group ids go to
 // consecutive XCDs) each walk one 128-row block across the column tiles: a block's activations
@@ -23,15 +31,22 @@ namespace {
 constexpr int kWideRows = 128, kWideCols = 256;
 constexpr size_t kWideSmemBytes = kBigLutBytes + 2 * (size_t)kWideRows * A_LD * 2;
 
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+  // D[32x32] += A[32x16] * B[16x32]; lane l holds A row l%32 / B column l%32, k = 8*(l/32)..+7;
+  // D: column l%32, rows 8*(r/4) + 4*(l/32) + r%4 for register r.
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
 template <int SPT>
 __global__ __launch_bounds__(256)
 void qgemm_wide_kernel(const QLArgs a) {
-  constexpr int NT = 4, MT = 8, PF = 3, AP = 8;
+  constexpr int RT = 4, CG = 2, PF = 3, AP = 8;   // 32-row tiles, 32-column groups per wave
   constexpr uint32_t ABYTES = kWideRows * A_LD * 2;
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wn = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int lm = lane & 15, lq = lane >> 4;
+  const int l32 = lane & 31, lh = lane >> 5;
   // LDS is addressed absolutely (table at 0)
   if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem != 0u) return;
   asm volatile("" ::"s"(a.M), "s"(a.K), "s"(a.N), "s"(a.qtype), "s"(a.x), "s"(a.codes), "s"(a.scales),
@@ -55,7 +70,7 @@ void qgemm_wide_kernel(const QLArgs a) {
     ntile = r / gm;
   }
   const int64_t m0 = (int64_t)mtile * kWideRows;
-  const int64_t ntile0 = ((int64_t)ntile * 4 + wn) * NT;
+  const int64_t ntile0 = ((int64_t)ntile * 4 + wn) * 4;   // first packed 16-column tile of this wave
   const int64_t ntiles = a.N / 16;
   const int ktiles = (int)(a.K / KTILE);
   const int rows_here = (int)min((int64_t)kWideRows, a.M - m0);
@@ -66,43 +81,50 @@ void qgemm_wide_kernel(const QLArgs a) {
   const uint64_t ntk = (uint64_t)ntiles * ktiles;
   const rsrc_t rc = make_rsrc(a.codes, ntk * 1024);
   const rsrc_t rs = make_rsrc(a.scales, ntk * 16 * SPT * 2 + 16);
-  uint32_t coff[NT], soff[NT];
+  // Lane l: column l % 32 of a group = column (l % 16) of packed tile 2 cg + (l % 32) / 16.  A
+  // packed tile holds, at chunk 16 q + c, the k-groups 8 q + 32 j (dword j) of its column c;
+  // slab u of the MFMA wants k-group 2 u + l / 32 from this lane: chunk q = l / 32 gives the
+  // even slabs (dword u / 2), chunk q = 2 + l / 32 the odd ones.  Column tiles past N start
+  // beyond the buffer and read zeros.
+  uint32_t coff[CG], soff[CG];
   const uint32_t xbase = ((uint32_t)(tid >> 4) * (uint32_t)a.K + (uint32_t)(tid & 15) * 8u) * 2u;
   const uint32_t xstride = 16u * (uint32_t)a.K * 2u;  // 16 rows further per pass
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-    const uint32_t tile0 = (uint32_t)(ntile0 + nt) * (uint32_t)ktiles;
-    coff[nt] = tile0 * 1024u + (uint32_t)lane * 16u;
-    soff[nt] = (tile0 * 16u + (uint32_t)lm) * (uint32_t)(SPT * 2);
+  for (int cg = 0; cg < CG; ++cg) {
+    const uint32_t tile0 = (uint32_t)(ntile0 + 2 * cg + (l32 >> 4)) * (uint32_t)ktiles;
+    coff[cg] = tile0 * 1024u + (uint32_t)(16 * lh + (l32 & 15)) * 16u;
+    soff[cg] = (tile0 * 16u + (uint32_t)(l32 & 15)) * (uint32_t)(SPT * 2);
   }
 
-  f32x4 acc[MT][NT];
+  f32x16 acc[RT][CG];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) zero_acc(acc[mt][nt]);
+    for (int cg = 0; cg < CG; ++cg)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[rt][cg][i] = 0.f;
 
   u32x4 a_next[AP];
-  u32x4 ring_c[PF][NT];
-  u32x2 ring_s[PF][NT];
-  float sc[PF][NT][SPT];
-  u32x4 af[2][MT];
-  u32x4 bfr[2][NT];
-  uint32_t lp[NT][4];
+  u32x4 ring_c[PF][CG][2];   // [.][.][0]: even slabs, [1]: odd slabs
+  u32x2 ring_s[PF][CG];
+  float sc[PF][CG][SPT];
+  u32x4 xf[2][RT];           // activation fragments of the current / next slab
+  u32x4 wf[2][CG];           // weight fragments of the current / next slab
+  uint32_t lp[CG][4];        // table entries (f16 level pairs) of the slab after the next
 
   // LoRA: the k-tile after the last one is the 128-row block of t = bf16(x . A), columns
   // [toff_a, +64) | [toff_b, +64) (the host sends only shapes whose work-groups span at most
-  // two adapter segments here); the B^T fragments of this wave's columns stay in registers.
+  // two adapter segments here); the B^T fragments of this lane's columns stay in registers.
   const bool lora = a.lora_rank > 0;
-  int toff[NT];
+  int toff[4];
   int toff_a = 0, toff_b = 0;
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) toff[nt] = 0;
+  for (int nt = 0; nt < 4; ++nt) toff[nt] = 0;
   if (lora) {
     if (a.lora_nseg < 0) {
       toff_b = a.lora_rank;
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) toff[nt] = (int)((ntile0 + nt) & 1) * a.lora_rank;
+      for (int nt = 0; nt < 4; ++nt) toff[nt] = (int)((ntile0 + nt) & 1) * a.lora_rank;
     } else {
       int e0 = (int)a.lora_seg_end[0], e1 = (int)a.lora_seg_end[1], e2 = (int)a.lora_seg_end[2];
       int t0 = a.lora_seg_toff[0], t1 = a.lora_seg_toff[1], t2 = a.lora_seg_toff[2], t3 = a.lora_seg_toff[3];
@@ -117,187 +139,144 @@ void qgemm_wide_kernel(const QLArgs a) {
         return pick(pick(pick(t0, t1, i == 1), t2, i == 2), t3, i == 3);
       };
       const int last = (int)ntiles - 1;
-      const int wg_nt0 = ntile * 4 * NT;
+      const int wg_nt0 = ntile * 16;
       toff_a = idx_toff(seg_idx(min(wg_nt0, last)));
-      toff_b = idx_toff(seg_idx(min(wg_nt0 + 4 * NT - 1, last)));
+      toff_b = idx_toff(seg_idx(min(wg_nt0 + 15, last)));
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) toff[nt] = idx_toff(seg_idx(min((int)ntile0 + nt, last)));
+      for (int nt = 0; nt < 4; ++nt) toff[nt] = idx_toff(seg_idx(min((int)ntile0 + nt, last)));
     }
   }
-  u32x4 lbv[NT][2];
+  u32x4 lbv[CG][4];          // B^T of the adapter: this lane's column, ranks 16 u + 8 (l / 32) ..+7
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt)
+  for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) lbv[nt][j] = u32x4{0, 0, 0, 0};
+    for (int u = 0; u < 4; ++u) lbv[cg][u] = u32x4{0, 0, 0, 0};
   uint32_t tbase = 0;
   if (lora) {
     const int ch = tid & 15;
     const int col = ((ch < 8) ? toff_a : toff_b) + min((ch & 7) * 8, a.lora_rank - 8);
     tbase = (uint32_t)((tid >> 4) * a.t_ld + col) * 2u;
   }
-  const rsrc_t rt = lora ? make_rsrc(a.t + m0 * a.t_ld, (uint64_t)rows_here * a.t_ld * 2) : rx;
+  const rsrc_t rt_ = lora ? make_rsrc(a.t + m0 * a.t_ld, (uint64_t)rows_here * a.t_ld * 2) : rx;
   const uint32_t tstride = (uint32_t)(16 * a.t_ld * 2);
 
   auto load_a = [&](int kt) {
     const bool ut = lora && kt >= ktiles;
     const int s = ut ? 0 : min(kt, ktiles - 1) * (KTILE * 2);
-    const rsrc_t r = ut ? rt : rx;
+    const rsrc_t r = ut ? rt_ : rx;
     const uint32_t m = 0u - (uint32_t)ut;
     const uint32_t base = xbase ^ ((xbase ^ tbase) & m), stride = xstride ^ ((xstride ^ tstride) & m);
 #pragma unroll
     for (int c = 0; c < AP; ++c)
       a_next[c] = __builtin_amdgcn_raw_buffer_load_b128(r, base + (uint32_t)c * stride, s, 0);
   };
+  auto load_scale = [&](auto Dc, int cg, int ktc) {
+    constexpr int D = decltype(Dc)::value;
+    if constexpr (SPT == 2) {
+      ring_s[D][cg][0] = __builtin_amdgcn_raw_buffer_load_b32(rs, soff[cg], ktc * (16 * SPT * 2), 0);
+    } else {
+      ring_s[D][cg] = __builtin_amdgcn_raw_buffer_load_b64(rs, soff[cg], ktc * (16 * SPT * 2), 0);
+    }
+  };
   auto load_w = [&](auto Dc, int kt) {
     constexpr int D = decltype(Dc)::value;
     const int ktc = min(kt, ktiles - 1);
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      ring_c[D][nt] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff[nt], ktc * 1024, 0);
-      if constexpr (SPT == 2) {
-        ring_s[D][nt][0] = __builtin_amdgcn_raw_buffer_load_b32(rs, soff[nt], ktc * (16 * SPT * 2), 0);
-      } else {
-        ring_s[D][nt] = __builtin_amdgcn_raw_buffer_load_b64(rs, soff[nt], ktc * (16 * SPT * 2), 0);
-      }
+    for (int cg = 0; cg < CG; ++cg) {
+      ring_c[D][cg][0] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff[cg], ktc * 1024, 0);
+      ring_c[D][cg][1] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff[cg] + 512u, ktc * 1024, 0);
+      load_scale(Dc, cg, ktc);
     }
   };
   auto expand_scales = [&](auto Dc, bool active) {
     constexpr int D = decltype(Dc)::value;
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
+    for (int cg = 0; cg < CG; ++cg) {
 #pragma unroll
       for (int j = 0; j < SPT; ++j) {
-        const uint32_t w = ring_s[D][nt][j >> 1];
-        sc[D][nt][j] = active ? ((j & 1) ? bfhi(w) : bflo(w)) : 0.f;
+        const uint32_t w = ring_s[D][cg][j >> 1];
+        sc[D][cg][j] = active ? ((j & 1) ? bfhi(w) : bflo(w)) : 0.f;
       }
     }
   };
-  auto lut_issue = [&](auto Dc, auto Jc, uint32_t (&dst)[NT][4]) {
-    constexpr int D = decltype(Dc)::value, J = decltype(Jc)::value;
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const uint32_t w = ring_c[D][nt][J];
-      dst[nt][0] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0400u));
-      dst[nt][1] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0500u));
-      dst[nt][2] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0600u));
-      dst[nt][3] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0700u));
-    }
-  };
-  auto convert = [&](auto Dc, auto Jc, u32x4 (&dst)[NT], const uint32_t (&src)[NT][4]) {
-    constexpr int D = decltype(Dc)::value, J = decltype(Jc)::value;
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const float s = sc[D][nt][SPT == 2 ? (J >> 1) : J];
-      u32x4 r;
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const h16x2 h = __builtin_bit_cast(h16x2, src[nt][b]);
-        r[b] = cvt_pk_bf16(__builtin_fmaf((float)h[0], s, 0.0f), __builtin_fmaf((float)h[1], s, 0.0f));
-      }
-      dst[nt] = r;
-    }
-  };
-  uint32_t a_rd = kBigLutBytes + (uint32_t)(lm * A_LD + lq * 8) * 2u;
+  uint32_t a_rd = kBigLutBytes + (uint32_t)(l32 * A_LD + lh * 8) * 2u;
   uint32_t a_rd_nxt = a_rd + ABYTES;
   uint32_t a_wr = kBigLutBytes + (uint32_t)((tid >> 4) * A_LD + (tid & 15) * 8) * 2u;
   uint32_t a_wr_nxt = a_wr + ABYTES;
-  auto read_a = [&](u32x4 (&dst)[MT], uint32_t base, auto Jc) {
-    constexpr int J = decltype(Jc)::value;
-#pragma unroll
-    for (int m = 0; m < MT; ++m) dst[m] = lds_ld128(base + (uint32_t)((m * 16 * A_LD + J * 32) * 2));
-  };
   auto store_a = [&](uint32_t base) {
 #pragma unroll
     for (int c = 0; c < AP; ++c) lds_st128(base + (uint32_t)(c * 16 * A_LD * 2), a_next[c]);
   };
-  // (the products are formed transposed: D[weight column][row] += W^T . x^T)
-  // One k-step = 32 slots, one matrix instruction each, written in the order they should issue
-  // (a wave that has its SIMD to itself hides nothing behind another wave: whatever does not
-  // issue in the shadow of a matrix instruction adds to the loop).  Slot i multiplies
-  // accumulator (row tile i % 8, column tile i / 8), and carries two vector instructions and at
-  // most two memory instructions:
-  //   even slots  the two f16 x scale products of code pair i / 2 of the NEXT step's weights,
-  //               an activation fragment read for the next step (i < 16), an LDS write of the
-  //               next activation tile (ST, i >= 16), a global load (LD);
-  //   odd slots   the bf16 pack of that pair, and the table look-up (address: one v_perm) of
-  //               the same pair of the step AFTER the next, which overwrites the entry the
-  //               even slot just consumed.
-  // Column tile nt of the next step's weights is complete after slot 8 nt + 7, and the next
-  // step uses it from its slot 8 nt on.  The group barriers restate the slot contents for the
-  // machine scheduler.
-  auto step = [&](auto CURc, auto Dcc, auto Jcc, auto Dlc, auto Jlc, uint32_t rd_base, auto Jrc, auto STc,
-                  auto LDc, auto EXc, int kt, bool ex_active) {
-    constexpr int CUR = decltype(CURc)::value, NXT = CUR ^ 1;
-    constexpr int DC = decltype(Dcc)::value, JC = decltype(Jcc)::value;
-    constexpr int DL = decltype(Dlc)::value, JL = decltype(Jlc)::value, JR = decltype(Jrc)::value;
-    constexpr bool ST = decltype(STc)::value != 0, LD = decltype(LDc)::value != 0;
-    constexpr int EX = decltype(EXc)::value;   // -1, or the ring stage whose scales to expand
-    float f0 = 0.f, f1 = 0.f;
-    const bool ut = lora && kt >= ktiles;      // LD: the tile to fetch is the adapter block
-    const int xs = ut ? 0 : min(kt, ktiles - 1) * (KTILE * 2);
-    const rsrc_t xr = ut ? rt : rx;
+
+  // One slab (16 k) = eight slots, one MFMA each (column group i / 4, row tile i % 4), written
+  // in the order they should issue.  Slot i also carries, for code pair (group i / 4, byte i % 4):
+  // the two f16 x scale products and the bf16 pack of that pair of the NEXT slab's weights, the
+  // table look-up (address: one v_perm) of the same pair of the slab AFTER the next, which
+  // overwrites the entry just consumed, and in even slots an activation fragment read for the
+  // next slab.  Slab 5 expands the next k-tile's scales, slab 6 stores the next activation tile
+  // (fetched by slab 7 of the tile before), the barrier sits between slabs 6 and 7 (the
+  // fragments slab 7 reads are the next tile's), and slab 7 issues the global loads:
+  // activations of k-tile kt + 2, weights of k-tile kt + PF into the ring stage this tile has
+  // finished with.
+  auto slab = [&](auto Uc, auto Dc, int kt, bool next_active) {
+    constexpr int U = decltype(Uc)::value, D = decltype(Dc)::value, DN = (D + 1) % PF;
+    constexpr int CUR = U & 1, NXT = CUR ^ 1;
+    constexpr int UC = (U + 1) & 7, DC = U < 7 ? D : DN;   // slab whose weights are converted here
+    constexpr int UL = (U + 2) & 7, DL = U < 6 ? D : DN;   // slab whose table entries are fetched here
+    constexpr bool ST = U == 6, LD = U == 7, EX = U == 5;
+    const uint32_t xb = (U < 7 ? a_rd : a_rd_nxt) + (uint32_t)(UC * 16 * 2);
+    const bool ut = lora && kt + 2 >= ktiles;      // LD: the activation tile to fetch is the adapter block
+    const int xs = ut ? 0 : min(kt + 2, ktiles - 1) * (KTILE * 2);
+    const rsrc_t xr = ut ? rt_ : rx;
     const uint32_t um = 0u - (uint32_t)ut;
-    const uint32_t xb = xbase ^ ((xbase ^ tbase) & um), xst = xstride ^ ((xstride ^ tstride) & um);
-    const int wkt = min(kt + (PF - 2), ktiles - 1);   // LD: weights of k-tile (this + PF)
+    const uint32_t xo = xbase ^ ((xbase ^ tbase) & um), xst = xstride ^ ((xstride ^ tstride) & um);
+    const int wkt = min(kt + PF, ktiles - 1);
 #pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      const int nt = i >> 3, m = i & 7, pr = i >> 1, pnt = pr >> 2, pb = pr & 3;
-      acc[m][nt] = mfma16(bfr[CUR][nt], af[CUR][m], acc[m][nt]);
-      if ((i & 1) == 0) {
-        const h16x2 h = __builtin_bit_cast(h16x2, lp[pnt][pb]);
-        const float sv = sc[DC][pnt][SPT == 2 ? (JC >> 1) : JC];
-        f0 = __builtin_fmaf((float)h[0], sv, 0.0f);
-        f1 = __builtin_fmaf((float)h[1], sv, 0.0f);
-        if (i < 16) af[NXT][i >> 1] = lds_ld128(rd_base + (uint32_t)(((i >> 1) * 16 * A_LD + JR * 32) * 2));
-        if (ST && i >= 16) lds_st128(a_wr_nxt + (uint32_t)(((i - 16) >> 1) * 16 * A_LD * 2), a_next[(i - 16) >> 1]);
-        if (LD) {
-          const int q = i >> 1;
-          if (q < 8) {
-            a_next[q] = __builtin_amdgcn_raw_buffer_load_b128(xr, xb + (uint32_t)q * xst, xs, 0);
-          } else if (q < 12) {
-            ring_c[DL == 0 ? PF - 1 : DL - 1][q - 8] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff[q - 8], wkt * 1024, 0);
-          } else if constexpr (SPT == 2) {
-            ring_s[DL == 0 ? PF - 1 : DL - 1][q - 12][0] =
-                __builtin_amdgcn_raw_buffer_load_b32(rs, soff[q - 12], wkt * (16 * SPT * 2), 0);
-          } else {
-            ring_s[DL == 0 ? PF - 1 : DL - 1][q - 12] =
-                __builtin_amdgcn_raw_buffer_load_b64(rs, soff[q - 12], wkt * (16 * SPT * 2), 0);
-          }
-        }
-      } else {
-        bfr[NXT][pnt][pb] = cvt_pk_bf16(f0, f1);
-        lp[pnt][pb] = lds_ld32(__builtin_amdgcn_perm(ring_c[DL][pnt][JL], lane_off, 0x0c0c0400u + ((uint32_t)pb << 8)));
+    for (int i = 0; i < 8; ++i) {
+      const int cg = i >> 2, rt = i & 3;
+      acc[rt][cg] = mfma32(wf[CUR][cg], xf[CUR][rt], acc[rt][cg]);
+      {
+        const h16x2 hh = __builtin_bit_cast(h16x2, lp[cg][rt]);
+        const float sv = sc[DC][cg][SPT == 2 ? (UC >> 2) : (UC >> 1)];
+        wf[NXT][cg][rt] = cvt_pk_bf16(__builtin_fmaf((float)hh[0], sv, 0.0f), __builtin_fmaf((float)hh[1], sv, 0.0f));
+        const uint32_t w = ring_c[DL][cg][UL & 1][UL >> 1];
+        lp[cg][rt] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0400u + ((uint32_t)rt << 8)));
       }
-      if (EX >= 0 && i < NT * SPT) {
-        const int ent = i / SPT, ej = i % SPT;
-        const uint32_t w = ring_s[EX < 0 ? 0 : EX][ent][ej >> 1];
-        sc[EX < 0 ? 0 : EX][ent][ej] = ex_active ? ((ej & 1) ? bfhi(w) : bflo(w)) : 0.f;
+      if ((i & 1) == 0) xf[NXT][i >> 1] = lds_ld128(xb + (uint32_t)((i >> 1) * 32 * A_LD * 2));
+      if (ST) lds_st128(a_wr_nxt + (uint32_t)(i * 16 * A_LD * 2), a_next[i]);
+      if (LD) {
+        a_next[i] = __builtin_amdgcn_raw_buffer_load_b128(xr, xo + (uint32_t)i * xst, xs, 0);
+        if (i < 4) ring_c[D][i >> 1][i & 1] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff[i >> 1] + (uint32_t)(i & 1) * 512u, wkt * 1024, 0);
+        else if (i < 6) load_scale(Dc, i - 4, wkt);
+      }
+      if (EX && i < CG * SPT) {
+        const uint32_t w = ring_s[DN][i / SPT][(i % SPT) >> 1];
+        sc[DN][i / SPT][i % SPT] = next_active ? (((i % SPT) & 1) ? bfhi(w) : bflo(w)) : 0.f;
       }
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-      if (EX >= 0 && i < NT * SPT) __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
-      if ((i & 1) == 1 || i < 16) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      if (ST && (i & 1) == 0 && i >= 16) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-      if (LD && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      if (EX && i < CG * SPT) __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if ((i & 1) == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if (ST) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      if (LD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      if (LD && i < 6) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-
-  // One k-tile of ring stage D.  On entry af[0] / bfr[0] hold the fragments of k-step 0 and lp
-  // the table entries of k-step 1.  Step 2 stores the next activation tile (fetched by step 3 of
-  // the tile before), the barrier sits before step 3 (whose fragment reads are the first of the
-  // next tile), and step 3 issues the global loads: activations of k-tile kt + 2, weights of
-  // k-tile kt + PF into the ring stage this tile has just finished with.
   auto tile = [&](auto Dc, int kt) {
-    constexpr int d = decltype(Dc)::value, dn = (d + 1) % PF;
     const bool next_active = kt + 1 < ktiles;
     __builtin_amdgcn_sched_barrier(0);
-    step(ic<0>{}, Dc, ic<1>{}, Dc, ic<2>{}, a_rd, ic<1>{}, ic<0>{}, ic<0>{}, ic<-1>{}, 0, false);
-    step(ic<1>{}, Dc, ic<2>{}, Dc, ic<3>{}, a_rd, ic<2>{}, ic<0>{}, ic<0>{}, ic<-1>{}, 0, false);
-    step(ic<0>{}, Dc, ic<3>{}, ic<dn>{}, ic<0>{}, a_rd, ic<3>{}, ic<1>{}, ic<0>{}, ic<dn>{}, 0, next_active);
+    slab(ic<0>{}, Dc, kt, next_active);
+    slab(ic<1>{}, Dc, kt, next_active);
+    slab(ic<2>{}, Dc, kt, next_active);
+    slab(ic<3>{}, Dc, kt, next_active);
+    slab(ic<4>{}, Dc, kt, next_active);
+    slab(ic<5>{}, Dc, kt, next_active);
+    slab(ic<6>{}, Dc, kt, next_active);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
-    step(ic<1>{}, ic<dn>{}, ic<0>{}, ic<dn>{}, ic<1>{}, a_rd_nxt, ic<0>{}, ic<0>{}, ic<1>{}, ic<-1>{}, kt + 2, false);
+    slab(ic<7>{}, Dc, kt, next_active);
     const uint32_t r = a_rd; a_rd = a_rd_nxt; a_rd_nxt = r;
     const uint32_t w = a_wr; a_wr = a_wr_nxt; a_wr_nxt = w;
   };
@@ -321,19 +300,36 @@ void qgemm_wide_kernel(const QLArgs a) {
   if (lora) {
     const rsrc_t rb = make_rsrc(a.lora_b, (uint64_t)a.N * a.lora_rank * 2);
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
+    for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-        if (j * 32 < a.lora_rank)
-          lbv[nt][j] = buf_load128(rb, (((uint32_t)(ntile0 + nt) * 16u + (uint32_t)lm) * (uint32_t)a.lora_rank +
-                                        (uint32_t)(j * 32 + lq * 8)) * 2u);
+      for (int u = 0; u < 4; ++u)
+        if (u * 16 < a.lora_rank)
+          lbv[cg][u] = buf_load128(rb, (((uint32_t)(ntile0 + 2 * cg) * 16u + (uint32_t)l32) * (uint32_t)a.lora_rank +
+                                        (uint32_t)(u * 16 + lh * 8)) * 2u);
   }
   expand_scales(ic<0>{}, true);
   __syncthreads();
-  lut_issue(ic<0>{}, ic<0>{}, lp);
-  read_a(af[0], a_rd, ic<0>{});
-  convert(ic<0>{}, ic<0>{}, bfr[0], lp);
-  lut_issue(ic<0>{}, ic<1>{}, lp);
+  // slab 0: table entries, conversion, fragments; then the table entries of slab 1
+#pragma unroll
+  for (int cg = 0; cg < CG; ++cg)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+      lp[cg][b] = lds_ld32(__builtin_amdgcn_perm(ring_c[0][cg][0][0], lane_off, 0x0c0c0400u + ((uint32_t)b << 8)));
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) xf[0][rt] = lds_ld128(a_rd + (uint32_t)(rt * 32 * A_LD * 2));
+#pragma unroll
+  for (int cg = 0; cg < CG; ++cg)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const h16x2 hh = __builtin_bit_cast(h16x2, lp[cg][b]);
+      const float sv = sc[0][cg][0];
+      wf[0][cg][b] = cvt_pk_bf16(__builtin_fmaf((float)hh[0], sv, 0.0f), __builtin_fmaf((float)hh[1], sv, 0.0f));
+    }
+#pragma unroll
+  for (int cg = 0; cg < CG; ++cg)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+      lp[cg][b] = lds_ld32(__builtin_amdgcn_perm(ring_c[0][cg][1][0], lane_off, 0x0c0c0400u + ((uint32_t)b << 8)));
   // whole turns of the ring without a branch inside (a conditional tile would make the waits
   // of the tile after it assume that its loads never happened), then the one or two tiles left
   int kt = 0;
@@ -348,61 +344,77 @@ void qgemm_wide_kernel(const QLArgs a) {
   }
 
   if (lora) {
-    // the t block sits in the activation buffer the last k-tile left as "next" (now a_rd)
+    // The t block sits in the activation buffer the last k-tile left as "next" (now a_rd).  The
+    // two 16-column halves of a group may belong to different adapters (always so for a
+    // gate | up pair): one pass per half then, the other half's lanes contributing zeros.
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const uint32_t base = a_rd + (uint32_t)((toff[nt] == toff_a ? 0 : 64) * 2);
-      f32x4 part[MT];
+    for (int cg = 0; cg < CG; ++cg) {
+      const bool same = toff[2 * cg] == toff[2 * cg + 1];
+      f32x16 part[RT];
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) zero_acc(part[mt]);
+      for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        if (j * 32 < a.lora_rank) {
+        for (int i = 0; i < 16; ++i) part[rt][i] = 0.f;
+      for (int p = 0; p < (same ? 1 : 2); ++p) {
+        const uint32_t base = a_rd + (uint32_t)((toff[2 * cg + p] == toff_a ? 0 : 64) * 2);
+        const bool mine = same || (l32 >> 4) == p;
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-            part[mt] = mfma16(lbv[nt][j], lds_ld128(base + (uint32_t)((mt * 16 * A_LD + j * 32) * 2)), part[mt]);
+        for (int u = 0; u < 4; ++u) {
+          if (u * 16 < a.lora_rank) {
+            const u32x4 lb = mine ? lbv[cg][u] : u32x4{0, 0, 0, 0};
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+              part[rt] = mfma32(lb, lds_ld128(base + (uint32_t)((rt * 32 * A_LD + u * 16) * 2)), part[rt]);
+          }
         }
       }
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+      for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[mt][nt][i] += a.lora_scale * part[mt][i];
+        for (int i = 0; i < 16; ++i) acc[rt][cg][i] += a.lora_scale * part[rt][i];
     }
   }
   __syncthreads();  // every wave is done with the activation buffers: they become the output stage
 
   // The bf16 tile goes through LDS (row stride cols + 8 elements) and leaves as 16-byte chunks
-  // of whole rows.  A lane holds, for row mt * 16 + lm, the four columns nt * 16 + lq * 4 + i.
+  // of whole rows.  A lane holds, for row rt * 32 + l % 32 and group cg, the columns
+  // 8 b + 4 (l / 32) + e of the group in register 4 b + e.
   const bool mul = a.epilogue == TNX_EPI_SILU_MUL || a.epilogue == TNX_EPI_GELU_MUL;
   const int cols = mul ? kWideCols / 2 : kWideCols;      // output columns of the work-group
   const int sld = cols + 8;
   const uint32_t stage = kBigLutBytes;
   if (mul) {
+    // a group is [16 gate columns | 16 up columns]: registers 4 b + e (b < 2) and 4 (b + 2) + e
 #pragma unroll
-    for (int p = 0; p < NT / 2; ++p)
+    for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        float v[4];
+      for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float g = rbf(acc[mt][2 * p][i]);
-          const float u = rbf(acc[mt][2 * p + 1][i]);
-          const float act = a.epilogue == TNX_EPI_SILU_MUL ? silu_bf16(g) : gelu_tanh_bf16(g);
-          v[i] = rbf(act) * u;
+        for (int b = 0; b < 2; ++b) {
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float g = rbf(acc[rt][cg][4 * b + e]);
+            const float u = rbf(acc[rt][cg][4 * (b + 2) + e]);
+            const float act = a.epilogue == TNX_EPI_SILU_MUL ? silu_bf16(g) : gelu_tanh_bf16(g);
+            v[e] = rbf(act) * u;
+          }
+          const u32x2 pk = {pack2bf(v[0], v[1]), pack2bf(v[2], v[3])};
+          const uint32_t at = stage + (uint32_t)(((rt * 32 + l32) * sld + wn * 32 + cg * 16 + 8 * b + 4 * lh) * 2);
+          *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(static_cast<uintptr_t>(at)) = pk;
         }
-        const u32x2 pk = {pack2bf(v[0], v[1]), pack2bf(v[2], v[3])};
-        const uint32_t at = stage + (uint32_t)(((mt * 16 + lm) * sld + wn * 32 + p * 16 + lq * 4) * 2);
-        *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(static_cast<uintptr_t>(at)) = pk;
-      }
   } else {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
+    for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const u32x2 pk = {pack2bf(acc[mt][nt][0], acc[mt][nt][1]), pack2bf(acc[mt][nt][2], acc[mt][nt][3])};
-        const uint32_t at = stage + (uint32_t)(((mt * 16 + lm) * sld + wn * 64 + nt * 16 + lq * 4) * 2);
-        *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(static_cast<uintptr_t>(at)) = pk;
-      }
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          const u32x2 pk = {pack2bf(acc[rt][cg][4 * b], acc[rt][cg][4 * b + 1]),
+                            pack2bf(acc[rt][cg][4 * b + 2], acc[rt][cg][4 * b + 3])};
+          const uint32_t at = stage + (uint32_t)(((rt * 32 + l32) * sld + wn * 64 + cg * 32 + 8 * b + 4 * lh) * 2);
+          *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(static_cast<uintptr_t>(at)) = pk;
+        }
   }
   __syncthreads();
   {
