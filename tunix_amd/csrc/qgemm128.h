@@ -130,7 +130,7 @@ void qgemm128_kernel(const QLArgs a) {
   float sc[PF][NT][SW];   // the scales of a ring stage as fp32
   u32x4 af[2][MT];        // activation fragments of this wave's two k-steps
   u32x4 bfr[2][NT];       // weight fragments of the two k-steps
-  uint32_t lp[NT][4];     // table entries (f16 level pairs) of the k-step after the next
+  uint32_t lp[2][NT][4];  // table entries (f16 level pairs): [s] is read by the steps of parity s, written by the others
 
   // LoRA delta through the activation pipeline: the "k-tile" after the last real one is the
   // 128-row block of t = bf16(x . A), columns [toff_a, +64) | [toff_b, +64) (the one or two
@@ -287,61 +287,97 @@ void qgemm128_kernel(const QLArgs a) {
 #pragma unroll
     for (int c = 0; c < AP; ++c) lds_st128(base + (uint32_t)(c * 32 * A_LD * 2), a_next[c]);
   };
-  auto mfmas = [&](auto Jc) {
-    constexpr int J = decltype(Jc)::value;
+  // One of this wave's two k-steps, written as NT * 8 units in the order they should issue: two
+  // units per code pair of the step.  The MT * NT MFMAs are spread evenly over the units
+  // (column tile-major: the first MT use the column tile whose conversion finished first).  An
+  // even unit forms the two f16 x scale products of its pair of the NEXT step's weights, the odd
+  // unit packs them to bf16.  The first half of the units also carries the LDS reads: one table
+  // look-up each (pair u of the step AFTER the next, into the other half of lp) and the
+  // activation fragments of the next step; the second half the stores of the next activation
+  // tile (ST, first step: issued seven units before the barrier behind the step asks for them)
+  // or the global loads (LD, second step).
+  // A scheduling barrier behind every unit keeps that order.
+  auto kstep = [&](auto CURc, auto Dcc, auto Jcc, auto Dlc, auto Jlc, uint32_t rd_base, auto Jrc, auto STc,
+                   auto LDc, auto EXc, int kt, bool ex_active) {
+    constexpr int CUR = decltype(CURc)::value, NXT = CUR ^ 1;
+    constexpr int DC = decltype(Dcc)::value, JC = decltype(Jcc)::value;
+    constexpr int DL = decltype(Dlc)::value, JL = decltype(Jlc)::value, JR = decltype(Jrc)::value;
+    constexpr bool ST = decltype(STc)::value != 0, LD = decltype(LDc)::value != 0;
+    constexpr int EX = decltype(EXc)::value;   // -1, or the ring stage whose scales to expand
+    constexpr int UNITS = NT * 8, MPS = MT * NT;
+    static_assert(UNITS % MPS == 0 && 4 + 2 * NT <= UNITS / 2 && AP <= 4, "unit layout");
+    float f0 = 0.f, f1 = 0.f;
+    const bool ut = lora_fast && kt >= kt_end;      // LD: the activation tile to fetch is the adapter block
+    const int xs = ut ? 0 : min(kt, ktiles - 1) * (KTILE * 2);
+    const rsrc_t xr = ut ? rt : rx;
+    const uint32_t um = 0u - (uint32_t)ut;
+    const uint32_t xo = xbase ^ ((xbase ^ tbase) & um), xst = xstride ^ ((xstride ^ tstride) & um);
+    const int wkt = min(kt + (PF - 2), ktiles - 1);   // LD: weights of k-tile (this + PF)
 #pragma unroll
-    for (int m = 0; m < MT; ++m)
+    for (int u = 0; u < UNITS; ++u) {
+      const int p = u >> 1, pnt = p >> 2, pb = p & 3;
+      if ((u * MPS) % UNITS == 0) {
+        const int mi = u * MPS / UNITS, nt = mi / MT, m = mi % MT;
+        acc[m][nt] = mfma16(af[CUR][m], bfr[CUR][nt], acc[m][nt]);
+      }
+      if ((u & 1) == 0) {
+        const h16x2 h = __builtin_bit_cast(h16x2, lp[CUR][pnt][pb]);
+        const float sv = sc[DC][pnt][SPT == 2 ? 0 : JC];
+        f0 = __builtin_fmaf((float)h[0], sv, 0.0f);
+        f1 = __builtin_fmaf((float)h[1], sv, 0.0f);
+      } else {
+        bfr[NXT][pnt][pb] = cvt_pk_bf16(f0, f1);
+      }
+      if (u < UNITS / 2) {   // all LDS reads in the first half: nothing of them is in flight at the barrier
+        lp[NXT][u >> 2][u & 3] =
+            lds_ld32(__builtin_amdgcn_perm(ring_c[DL][u >> 2][JL], lane_off, 0x0c0c0400u + ((uint32_t)(u & 3) << 8)));
+        if (u < MT) af[NXT][u] = lds_ld128(rd_base + (uint32_t)((u * 16 * A_LD + JR * 32) * 2));
+      } else {
+        const int q = u - UNITS / 2;
+        if (ST && q == 0) {
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) acc[m][nt] = mfma16(af[J][m], bfr[J][nt], acc[m][nt]);
+          for (int c = 0; c < AP; ++c) lds_st128(a_wr_nxt + (uint32_t)(c * 32 * A_LD * 2), a_next[c]);
+        }
+        if (LD) {
+          constexpr int DW = DL == 0 ? PF - 1 : DL - 1;   // the ring stage this k-tile has finished with
+          if (q < AP) {
+            a_next[q] = __builtin_amdgcn_raw_buffer_load_b128(xr, xo + (uint32_t)q * xst, xs, 0);
+          } else if (q >= 4 && q < 4 + NT) {
+            ring_c[DW][q - 4] = __builtin_amdgcn_raw_buffer_load_b64(rc, coff[q - 4], wkt * 1024, 0);
+          } else if (q >= 4 + NT && q < 4 + 2 * NT) {
+            ring_s[DW][q - 4 - NT] = __builtin_amdgcn_raw_buffer_load_b32(rs, soff[q - 4 - NT], wkt * (16 * SPT * 2), 0);
+          }
+        }
+      }
+      if (EX >= 0 && u < NT * SW) {
+        constexpr int E = EX < 0 ? 0 : EX;
+        const int ent = u / SW, ej = u % SW;
+        const uint32_t w = ring_s[E][ent];
+        if constexpr (SPT == 2) {
+          const uint32_t bits = kh ? (w & 0xffff0000u) : (w << 16);
+          sc[E][ent][0] = ex_active ? __builtin_bit_cast(float, bits) : 0.f;
+        } else {
+          sc[E][ent][ej] = ex_active ? (ej ? bfhi(w) : bflo(w)) : 0.f;
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);   // units issue in the order written
+    }
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   // One k-tile of ring stage D = this wave's two k-steps.  On entry af[0] holds the activation
   // fragments of the first step, bfr[0] its weights and lp the table entries of the second.
-  // Step 0 converts the weights of step 1, issues the look-ups of the next k-tile's first step,
-  // reads the fragments of step 1 and stores the next activation tile; step 1, behind the one
-  // barrier of the k-tile (every wave has finished reading this tile and stored the next),
-  // does the same one step further and issues the global loads.  Two waves share a SIMD, so
-  // one's conversions overlap the other's MFMAs; the group barriers only keep the memory
-  // operations spread between the MFMAs.
+  // The one barrier of the k-tile sits between the steps (every wave has finished reading this
+  // tile and stored the next); the second step issues the global loads: activations of k-tile
+  // kt + 2, weights of k-tile kt + PF into the ring stage this tile has finished with.
   auto tile = [&](auto Dc, int kt) {
     constexpr int d = decltype(Dc)::value, dn = (d + 1) % PF;
     const bool next_active = kt + 1 < kt_end;
     __builtin_amdgcn_sched_barrier(0);
-    expand_scales(ic<dn>{}, next_active);
-    convert(Dc, ic<1>{}, bfr[1], lp);
-    mfmas(ic<0>{});
-    lut_issue(ic<dn>{}, ic<0>{}, lp);
-    read_a(af[1], a_rd, ic<1>{});
-    store_a(a_wr_nxt);
-    if constexpr (MT == 8) {
-#pragma unroll
-      for (int i = 0; i < 8 * NT; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-        if (i < 4) __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        if (i >= 8 && i < 8 + AP) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-      }
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    kstep(ic<0>{}, Dc, ic<1>{}, ic<dn>{}, ic<0>{}, a_rd, ic<1>{}, ic<1>{}, ic<0>{}, ic<dn>{}, 0, next_active);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
-    convert(ic<dn>{}, ic<0>{}, bfr[0], lp);
-    mfmas(ic<1>{});
-    lut_issue(ic<dn>{}, ic<1>{}, lp);
-    read_a(af[0], a_rd_nxt, ic<0>{});
-    load_a(kt + 2);
-    load_w(Dc, kt + PF);
-    if constexpr (MT == 8) {
-#pragma unroll
-      for (int i = 0; i < 8 * NT; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        if (i >= 4 && i < 4 + AP + 2 * NT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      }
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    kstep(ic<1>{}, ic<dn>{}, ic<0>{}, ic<dn>{}, ic<1>{}, a_rd_nxt, ic<0>{}, ic<0>{}, ic<1>{}, ic<-1>{}, kt + 2, false);
     const uint32_t r = a_rd; a_rd = a_rd_nxt; a_rd_nxt = r;
     const uint32_t w = a_wr; a_wr = a_wr_nxt; a_wr_nxt = w;
   };
@@ -375,10 +411,10 @@ void qgemm128_kernel(const QLArgs a) {
     for (int c = 0; c < AP; ++c) lds_st128(a_wr + (uint32_t)(c * 32 * A_LD * 2), a_first[c]);
     expand_scales(ic<0>{}, true);
     __syncthreads();  // table and first activation tile
-    lut_issue(ic<0>{}, ic<0>{}, lp);
+    lut_issue(ic<0>{}, ic<0>{}, lp[1]);
     read_a(af[0], a_rd, ic<0>{});
-    convert(ic<0>{}, ic<0>{}, bfr[0], lp);
-    lut_issue(ic<0>{}, ic<1>{}, lp);
+    convert(ic<0>{}, ic<0>{}, bfr[0], lp[1]);
+    lut_issue(ic<0>{}, ic<1>{}, lp[0]);
     if (lora_fast) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
