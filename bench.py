@@ -132,9 +132,9 @@ def kernel_breakdown(model, runner, st, ctx, iters):
 
 
 # HBM bytes of one qgemm128 launch on the default workload (batch 128, Llama-3.1-8B shapes, mean
-# over the four linears): rocprofv3 FETCH_SIZE + WRITE_SIZE, (22833 + 12939) KiB, both counters
+# over the four linears): rocprofv3 FETCH_SIZE + WRITE_SIZE, (22190 + 12947) KiB, both counters
 # scaled by 1.000 against a plain copy of known size (profiles/qgemm128_kernel_llama8b_decode_b128.md).
-QGEMM128_TRAFFIC_BYTES_B128 = 36_630_528
+QGEMM128_TRAFFIC_BYTES_B128 = 35_980_288
 
 
 def rooflines(kern, default_workload=False):

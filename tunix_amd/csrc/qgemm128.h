@@ -294,8 +294,9 @@ void qgemm128_kernel(const QLArgs a) {
   // unit packs them to bf16.  The first half of the units also carries the LDS reads: one table
   // look-up each (pair u of the step AFTER the next, into the other half of lp) and the
   // activation fragments of the next step; the second half the stores of the next activation
-  // tile (ST, first step: issued seven units before the barrier behind the step asks for them)
-  // or the global loads (LD, second step).
+  // tile (ST, first step: issued seven units before the barrier behind the step asks for them),
+  // followed at once by the loads of the activation tile after that one into the same registers
+  // (a whole k-tile before their store), or the weight loads (LD, second step).
   // A scheduling barrier behind every unit keeps that order.
   auto kstep = [&](auto CURc, auto Dcc, auto Jcc, auto Dlc, auto Jlc, uint32_t rd_base, auto Jrc, auto STc,
                    auto LDc, auto EXc, int kt, bool ex_active) {
@@ -338,11 +339,11 @@ void qgemm128_kernel(const QLArgs a) {
 #pragma unroll
           for (int c = 0; c < AP; ++c) lds_st128(a_wr_nxt + (uint32_t)(c * 32 * A_LD * 2), a_next[c]);
         }
+        if (ST && q >= 1 && q <= AP)   // the registers just stored take the activation tile after the next
+          a_next[q - 1] = __builtin_amdgcn_raw_buffer_load_b128(xr, xo + (uint32_t)(q - 1) * xst, xs, 0);
         if (LD) {
           constexpr int DW = DL == 0 ? PF - 1 : DL - 1;   // the ring stage this k-tile has finished with
-          if (q < AP) {
-            a_next[q] = __builtin_amdgcn_raw_buffer_load_b128(xr, xo + (uint32_t)q * xst, xs, 0);
-          } else if (q >= 4 && q < 4 + NT) {
+          if (q >= 4 && q < 4 + NT) {
             ring_c[DW][q - 4] = __builtin_amdgcn_raw_buffer_load_b64(rc, coff[q - 4], wkt * 1024, 0);
           } else if (q >= 4 + NT && q < 4 + 2 * NT) {
             ring_s[DW][q - 4 - NT] = __builtin_amdgcn_raw_buffer_load_b32(rs, soff[q - 4 - NT], wkt * (16 * SPT * 2), 0);
@@ -368,13 +369,13 @@ void qgemm128_kernel(const QLArgs a) {
   // One k-tile of ring stage D = this wave's two k-steps.  On entry af[0] holds the activation
   // fragments of the first step, bfr[0] its weights and lp the table entries of the second.
   // The one barrier of the k-tile sits between the steps (every wave has finished reading this
-  // tile and stored the next); the second step issues the global loads: activations of k-tile
-  // kt + 2, weights of k-tile kt + PF into the ring stage this tile has finished with.
+  // tile and stored the next).  The first step fetches the activations of k-tile kt + 2, the
+  // second the weights of k-tile kt + PF into the ring stage this tile has finished with.
   auto tile = [&](auto Dc, int kt) {
     constexpr int d = decltype(Dc)::value, dn = (d + 1) % PF;
     const bool next_active = kt + 1 < kt_end;
     __builtin_amdgcn_sched_barrier(0);
-    kstep(ic<0>{}, Dc, ic<1>{}, ic<dn>{}, ic<0>{}, a_rd, ic<1>{}, ic<1>{}, ic<0>{}, ic<dn>{}, 0, next_active);
+    kstep(ic<0>{}, Dc, ic<1>{}, ic<dn>{}, ic<0>{}, a_rd, ic<1>{}, ic<1>{}, ic<0>{}, ic<dn>{}, kt + 2, next_active);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     kstep(ic<1>{}, ic<dn>{}, ic<0>{}, ic<dn>{}, ic<1>{}, a_rd_nxt, ic<0>{}, ic<0>{}, ic<1>{}, ic<-1>{}, kt + 2, false);
