@@ -34,7 +34,10 @@ def assert_bf16_close(got, ref, atol=1e-6, min_equal=0.97, what="", mag=None, ul
   results computed from several rounded intermediates, each of which may be one ulp off."""
   got, ref = got.float().cpu(), ref.float().cpu()
   diff = (got - ref).abs()
-  tol = (ref.abs() if mag is None else torch.maximum(ref.abs(), mag.float().cpu().abs())) * (ulps * 2.0 ** -7) + atol
+  # one ulp of the larger of the two values (the spacing doubles at a power of two: two
+  # neighbouring bf16 values on either side of it differ by the ulp of the upper one)
+  big = torch.maximum(ref.abs(), got.abs())
+  tol = (big if mag is None else torch.maximum(big, mag.float().cpu().abs())) * (ulps * 2.0 ** -7) + atol
   bad = (diff > tol).sum().item()
   eq = (got == ref).float().mean().item()
   assert bad == 0, f"{what}: {bad} elements beyond one bf16 ulp, max diff {diff.max().item()}"
@@ -130,18 +133,34 @@ def test_qlinear_many_rows_matches_oracle(gpu, M, K, N, group, qtype, r, seg_wid
   mul = epi in ("silu", "gelu")
   widths = seg_widths or ([N // 2, N // 2] if mul else [N])
   rp = (r + 31) // 32 * 32 if r else 0
-  ref = torch.empty(M, N)
+  gx = bf(x).to(gpu)
   a_t = torch.zeros(len(widths) * max(rp, 1), K)
   b_full = torch.zeros(N, max(rp, 1))
+  lora = []
   off = 0
   for i, wd in enumerate(widths):
-    a = b = None
     if r:
       a, b = _lora(K, wd, r, 30 + 2 * i)
       a_t[i * rp: i * rp + r] = a.t()
       b_full[off: off + wd, :r] = b.t()
-    ref[:, off: off + wd] = Q.qlinear_lora(x, codes[:, off: off + wd], scale[:, off: off + wd], group, qtype,
-                                           a, b, lora_scale=0.5)
+      lora.append(b)
+    off += wd
+  t = t_host = None
+  if r:
+    # t = bf16(x . A) by the kernel for these row counts (128-row MFMA tiles), checked on its own;
+    # the linear's reference then uses the kernel's t, so that a t element rounded the other way
+    # (one bf16 ulp, allowed) is not counted against the linear
+    t = torch.zeros(M, len(widths) * rp, dtype=torch.bfloat16, device=gpu)
+    ops.lora_down(gx, bf(a_t).to(gpu), t)
+    assert_bf16_close(t, Q.rb((x.double() @ a_t.t().double()).float()), what="lora_down, many rows")
+    t_host = t.float().cpu()
+  ref = torch.empty(M, N)
+  off = 0
+  for i, wd in enumerate(widths):
+    seg = Q.qlinear_lora(x, codes[:, off: off + wd], scale[:, off: off + wd], group, qtype).double()
+    if r:
+      seg = seg + 0.5 * (t_host[:, i * rp: i * rp + r].double() @ lora[i].double())
+    ref[:, off: off + wd] = seg.float()
     off += wd
   ref = Q.rb(ref)
   res = mag = None
@@ -154,13 +173,10 @@ def test_qlinear_many_rows_matches_oracle(gpu, M, K, N, group, qtype, r, seg_wid
     act = Q.rb(gte * Q.rb(torch.sigmoid(gte))) if epi == "silu" else \
         Q.rb(torch.nn.functional.gelu(gte, approximate="tanh"))
     ref = Q.rb(act * up)
-  gx = bf(x).to(gpu)
   c, s = ops.quantize_pack(bf(w).to(gpu), group, qtype, mul)
   y = torch.empty(M, N // 2 if mul else N, dtype=torch.bfloat16, device=gpu)
   kw = {}
   if r:
-    t = torch.zeros(M, len(widths) * rp, dtype=torch.bfloat16, device=gpu)
-    ops.lora_down(gx, bf(a_t).to(gpu), t)
     b_t = b_full
     if mul:
       b_t = torch.zeros_like(b_full)
@@ -178,6 +194,18 @@ def test_qlinear_many_rows_matches_oracle(gpu, M, K, N, group, qtype, r, seg_wid
   torch.cuda.synchronize()
   assert_bf16_close(y, ref, atol=1e-5 if mul else 1e-6, min_equal=0.9 if mul else 0.97, what=f"wide {epi}", mag=mag,
                     ulps=3 if mul else 1)   # act(gate) * up: gate and up may each be one ulp off
+
+
+@pytest.mark.parametrize("M,K,R", [(12300, 256, 192), (6200, 384, 128), (700, 128, 32)])
+def test_lora_down_many_rows(gpu, M, K, R):
+  """The MFMA flavours of the LoRA down-projection (128-, 64- and 32-row tiles, chosen by how many
+  work-groups the shape yields) against the oracle; t is written only in its R columns."""
+  from tunix_amd import ops
+  x, a_t = rnd((M, K), 41), rnd((R, K), 42, 0.02)
+  t = torch.full((M, R + 32), 7.0, dtype=torch.bfloat16, device=gpu)
+  ops.lora_down(bf(x).to(gpu), bf(a_t).to(gpu), t)
+  assert_bf16_close(t[:, :R], Q.rb((x.double() @ a_t.t().double()).float()), what="lora_down rows")
+  assert (t[:, R:].float() == 7.0).all()
 
 
 def test_qlinear_invariants(gpu):

@@ -409,6 +409,38 @@ int check_desc(const tnx_qlinear_desc* d) {
   return TNX_OK;
 }
 
+// The same product for many rows (prefill, per-token logps): 16 * MT rows x 64 adapter columns
+// per work-group through the dense main loop (x staged in LDS, A^T fragments straight from
+// global memory, MFMA), instead of tiles sized for a decode batch that re-read K-long rows per
+// tile.
+template <int MT>
+__global__ __launch_bounds__(256) void lora_down_rows_kernel(const uint16_t* x, int64_t M, int64_t K,
+                                                             const uint16_t* a_t, int R, uint16_t* t,
+                                                             int64_t t_ld) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  uint16_t* sA = reinterpret_cast<uint16_t*>(smem);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, lm = lane & 15, lq = lane >> 4;
+  TileSrc s;
+  s.M = M; s.K = K; s.x = x; s.row_index = nullptr; s.row_div = 1; s.x_rows = M;
+  s.w_bf16 = a_t; s.codes = nullptr; s.scales = nullptr; s.group = 0; s.qtype = 0;
+  s.ntiles = R / 16; s.lora_rank = 0; s.t = nullptr; s.t_ld = 0; s.lora_b = nullptr; s.lora_scale = 0.f;
+  const int64_t m0 = (int64_t)blockIdx.x * (16 * MT);
+  const int64_t ntile0 = (int64_t)blockIdx.y * 4 + wave;
+  f32x4 acc[MT][1];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) zero_acc(acc[mt][0]);
+  tile_mainloop<MT, 1, true>(s, m0, ntile0, 0, (int)(K / KTILE), sA, nullptr, acc);
+  if (ntile0 >= s.ntiles) return;
+  const int64_t col = ntile0 * 16 + lm;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t row = m0 + mt * 16 + lq * 4 + i;
+      if (row < M) t[row * t_ld + col] = f2bf(acc[mt][0][i]);
+    }
+}
+
 template <class Kern>
 int raise_lds_limit(Kern kern, size_t bytes) {
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -575,6 +607,26 @@ extern "C" int tnx_lora_down(void* stream, const uint16_t* x, int64_t M, int64_t
   TNX_REQUIRE(x && a_t && t, "lora_down: null pointer");
   TNX_REQUIRE(M > 0 && K > 0 && K % 32 == 0, "lora_down: K=%lld must be a multiple of 32", (long long)K);
   TNX_REQUIRE(R > 0 && R % 16 == 0 && t_ld >= R, "lora_down: R=%d must be a multiple of 16 and <= t_ld", R);
+  if (M >= 512 && K % KTILE == 0 && (uint64_t)(M + 128) * (uint64_t)K * 2 < (1ull << 32)) {
+    // many rows: MFMA tiles of 128 rows, or of 64 / 32 where that is what it takes to fill the
+    // device (32-bit buffer offsets: the activations must stay below 4 GiB)
+    const int64_t cols = cdiv(R, 64);
+    auto launch = [&](auto MTc) -> int {
+      constexpr int MT = decltype(MTc)::value;
+      constexpr size_t kSmem = 2 * (size_t)MT * 16 * A_LD * sizeof(uint16_t);
+      static std::once_flag once;
+      static int attr_rc = TNX_OK;
+      std::call_once(once, [] { attr_rc = raise_lds_limit(&lora_down_rows_kernel<MT>, kSmem); });
+      if (attr_rc) return attr_rc;
+      dim3 grid((unsigned)cdiv(M, 16 * MT), (unsigned)cols);
+      hipLaunchKernelGGL((lora_down_rows_kernel<MT>), grid, dim3(256), kSmem, as_stream(stream), x, M, K, a_t, R, t, t_ld);
+      TNX_CHECK_LAUNCH("lora_down_rows");
+      return TNX_OK;
+    };
+    if (cdiv(M, 128) * cols >= 192) return launch(std::integral_constant<int, 8>{});
+    if (cdiv(M, 64) * cols >= 192) return launch(std::integral_constant<int, 4>{});
+    return launch(std::integral_constant<int, 2>{});
+  }
   // smallest tm + tn whose grid still fits the device once; 16 x 16 when nothing does
   int tm = 16, tn = 16;
   {
