@@ -123,10 +123,10 @@ typedef struct tnx_qlinear_desc {
   float* ws;                /* fp32 [split_k, M, N] workspace (need not be initialised);
                                required when split_k > 1; tnx_splitk_finish adds the
                                partial tiles in split order and applies the epilogue        */
-  /* Optional (next_tpart != NULL), *_MUL epilogues with split_k == 1 and M > 64 only: the LoRA
+  /* Optional (next_tpart != NULL), *_MUL epilogues with split_k == 1 only: the LoRA
    * down-projection of the NEXT linear -- the one that consumes y, e.g. down_proj after
-   * gate|up -- fused into this epilogue.  Each 128-row x 128-column work-group tile leaves its
-   * share of y . A_next as one fp32 fragment plane; tnx_lora_reduce adds the planes in a fixed
+   * gate|up -- fused into this epilogue.  Each (up to) 128-row x 128-column work-group tile leaves
+   * its share of y . A_next as one fp32 fragment plane; tnx_lora_reduce adds the planes in a fixed
    * order and writes t_next = bf16(y . A_next), which tnx_lora_down would have produced.    */
   const uint16_t* next_a_t; /* bf16 [next_rank, N/2]: A_next transposed                     */
   int next_rank;            /* multiple of 16, <= 64                                        */
