@@ -439,11 +439,40 @@ void qgemm128_kernel(const QLArgs a) {
   }
   TNX_STAMP(3);
 
+  const bool has_rows = MT > 1 || kh == 0;
+  const int64_t m0w = m0 + kh * (HM * 16);   // first row of the tile this wave finishes
+  const uint32_t row_lds = (uint32_t)(kh * (HM * 16) * A_LD * 2);
+
+  // The adapter's share of the rows this wave will finish, before the k halves meet: it needs
+  // nothing from the partner (the t block sits in the activation buffer the last k-tile left
+  // as "next", the B^T fragments in LDS since the prologue), so it runs while slower waves are
+  // still in their last k-tile.
+  f32x4 part[HM][NT];
+#pragma unroll
+  for (int mt = 0; mt < HM; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) zero_acc(part[mt][nt]);
+  if (lora_fast && has_rows) {
+    const uint32_t tb = a_rd - (uint32_t)(kh * 64 * 2) + row_lds;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const uint32_t base = tb + (uint32_t)((toff[nt] == toff_a ? 0 : 64) * 2);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (j * 32 < a.lora_rank) {
+          const u32x4 lbf = lds_ld128(lb_lds + (uint32_t)((nt * 2 + j) * 1024));
+#pragma unroll
+          for (int mt = 0; mt < HM; ++mt)
+            part[mt][nt] = mfma16(lds_ld128(base + (uint32_t)((mt * 16 * A_LD + j * 32) * 2)), lbf, part[mt][nt]);
+        }
+      }
+    }
+  }
+
   // The two k halves meet: each wave keeps the row half kh of its column group (row tiles
   // [kh * HM, ...); with a single row tile the first wave keeps it and the second keeps none),
   // hands the other tiles to its partner through the (now idle) table area and adds what the
   // partner hands over.
-  const bool has_rows = MT > 1 || kh == 0;
   f32x4 out[HM][NT];
   {
     __syncthreads();  // every wave is done with the table
@@ -466,32 +495,13 @@ void qgemm128_kernel(const QLArgs a) {
         out[m][nt] = own + got;
       }
   }
-  const int64_t m0w = m0 + kh * (HM * 16);   // first row of this wave's tile
-  const uint32_t row_lds = (uint32_t)(kh * (HM * 16) * A_LD * 2);
-
   if (lora_fast && has_rows) {
-    // the t block sits in the activation buffer the last k-tile left as "next"
-    const uint32_t tb = a_rd - (uint32_t)(kh * 64 * 2) + row_lds;
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const uint32_t base = tb + (uint32_t)((toff[nt] == toff_a ? 0 : 64) * 2);
-      f32x4 part[HM];
+    for (int mt = 0; mt < HM; ++mt)
 #pragma unroll
-      for (int mt = 0; mt < HM; ++mt) zero_acc(part[mt]);
+      for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        if (j * 32 < a.lora_rank) {
-          const u32x4 lbf = lds_ld128(lb_lds + (uint32_t)((nt * 2 + j) * 1024));
-#pragma unroll
-          for (int mt = 0; mt < HM; ++mt)
-            part[mt] = mfma16(lds_ld128(base + (uint32_t)((mt * 16 * A_LD + j * 32) * 2)), lbf, part[mt]);
-        }
-      }
-#pragma unroll
-      for (int mt = 0; mt < HM; ++mt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) out[mt][nt][i] += a.lora_scale * part[mt][i];
-    }
+        for (int i = 0; i < 4; ++i) out[mt][nt][i] += a.lora_scale * part[mt][nt][i];
   } else if (a.lora_rank > 0 && blockIdx.z == 0 && !lora_fast && has_rows) {
     TileSrc s;
     s.M = a.M; s.K = a.K; s.x = a.x; s.row_index = nullptr; s.row_div = 1; s.x_rows = a.M;
