@@ -131,6 +131,40 @@ def kernel_breakdown(model, runner, st, ctx, iters):
   return out
 
 
+def many_rows_breakdown(model, rows, iters):
+  """The four linears of a layer at `rows` activation rows (one prefill / per-token-logps chunk):
+  the regime of the 128 x 256-tile GEMM kernel, bound by the matrix pipe.  Returns per-linear
+  microseconds and TFLOP/s and their mean as a fraction of the dense bf16 MFMA peak."""
+  import torch
+
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  dev, ly = model.device, model.layers[0]
+  bf = torch.bfloat16
+  out = {}
+  for key, epi in (("qkv", L.TNX_EPI_STORE), ("o", L.TNX_EPI_STORE), ("gu", L.TNX_EPI_SILU_MUL),
+                   ("down", L.TNX_EPI_STORE)):
+    f = ly[key]
+    x = torch.randn(rows, f.K, device=dev).to(bf)
+    y = torch.empty(rows, f.N // (2 if f.interleave2 else 1), dtype=bf, device=dev)
+    t = torch.randn(rows, max(f.rp * len(f.names), 32), device=dev).to(bf) if f.has_lora else None
+    d = ops.make_qlinear_desc(
+        M=rows, K=f.K, N=f.N, group=f.group, qtype=f.qtype, x=x, codes=f.codes, scales=f.scales, y=y,
+        epilogue=epi, lora_rank=f.rp, lora_nseg=(-1 if f.interleave2 else len(f.names)),
+        lora_seg_end=f.seg_end, lora_seg_toff=f.seg_toff, t=t, t_ld=t.shape[1] if t is not None else 0,
+        lora_b=f.b_t if f.has_lora else None, lora_scale=f.lora_scale)
+    ms = time_loop(lambda: ops.qlinear(d), iters, per_graph=2, warm=1)
+    flops = 2.0 * rows * f.K * f.N
+    out[key] = {"us": round(ms * 1e3, 1), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1)}
+    del x, y, t
+  tot_flops = sum(2.0 * rows * ly[k].K * ly[k].N for k in out)
+  tot_s = sum(v["us"] for v in out.values()) * 1e-6
+  tf = tot_flops / tot_s / 1e12
+  return {"kernel": "qgemm_wide_kernel", "rows": rows, "bound": "mfma", "achieved": round(tf, 1),
+          "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+          "linears": out}
+
+
 # HBM bytes of one qgemm128 launch on the default workload (batch 128, Llama-3.1-8B shapes, mean
 # over the four linears): rocprofv3 FETCH_SIZE + WRITE_SIZE, (22190 + 12947) KiB, both counters
 # scaled by 1.000 against a plain copy of known size (profiles/qgemm128_kernel_llama8b_decode_b128.md).
@@ -297,8 +331,9 @@ def main():
     for _ in range(3):
       dst.copy_(src)
     torch.cuda.synchronize()
+    many = many_rows_breakdown(model, 8192, max(2, args.kernel_iters // 5))
     print(json.dumps({"kernels_only": True, "context": P + T // 2, "roofline": roofline,
-                      "roofline_hbm": roofline_hbm,
+                      "roofline_hbm": roofline_hbm, "roofline_many_rows": many,
                       "kernels": {k: {"us": round(v["ms"] * 1e3, 2),
                                       "gemm_us": round(v.get("kernel_ms", v["ms"]) * 1e3, 2)}
                                   for k, v in kern.items()}}), flush=True)
@@ -380,6 +415,8 @@ def main():
     log(f"  {name:16s} {v['ms'] * 1e3:8.1f} us/launch  {v['gbs']:7.0f} GB/s  {v['tflops']:7.1f} TFLOP/s"
         f"  x{v['per_step']} = {v['step_ms']:.3f} ms/step")
   roofline, roofline_linears = rooflines(kern, default_workload=(B == 128 and not args.layers))
+  many = many_rows_breakdown(model, 8192, max(2, args.kernel_iters // 5))
+  log(f"  linears at 8192 rows (prefill / logps chunk): {many['achieved']} TFLOP/s, {many['linears']}")
   wb = model.weight_bytes()
   step_bytes = (wb["quantized"] + wb["lora"] + wb["head"]
                 + B * cfg.num_kv_heads * mean_ctx * cfg.head_dim * 4 * cfg.num_layers)
@@ -393,7 +430,7 @@ def main():
                  "context_range": [step_first + 1, step_last + 1], "parallelism": "single GPU"},
       "hbm_roofline_frac_step": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
       "step_bytes": int(step_bytes), "prefill_s": round(prefill_s, 3),
-      "roofline": roofline, "roofline_hbm": roofline_linears,
+      "roofline": roofline, "roofline_hbm": roofline_linears, "roofline_many_rows": many,
       "kernels": {k: {"us": round(v["ms"] * 1e3, 2), "GBps": round(v["gbs"], 1),
                       "TFLOPs": round(v["tflops"], 1), "ms_per_step": round(v["step_ms"], 4)}
                   for k, v in kern.items()},
