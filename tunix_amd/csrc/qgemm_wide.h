@@ -16,7 +16,7 @@
 //     operand), so that a lane owns runs of four consecutive output columns of one row and the
 //     tile leaves through LDS as whole 16-byte row chunks.
 //   * a slab is written as eight slots in issue order, one MFMA each with its share of the
-//     work for the following slabs; group barriers restate the slots for the scheduler.
+//     work for the following slabs; a scheduling barrier behind every slot keeps that order.
 //
 // Work-groups are numbered so that the eight XCDs (consecutive work-group ids go to
 // consecutive XCDs) each walk one 128-row block across the column tiles: a block's activations
@@ -111,6 +111,7 @@ void qgemm_wide_kernel(const QLArgs a) {
   u32x4 xf[2][RT];           // activation fragments of the current / next slab
   u32x4 wf[2][CG];           // weight fragments of the current / next slab
   uint32_t lp[CG][4];        // table entries (f16 level pairs) of the slab after the next
+  float cf0 = 0.f, cf1 = 0.f;  // products of the pair whose pack is still to come
 
   // LoRA: the k-tile after the last one is the 128-row block of t = bf16(x . A), columns
   // [toff_a, +64) | [toff_b, +64) (the host sends only shapes whose work-groups span at most
@@ -236,9 +237,15 @@ void qgemm_wide_kernel(const QLArgs a) {
       const int cg = i >> 2, rt = i & 3;
       acc[rt][cg] = mfma32(wf[CUR][cg], xf[CUR][rt], acc[rt][cg]);
       {
+        // the pack of the pair before this one (a slot behind its products: packed in the same
+        // slot it would wait on them); slot 0 packs the last pair of the slab before, which
+        // belongs to the fragment the MFMAs of slots 4-7 of THIS slab multiply
+        if (i == 0) wf[CUR][CG - 1][3] = cvt_pk_bf16(cf0, cf1);
+        else wf[NXT][(i - 1) >> 2][(i - 1) & 3] = cvt_pk_bf16(cf0, cf1);
         const h16x2 hh = __builtin_bit_cast(h16x2, lp[cg][rt]);
         const float sv = sc[DC][cg][SPT == 2 ? (UC >> 2) : (UC >> 1)];
-        wf[NXT][cg][rt] = cvt_pk_bf16(__builtin_fmaf((float)hh[0], sv, 0.0f), __builtin_fmaf((float)hh[1], sv, 0.0f));
+        cf0 = __builtin_fmaf((float)hh[0], sv, 0.0f);
+        cf1 = __builtin_fmaf((float)hh[1], sv, 0.0f);
         const uint32_t w = ring_c[DL][cg][UL & 1][UL >> 1];
         lp[cg][rt] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0400u + ((uint32_t)rt << 8)));
       }
@@ -253,14 +260,7 @@ void qgemm_wide_kernel(const QLArgs a) {
         const uint32_t w = ring_s[DN][i / SPT][(i % SPT) >> 1];
         sc[DN][i / SPT][i % SPT] = next_active ? (((i % SPT) & 1) ? bfhi(w) : bflo(w)) : 0.f;
       }
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-      if (EX && i < CG * SPT) __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      if ((i & 1) == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      if (ST) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-      if (LD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-      if (LD && i < 6) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      __builtin_amdgcn_sched_barrier(0);   // slots issue in the order written
     }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -323,7 +323,9 @@ void qgemm_wide_kernel(const QLArgs a) {
     for (int b = 0; b < 4; ++b) {
       const h16x2 hh = __builtin_bit_cast(h16x2, lp[cg][b]);
       const float sv = sc[0][cg][0];
-      wf[0][cg][b] = cvt_pk_bf16(__builtin_fmaf((float)hh[0], sv, 0.0f), __builtin_fmaf((float)hh[1], sv, 0.0f));
+      cf0 = __builtin_fmaf((float)hh[0], sv, 0.0f);
+      cf1 = __builtin_fmaf((float)hh[1], sv, 0.0f);
+      if (cg < CG - 1 || b < 3) wf[0][cg][b] = cvt_pk_bf16(cf0, cf1);   // the last pair: slot 0 of the loop
     }
 #pragma unroll
   for (int cg = 0; cg < CG; ++cg)
