@@ -8,7 +8,9 @@
 //     g run, the same wave converts the weights of step g+1 (two v_fma_mix_f32 + one
 //     v_cvt_pk_bf16_f32 per code pair), issues the table look-ups of step g+2 and reads the
 //     activation fragments of step g+1 -- a three-deep software pipeline that runs across
-//     k-tile boundaries;
+//     k-tile boundaries.  A step is written as units in issue order (one MFMA with its share
+//     of that work each) behind scheduling barriers: left to the scheduler, the conversions
+//     bunch up and pull look-ups that have not returned yet into waits;
 //   * the code book is an LDS table of f16 level pairs indexed by a code byte, replicated 64
 //     times with a 256-byte entry stride, so that the LDS address of a look-up is one
 //     v_perm_b32: (byte << 8) | (lane << 2); every bf16-rounded level is exact in f16, and
