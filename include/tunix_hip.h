@@ -172,6 +172,16 @@ int tnx_rmsnorm(void* stream, const uint16_t* x, const uint16_t* res_pre, uint16
 int tnx_rmsnorm_splitk(void* stream, const float* ws, int split_k, const uint16_t* res_pre,
                        uint16_t* h_out, const uint16_t* w, const uint16_t* res_post, uint16_t* y,
                        int64_t M, int64_t D, float eps, int flavor);
+/* Two norms in a row in one launch: y as above (input x, or the partial planes ws of a split-k
+ * linear when x is NULL), then y2 = norm(y) with weight w2.  Gemma-3's block applies
+ * post_attention_norm, adds the residual and applies pre_ffw_norm to the sum, and likewise
+ * post_ffw_norm + residual followed by the next block's pre_attention_norm
+ * (gemma3/model.py:882-898): y = h + norm(x) . w is the new residual stream, y2 the next
+ * linear's input.  Results equal those of two tnx_rmsnorm launches bit for bit.  D % 8 == 0. */
+int tnx_rmsnorm_pair(void* stream, const uint16_t* x, const float* ws, int split_k,
+                     const uint16_t* res_pre, uint16_t* h_out, const uint16_t* w,
+                     const uint16_t* res_post, uint16_t* y, const uint16_t* w2, uint16_t* y2,
+                     int64_t M, int64_t D, float eps, int flavor);
 
 /* ---------------------------------------------------------------------------------------
  * Per-head q/k RMSNorm (optional) + RoPE + KV-cache write for T tokens per row.

@@ -799,6 +799,50 @@ def test_rmsnorm_splitk_equals_finish_then_norm(gpu, family):
   assert torch.equal(y1, y2)
 
 
+@pytest.mark.parametrize("family", ["llama3", "qwen3", "gemma3"])
+@pytest.mark.parametrize("planes", [False, True])
+def test_rmsnorm_pair_equals_two_norms(gpu, family, planes):
+  """Post-norm + residual + next pre-norm in one launch (Gemma-3's block structure) against the
+  launches it replaces -- split-k finishing pass, norm with residual, norm -- bit for bit, and
+  the first norm against the oracle."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  from tunix_amd.model import _NORM
+  M, K, D, g, split = 70, 1024, 1152, 128, 4
+  x, res = rnd((M, K), 90), rnd((M, D), 91)
+  w = rnd((K, D), 92, 0.02)
+  w1 = bf(rnd((D,), 93, 0.3) + 1.0).to(gpu)
+  w2 = bf(rnd((D,), 94, 0.3) + 1.0).to(gpu)
+  c, s = ops.quantize_pack(bf(w).to(gpu), g, Q.INT4)
+  gx = bf(x).to(gpu)
+  ws = torch.empty(split * M * D, dtype=torch.float32, device=gpu)
+  tmp = torch.empty(M, D, dtype=torch.bfloat16, device=gpu)
+  d = ops.make_qlinear_desc(M=M, K=K, N=D, group=g, qtype=Q.INT4, x=gx, codes=c, scales=s, y=tmp,
+                            split_k=split, ws=ws)
+  ops.qlinear(d)                                   # planes + finishing pass -> tmp
+  h1 = bf(res).to(gpu)
+  xn1 = torch.empty_like(tmp)
+  ops.rmsnorm(tmp, w1, h1, 1e-6, _NORM[family], res_post=h1)
+  ops.rmsnorm(h1, w2, xn1, 1e-6, _NORM[family])
+  h2 = bf(res).to(gpu)
+  xn2 = torch.empty_like(tmp)
+  if planes:
+    ops.qlinear(d, finish=False)
+    ops.rmsnorm_pair(w1, h2, w2, xn2, 1e-6, _NORM[family], M, D, ws=ws, split_k=split, res_post=h2)
+  else:
+    ops.rmsnorm_pair(w1, h2, w2, xn2, 1e-6, _NORM[family], M, D, x=tmp, res_post=h2)
+  torch.cuda.synchronize()
+  assert torch.equal(h1, h2)
+  assert torch.equal(xn1, xn2)
+  ref_m = MR.RefModel.__new__(MR.RefModel)
+  ref_m.cfg, ref_m.bf16 = _Cfg(family, 1e-6), True
+  ref_h = Q.rb(ref_m.rmsnorm(tmp.float().cpu(), w1.float().cpu()) + Q.rb(res))
+  assert_bf16_close(h2, ref_h, min_equal=0.95, what="pair: first norm + residual")
+  assert_bf16_close(xn2, ref_m.rmsnorm(h2.float().cpu(), w2.float().cpu()), min_equal=0.95, what="pair: second norm")
+  with pytest.raises(ValueError):
+    ops.rmsnorm_pair(w1, h2, w2, xn2, 1e-6, _NORM[family], M, D, res_post=h2)   # neither x nor ws
+
+
 @pytest.mark.parametrize("kv_chunk,window,planes", [(0, 0, False), (32, 0, True), (0, 40, True), (64, 0, False)])
 def test_attention_with_fused_rope_equals_rope_then_attention(gpu, kv_chunk, window, planes):
   """Decode attention that rotates q / k and writes the step's key / value itself (from the qkv

@@ -86,7 +86,8 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
                                                           uint16_t* h_out, const uint16_t* w,
                                                           const uint16_t* res_post, uint16_t* y,
                                                           int64_t D, float eps, int flavor,
-                                                          const float* ws, int split_k, int64_t plane) {
+                                                          const float* ws, int split_k, int64_t plane,
+                                                          const uint16_t* w2, uint16_t* y2) {
   __shared__ float red[4];
   const int64_t row = blockIdx.x;
   const int nchunks = (int)(D / 8);
@@ -143,6 +144,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
   }
   ss = block_sum(ss, red);
   const float ms = finish_ms(ss, (float)D, flavor);
+  float ss2 = 0.f;
 #pragma unroll
   for (int c = 0; c < kNormMaxChunks; ++c) {
     const int ch = c * 256 + threadIdx.x;
@@ -162,6 +164,32 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
 #pragma unroll
       for (int j = 0; j < 4; ++j) q[j] = pack2bf(v[2 * j], v[2 * j + 1]);
       *reinterpret_cast<u32x4*>(y + o) = q;
+      if (w2) {   // the row just written is the input of a second norm: keep it, as rounded
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          h[c][j] = rbf(v[j]);
+          ss2 += sq_term(h[c][j], flavor);
+        }
+      }
+    }
+  }
+  if (!w2) return;
+  // y2 = norm(y) with its own weight, the row still in registers (same thread -> chunk map and
+  // reduction order as a launch of its own would use: the results are identical)
+  ss2 = block_sum(ss2, red);
+  const float ms2 = finish_ms(ss2, (float)D, flavor);
+#pragma unroll
+  for (int c = 0; c < kNormMaxChunks; ++c) {
+    const int ch = c * 256 + threadIdx.x;
+    if (ch < nchunks) {
+      float wv[8];
+      unpack8(*reinterpret_cast<const u32x4*>(w2 + (int64_t)ch * 8), wv);
+      u32x4 q;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        q[j] = pack2bf(norm_elem(h[c][2 * j], wv[2 * j], ms2, eps, flavor),
+                       norm_elem(h[c][2 * j + 1], wv[2 * j + 1], ms2, eps, flavor));
+      *reinterpret_cast<u32x4*>(y2 + row * D + (int64_t)ch * 8) = q;
     }
   }
 }
@@ -327,7 +355,8 @@ extern "C" int tnx_rmsnorm(void* stream, const uint16_t* x, const uint16_t* res_
   TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm: bad flavor %d", flavor);
   if (D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks)
     hipLaunchKernelGGL(rmsnorm_vec_kernel, dim3((unsigned)M), dim3(256), 0, as_stream(stream), x, res_pre,
-                       h_out, w, res_post, y, D, eps, flavor, (const float*)nullptr, 0, (int64_t)0);
+                       h_out, w, res_post, y, D, eps, flavor, (const float*)nullptr, 0, (int64_t)0,
+                       (const uint16_t*)nullptr, (uint16_t*)nullptr);
   else
     hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)M), dim3(256), (size_t)D * sizeof(float),
                        as_stream(stream), x, res_pre, h_out, w, res_post, y, D, eps, flavor);
@@ -345,8 +374,24 @@ extern "C" int tnx_rmsnorm_splitk(void* stream, const float* ws, int split_k, co
   TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm_splitk: bad flavor %d", flavor);
   hipLaunchKernelGGL(rmsnorm_vec_kernel, dim3((unsigned)M), dim3(256), 0, as_stream(stream),
                      (const uint16_t*)nullptr, res_pre, h_out, w, res_post, y, D, eps, flavor, ws, split_k,
-                     (int64_t)(M * D));
+                     (int64_t)(M * D), (const uint16_t*)nullptr, (uint16_t*)nullptr);
   TNX_CHECK_LAUNCH("rmsnorm_splitk");
+  return TNX_OK;
+}
+
+extern "C" int tnx_rmsnorm_pair(void* stream, const uint16_t* x, const float* ws, int split_k,
+                                const uint16_t* res_pre, uint16_t* h_out, const uint16_t* w,
+                                const uint16_t* res_post, uint16_t* y, const uint16_t* w2, uint16_t* y2,
+                                int64_t M, int64_t D, float eps, int flavor) {
+  TNX_REQUIRE((x != nullptr) != (ws != nullptr), "rmsnorm_pair: exactly one of x and ws must be given");
+  TNX_REQUIRE(w && y && w2 && y2, "rmsnorm_pair: null pointer");
+  if (ws) TNX_REQUIRE(split_k >= 1, "rmsnorm_pair: split_k must be >= 1");
+  TNX_REQUIRE(M > 0 && D > 0 && D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks,
+              "rmsnorm_pair: D=%lld must be a multiple of 8 and <= 16384", (long long)D);
+  TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm_pair: bad flavor %d", flavor);
+  hipLaunchKernelGGL(rmsnorm_vec_kernel, dim3((unsigned)M), dim3(256), 0, as_stream(stream), x, res_pre, h_out,
+                     w, res_post, y, D, eps, flavor, ws, ws ? split_k : 0, (int64_t)(M * D), w2, y2);
+  TNX_CHECK_LAUNCH("rmsnorm_pair");
   return TNX_OK;
 }
 

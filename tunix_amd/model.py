@@ -344,6 +344,14 @@ class Runner:
     else:
       ops.rmsnorm(self.h, w, self.xn, cfg.norm_eps, flavor, M=M)
 
+  def norm_pair(self, pending: int, w, w2, M):
+    """self.h += norm(self.tmp) . w (self.tmp = a linear's output, or its `pending` partial planes);
+    self.xn = norm(self.h) . w2 -- Gemma-3's post-norm + residual + next pre-norm in one launch."""
+    cfg = self.cfg
+    kw = dict(ws=self.splitk_ws, split_k=pending) if pending > 1 else dict(x=self.tmp)
+    ops.rmsnorm_pair(w, self.h, w2, self.xn, cfg.norm_eps, _NORM[cfg.family], M, cfg.embed_dim,
+                     res_post=self.h, **kw)
+
   def forward_hidden(self, tokens, positions, col_ptr, kcache, vcache, B=None, T=None):
     """Runs all layers for tokens[b, col .. col+T) of each row; leaves the final-normed hidden
     state in self.xn[:B*T].  kcache/vcache: lists of [B,Hkv,S,dh] tensors."""
@@ -359,9 +367,11 @@ class Runner:
         and _ROPE[cfg.family] == L.TNX_ROPE_LLAMA and cfg.head_dim == 128):
       # one table of this step's sines / cosines for all layers (they share theta)
       ops.rope_table(positions, col_ptr, B, m.layers[0]["timescale"], cfg.head_dim, self.rope_sin, self.rope_cos)
+    xn_ready = False   # gemma3: the block before has already normed the residual stream into self.xn
     for i, ly in enumerate(m.layers):
-      self.norm_after(pending, ly["attn_norm"], M)
-      pending = 1
+      if not xn_ready:
+        self.norm_after(pending, ly["attn_norm"], M)
+      pending, xn_ready = 1, False
       qkv_split = self.linear(ly["qkv"], self.xn, self.qkv, M, defer=True)
       # decode step of a model without q/k norm and with the Llama rotation: the attention kernel
       # rotates q / k and writes the cache itself, and the stand-alone launch is dropped
@@ -404,10 +414,10 @@ class Runner:
         ad.rope_sin, ad.rope_cos = self.rope_sin.data_ptr(), self.rope_cos.data_ptr()
       ops.gqa_attn(ad)
       if cfg.family == "gemma3":
-        self.linear(ly["o"], self.attn, self.tmp, M)
-        ops.rmsnorm(self.tmp, ly["post_attn_norm"], self.h, cfg.norm_eps, flavor, M=M,
-                    res_post=self.h)
-        ops.rmsnorm(self.h, ly["mlp_norm"], self.xn, cfg.norm_eps, flavor, M=M)
+        # h += post_attn_norm(o_proj); xn = mlp_norm(h): one launch, which also sums the
+        # projection's partial planes when it ran split
+        po = self.linear(ly["o"], self.attn, self.tmp, M, defer=True)
+        self.norm_pair(po, ly["post_attn_norm"], ly["mlp_norm"], M)
       else:
         po = self.linear(ly["o"], self.attn, self.h, M, epilogue=L.TNX_EPI_RESIDUAL, residual=self.h,
                          defer=True)
@@ -417,15 +427,18 @@ class Runner:
       elif cfg.family == "gemma3":
         fused = self.fuses_next(ly["gu"], ly["down"], M, L.TNX_EPI_GELU_MUL)
         self.linear(ly["gu"], self.xn, self.act, M, epilogue=L.TNX_EPI_GELU_MUL, next_f=ly["down"])
-        self.linear(ly["down"], self.act, self.tmp, M, t_ready=fused)
-        ops.rmsnorm(self.tmp, ly["post_ffw_norm"], self.h, cfg.norm_eps, flavor, M=M,
-                    res_post=self.h)
+        pd = self.linear(ly["down"], self.act, self.tmp, M, t_ready=fused, defer=True)
+        # h += post_ffw_norm(down_proj); xn = the next block's attn_norm (or the final norm) of h
+        nxt = m.layers[i + 1]["attn_norm"] if i + 1 < len(m.layers) else m.final_norm
+        self.norm_pair(pd, ly["post_ffw_norm"], nxt, M)
+        xn_ready = True
       else:
         fused = self.fuses_next(ly["gu"], ly["down"], M, L.TNX_EPI_SILU_MUL)
         self.linear(ly["gu"], self.xn, self.act, M, epilogue=L.TNX_EPI_SILU_MUL, next_f=ly["down"])
         pending = self.linear(ly["down"], self.act, self.h, M, epilogue=L.TNX_EPI_RESIDUAL,
                               residual=self.h, defer=True, t_ready=fused)
-    self.norm_after(pending, m.final_norm, M)
+    if not xn_ready:
+      self.norm_after(pending, m.final_norm, M)
     return self.xn
 
   def _moe(self, ex: ExpertBank, M: int):

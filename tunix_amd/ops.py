@@ -121,6 +121,14 @@ def rmsnorm_splitk(ws, split_k, w, y, eps, flavor, M, D, res_pre=None, h_out=Non
           "tnx_rmsnorm_splitk")
 
 
+def rmsnorm_pair(w, y, w2, y2, eps, flavor, M, D, x=None, ws=None, split_k=0, res_pre=None, h_out=None,
+                 res_post=None):
+  """y = [res_post +] norm(h) . w with h from x (or the split-k planes ws) [+ res_pre]; y2 = norm(y) . w2."""
+  L.check(L.lib().tnx_rmsnorm_pair(_stream(), _ptr(x), _ptr(ws), split_k, _ptr(res_pre), _ptr(h_out),
+                                   _ptr(w), _ptr(res_post), _ptr(y), _ptr(w2), _ptr(y2), M, D, float(eps),
+                                   flavor), "tnx_rmsnorm_pair")
+
+
 def rope_kvwrite(desc: L.RopeDesc):
   L.check(L.lib().tnx_qknorm_rope_kvwrite(_stream(), C.byref(desc)), "tnx_qknorm_rope_kvwrite")
 
