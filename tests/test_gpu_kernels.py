@@ -690,6 +690,27 @@ def test_grpo_ratio_matches_oracle(gpu):
   assert torch.all(ratio == 1.0)
 
 
+@pytest.mark.parametrize("n_tok,k,E", [(64, 8, 128), (1, 1, 1), (700, 8, 128), (3000, 2, 7), (33, 4, 640)])
+def test_moe_sort_routes_is_a_stable_counting_sort(gpu, n_tok, k, E):
+  """Routes sorted by expert, ties in route order, counts and offsets: against numpy's stable
+  argsort -- one batch of 1024 routes and several, few and many experts (more than 512 experts
+  take the general kernel), experts that receive nothing."""
+  from tunix_amd import ops
+  rng = np.random.Generator(np.random.PCG64(1000 + n_tok))
+  ids = rng.integers(0, max(1, E - 1 if E > 2 else E), size=(n_tok, k)).astype(np.int32)   # the last expert stays empty
+  ti = torch.from_numpy(ids).to(gpu)
+  counts = torch.full((E,), -1, dtype=torch.int32, device=gpu)
+  offs = torch.full((E + 1,), -1, dtype=torch.int32, device=gpu)
+  sr = torch.full((n_tok * k,), -1, dtype=torch.int32, device=gpu)
+  for _ in range(2):   # the second call sees the first call's leftovers in nothing it reads
+    ops.moe_sort_routes(ti, E, counts, offs, sr)
+  flat = ids.reshape(-1)
+  np.testing.assert_array_equal(sr.cpu().numpy(), np.argsort(flat, kind="stable"))
+  cnt = np.bincount(flat, minlength=E)
+  np.testing.assert_array_equal(counts.cpu().numpy(), cnt)
+  np.testing.assert_array_equal(offs.cpu().numpy(), np.concatenate([[0], np.cumsum(cnt)]))
+
+
 def test_moe_route_sort_gmm_combine(gpu):
   from tunix_amd import _lib as L
   from tunix_amd import ops

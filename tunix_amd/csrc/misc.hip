@@ -110,10 +110,11 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const uint16_t* scores, i
   }
 }
 
-// Counting sort of routes by expert; single work-group, stable in route order.
-__global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* topk_id, int64_t n_routes,
-                                                        int E, int32_t* counts, int32_t* offsets,
-                                                        int32_t* sorted_route) {
+// Counting sort of routes by expert; single work-group, stable in route order.  General form
+// (any E): one thread per expert scans the routes.
+__global__ __launch_bounds__(1024) void moe_sort_scan_kernel(const int32_t* topk_id, int64_t n_routes,
+                                                             int E, int32_t* counts, int32_t* offsets,
+                                                             int32_t* sorted_route) {
   extern __shared__ int32_t sh[];  // [E] counts, then [E] cursors
   int32_t* cnt = sh;
   int32_t* cur = sh + E;
@@ -137,6 +138,72 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* topk_id, 
     int32_t pos = cur[e];
     for (int64_t r = 0; r < n_routes; ++r)
       if (topk_id[r] == e) sorted_route[pos++] = (int32_t)r;
+  }
+}
+
+// The same for E <= 512 (every model on the path), one thread per ROUTE: the routes are walked
+// 1024 at a time; within a wave, lanes of the same expert find each other by ballots and number
+// themselves; a per-wave, per-expert count table in LDS gives each wave the routes of its
+// expert in the waves before it; a cursor per expert carries over from one batch of 1024 to
+// the next.  Three barriers per batch, no scan over the routes per expert.
+constexpr int kSortMaxE = 512;
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* topk_id, int64_t n_routes,
+                                                        int E, int32_t* counts, int32_t* offsets,
+                                                        int32_t* sorted_route) {
+  extern __shared__ int32_t sh[];  // [E] cursors, [16][E] per-wave counts of the current batch
+  int32_t* cur = sh;
+  int32_t* wcnt = sh + E;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < 17 * E; i += 1024) sh[i] = 0;
+  __syncthreads();
+  for (int64_t r = tid; r < n_routes; r += 1024) atomicAdd(&cur[topk_id[r]], 1);
+  __syncthreads();
+  if (tid == 0) {   // counts -> exclusive offsets (E <= 512: a few microseconds)
+    int32_t acc = 0;
+    for (int e = 0; e < E; ++e) {
+      const int32_t c = cur[e];
+      counts[e] = c;
+      offsets[e] = acc;
+      cur[e] = acc;
+      acc += c;
+    }
+    offsets[E] = acc;
+  }
+  __syncthreads();
+  const uint64_t below = lane ? (~0ull >> (64 - lane)) : 0ull;
+  for (int64_t r0 = 0; r0 < n_routes; r0 += 1024) {
+    const int64_t r = r0 + tid;
+    const int e = r < n_routes ? topk_id[r] : -1;
+    int rank = 0, mine = 0;
+    bool leader = false;
+    uint64_t todo = __ballot(e >= 0);
+    while (todo) {   // wave-uniform: one turn per distinct expert in the wave
+      const int l = __builtin_amdgcn_readfirstlane(__ffsll((long long)todo) - 1);
+      const int le = __builtin_amdgcn_readlane(e, l);
+      const uint64_t m = __ballot(e == le);
+      if (e == le) {
+        rank = __popcll(m & below);
+        mine = __popcll(m);
+        leader = lane == l;
+      }
+      todo &= ~m;
+    }
+    if (leader) wcnt[wave * E + e] = mine;
+    __syncthreads();
+    if (e >= 0) {
+      int32_t base = cur[e];
+      for (int w = 0; w < wave; ++w) base += wcnt[w * E + e];
+      sorted_route[base + rank] = (int32_t)r;
+    }
+    __syncthreads();
+    for (int x = tid; x < E; x += 1024) {
+      int32_t s = 0;
+#pragma unroll
+      for (int w = 0; w < 16; ++w) s += wcnt[w * E + x];
+      cur[x] += s;
+    }
+    __syncthreads();
+    if (leader) wcnt[wave * E + e] = 0;
   }
 }
 
@@ -198,8 +265,12 @@ extern "C" int tnx_moe_sort_routes(void* stream, const int32_t* topk_id, int64_t
                                    int32_t* counts, int32_t* offsets, int32_t* sorted_route) {
   TNX_REQUIRE(topk_id && counts && offsets && sorted_route, "moe_sort: null pointer");
   TNX_REQUIRE(M > 0 && k > 0 && E > 0 && E <= 4096 && M * k <= (1 << 20), "moe_sort: bad shape");
-  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), (size_t)(2 * E) * sizeof(int32_t),
-                     as_stream(stream), topk_id, M * k, E, counts, offsets, sorted_route);
+  if (E <= kSortMaxE)
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), (size_t)(17 * E) * sizeof(int32_t),
+                       as_stream(stream), topk_id, M * k, E, counts, offsets, sorted_route);
+  else
+    hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(1), dim3(1024), (size_t)(2 * E) * sizeof(int32_t),
+                       as_stream(stream), topk_id, M * k, E, counts, offsets, sorted_route);
   TNX_CHECK_LAUNCH("moe_sort");
   return TNX_OK;
 }

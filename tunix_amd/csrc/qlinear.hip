@@ -667,10 +667,15 @@ extern "C" int tnx_moe_int4_gmm(void* stream, const tnx_moe_gmm_desc* d) {
   a.codes_stride = (int64_t)(cb / 4); a.scales_stride = (int64_t)(sb / 2);
   // Any expert can receive up to all rows (one route per token and expert): the grid covers
   // that bound and blocks past an expert's count exit at once.
+  // The row tile follows the rows an expert gets on average (n_routes / E: 4 for a decode batch of
+  // 64 with top-8 routing over 128 experts): the dequantisation per k-tile is the same for every
+  // tile height, the MFMA, staging and LDS work is not, and two 16-row work-groups share a
+  // compute unit.  An expert with more rows than one tile takes several (weights read again).
   const int64_t max_rows = d->n_routes / d->k;
+  const int64_t avg_rows = cdiv(d->n_routes, (int64_t)d->E);
   hipStream_t st = as_stream(stream);
-  if (max_rows <= 16) return launch_moe<1, 2>(st, a, d->E, max_rows);
-  if (max_rows <= 32) return launch_moe<2, 2>(st, a, d->E, max_rows);
+  if (max_rows <= 16 || avg_rows <= 8) return launch_moe<1, 2>(st, a, d->E, max_rows);
+  if (max_rows <= 32 || avg_rows <= 24) return launch_moe<2, 2>(st, a, d->E, max_rows);
   return launch_moe<4, 2>(st, a, d->E, max_rows);
 }
 
