@@ -219,6 +219,49 @@ __global__ void moe_combine_kernel(const uint16_t* y, const uint16_t* topk_w, in
   }
 }
 
+// The same for D % 8 == 0 and k <= 16: eight columns per thread, the k expert rows fetched with
+// independent 16-byte loads (same summation order per element: j ascending).
+__global__ __launch_bounds__(256) void moe_combine_vec_kernel(const uint16_t* y, const uint16_t* topk_w, int k,
+                                                              int64_t D, const uint16_t* residual,
+                                                              uint16_t* out) {
+  const int64_t m = blockIdx.x;
+  const int64_t d0 = ((int64_t)blockIdx.y * 256 + threadIdx.x) * 8;
+  if (d0 >= D) return;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  for (int j0 = 0; j0 < k; j0 += 8) {
+    u32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      v[u] = *reinterpret_cast<const u32x4*>(y + (m * k + min(j0 + u, k - 1)) * D + d0);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (j0 + u < k) {
+        const float w = bf2f(topk_w[m * k + j0 + u]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          acc[2 * q] += w * bflo(v[u][q]);
+          acc[2 * q + 1] += w * bfhi(v[u][q]);
+        }
+      }
+    }
+  }
+  u32x4 r = {0, 0, 0, 0};
+  if (residual) r = *reinterpret_cast<const u32x4*>(residual + m * D + d0);
+  u32x4 o;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    float lo = rbf(acc[2 * q]), hi = rbf(acc[2 * q + 1]);
+    if (residual) {
+      lo = rbf(lo + bflo(r[q]));
+      hi = rbf(hi + bfhi(r[q]));
+    }
+    o[q] = pack2bf(lo, hi);
+  }
+  *reinterpret_cast<u32x4*>(out + m * D + d0) = o;
+}
+
 }  // namespace
 
 extern "C" int tnx_fill_u32(void* stream, uint32_t* p, int64_t n, uint32_t value) {
@@ -278,8 +321,12 @@ extern "C" int tnx_moe_sort_routes(void* stream, const int32_t* topk_id, int64_t
 extern "C" int tnx_moe_combine(void* stream, const uint16_t* y, const uint16_t* topk_w, int64_t M,
                                int k, int64_t D, const uint16_t* residual, uint16_t* out) {
   TNX_REQUIRE(y && topk_w && out && M > 0 && k > 0 && D > 0, "moe_combine: bad arguments");
-  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)M), dim3(256), 0, as_stream(stream), y,
-                     topk_w, k, D, residual, out);
+  if (D % 8 == 0 && D <= 2048 * 65535)
+    hipLaunchKernelGGL(moe_combine_vec_kernel, dim3((unsigned)M, (unsigned)cdiv(D, 2048)), dim3(256), 0,
+                       as_stream(stream), y, topk_w, k, D, residual, out);
+  else
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)M), dim3(256), 0, as_stream(stream), y,
+                       topk_w, k, D, residual, out);
   TNX_CHECK_LAUNCH("moe_combine");
   return TNX_OK;
 }
