@@ -78,28 +78,23 @@ __device__ __forceinline__ float code_level_imm(int qtype, int code) {
 // (a group of 128 or more repeats its scale), so that a lane's scales are one aligned 4- or 8-byte word.
 __host__ __device__ inline int scales_per_tile(int group) { return group >= 64 ? 2 : 128 / group; }
 
-// LDS look-up table: byte (two codes) -> two bf16 levels, replicated so that lane l reads
-// entry [byte][l % 32] and every lane of a half-wave hits its own bank.
+// LDS look-up table: byte (two codes) -> two levels as an f16 pair (every bf16-rounded level is
+// exact in f16, and v_fma_mix_f32 converts the half it selects and multiplies it with the fp32
+// scale in one instruction), replicated so that lane l reads entry [byte][l % 32] and every
+// lane of a half-wave hits its own bank.
 #define TNX_LUT_COPIES 32
 #define TNX_LUT_WORDS (256 * TNX_LUT_COPIES)
 __device__ __forceinline__ void build_lut(uint32_t* lut, int qtype, int tid, int nthreads) {
   // thread `byte` looks its two levels up once and writes all copies of its entry
   for (int byte = tid; byte < 256; byte += nthreads) {
-    const uint32_t v = pack2bf(code_level(qtype, byte & 15), code_level(qtype, byte >> 4));
+    typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+    const f16x2_t hv = {(_Float16)rbf(code_level(qtype, byte & 15)), (_Float16)rbf(code_level(qtype, byte >> 4))};
+    const uint32_t v = __builtin_bit_cast(uint32_t, hv);
 #pragma unroll
     for (int c = 0; c < TNX_LUT_COPIES; ++c)  // rotated so that the lanes hit different banks
       lut[byte * TNX_LUT_COPIES + ((c + tid) & (TNX_LUT_COPIES - 1))] = v;
   }
 }
-__device__ __forceinline__ u32x4 dequant8(uint32_t w, const uint32_t* lut_lane) {
-  u32x4 r;
-  r[0] = lut_lane[(w & 0xffu) * TNX_LUT_COPIES];
-  r[1] = lut_lane[((w >> 8) & 0xffu) * TNX_LUT_COPIES];
-  r[2] = lut_lane[((w >> 16) & 0xffu) * TNX_LUT_COPIES];
-  r[3] = lut_lane[(w >> 24) * TNX_LUT_COPIES];
-  return r;
-}
-
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
@@ -110,8 +105,9 @@ __device__ __forceinline__ u32x4 dequant8_scaled(uint32_t w, const uint32_t* lut
   u32x4 r;
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
-    const uint32_t p = lut_lane[((w >> (8 * b)) & 0xffu) * TNX_LUT_COPIES];
-    r[b] = cvt_pk_bf16(bflo(p) * scale, bfhi(p) * scale);
+    typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+    const f16x2_t h = __builtin_bit_cast(f16x2_t, lut_lane[((w >> (8 * b)) & 0xffu) * TNX_LUT_COPIES]);
+    r[b] = cvt_pk_bf16(__builtin_fmaf((float)h[0], scale, 0.0f), __builtin_fmaf((float)h[1], scale, 0.0f));
   }
   return r;
 }

@@ -146,6 +146,59 @@ __device__ __forceinline__ void tile_mainloop(const TileSrc& s, int64_t m0, int6
         sc[nt] = __builtin_amdgcn_raw_buffer_load_b64(rs, (tile * 16u + (uint32_t)lm) * (uint32_t)spt * 2u, 0, 0);
       }
     };
+    if constexpr (MT == 1) {
+      // One 16-row tile (a decode batch, the few rows an expert gets): every wave fetches the
+      // activation fragments of its MFMAs itself, straight from global memory in fragment
+      // layout (16 rows x 64 bytes per load, the four waves' requests meet in L1) -- no LDS
+      // staging, no barrier in the loop, the waves drift apart and hide each other's waits.
+      constexpr int PX = 3;
+      int64_t src = m0 + lm;
+      if (s.row_index) src = s.row_index[src < s.M ? src : s.M - 1] / s.row_div;   // gather; rows past M: a clamped row, never stored
+      const uint32_t xoff = ((uint32_t)src * (uint32_t)s.K + (uint32_t)(lq * 8)) * 2u;   // rows past M (no gather) lie beyond the resource: zeros
+      u32x4 xr[PX][4], rc3[PX][NT];
+      u32x2 rs3[PX][NT];
+      auto load_x = [&](u32x4 (&dst)[4], int kt) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          dst[j] = __builtin_amdgcn_raw_buffer_load_b128(rx, xoff, (kt * KTILE + j * 32) * 2, 0);
+      };
+      const int kt_last = ktiles - 1;
+#pragma unroll
+      for (int d = 0; d < PX; ++d) {
+        load_x(xr[d], min(kt_begin + d, kt_last));
+        load_w(rc3[d], rs3[d], min(kt_begin + d, kt_last));
+      }
+      __syncthreads();  // the code-book table (built by the caller just before) is complete
+      for (int kt0 = kt_begin; kt0 < kt_end; kt0 += PX) {
+#pragma unroll
+        for (int d = 0; d < PX; ++d) {
+          const int kt = kt0 + d;
+          const bool active = kt < kt_end;
+          u32x4 cw[NT], xf[4];
+          float sc[NT][4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) xf[j] = xr[d][j];
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            cw[nt] = rc3[d][nt];
+            const u32x2 p = rs3[d][nt];
+            float f[4] = {bflo(p[0]), bfhi(p[0]), bflo(p[1]), bfhi(p[1])};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sc[nt][j] = spt == 2 ? f[j >> 1] : f[j];
+          }
+          load_x(xr[d], min(kt + PX, kt_last));
+          load_w(rc3[d], rs3[d], min(kt + PX, kt_last));
+          if (active)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+              for (int nt = 0; nt < NT; ++nt)
+                acc[0][nt] = mfma16(xf[j], dequant8_scaled(cw[nt][j], lut_lane, sc[nt][j]), acc[0][nt]);
+            }
+        }
+      }
+      return;
+    }
     // Loads are never predicated (k-tiles past the end read unused neighbouring or zero data)
     // and the trip count is padded to a multiple of PF, so every wait is counted exactly.
     load_a<MT>(s, rx, m0, kt_begin, tid, a_next);
