@@ -427,7 +427,7 @@ def test_gqa_attention_matches_oracle(gpu, B, T, S, Hq, Hkv, dh, col, chunk, win
 
 
 @pytest.mark.parametrize("M,D,V,dense", [(8, 512, 32000, True), (128, 512, 4096, True),
-                                         (130, 256, 1040, True),   # 256-column tiles, odd block count
+                                         (130, 256, 1040, True),   # two row blocks, partial last column block
                                          (50, 256, 1040, False), (130, 256, 4096, False)])
 def test_lmhead_greedy_and_logp(gpu, M, D, V, dense):
   from tunix_amd import _lib as L
