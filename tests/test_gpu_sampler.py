@@ -159,6 +159,45 @@ def test_sampler_contract(tiny, gpu):
     sampler(["5"], 2, beam_size=2)
 
 
+def test_single_step_forbidden_ids_and_prompt_length(tiny, gpu):
+  """The cases of tests/generate/sampler_test.py:412-466 (one generation step: the decode loop
+  adds nothing after the prefill), :632-665 (forbidden ids never appear, in greedy mode and when
+  drawing) and :100-152 (an explicit max_prompt_length at least as long as the prompts is used
+  as given, a shorter one is replaced by the next power of two)."""
+  from tunix_amd.generate import CacheConfig, Sampler
+  from tunix_amd.generate.utils import IdTokenizer
+  cfg, w, model = tiny
+  V = cfg.vocab_size
+  tok = IdTokenizer(V, pad_id=0, eos_id=1)
+  sampler = Sampler(model, tok, CacheConfig(64, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim))
+  prompts = ["5 6 7", "9 10 11 12 13"]
+  ref = sampler(prompts, max_generation_steps=6, eos_tokens=[-1])
+  one = sampler(prompts, max_generation_steps=1, eos_tokens=[-1], return_logprobs=True)
+  assert [len(t) for t in one.tokens] == [1, 1]
+  assert [int(t[0]) for t in one.tokens] == [int(t[0]) for t in ref.tokens]
+  assert all(len(lp) == 1 and np.isfinite(lp).all() for lp in one.logprobs)
+
+  allowed = V // 4
+  forbidden = set(range(allowed, V)) | {tok.eos_id()}
+  steps = 40
+  for kw in (dict(temperature=1.0, seed=123),                       # greedy: no top_p given
+             dict(temperature=1.0, top_p=1.0, seed=123),             # categorical draw in the head
+             dict(temperature=0.8, top_p=0.9, top_k=20, seed=7)):    # top-k / top-p kernel
+    out = sampler(["5 6 7"], max_generation_steps=steps, forbidden_tokens=forbidden, **kw)
+    assert len(out.tokens[0]) == steps, kw
+    assert not (set(out.tokens[0].tolist()) & forbidden), kw
+
+  wide = sampler(prompts, max_generation_steps=4, max_prompt_length=16, eos_tokens=[-1])
+  assert wide.padded_prompt_tokens.shape == (2, 16)
+  assert wide.padded_prompt_tokens[1].tolist() == [0] * 11 + [9, 10, 11, 12, 13]
+  short = sampler(prompts, max_generation_steps=4, max_prompt_length=2, eos_tokens=[-1])
+  assert short.padded_prompt_tokens.shape == (2, 8)
+  # left padding is masked out: the continuation does not depend on the padded width
+  for b in range(2):
+    np.testing.assert_array_equal(wide.tokens[b], ref.tokens[b][:4])
+    np.testing.assert_array_equal(short.tokens[b], ref.tokens[b][:4])
+
+
 @pytest.mark.parametrize("top_k,top_p", [(50, 0.95), (None, 0.9), (None, 1.0)])
 def test_top_p_sampling_against_oracle(tiny, gpu, top_k, top_p):
   """temperature / top-k / top-p, top-p over the whole vocabulary (no top-k) and the plain
