@@ -390,6 +390,30 @@ int tnx_grpo_ratio(void* stream, const float* logp, const float* old_logp, const
                    int64_t N, int64_t tokens_per_seq, float eps_lo, float eps_hi, float* ratio,
                    float* loss, int32_t* clipped);
 
+/* Per-token KL estimators between the trained and the reference policy
+ * (tunix/rl/common.py:135-184): TNX_KL_KL logp - ref; TNX_KL_MSE 0.5 * (logp - ref)^2;
+ * TNX_KL_LOW_VAR exp(d) - d - 1 with d = ref - logp.  clamp >= 0 clips the result to
+ * [-clamp, clamp]; a negative clamp means none (the reference's clamp_value=None). */
+enum { TNX_KL_KL = 0, TNX_KL_MSE = 1, TNX_KL_LOW_VAR = 2 };
+int tnx_kl_divergence(void* stream, const float* logp, const float* ref_logp, int64_t N, int method,
+                      float clamp, float* kl);
+
+/* Loss aggregation without packing segments (tunix/rl/common.py:763-854): out[0] = unreduced sum,
+ * out[1] = denominator of the mode; the caller divides as WeightedMetric.compute does
+ * (tunix/sft/utils.py:201-219).  per_token_loss, mask: fp32 [B, T]; row_ws: [B, 2] fp32 workspace
+ * (per-row sum of loss * mask, per-row sum of mask).  norm: the `norm` keyword of the two modes
+ * that take one (the caller passes the reference's default, T or B, when the keyword is absent).
+ * Sums run in a fixed order: the result is the same on every launch. */
+enum {
+  TNX_AGG_TOKEN_MEAN = 0,              /* "token-mean" */
+  TNX_AGG_SEQ_MEAN_TOKEN_MEAN = 1,     /* "sequence-mean-token-mean" */
+  TNX_AGG_SEQ_MEAN_TOKEN_SCALE = 2,    /* "sequence-mean-token-scale" */
+  TNX_AGG_SEQ_MEAN_TOKEN_SUM = 3,      /* "seq-mean-token-sum" */
+  TNX_AGG_SEQ_MEAN_TOKEN_SUM_NORM = 4  /* "sequence-mean-token-sum-norm" */
+};
+int tnx_aggregate_loss(void* stream, const float* per_token_loss, const float* mask, int64_t B, int64_t T,
+                       int mode, float norm, float* row_ws, float* out);
+
 /* Fill n 32-bit words with `value` (graph-capturable replacement for hipMemsetAsync). */
 int tnx_fill_u32(void* stream, uint32_t* p, int64_t n, uint32_t value);
 

@@ -13,6 +13,8 @@ tree).  Pinning status of each part:
                  scipy.special.logsumexp / torch.log_softmax and the chunk-invariance property of
                  tests/rl/common_test.py:340-399; GRPO ratio: closed form + the old=None case of
                  tests/rl/algo_core_test.py:51-143 (ratio == 1).
+                 aggregate_loss (five modes, no packing segments) and WeightedMetric.compute:
+                 pinned by the thirteen literal cases of tests/rl/common_test.py:457-576.
   model_ref      RMSNorm / RoPE / GQA attention / SwiGLU / full decoder: pinned against
                  transformers' Qwen3 / Llama / Gemma3 / Qwen3Moe random-init models in fp32
                  (tol 1e-3, the equivalence tests/model_alignment/qwen_align_test.py:113-200

@@ -1,6 +1,8 @@
-"""Per-token log-probabilities, KL estimators and the GRPO clipped ratio (oracle; tests only).
+"""Per-token log-probabilities, KL estimators, loss aggregation and the GRPO clipped ratio
+(oracle; tests only).
 
-Follows tunix/rl/common.py:135-203, :234-291, :326-571 and tunix/rl/algo_core.py:440-489.
+Follows tunix/rl/common.py:135-203, :234-291, :326-571, :763-854 and
+tunix/rl/algo_core.py:440-489.
 """
 from __future__ import annotations
 
@@ -97,3 +99,50 @@ def grpo_ratio(logp, old_logp, adv, eps_lo, eps_hi):
   l1 = -a * ratio
   l2 = -a * np.clip(ratio, np.float32(1 - eps_lo), np.float32(1 + eps_hi))
   return ratio, np.maximum(l1, l2).astype(np.float32), (l2 > l1)
+
+
+def aggregate_loss(per_token_loss, completion_mask, loss_agg_mode, **kwargs):
+  """tunix/rl/common.py:763-854 without packing segments, in float64:
+  (unreduced_sum, denominator, min_denom)."""
+  loss = np.asarray(per_token_loss, dtype=np.float64)
+  mask = np.asarray(completion_mask, dtype=np.float64)
+
+  def get_norm(default):  # tunix/rl/common.py:1151-1177
+    if "norm" in kwargs:
+      try:
+        norm = float(kwargs["norm"])
+      except (ValueError, TypeError):
+        raise ValueError(f"Invalid 'norm' value: {kwargs['norm']}. Must be a positive number.")
+      if norm <= 0:
+        raise ValueError(f"Invalid 'norm' value: {norm}. Must be a positive number.")
+      return norm
+    return default
+
+  if loss_agg_mode == "token-mean":
+    return (loss * mask).sum(), mask.sum(), 1.0
+  if loss_agg_mode == "sequence-mean-token-mean":
+    seq_mask = mask.sum(axis=-1)
+    seq_loss = (loss * mask).sum(axis=-1) / np.clip(seq_mask, 1.0, None)
+    return seq_loss.sum(), float((seq_mask > 0).sum()), 1.0
+  if loss_agg_mode == "sequence-mean-token-scale":
+    norm = get_norm(loss.shape[-1])
+    seq_loss = (loss * mask).sum(axis=-1) / max(norm, 1e-6)
+    return seq_loss.sum(), float((mask.sum(axis=-1) > 0).sum()), 1.0
+  if loss_agg_mode == "seq-mean-token-sum":
+    seq_loss = (loss * mask).sum(axis=-1)
+    seq_mask = (mask.sum(axis=-1) > 0).astype(np.float64)
+    return (seq_loss * seq_mask).sum(), seq_mask.sum(), 1e-6
+  if loss_agg_mode == "sequence-mean-token-sum-norm":
+    norm = get_norm(loss.shape[0])
+    return (loss * mask).sum(), float(norm), 1e-6
+  raise ValueError(f"Unsupported loss aggregation mode: {loss_agg_mode}.")
+
+
+def weighted_metric_compute(unreduced_sum, denominator, min_denom=None, eps=None):
+  """WeightedMetric.compute, tunix/sft/utils.py:201-219."""
+  denom = float(denominator)
+  if eps is not None:
+    denom = denom + eps
+  if min_denom is not None:
+    denom = max(denom, min_denom)
+  return 0.0 if denom == 0 else float(unreduced_sum) / denom

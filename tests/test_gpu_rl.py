@@ -223,3 +223,93 @@ def test_fused_head_logps_training_scale_shapes(gpu):
   r_ref, l_ref, _ = R.grpo_ratio(tlp.view(-1, 64).numpy(), old.view(-1, 64).numpy(), adv.numpy(), 0.2, 0.2)
   np.testing.assert_allclose(ratio.cpu().numpy(), r_ref, rtol=2e-6)
   np.testing.assert_allclose(loss.cpu().numpy(), l_ref, rtol=2e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("method", ["kl", "mse_kl", "low_var_kl"])
+@pytest.mark.parametrize("clamp", [None, 0.05])
+def test_kl_divergence_matches_oracle(gpu, method, clamp):
+  """tnx_kl_divergence against the oracle (itself pinned to the reference's KL tables): fp32
+  arithmetic, so 1e-6 absolute (expf against numpy's exp in exp(d) - d - 1) plus 1e-6 relative;
+  closed forms at equal inputs; the training-scale size of 128 x 1024 tokens."""
+  from tunix_amd.rl import common as C
+  rng = np.random.default_rng(5)
+  for shape in ((3, 7), (128, 1024)):
+    lp = (-rng.gamma(2.0, 1.5, size=shape)).astype(np.float32)
+    ref = (lp + rng.normal(0, 0.3, size=shape)).astype(np.float32)
+    ref[0, 0] = lp[0, 0] - 30.0 if method != "low_var_kl" else lp[0, 0] + 30.0   # an outlier for the clamp
+    got = C.compute_kl_divergence(torch.from_numpy(lp).to(gpu), torch.from_numpy(ref).to(gpu), method, clamp)
+    want = R.compute_kl_divergence(lp, ref, method, clamp)
+    assert got.shape == shape and got.dtype == torch.float32
+    np.testing.assert_allclose(got.cpu().numpy(), want, rtol=2e-6, atol=1e-6)
+    if clamp is not None:
+      assert got.abs().max().item() <= float(np.float32(clamp))
+    same = C.compute_kl_divergence(torch.from_numpy(lp).to(gpu), torch.from_numpy(lp).to(gpu), method)
+    assert (same == 0).all()
+  with pytest.raises(ValueError, match="must be one of"):
+    C.compute_kl_divergence(torch.zeros(2, device=gpu), torch.zeros(2, device=gpu), "reverse")
+
+
+def _agg_cases():
+  import json
+  import os
+  with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "aggregate_loss_cases.json")) as f:
+    return [(c["mode"], c["loss"], c["mask"], c["kwargs"], c["expected"]) for c in json.load(f)]
+
+
+@pytest.mark.parametrize("mode,loss,mask,kwargs,expected", _agg_cases())
+def test_aggregate_loss_literal_cases(gpu, mode, loss, mask, kwargs, expected):
+  """The cases of tests/rl/common_test.py:457-576 through tnx_aggregate_loss, same tolerance."""
+  from tunix_amd.rl import common as C
+  m = C.aggregate_loss(torch.tensor(loss, device=gpu), torch.tensor(mask, device=gpu), mode, **kwargs)
+  np.testing.assert_allclose(m.compute().item(), expected, rtol=1e-6, atol=1e-6)
+
+
+AGG_MODES = ["token-mean", "sequence-mean-token-mean", "sequence-mean-token-scale", "seq-mean-token-sum",
+             "sequence-mean-token-sum-norm"]
+
+
+@pytest.mark.parametrize("mode", AGG_MODES)
+def test_aggregate_loss_training_scale(gpu, mode):
+  """128 x 1024 tokens with ragged masks and two empty rows against the float64 oracle (fp32 sums
+  of 1e5 terms: 1e-5 relative), and what holds at any size: the result is linear in the loss,
+  the same on every launch, and zero under an all-zero mask."""
+  from tunix_amd.rl import common as C
+  rng = np.random.default_rng(11)
+  B, T = 128, 1024
+  loss = rng.normal(0.3, 1.0, size=(B, T)).astype(np.float32)
+  lens = rng.integers(1, T + 1, size=B)
+  lens[[5, 77]] = 0
+  mask = (np.arange(T)[None, :] < lens[:, None])
+  kwargs = {"norm": 37.5} if "norm" in mode or "scale" in mode else {}
+  gl, gm = torch.from_numpy(loss).to(gpu), torch.from_numpy(mask).to(gpu)
+  m = C.aggregate_loss(gl, gm, mode, **kwargs)
+  num, den, min_denom = R.aggregate_loss(loss, mask, mode, **kwargs)
+  assert m.min_denom == min_denom
+  np.testing.assert_allclose(m.unreduced_sum.item(), num, rtol=1e-5, atol=1e-4)
+  np.testing.assert_allclose(m.denominator.item(), den, rtol=1e-7)
+  np.testing.assert_allclose(m.compute().item(), R.weighted_metric_compute(num, den, min_denom), rtol=1e-5,
+                             atol=1e-6)
+  again = C.aggregate_loss(gl, gm, mode, **kwargs)
+  assert again.unreduced_sum.item() == m.unreduced_sum.item()
+  scaled = C.aggregate_loss(gl * 4.0, gm, mode, **kwargs)          # a power of two: exact
+  assert scaled.unreduced_sum.item() == 4.0 * m.unreduced_sum.item()
+  zero = C.aggregate_loss(gl, torch.zeros_like(gm), mode, **kwargs)
+  assert zero.compute().item() == 0.0
+  # an integer or bf16 mask and a bf16 loss are converted, as the reference's astype does
+  m16 = C.aggregate_loss(gl.to(torch.bfloat16), gm.to(torch.int32), mode, **kwargs)
+  num16, _, _ = R.aggregate_loss(gl.to(torch.bfloat16).float().cpu().numpy(), mask, mode, **kwargs)
+  np.testing.assert_allclose(m16.unreduced_sum.item(), num16, rtol=1e-5, atol=1e-4)
+
+
+def test_aggregate_loss_argument_errors(gpu):
+  from tunix_amd.rl import common as C
+  x, k = torch.ones(2, 3, device=gpu), torch.ones(2, 3, device=gpu)
+  with pytest.raises(ValueError, match="Unsupported loss aggregation mode"):
+    C.aggregate_loss(x, k, "mean")
+  for bad in (0, -2.0, "x"):
+    with pytest.raises(ValueError, match="Invalid 'norm' value"):
+      C.aggregate_loss(x, k, "sequence-mean-token-sum-norm", norm=bad)
+  with pytest.raises(NotImplementedError):
+    C.aggregate_loss(x, k, "token-mean", segment_ids=torch.ones(2, 3, dtype=torch.int32, device=gpu), num_segments=2)
+  with pytest.raises(ValueError):
+    C.aggregate_loss(x, k[:, :2], "token-mean")

@@ -161,3 +161,29 @@ def test_entropy_from_logits_closed_forms():
   lg = torch.randn(6, 101, generator=g) * 3
   want = scipy.stats.entropy(torch.softmax(lg.double(), -1).numpy(), axis=-1)
   np.testing.assert_allclose(rl_ref.compute_entropy_from_logits(lg).numpy(), want, rtol=1e-5)
+
+
+def _aggregate_loss_cases():
+  import json
+  import os
+  with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "aggregate_loss_cases.json")) as f:
+    return [(c["mode"], c["loss"], c["mask"], c["kwargs"], c["expected"]) for c in json.load(f)]
+
+
+AGGREGATE_LOSS_CASES = _aggregate_loss_cases()
+
+
+@pytest.mark.parametrize("mode,loss,mask,kwargs,expected", AGGREGATE_LOSS_CASES)
+def test_aggregate_loss_literal_cases(mode, loss, mask, kwargs, expected):
+  """tests/rl/common_test.py:457-576, same tolerance."""
+  num, den, min_denom = R.aggregate_loss(loss, mask, mode, **kwargs)
+  got = R.weighted_metric_compute(num, den, min_denom=min_denom)
+  np.testing.assert_allclose(got, expected, rtol=1e-6, atol=1e-6)
+
+
+def test_aggregate_loss_bad_arguments():
+  with pytest.raises(ValueError, match="Unsupported loss aggregation mode"):
+    R.aggregate_loss([[0.1]], [[1]], "mean")
+  for bad in (0, -1.0, "x"):
+    with pytest.raises(ValueError, match="Invalid 'norm' value"):
+      R.aggregate_loss([[0.1]], [[1]], "sequence-mean-token-scale", norm=bad)

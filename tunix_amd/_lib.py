@@ -116,6 +116,8 @@ SIGNATURES = {
     "tnx_moe_int4_gmm": (_i32, [_p, C.POINTER(MoeGmmDesc)]),
     "tnx_moe_combine": (_i32, [_p, _p, _p, _i64, _i32, _i64, _p, _p]),
     "tnx_grpo_ratio": (_i32, [_p, _p, _p, _p, _i64, _i64, _f32, _f32, _p, _p, _p]),
+    "tnx_kl_divergence": (_i32, [_p, _p, _p, _i64, _i32, _f32, _p]),
+    "tnx_aggregate_loss": (_i32, [_p, _p, _p, _i64, _i64, _i32, _f32, _p, _p]),
     "tnx_fill_u32": (_i32, [_p, _p, _i64, C.c_uint32]),
 }
 

@@ -62,6 +62,88 @@ __global__ void grpo_ratio_kernel(const float* logp, const float* old_logp, cons
   if (clipped) clipped[i] = l2 > l1 ? 1 : 0;
 }
 
+// Per-token KL estimators: logp - ref ("kl"), half the squared difference ("mse_kl"),
+// exp(d) - d - 1 with d = ref - logp ("low_var_kl"); optional symmetric clamp.
+__global__ void kl_divergence_kernel(const float* logp, const float* ref_logp, int64_t N, int method,
+                                     float clamp, float* kl) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= N) return;
+  const float p = logp[i], q = ref_logp[i];
+  float v;
+  if (method == TNX_KL_KL) {
+    v = p - q;
+  } else if (method == TNX_KL_MSE) {
+    const float d = p - q;
+    v = 0.5f * (d * d);
+  } else {
+    const float d = q - p;
+    v = expf(d) - d - 1.0f;
+  }
+  if (clamp >= 0.f) v = fminf(fmaxf(v, -clamp), clamp);
+  kl[i] = v;
+}
+
+// Sum of 256 values, one per thread, in a fixed order: every launch adds the same numbers in
+// the same tree, so the aggregates do not change between runs.
+__device__ __forceinline__ float block_sum256(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();   // red may still be read from an earlier call
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// Row b: (sum of loss * mask, sum of mask) -> row_ws[b][0..1].
+__global__ __launch_bounds__(256) void agg_rows_kernel(const float* loss, const float* mask, int64_t T,
+                                                       float* row_ws) {
+  __shared__ float red[4];
+  const int64_t b = blockIdx.x;
+  float s = 0.f, c = 0.f;
+  for (int64_t t = threadIdx.x; t < T; t += 256) {
+    const float m = mask[b * T + t];
+    s += loss[b * T + t] * m;
+    c += m;
+  }
+  s = block_sum256(s, red);
+  c = block_sum256(c, red);
+  if (threadIdx.x == 0) {
+    row_ws[2 * b] = s;
+    row_ws[2 * b + 1] = c;
+  }
+}
+
+// The rows' sums -> (unreduced sum, denominator) of the aggregation mode.
+__global__ __launch_bounds__(256) void agg_finish_kernel(const float* row_ws, int64_t B, int mode,
+                                                         float norm, float* out) {
+  __shared__ float red[4];
+  float num = 0.f, den = 0.f;
+  for (int64_t b = threadIdx.x; b < B; b += 256) {
+    const float s = row_ws[2 * b], c = row_ws[2 * b + 1];
+    const float nonempty = c > 0.f ? 1.f : 0.f;
+    if (mode == TNX_AGG_TOKEN_MEAN) {
+      num += s;
+      den += c;
+    } else if (mode == TNX_AGG_SEQ_MEAN_TOKEN_MEAN) {
+      num += s / fmaxf(c, 1.0f);
+      den += nonempty;
+    } else if (mode == TNX_AGG_SEQ_MEAN_TOKEN_SCALE) {
+      num += s / fmaxf(norm, 1e-6f);
+      den += nonempty;
+    } else if (mode == TNX_AGG_SEQ_MEAN_TOKEN_SUM) {
+      num += s * nonempty;
+      den += nonempty;
+    } else {
+      num += s;
+    }
+  }
+  num = block_sum256(num, red);
+  den = block_sum256(den, red);
+  if (threadIdx.x == 0) {
+    out[0] = num;
+    out[1] = mode == TNX_AGG_SEQ_MEAN_TOKEN_SUM_NORM ? norm : den;
+  }
+}
+
 // Router: fp32 softmax of the bf16 scores, top-k (descending, lower expert id first among
 // equals), renormalise, cast to bf16.  One wave per token; E <= 1024.
 __global__ __launch_bounds__(64) void moe_route_kernel(const uint16_t* scores, int E, int k,
@@ -291,6 +373,31 @@ extern "C" int tnx_grpo_ratio(void* stream, const float* logp, const float* old_
                      as_stream(stream), logp, old_logp, adv, N, tokens_per_seq, eps_lo, eps_hi,
                      ratio, loss, clipped);
   TNX_CHECK_LAUNCH("grpo_ratio");
+  return TNX_OK;
+}
+
+extern "C" int tnx_kl_divergence(void* stream, const float* logp, const float* ref_logp, int64_t N,
+                                 int method, float clamp, float* kl) {
+  TNX_REQUIRE(logp && ref_logp && kl && N > 0, "kl_divergence: bad arguments");
+  TNX_REQUIRE(method >= TNX_KL_KL && method <= TNX_KL_LOW_VAR, "kl_divergence: bad method %d", method);
+  hipLaunchKernelGGL(kl_divergence_kernel, dim3((unsigned)cdiv(N, 256)), dim3(256), 0, as_stream(stream),
+                     logp, ref_logp, N, method, clamp, kl);
+  TNX_CHECK_LAUNCH("kl_divergence");
+  return TNX_OK;
+}
+
+extern "C" int tnx_aggregate_loss(void* stream, const float* per_token_loss, const float* mask, int64_t B,
+                                  int64_t T, int mode, float norm, float* row_ws, float* out) {
+  TNX_REQUIRE(per_token_loss && mask && row_ws && out, "aggregate_loss: null pointer");
+  TNX_REQUIRE(B > 0 && T > 0 && B <= 0x7fffffffLL, "aggregate_loss: bad shape");
+  TNX_REQUIRE(mode >= TNX_AGG_TOKEN_MEAN && mode <= TNX_AGG_SEQ_MEAN_TOKEN_SUM_NORM, "aggregate_loss: bad mode %d", mode);
+  if (mode == TNX_AGG_SEQ_MEAN_TOKEN_SCALE || mode == TNX_AGG_SEQ_MEAN_TOKEN_SUM_NORM)
+    TNX_REQUIRE(norm > 0.f, "aggregate_loss: norm must be positive");
+  hipLaunchKernelGGL(agg_rows_kernel, dim3((unsigned)B), dim3(256), 0, as_stream(stream), per_token_loss, mask,
+                     T, row_ws);
+  TNX_CHECK_LAUNCH("aggregate_loss rows");
+  hipLaunchKernelGGL(agg_finish_kernel, dim3(1), dim3(256), 0, as_stream(stream), row_ws, B, mode, norm, out);
+  TNX_CHECK_LAUNCH("aggregate_loss finish");
   return TNX_OK;
 }
 

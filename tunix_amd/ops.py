@@ -210,6 +210,22 @@ def grpo_ratio(logp, old_logp, adv, tokens_per_seq, eps_lo, eps_hi, ratio=None, 
                                  _ptr(loss), _ptr(clipped)), "tnx_grpo_ratio")
 
 
+KL_METHODS = {"kl": 0, "mse_kl": 1, "low_var_kl": 2}
+AGG_MODES = {"token-mean": 0, "sequence-mean-token-mean": 1, "sequence-mean-token-scale": 2,
+             "seq-mean-token-sum": 3, "sequence-mean-token-sum-norm": 4}
+
+
+def kl_divergence(logp, ref_logp, method: int, clamp: float, out):
+  L.check(L.lib().tnx_kl_divergence(_stream(), _ptr(logp), _ptr(ref_logp), logp.numel(), method,
+                                    float(clamp), _ptr(out)), "tnx_kl_divergence")
+
+
+def aggregate_loss(per_token_loss, mask, mode: int, norm: float, row_ws, out):
+  B, T = per_token_loss.shape
+  L.check(L.lib().tnx_aggregate_loss(_stream(), _ptr(per_token_loss), _ptr(mask), B, T, mode,
+                                     float(norm), _ptr(row_ws), _ptr(out)), "tnx_aggregate_loss")
+
+
 def fill_u32(t: torch.Tensor, value: int = 0):
   assert t.element_size() == 4
   L.check(L.lib().tnx_fill_u32(_stream(), _ptr(t), t.numel(), value), "tnx_fill_u32")

@@ -1,6 +1,7 @@
-"""Per-token log-probabilities and the GRPO clipped ratio on the quantized model
-(mirrors tunix/rl/common.py:187-203 selective_log_softmax, :326-482 compute_per_token_logps,
-:485-571 compute_chunked_logps and the ratio of tunix/rl/algo_core.py:440-489).
+"""Per-token log-probabilities, the GRPO clipped ratio, KL estimators and loss aggregation on
+the quantized model (mirrors tunix/rl/common.py:187-203 selective_log_softmax, :326-482
+compute_per_token_logps, :485-571 compute_chunked_logps, :135-184 compute_kl_divergence,
+:763-854 aggregate_loss and the ratio of tunix/rl/algo_core.py:440-489).
 
 compute_per_token_logps runs one full forward over prompt + completion (no cache reuse, the
 reference does the same), then feeds the hidden states of the positions that predict the
@@ -8,6 +9,9 @@ completion tokens to the fused lm_head -> log-softmax -> gather kernel: full-voc
 are never written to HBM, so `chunk_size` only bounds the number of rows per launch.
 """
 from __future__ import annotations
+
+import dataclasses
+from typing import Any
 
 import numpy as np
 import torch
@@ -115,3 +119,90 @@ def grpo_clipped_ratio(logp: torch.Tensor, old_logp: torch.Tensor | None, advant
   clipped = torch.empty(B, T, dtype=torch.int32, device=lp.device)
   ops.grpo_ratio(lp, old, adv, T, epsilon, eps_hi, ratio=ratio, loss=loss, clipped=clipped)
   return ratio, loss, clipped.bool()
+
+
+def compute_kl_divergence(per_token_logps: torch.Tensor, ref_per_token_logps: torch.Tensor,
+                          method: str = "low_var_kl", clamp_value: float | None = None) -> torch.Tensor:
+  """Per-token KL between the trained and the reference policy (tunix/rl/common.py:135-184):
+  "kl" logp - ref, "mse_kl" 0.5 (logp - ref)^2, "low_var_kl" exp(d) - d - 1 with d = ref - logp;
+  clamp_value clips the result symmetrically."""
+  if method not in ops.KL_METHODS:
+    raise ValueError("`method` must be one of 'kl', 'mse_kl', 'low_var_kl'. Received:"
+                     f" {method}")
+  if clamp_value is not None and clamp_value < 0:
+    raise ValueError("clamp_value must not be negative")  # clip(x, c, -c) with c < 0 has no meaning
+  lp = per_token_logps.to(torch.float32).contiguous()
+  ref = ref_per_token_logps.to(torch.float32).contiguous()
+  if lp.shape != ref.shape:
+    raise ValueError(f"shapes differ: {tuple(lp.shape)} vs {tuple(ref.shape)}")
+  out = torch.empty_like(lp)
+  if lp.numel():
+    ops.kl_divergence(lp, ref, ops.KL_METHODS[method], -1.0 if clamp_value is None else clamp_value, out)
+  return out
+
+
+@dataclasses.dataclass
+class WeightedMetric:
+  """A sum and the weight to divide it by (tunix/sft/utils.py:185-219); both stay on the device."""
+  unreduced_sum: torch.Tensor
+  denominator: torch.Tensor
+  eps: float | None = None
+  min_denom: float | None = None
+
+  def compute_scale(self) -> torch.Tensor:
+    denom = self.denominator
+    if self.eps is not None:
+      denom = denom + self.eps
+    if self.min_denom is not None:
+      denom = torch.clamp(denom, min=self.min_denom)
+    safe = torch.where(denom == 0, torch.ones_like(denom), denom)
+    return torch.where(denom == 0, torch.zeros_like(denom), 1.0 / safe)
+
+  def compute(self) -> torch.Tensor:
+    return self.unreduced_sum * self.compute_scale()
+
+
+def _check_get_norm(arguments: dict[str, Any], default: float) -> float:
+  """The `norm` keyword or its default (tunix/rl/common.py:1151-1177)."""
+  if "norm" in arguments:
+    try:
+      norm = float(arguments["norm"])
+    except (ValueError, TypeError):
+      raise ValueError(f"Invalid 'norm' value: {arguments['norm']}. Must be a positive number.")
+    if norm <= 0:
+      raise ValueError(f"Invalid 'norm' value: {norm}. Must be a positive number.")
+    return norm
+  return float(default)
+
+
+def aggregate_loss(per_token_loss: torch.Tensor, completion_mask: torch.Tensor, loss_agg_mode: str,
+                   segment_ids=None, num_segments=None, **kwargs: Any) -> WeightedMetric:
+  """Aggregates a [B, T] per-token loss under its completion mask (tunix/rl/common.py:763-854).
+  Packing segments (`segment_ids`) belong to the trainer's packed batches and are not part of
+  this build."""
+  if segment_ids is not None:
+    raise NotImplementedError("aggregate_loss over packing segments is outside this build")
+  if loss_agg_mode not in ops.AGG_MODES:
+    raise ValueError(
+        f"Unsupported loss aggregation mode: {loss_agg_mode}. Supported modes:"
+        " 'token-mean', 'sequence-mean-token-mean',"
+        " 'sequence-mean-token-scale', 'seq-mean-token-sum',"
+        " 'sequence-mean-token-sum-norm'.")
+  if per_token_loss.dim() != 2 or per_token_loss.shape != completion_mask.shape:
+    raise ValueError("per_token_loss and completion_mask must both be [batch_size, sequence_len]")
+  B, T = per_token_loss.shape
+  norm = 1.0
+  if loss_agg_mode == "sequence-mean-token-scale":
+    norm = _check_get_norm(kwargs, T)
+  elif loss_agg_mode == "sequence-mean-token-sum-norm":
+    norm = _check_get_norm(kwargs, B)
+  min_denom = 1e-6 if loss_agg_mode in ("seq-mean-token-sum", "sequence-mean-token-sum-norm") else 1.0
+  loss = per_token_loss.to(torch.float32).contiguous()
+  mask = completion_mask.to(torch.float32).contiguous()
+  out = torch.zeros(2, dtype=torch.float32, device=loss.device)
+  if B and T:
+    row_ws = torch.empty(B, 2, dtype=torch.float32, device=loss.device)
+    ops.aggregate_loss(loss, mask, ops.AGG_MODES[loss_agg_mode], norm, row_ws, out)
+  elif loss_agg_mode == "sequence-mean-token-sum-norm":
+    out[1] = norm
+  return WeightedMetric(out[0], out[1], min_denom=min_denom)
