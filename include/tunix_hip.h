@@ -414,6 +414,16 @@ enum {
 int tnx_aggregate_loss(void* stream, const float* per_token_loss, const float* mask, int64_t B, int64_t T,
                        int mode, float norm, float* row_ws, float* out);
 
+/* Agreement between the log-probabilities the rollout recorded and the ones the trainer
+ * recomputes for the same tokens (tunix/rl/grpo/grpo_learner.py:405-440), over the positions
+ * where mask != 0.  rollout_logp, trainer_logp, mask: fp32 [B, T].  out5 = { mean |dlogp|,
+ * max |dlogp|, mean |dp|, max |dp|, Pearson correlation of the probabilities } with
+ * p = exp(logp), means over max(mask count, 1), correlation = cov / sqrt(max(var_r * var_t, 1e-12)).
+ * ws: tnx_logp_drift_ws_bytes(B) bytes, 8-byte aligned.  The moments are accumulated in double. */
+size_t tnx_logp_drift_ws_bytes(int64_t B);
+int tnx_logp_drift(void* stream, const float* rollout_logp, const float* trainer_logp, const float* mask,
+                   int64_t B, int64_t T, void* ws, float* out5);
+
 /* Fill n 32-bit words with `value` (graph-capturable replacement for hipMemsetAsync). */
 int tnx_fill_u32(void* stream, uint32_t* p, int64_t n, uint32_t value);
 

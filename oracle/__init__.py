@@ -15,6 +15,10 @@ tree).  Pinning status of each part:
                  tests/rl/algo_core_test.py:51-143 (ratio == 1).
                  aggregate_loss (five modes, no packing segments) and WeightedMetric.compute:
                  pinned by the thirteen literal cases of tests/rl/common_test.py:457-576.
+                 sampler_trainer_agreement (grpo_learner.py:405-440; the reference holds no
+                 vector for it): pinned by numpy.corrcoef / masked means and maxima over the
+                 masked subset, and by the closed forms (equal inputs, a constant log offset,
+                 an anti-correlated pair, an empty mask).
   model_ref      RMSNorm / RoPE / GQA attention / SwiGLU / full decoder: pinned against
                  transformers' Qwen3 / Llama / Gemma3 / Qwen3Moe random-init models in fp32
                  (tol 1e-3, the equivalence tests/model_alignment/qwen_align_test.py:113-200

@@ -1,8 +1,8 @@
 """Per-token log-probabilities, KL estimators, loss aggregation and the GRPO clipped ratio
 (oracle; tests only).
 
-Follows tunix/rl/common.py:135-203, :234-291, :326-571, :763-854 and
-tunix/rl/algo_core.py:440-489.
+Follows tunix/rl/common.py:135-203, :234-291, :326-571, :763-854,
+tunix/rl/algo_core.py:440-489 and tunix/rl/grpo/grpo_learner.py:405-440.
 """
 from __future__ import annotations
 
@@ -146,3 +146,31 @@ def weighted_metric_compute(unreduced_sum, denominator, min_denom=None, eps=None
   if min_denom is not None:
     denom = max(denom, min_denom)
   return 0.0 if denom == 0 else float(unreduced_sum) / denom
+
+
+def sampler_trainer_agreement(rollout_logps, trainer_logps, completion_mask):
+  """tunix/rl/grpo/grpo_learner.py:405-440, fp32 as there: how far the log-probabilities recorded
+  by the rollout are from the ones the trainer recomputes, over the completion tokens."""
+  a = np.asarray(rollout_logps, dtype=np.float32)
+  b = np.asarray(trainer_logps, dtype=np.float32)
+  mask = np.asarray(completion_mask).astype(bool)
+  mask_f = mask.astype(np.float32)
+  mask_sum = np.maximum(mask_f.sum(dtype=np.float32), np.float32(1.0))
+  diff = np.abs(a - b)
+  rp, tp = np.exp(a), np.exp(b)
+  prob_diff = np.abs(rp - tp)
+  rp_flat, tp_flat, mf = rp.reshape(-1), tp.reshape(-1), mask_f.reshape(-1)
+  rp_mean = (rp_flat * mf).sum(dtype=np.float32) / mask_sum
+  tp_mean = (tp_flat * mf).sum(dtype=np.float32) / mask_sum
+  rp_d = (rp_flat - rp_mean) * mf
+  tp_d = (tp_flat - tp_mean) * mf
+  cov = (rp_d * tp_d).sum(dtype=np.float32) / mask_sum
+  rp_var = (rp_d * rp_d).sum(dtype=np.float32) / mask_sum
+  tp_var = (tp_d * tp_d).sum(dtype=np.float32) / mask_sum
+  return {
+      "sampler_trainer/logp_diff_mean": float((diff * mask_f).sum(dtype=np.float32) / mask_sum),
+      "sampler_trainer/logp_diff_max": float(np.where(mask, diff, 0.0).max()),
+      "sampler_trainer/prob_diff_mean": float((prob_diff * mask_f).sum(dtype=np.float32) / mask_sum),
+      "sampler_trainer/prob_diff_max": float(np.where(mask, prob_diff, 0.0).max()),
+      "sampler_trainer/probs_pearson_corr": float(cov / np.sqrt(np.maximum(rp_var * tp_var, np.float32(1e-12)))),
+  }

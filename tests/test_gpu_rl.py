@@ -313,3 +313,61 @@ def test_aggregate_loss_argument_errors(gpu):
     C.aggregate_loss(x, k, "token-mean", segment_ids=torch.ones(2, 3, dtype=torch.int32, device=gpu), num_segments=2)
   with pytest.raises(ValueError):
     C.aggregate_loss(x, k[:, :2], "token-mean")
+
+
+def test_sampler_trainer_agreement_matches_oracle(gpu):
+  """tnx_logp_drift against the oracle (fp32 two-pass moments there, double raw moments here:
+  1e-5 relative, 1e-4 on the correlation), at the training-scale size, on the closed forms, and
+  with an empty mask."""
+  from tunix_amd.rl import common as C
+  rng = np.random.default_rng(9)
+  for shape in ((3, 7), (128, 512)):
+    a = -rng.gamma(2.0, 1.0, size=shape).astype(np.float32)
+    b = (a + rng.normal(0, 0.05, size=shape)).astype(np.float32)
+    lens = rng.integers(0, shape[1] + 1, size=shape[0])
+    mask = np.arange(shape[1])[None, :] < lens[:, None]
+    b[~mask] -= 3.0
+    ga, gb, gm = (torch.from_numpy(v).to(gpu) for v in (a, b, mask))
+    got = C.sampler_trainer_agreement(ga, gb, gm)
+    want = R.sampler_trainer_agreement(a, b, mask)
+    assert list(got) == list(want)
+    for k in want:
+      np.testing.assert_allclose(got[k], want[k], rtol=1e-4 if k.endswith("corr") else 1e-5, atol=1e-7, err_msg=k)
+    same = C.sampler_trainer_agreement(ga, ga, gm)
+    assert same["sampler_trainer/logp_diff_max"] == 0 and same["sampler_trainer/prob_diff_max"] == 0
+    np.testing.assert_allclose(same["sampler_trainer/probs_pearson_corr"], 1.0, rtol=1e-5)
+    empty = C.sampler_trainer_agreement(ga, gb, torch.zeros_like(gm))
+    assert all(v == 0 for v in empty.values())
+  anti = C.sampler_trainer_agreement(torch.tensor([[0.2, 0.8]], device=gpu).log(),
+                                     torch.tensor([[0.8, 0.2]], device=gpu).log(),
+                                     torch.ones(1, 2, device=gpu))
+  np.testing.assert_allclose(anti["sampler_trainer/probs_pearson_corr"], -1.0, rtol=1e-5)
+  with pytest.raises(ValueError):
+    C.sampler_trainer_agreement(torch.zeros(2, 3, device=gpu), torch.zeros(2, 4, device=gpu),
+                                torch.ones(2, 3, device=gpu))
+
+
+def test_rollout_and_logps_paths_agree_by_the_drift_monitor(tiny, gpu):
+  """The monitor on the two paths of this package: the log-probabilities the decode loop records
+  and compute_per_token_logps over the same tokens differ by bf16 rounding only."""
+  from tunix_amd.generate import CacheConfig, Sampler
+  from tunix_amd.generate.utils import IdTokenizer
+  from tunix_amd.rl import common as C
+  cfg, w, model = tiny
+  tok = IdTokenizer(cfg.vocab_size, pad_id=0, eos_id=1)
+  sampler = Sampler(model, tok, CacheConfig(64, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim))
+  T = 12
+  out = sampler(["5 6 7 8", "9 10 11", "40 41 42 43 44 45"], max_generation_steps=T, return_logprobs=True,
+                eos_tokens=[-1], pad_output=True)
+  comp = torch.from_numpy(np.stack(out.tokens).astype(np.int32)).to(gpu)
+  prompt = torch.from_numpy(out.padded_prompt_tokens.astype(np.int32)).to(gpu)
+  rollout_lp = torch.from_numpy(np.stack(out.logprobs).astype(np.float32)).to(gpu)
+  trainer_lp = C.compute_per_token_logps(model, prompt, comp, pad_id=0)
+  m = C.sampler_trainer_agreement(rollout_lp, trainer_lp, torch.ones_like(comp))
+  assert m["sampler_trainer/logp_diff_max"] <= 2e-2, m
+  assert m["sampler_trainer/prob_diff_max"] <= 1e-3, m
+  # (with these N(0, 0.02) weights every probability is close to 1 / V, the variances lie below
+  # the 1e-12 floor of the formula and the correlation figure carries no information)
+  want = R.sampler_trainer_agreement(rollout_lp.cpu().numpy(), trainer_lp.cpu().numpy(), np.ones((3, T)))
+  for k in want:
+    np.testing.assert_allclose(m[k], want[k], rtol=1e-4, atol=1e-6, err_msg=k)

@@ -187,3 +187,32 @@ def test_aggregate_loss_bad_arguments():
   for bad in (0, -1.0, "x"):
     with pytest.raises(ValueError, match="Invalid 'norm' value"):
       R.aggregate_loss([[0.1]], [[1]], "sequence-mean-token-scale", norm=bad)
+
+
+def test_sampler_trainer_agreement_against_library_routines_and_closed_forms():
+  """The reference holds no vector for grpo_learner.py:405-440: the oracle is checked against
+  numpy.corrcoef and plain masked means / maxima over the masked subset, and against cases with
+  a known answer."""
+  rng = np.random.default_rng(3)
+  a = -rng.gamma(2.0, 1.0, size=(6, 40)).astype(np.float32)
+  b = (a + rng.normal(0, 0.2, size=a.shape)).astype(np.float32)
+  mask = rng.random(a.shape) < 0.6
+  b[~mask] += 5.0                                   # masked-out positions must not count
+  m = R.sampler_trainer_agreement(a, b, mask)
+  pa, pb = np.exp(a[mask].astype(np.float64)), np.exp(b[mask].astype(np.float64))
+  np.testing.assert_allclose(m["sampler_trainer/logp_diff_mean"], np.abs(a[mask] - b[mask]).mean(), rtol=1e-5)
+  np.testing.assert_allclose(m["sampler_trainer/logp_diff_max"], np.abs(a[mask] - b[mask]).max(), rtol=1e-6)
+  np.testing.assert_allclose(m["sampler_trainer/prob_diff_mean"], np.abs(pa - pb).mean(), rtol=1e-5)
+  np.testing.assert_allclose(m["sampler_trainer/prob_diff_max"], np.abs(pa - pb).max(), rtol=1e-5)
+  np.testing.assert_allclose(m["sampler_trainer/probs_pearson_corr"], np.corrcoef(pa, pb)[0, 1], rtol=1e-4)
+  same = R.sampler_trainer_agreement(a, a, mask)
+  assert same["sampler_trainer/logp_diff_max"] == 0 and same["sampler_trainer/prob_diff_mean"] == 0
+  np.testing.assert_allclose(same["sampler_trainer/probs_pearson_corr"], 1.0, rtol=1e-5)
+  off = R.sampler_trainer_agreement(a, a + np.float32(np.log(0.5)), mask)      # p_t = p_r / 2
+  np.testing.assert_allclose(off["sampler_trainer/logp_diff_mean"], np.log(2.0), rtol=1e-5)
+  np.testing.assert_allclose(off["sampler_trainer/probs_pearson_corr"], 1.0, rtol=1e-4)
+  anti = R.sampler_trainer_agreement(np.log([[0.2, 0.8]]), np.log([[0.8, 0.2]]), [[1, 1]])
+  np.testing.assert_allclose(anti["sampler_trainer/probs_pearson_corr"], -1.0, rtol=1e-5)
+  np.testing.assert_allclose(anti["sampler_trainer/prob_diff_max"], 0.6, rtol=1e-5)
+  empty = R.sampler_trainer_agreement(a, b, np.zeros_like(mask))
+  assert all(v == 0 for v in empty.values())

@@ -118,6 +118,8 @@ SIGNATURES = {
     "tnx_grpo_ratio": (_i32, [_p, _p, _p, _p, _i64, _i64, _f32, _f32, _p, _p, _p]),
     "tnx_kl_divergence": (_i32, [_p, _p, _p, _i64, _i32, _f32, _p]),
     "tnx_aggregate_loss": (_i32, [_p, _p, _p, _i64, _i64, _i32, _f32, _p, _p]),
+    "tnx_logp_drift_ws_bytes": (C.c_size_t, [_i64]),
+    "tnx_logp_drift": (_i32, [_p, _p, _p, _p, _i64, _i64, _p, _p]),
     "tnx_fill_u32": (_i32, [_p, _p, _i64, C.c_uint32]),
 }
 

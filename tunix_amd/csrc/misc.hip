@@ -144,6 +144,95 @@ __global__ __launch_bounds__(256) void agg_finish_kernel(const float* row_ws, in
   }
 }
 
+// Agreement of two sets of per-token log-probabilities under a mask.  Row pass: eight masked
+// sums in double (count, |dlogp|, |dp|, p_r, p_t, p_r^2, p_t^2, p_r * p_t) and two maxima per
+// row; the finishing work-group adds the rows in order and forms the five figures.
+constexpr int kDriftSums = 8;
+__device__ __forceinline__ double block_sum256d(double v, double* red) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+__device__ __forceinline__ float block_max256(float v, float* red) {
+  v = wave_max(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+__global__ __launch_bounds__(256) void drift_rows_kernel(const float* a, const float* b, const float* mask,
+                                                         int64_t T, double* row_ws) {
+  __shared__ double redd[4];
+  __shared__ float redf[4];
+  const int64_t row = blockIdx.x;
+  double s[kDriftSums] = {0, 0, 0, 0, 0, 0, 0, 0};
+  float mx_d = 0.f, mx_p = 0.f;
+  for (int64_t t = threadIdx.x; t < T; t += 256) {
+    if (mask[row * T + t] == 0.f) continue;
+    const float la = a[row * T + t], lb = b[row * T + t];
+    const float d = fabsf(la - lb);
+    const float pa = expf(la), pb = expf(lb);
+    const float dp = fabsf(pa - pb);
+    s[0] += 1.0;
+    s[1] += d;
+    s[2] += dp;
+    s[3] += pa;
+    s[4] += pb;
+    s[5] += (double)pa * pa;
+    s[6] += (double)pb * pb;
+    s[7] += (double)pa * pb;
+    mx_d = fmaxf(mx_d, d);
+    mx_p = fmaxf(mx_p, dp);
+  }
+#pragma unroll
+  for (int i = 0; i < kDriftSums; ++i) s[i] = block_sum256d(s[i], redd);
+  mx_d = block_max256(mx_d, redf);
+  mx_p = block_max256(mx_p, redf);
+  if (threadIdx.x == 0) {
+    double* o = row_ws + row * (kDriftSums + 2);
+#pragma unroll
+    for (int i = 0; i < kDriftSums; ++i) o[i] = s[i];
+    o[kDriftSums] = mx_d;
+    o[kDriftSums + 1] = mx_p;
+  }
+}
+
+__global__ __launch_bounds__(256) void drift_finish_kernel(const double* row_ws, int64_t B, float* out) {
+  __shared__ double redd[4];
+  __shared__ float redf[4];
+  double s[kDriftSums] = {0, 0, 0, 0, 0, 0, 0, 0};
+  float mx_d = 0.f, mx_p = 0.f;
+  for (int64_t r = threadIdx.x; r < B; r += 256) {
+    const double* o = row_ws + r * (kDriftSums + 2);
+#pragma unroll
+    for (int i = 0; i < kDriftSums; ++i) s[i] += o[i];
+    mx_d = fmaxf(mx_d, (float)o[kDriftSums]);
+    mx_p = fmaxf(mx_p, (float)o[kDriftSums + 1]);
+  }
+#pragma unroll
+  for (int i = 0; i < kDriftSums; ++i) s[i] = block_sum256d(s[i], redd);
+  mx_d = block_max256(mx_d, redf);
+  mx_p = block_max256(mx_p, redf);
+  if (threadIdx.x == 0) {
+    const double n = s[0] > 1.0 ? s[0] : 1.0;   // max(mask sum, 1)
+    const double ma = s[3] / n, mb = s[4] / n;
+    // sums of (p - mean)^2 * mask and of the cross term, from the raw moments (in double)
+    const double va = (s[5] - 2.0 * ma * s[3] + ma * ma * s[0]) / n;
+    const double vb = (s[6] - 2.0 * mb * s[4] + mb * mb * s[0]) / n;
+    const double cov = (s[7] - ma * s[4] - mb * s[3] + ma * mb * s[0]) / n;
+    const double vv = va * vb > 1e-12 ? va * vb : 1e-12;
+    out[0] = (float)(s[1] / n);
+    out[1] = mx_d;
+    out[2] = (float)(s[2] / n);
+    out[3] = mx_p;
+    out[4] = (float)(cov / sqrt(vv));
+  }
+}
+
 // Router: fp32 softmax of the bf16 scores, top-k (descending, lower expert id first among
 // equals), renormalise, cast to bf16.  One wave per token; E <= 1024.
 __global__ __launch_bounds__(64) void moe_route_kernel(const uint16_t* scores, int E, int k,
@@ -398,6 +487,23 @@ extern "C" int tnx_aggregate_loss(void* stream, const float* per_token_loss, con
   TNX_CHECK_LAUNCH("aggregate_loss rows");
   hipLaunchKernelGGL(agg_finish_kernel, dim3(1), dim3(256), 0, as_stream(stream), row_ws, B, mode, norm, out);
   TNX_CHECK_LAUNCH("aggregate_loss finish");
+  return TNX_OK;
+}
+
+extern "C" size_t tnx_logp_drift_ws_bytes(int64_t B) {
+  return B > 0 ? (size_t)B * (kDriftSums + 2) * sizeof(double) : 0;
+}
+
+extern "C" int tnx_logp_drift(void* stream, const float* rollout_logp, const float* trainer_logp,
+                              const float* mask, int64_t B, int64_t T, void* ws, float* out5) {
+  TNX_REQUIRE(rollout_logp && trainer_logp && mask && ws && out5, "logp_drift: null pointer");
+  TNX_REQUIRE(B > 0 && T > 0 && B <= 0x7fffffffLL, "logp_drift: bad shape");
+  TNX_REQUIRE(((uintptr_t)ws & 7) == 0, "logp_drift: the workspace must be 8-byte aligned");
+  hipLaunchKernelGGL(drift_rows_kernel, dim3((unsigned)B), dim3(256), 0, as_stream(stream), rollout_logp,
+                     trainer_logp, mask, T, (double*)ws);
+  TNX_CHECK_LAUNCH("logp_drift rows");
+  hipLaunchKernelGGL(drift_finish_kernel, dim3(1), dim3(256), 0, as_stream(stream), (const double*)ws, B, out5);
+  TNX_CHECK_LAUNCH("logp_drift finish");
   return TNX_OK;
 }
 

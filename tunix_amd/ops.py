@@ -226,6 +226,13 @@ def aggregate_loss(per_token_loss, mask, mode: int, norm: float, row_ws, out):
                                      float(norm), _ptr(row_ws), _ptr(out)), "tnx_aggregate_loss")
 
 
+def logp_drift(rollout_logp, trainer_logp, mask, out5):
+  B, T = rollout_logp.shape
+  ws = torch.empty(int(L.lib().tnx_logp_drift_ws_bytes(B)) // 8, dtype=torch.float64, device=out5.device)
+  L.check(L.lib().tnx_logp_drift(_stream(), _ptr(rollout_logp), _ptr(trainer_logp), _ptr(mask), B, T,
+                                 _ptr(ws), _ptr(out5)), "tnx_logp_drift")
+
+
 def fill_u32(t: torch.Tensor, value: int = 0):
   assert t.element_size() == 4
   L.check(L.lib().tnx_fill_u32(_stream(), _ptr(t), t.numel(), value), "tnx_fill_u32")

@@ -1,7 +1,8 @@
 """Per-token log-probabilities, the GRPO clipped ratio, KL estimators and loss aggregation on
 the quantized model (mirrors tunix/rl/common.py:187-203 selective_log_softmax, :326-482
 compute_per_token_logps, :485-571 compute_chunked_logps, :135-184 compute_kl_divergence,
-:763-854 aggregate_loss and the ratio of tunix/rl/algo_core.py:440-489).
+:763-854 aggregate_loss, the ratio of tunix/rl/algo_core.py:440-489 and the rollout-against-trainer
+agreement figures of tunix/rl/grpo/grpo_learner.py:405-440).
 
 compute_per_token_logps runs one full forward over prompt + completion (no cache reuse, the
 reference does the same), then feeds the hidden states of the positions that predict the
@@ -206,3 +207,25 @@ def aggregate_loss(per_token_loss: torch.Tensor, completion_mask: torch.Tensor, 
   elif loss_agg_mode == "sequence-mean-token-sum-norm":
     out[1] = norm
   return WeightedMetric(out[0], out[1], min_denom=min_denom)
+
+
+DRIFT_METRICS = ("sampler_trainer/logp_diff_mean", "sampler_trainer/logp_diff_max",
+                 "sampler_trainer/prob_diff_mean", "sampler_trainer/prob_diff_max",
+                 "sampler_trainer/probs_pearson_corr")
+
+
+def sampler_trainer_agreement(rollout_per_token_logps: torch.Tensor, trainer_per_token_logps: torch.Tensor,
+                              completion_mask: torch.Tensor) -> dict[str, float]:
+  """How far the log-probabilities the rollout recorded are from the ones recomputed for the same
+  tokens, over the completion positions (tunix/rl/grpo/grpo_learner.py:405-440, same metric
+  names): mean / max |dlogp|, mean / max |dp| and the Pearson correlation of the probabilities.
+  With the rollout's own log-probabilities and compute_per_token_logps of this package it is the
+  running check that the decode path and the many-row path agree."""
+  a = rollout_per_token_logps.to(torch.float32).contiguous()
+  b = trainer_per_token_logps.to(torch.float32).contiguous()
+  if a.dim() != 2 or a.shape != b.shape or a.shape != completion_mask.shape:
+    raise ValueError("log-probabilities and mask must share one [batch_size, sequence_len] shape")
+  out = torch.zeros(5, dtype=torch.float32, device=a.device)
+  if a.numel():
+    ops.logp_drift(a, b, completion_mask.to(torch.bool).to(torch.float32).contiguous(), out)
+  return dict(zip(DRIFT_METRICS, out.tolist()))
