@@ -267,6 +267,67 @@ def summarize_step_trace(path):
     print(f"| {name:34s} | {n:5d} | {busy / 1e3:8.1f} | {busy / n / 1e3:7.2f} | {span / n / 1e3:22.2f} |")
 
 
+def fused_logps_workload(rows, chunk, iters):
+  """The standalone per-token log-probability case at training scale: hidden states
+  [rows, 4096] bf16 N(0,1) x an int4 (group 128) + LoRA r64 lm_head of 128256 columns ->
+  log-softmax -> gather at random targets -> GRPO clipped ratio; logits never reach HBM.
+  Timed with HIP events around `iters` passes after one warm-up pass."""
+  import torch
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  dev = torch.device("cuda:0")
+  D, V, r, group = 4096, 128256, 64, 128
+  g = torch.Generator(device=dev).manual_seed(20254)
+  x = torch.randn(rows, D, generator=g, device=dev).to(torch.bfloat16)
+  w = (torch.randn(D, V, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+  a_t = (torch.randn(r, D, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+  b_t = (torch.randn(V, r, generator=g, device=dev) * 0.01).to(torch.bfloat16)
+  targets = torch.randint(0, V, (rows,), generator=g, device=dev, dtype=torch.int32)
+  codes, scales = ops.quantize_pack(w, group, 0)
+  del w
+  t = torch.zeros(rows, r, dtype=torch.bfloat16, device=dev)
+  nvb = ops.lmhead_nblocks(V)
+  part = torch.empty(chunk * nvb * 4, dtype=torch.float32, device=dev)
+  logp = torch.empty(rows, dtype=torch.float32, device=dev)
+  ref = torch.empty(rows, dtype=torch.float32, device=dev)
+  adv = torch.randn(max(rows // 4096, 1), generator=g, device=dev)
+  ratio, loss = torch.empty(rows, device=dev), torch.empty(rows, device=dev)
+
+  def one_pass():
+    ops.lora_down(x, a_t, t)
+    for r0 in range(0, rows, chunk):
+      d = L.LmHeadDesc()
+      d.M, d.D, d.V = min(chunk, rows - r0), D, V
+      d.x, d.codes, d.scales, d.group, d.qtype = x[r0:].data_ptr(), codes.data_ptr(), scales.data_ptr(), group, 0
+      d.lora_rank, d.t, d.t_ld, d.lora_b, d.lora_scale = r, t[r0:].data_ptr(), r, b_t.data_ptr(), 1.0
+      d.temperature = 1.0
+      d.targets, d.part, d.target_logp = targets[r0:].data_ptr(), part.data_ptr(), logp[r0:].data_ptr()
+      ops.lmhead(d)
+    ops.grpo_ratio(logp, ref, adv, min(4096, rows), 0.2, 0.2, ratio=ratio, loss=loss)
+
+  one_pass()
+  ref.copy_(logp + 0.05 * torch.randn(rows, generator=g, device=dev))
+  torch.cuda.synchronize()
+  e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+  e0.record()
+  for _ in range(iters):
+    one_pass()
+  e1.record()
+  torch.cuda.synchronize()
+  ms = e0.elapsed_time(e1) / iters
+  flops = 2.0 * rows * D * V + 2.0 * rows * r * (D + V)
+  assert bool(torch.isfinite(logp).all()) and bool(torch.isfinite(loss).all())
+  print(json.dumps({
+      "metric": "fused per-token logps rows/sec @1 MI355X (int4 g128 + LoRA r64 head, 4096 x 128256)",
+      "value": round(rows / (ms * 1e-3), 1), "unit": "rows/s", "n_gpus": 1, "steps": iters, "warmup": 1,
+      "ms_per_step": round(ms, 3), "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+      "config": {"workload": "standalone fused lm_head -> log-softmax -> gather -> GRPO ratio", "rows": rows,
+                 "rows_per_launch": chunk},
+      "roofline": {"kernel": "qgemm_wide_kernel (statistics epilogue)", "bound": "mfma",
+                   "achieved": round(flops / (ms * 1e-3) / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                   "frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}}), flush=True)
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -283,9 +344,18 @@ def main():
   ap.add_argument("--kernels-only", action="store_true",
                   help="profiling aid: one layer, no prefill / decode; only the per-kernel loops at "
                        "context prompt + gen / 2 (prints the kernel table, not the metric)")
+  ap.add_argument("--fused-logps", action="store_true",
+                  help="instead of the decode benchmark: the standalone fused per-token log-probability "
+                       "workload (32 x 4096 rows, quantised 128256-column head), its own JSON line")
+  ap.add_argument("--fused-logps-rows", type=int, default=131072)
   ap.add_argument("--summarize-trace", metavar="CSV", default=None,
                   help="no GPU work: tabulate one decode step of a rocprofv3 kernel-trace csv of this script")
   args = ap.parse_args()
+  if args.fused_logps:
+    if args.gpus != 1:
+      sys.exit("bench.py measures one GPU; --gpus must be 1")
+    fused_logps_workload(args.fused_logps_rows, 16384, max(1, args.kernel_iters // 10))
+    return
   if args.summarize_trace:
     summarize_step_trace(args.summarize_trace)
     return

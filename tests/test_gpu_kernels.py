@@ -489,6 +489,69 @@ def test_lmhead_greedy_and_logp(gpu, M, D, V, dense):
   assert (tlp.cpu() - ref_t2).abs().max().item() < 2e-2
 
 
+@pytest.mark.parametrize("M,D,V,group,qtype,r,entropy", [(1030, 256, 8208, 128, Q.INT4, 64, True),
+                                                         (2048, 384, 4096, 64, Q.NF4, 0, False),
+                                                         (640, 256, 16384, 64, Q.NF4, 32, True)])
+def test_lmhead_many_rows_quantized_head(gpu, M, D, V, group, qtype, r, entropy):
+  """The quantised head from 512 rows on (per-token log-probabilities at training scale) runs on
+  the many-rows GEMM kernel with a statistics epilogue.  Tight check: the plain linear of the
+  same kernel materialises the very logits the epilogue sees, and arg-max, logsumexp, target
+  log-probability and entropy must follow from them (ids exact, 2e-5).  Against the oracle's
+  logits: the tolerance of the bf16 path (2e-2).  Cases: a partial last row tile and a last
+  column tile of 16 columns; no adapter; an odd temperature."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  x = rnd((M, D), 60)
+  w = rnd((D, V), 61, 0.05)
+  g = torch.Generator().manual_seed(62)
+  targets = torch.randint(0, V, (M,), generator=g, dtype=torch.int32)
+  gx = bf(x).to(gpu)
+  c, s = ops.quantize_pack(bf(w).to(gpu), group, qtype)
+  codes, scale = Q.quantize(w.numpy(), group, qtype)
+  kw, a, b = {}, None, None
+  d = L.LmHeadDesc()
+  if r:
+    a, b = _lora(D, V, r, 63)
+    a_t, b_t = _pad_lora(a, b, r)
+    t = torch.zeros(M, r, dtype=torch.bfloat16, device=gpu)
+    ops.lora_down(gx, bf(a_t).to(gpu), t)
+    gb = bf(b_t).to(gpu)
+    kw = dict(lora_rank=r, lora_nseg=1, lora_seg_end=[V], lora_seg_toff=[0], t=t, t_ld=r, lora_b=gb, lora_scale=1.0)
+    d.lora_rank, d.t, d.t_ld, d.lora_b, d.lora_scale = r, t.data_ptr(), r, gb.data_ptr(), 1.0
+  y = torch.empty(M, V, dtype=torch.bfloat16, device=gpu)
+  ops.qlinear(ops.make_qlinear_desc(M=M, K=D, N=V, group=group, qtype=qtype, x=gx, codes=c, scales=s, y=y,
+                                    epilogue=L.TNX_EPI_STORE, **kw))
+  temperature = 0.7
+  d.M, d.D, d.V, d.x = M, D, V, gx.data_ptr()
+  d.codes, d.scales, d.group, d.qtype = c.data_ptr(), s.data_ptr(), group, qtype
+  d.temperature = temperature
+  nvb = ops.lmhead_nblocks(V)
+  part = torch.full((M * nvb * 4,), float("nan"), dtype=torch.float32, device=gpu)
+  pent = torch.full((M * nvb,), float("nan"), dtype=torch.float32, device=gpu)
+  best = torch.empty(M, dtype=torch.int32, device=gpu)
+  blp, tlp, lse, ent = (torch.empty(M, dtype=torch.float32, device=gpu) for _ in range(4))
+  gt = targets.to(gpu)
+  d.targets, d.part, d.best_id, d.best_logp = gt.data_ptr(), part.data_ptr(), best.data_ptr(), blp.data_ptr()
+  d.target_logp, d.lse = tlp.data_ptr(), lse.data_ptr()
+  if entropy:
+    d.part_entropy, d.entropy = pent.data_ptr(), ent.data_ptr()
+  ops.lmhead(d)
+  torch.cuda.synchronize()
+  assert not torch.isnan(part).any(), "every (row, block) statistic is written"
+  got = (y.float() / np.float32(temperature)).cpu()
+  assert torch.equal(best.cpu().long(), torch.argmax(got, dim=-1)), "arg-max (first maximal index)"
+  ref_lse = torch.logsumexp(got, dim=-1)
+  np.testing.assert_allclose(lse.cpu().numpy(), ref_lse.numpy(), rtol=0, atol=2e-5)
+  np.testing.assert_allclose(tlp.cpu().numpy(), rl_ref.selective_log_softmax(got, targets).numpy(), rtol=0, atol=2e-5)
+  np.testing.assert_allclose(blp.cpu().numpy(), (got.max(-1).values - ref_lse).numpy(), atol=2e-5)
+  if entropy:
+    np.testing.assert_allclose(ent.cpu().numpy(), rl_ref.compute_entropy_from_logits(got).numpy(), rtol=0, atol=5e-5)
+  logits = Q.rb(Q.qlinear_lora(x, codes, scale, group, qtype, a, b, lora_scale=1.0) if r else
+                Q.qlinear_lora(x, codes, scale, group, qtype, None, None, lora_scale=0.0))
+  ref_t = rl_ref.selective_log_softmax(logits / np.float32(temperature), targets)
+  assert (tlp.cpu() - ref_t).abs().max().item() < 2e-2
+
+
 def test_lmhead_forbidden_and_ties(gpu):
   """Equal maxima resolve to the lowest index; forbidden ids are never chosen."""
   from tunix_amd import _lib as L

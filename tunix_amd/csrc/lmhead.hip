@@ -10,6 +10,10 @@
 #include "gemm_tile.h"
 #include "rng.h"
 
+// defined beside the 128 x 256 GEMM kernel: 0 = launched, 1 = not a shape it takes, < 0 = error
+int tnx_internal_wide_head(hipStream_t st, const tnx_lmhead_desc* d, float temperature, int64_t nvb,
+                           float* part_ent);
+
 namespace {
 
 struct LHArgs {
@@ -335,10 +339,15 @@ extern "C" int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* d) {
   hipStream_t st = as_stream(stream);
   int rc;
   const bool dense = d->w_bf16 != nullptr;
-  if (d->M <= 16) rc = dense ? launch_lmhead<1, true>(st, a) : launch_lmhead<1, false>(st, a);
-  else if (d->M <= 32) rc = dense ? launch_lmhead<2, true>(st, a) : launch_lmhead<2, false>(st, a);
-  else if (d->M <= 64) rc = dense ? launch_lmhead<4, true>(st, a) : launch_lmhead<4, false>(st, a);
-  else rc = dense ? launch_lmhead<8, true>(st, a) : launch_lmhead<8, false>(st, a);
+  // many rows on a quantised head (per-token log-probabilities at training scale): the
+  // 128 x 256 GEMM kernel with a statistics epilogue, when the request is one it covers
+  rc = tnx_internal_wide_head(st, d, a.temperature, a.nvb, a.part_ent);
+  if (rc == 1) {
+    if (d->M <= 16) rc = dense ? launch_lmhead<1, true>(st, a) : launch_lmhead<1, false>(st, a);
+    else if (d->M <= 32) rc = dense ? launch_lmhead<2, true>(st, a) : launch_lmhead<2, false>(st, a);
+    else if (d->M <= 64) rc = dense ? launch_lmhead<4, true>(st, a) : launch_lmhead<4, false>(st, a);
+    else rc = dense ? launch_lmhead<8, true>(st, a) : launch_lmhead<8, false>(st, a);
+  }
   if (rc) return rc;
   hipLaunchKernelGGL(lmhead_finish_kernel, dim3((unsigned)d->M), dim3(64), 0, st, a.part, a.nvb,
                      d->best_id, d->best_logp, d->target_logp, d->lse, a.part_ent, d->entropy, a.part_draw,

@@ -40,7 +40,7 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
 
 template <int SPT>
 __global__ __launch_bounds__(256)
-void qgemm_wide_kernel(const QLArgs a) {
+void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   constexpr int RT = 4, CG = 2, PF = 3, AP = 8;   // 32-row tiles, 32-column groups per wave
   constexpr uint32_t ABYTES = kWideRows * A_LD * 2;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -419,6 +419,59 @@ void qgemm_wide_kernel(const QLArgs a) {
         }
   }
   __syncthreads();
+  if (h.part != nullptr) {
+    // lm_head: thread (row, half) reduces the row's 128 staged logits of column block
+    // 2 * ntile + half to (max, first arg-max, sum of exp(l - max), logit of the row's target)
+    const int row = tid & 127, half = tid >> 7;
+    const int64_t pb = (int64_t)ntile * 2 + half;
+    if (row >= rows_here || pb >= h.nvb) return;
+    const int64_t grow = m0 + row, c0 = pb * 128;
+    const int tg = h.targets ? h.targets[grow] : -1;
+    const uint32_t base = stage + (uint32_t)((row * sld + half * 128) * 2);
+    const float ninf = -__builtin_inff();
+    float mx = ninf, tgt = ninf;
+    int idx = (int)c0;
+#pragma unroll 4
+    for (int ch = 0; ch < 16; ++ch) {
+      const u32x4 v = lds_ld128(base + (uint32_t)(ch * 16));
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const int64_t col = c0 + ch * 8 + q;
+        const float raw = (q & 1) ? bfhi(v[q >> 1]) : bflo(v[q >> 1]);
+        const float l = col < a.N ? __fdiv_rn(raw, h.temperature) : ninf;
+        if (l > mx) {   // columns ascend: the first maximal index stays
+          mx = l;
+          idx = (int)col;
+        }
+        if ((int)col == tg) tgt = l;
+      }
+    }
+    float se = 0.f, we = 0.f;
+    if (mx != ninf) {
+#pragma unroll 4
+      for (int ch = 0; ch < 16; ++ch) {
+        const u32x4 v = lds_ld128(base + (uint32_t)(ch * 16));
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          const int64_t col = c0 + ch * 8 + q;
+          const float raw = (q & 1) ? bfhi(v[q >> 1]) : bflo(v[q >> 1]);
+          if (col < a.N) {
+            const float l = __fdiv_rn(raw, h.temperature);
+            const float e = __expf(l - mx);
+            se += e;
+            we += e * l;
+          }
+        }
+      }
+    }
+    float* p = h.part + (grow * h.nvb + pb) * 4;
+    p[0] = mx;
+    p[1] = __int_as_float(idx);
+    p[2] = se;
+    p[3] = tgt;
+    if (h.part_ent) h.part_ent[grow * h.nvb + pb] = we;
+    return;
+  }
   {
     const int64_t ldy = mul ? a.N / 2 : a.N;
     const int64_t col0 = (int64_t)ntile * cols;

@@ -38,6 +38,15 @@ struct QLArgs {
   int next_rank;
   float* next_tpart;
 };
+// Second argument of the 128 x 256 kernel: with `part` set it reduces its tile to lm_head
+// statistics instead of storing it.
+struct WideHead {
+  float* part;               // [M, nvb, 4]: max, first arg-max, sum of exp, target logit
+  float* part_ent;           // optional [M, nvb]: sum of exp(l - max) * l
+  const int32_t* targets;    // optional [M]
+  int64_t nvb;               // 128-column blocks of the vocabulary
+  float temperature;
+};
 
 __device__ __forceinline__ float silu_bf16(float g) {
   // jax.nn.silu = x * sigmoid(x) as two bf16 HLO ops.
@@ -466,13 +475,13 @@ int launch_qgemm128(hipStream_t st, const QLArgs& a) {
 }
 
 template <int SPT>
-int launch_qgemm_wide(hipStream_t st, const QLArgs& a) {
+int launch_qgemm_wide(hipStream_t st, const QLArgs& a, const WideHead& h = WideHead{nullptr, nullptr, nullptr, 0, 1.0f}) {
   static std::once_flag once;
   static int attr_rc = TNX_OK;
   std::call_once(once, [] { attr_rc = raise_lds_limit(&qgemm_wide_kernel<SPT>, kWideSmemBytes); });
   if (attr_rc) return attr_rc;
   const unsigned wgs = (unsigned)(cdiv(a.M, kWideRows) * cdiv(a.N, kWideCols));
-  hipLaunchKernelGGL((qgemm_wide_kernel<SPT>), dim3(wgs), dim3(256), kWideSmemBytes, st, a);
+  hipLaunchKernelGGL((qgemm_wide_kernel<SPT>), dim3(wgs), dim3(256), kWideSmemBytes, st, a, h);
   TNX_CHECK_LAUNCH("qgemm_wide");
   return TNX_OK;
 }
@@ -576,6 +585,30 @@ extern "C" int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* d) {
   if (a.M <= 32) return s2 ? launch_qgemm128<2, 2, 2>(st, a) : launch_qgemm128<2, 4, 2>(st, a);
   if (a.M <= 64) return s2 ? launch_qgemm128<2, 2, 4>(st, a) : launch_qgemm128<2, 4, 4>(st, a);
   return s2 ? launch_qgemm128<2, 2, 8>(st, a) : launch_qgemm128<2, 4, 8>(st, a);
+}
+
+// The quantised lm_head over many rows on the 128 x 256 kernel: per 128-column block statistics
+// in the layout lmhead_kernel writes, so the same finishing kernel merges them.  Returns 1 when
+// the shape is not one the kernel takes (the caller then uses its own kernel), 0 when launched.
+int tnx_internal_wide_head(hipStream_t st, const tnx_lmhead_desc* d, float temperature, int64_t nvb,
+                           float* part_ent) {
+  if (d->w_bf16 || d->logits_out || d->forbidden || d->draw_id) return 1;
+  if (d->group < 32 || d->group % 32 != 0 || (d->group <= KTILE ? KTILE % d->group != 0 : d->group % KTILE != 0) ||
+      d->D % d->group != 0)
+    return 1;
+  if ((uint64_t)d->D * (uint64_t)d->V / 2 >= (1ull << 32)) return 1;
+  QLArgs a;
+  memset(&a, 0, sizeof(a));
+  a.M = d->M; a.K = d->D; a.N = d->V; a.group = d->group; a.qtype = d->qtype;
+  a.x = d->x; a.codes = d->codes; a.scales = d->scales;
+  a.lora_rank = d->lora_rank; a.lora_nseg = 1; a.lora_seg_end[0] = d->V;
+  a.t_ld = d->t_ld; a.t = d->t; a.lora_b = d->lora_b; a.lora_scale = d->lora_scale;
+  a.epilogue = TNX_EPI_STORE; a.y = d->part;   // the shape test looks at a stored tile
+  a.split_k = 1; a.ktiles_per_split = (int)(d->D / KTILE); a.x_div = 1;
+  if (!wide_shape(a)) return 1;
+  a.y = nullptr;
+  const WideHead h{d->part, part_ent, d->targets, nvb, temperature};
+  return scales_per_tile(a.group) == 2 ? launch_qgemm_wide<2>(st, a, h) : launch_qgemm_wide<4>(st, a, h);
 }
 
 extern "C" int tnx_splitk_finish(void* stream, const tnx_qlinear_desc* d) {
