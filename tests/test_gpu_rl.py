@@ -193,7 +193,10 @@ def test_fused_head_logps_training_scale_shapes(gpu):
       lse2 = torch.empty(n, dtype=torch.float32, device=gpu)
       d2.target_logp, d2.lse = tlp2.data_ptr(), lse2.data_ptr()
       ops.lmhead(d2)
-      assert torch.equal(tlp2, tlp[:n]) and torch.equal(lse2, lse[:n])
+      # from 512 rows on the many-rows kernel computes the statistics, the launch that materialises
+      # the logits of a few rows does not: same logits up to the fp32 accumulation order
+      torch.testing.assert_close(tlp2, tlp[:n], rtol=0, atol=2e-5 if rows < 512 else 1e-2)
+      torch.testing.assert_close(lse2, lse[:n], rtol=0, atol=2e-5)
     torch.cuda.synchronize()
     return x, w, a, b, targets, tlp.cpu(), lse.cpu(), (None if lg is None else lg.cpu())
 
@@ -212,7 +215,8 @@ def test_fused_head_logps_training_scale_shapes(gpu):
   ref_lse = torch.logsumexp(lg, -1)
   np.testing.assert_allclose(lse[:8].numpy(), ref_lse.numpy(), atol=2e-5)
   sel = lg[torch.arange(8), targets[:8].long()] - ref_lse
-  np.testing.assert_allclose(tlp[:8].numpy(), sel.numpy(), atol=2e-5)
+  # one bf16 ulp of a logit of magnitude <= 2 (2^-7) where the two kernels round a target logit apart
+  np.testing.assert_allclose(tlp[:8].numpy(), sel.numpy(), atol=1e-2)
   np.testing.assert_allclose(torch.exp(lg - ref_lse[:, None]).sum(-1).numpy(), 1.0, atol=1e-4)
   # (3) GRPO ratio against noisy reference log-probabilities (eps 0.2)
   from tunix_amd.rl import common
