@@ -424,6 +424,18 @@ size_t tnx_logp_drift_ws_bytes(int64_t B);
 int tnx_logp_drift(void* stream, const float* rollout_logp, const float* trainer_logp, const float* mask,
                    int64_t B, int64_t T, void* ws, float* out5);
 
+/* tnx_logp_drift for callers that cannot allocate device memory (code under HIP-graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): no counterpart in the reference.  Same
+ * arguments and results as tnx_logp_drift without the workspace: the per-row moments go to an
+ * array built into the library (tnx_logp_drift_static_max_rows() = 4096 rows, 320 KiB, one copy
+ * per GPU for the life of the process).  B above that limit returns TNX_EINVAL.  The call
+ * allocates and frees nothing; its first call on a device looks the array's address up
+ * (hipGetSymbolAddress), so make that call outside a capture.  Every call on one GPU shares
+ * that GPU's array: calls that overlap on one GPU (different streams, no ordering) race. */
+int64_t tnx_logp_drift_static_max_rows(void);
+int tnx_logp_drift_static(void* stream, const float* rollout_logp, const float* trainer_logp,
+                          const float* mask, int64_t B, int64_t T, float* out5);
+
 /* Fill n 32-bit words with `value` (graph-capturable replacement for hipMemsetAsync). */
 int tnx_fill_u32(void* stream, uint32_t* p, int64_t n, uint32_t value);
 

@@ -120,6 +120,8 @@ SIGNATURES = {
     "tnx_aggregate_loss": (_i32, [_p, _p, _p, _i64, _i64, _i32, _f32, _p, _p]),
     "tnx_logp_drift_ws_bytes": (C.c_size_t, [_i64]),
     "tnx_logp_drift": (_i32, [_p, _p, _p, _p, _i64, _i64, _p, _p]),
+    "tnx_logp_drift_static_max_rows": (_i64, []),
+    "tnx_logp_drift_static": (_i32, [_p, _p, _p, _p, _i64, _i64, _p]),
     "tnx_fill_u32": (_i32, [_p, _p, _i64, C.c_uint32]),
 }
 

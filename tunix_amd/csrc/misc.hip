@@ -3,6 +3,8 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "common.h"
 
 namespace {
@@ -504,6 +506,54 @@ extern "C" int tnx_logp_drift(void* stream, const float* rollout_logp, const flo
   TNX_CHECK_LAUNCH("logp_drift rows");
   hipLaunchKernelGGL(drift_finish_kernel, dim3(1), dim3(256), 0, as_stream(stream), (const double*)ws, B, out5);
   TNX_CHECK_LAUNCH("logp_drift finish");
+  return TNX_OK;
+}
+
+// The row moments of tnx_logp_drift_static live in this array instead of a caller's workspace.
+// Each GPU the library runs on holds its own copy (kDriftStaticMaxRows * 10 doubles = 320 KiB)
+// until the process ends.  Host code never uses the array's name as an address: the device
+// address is looked up once per device and kept in g_drift_scratch_ptr.
+constexpr int64_t kDriftStaticMaxRows = 4096;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) double drift_scratch[kDriftStaticMaxRows * (kDriftSums + 2)];
+static double* g_drift_scratch_ptr[kMaxDevices] = {};
+static std::mutex g_drift_scratch_mu;
+
+extern "C" int64_t tnx_logp_drift_static_max_rows(void) { return kDriftStaticMaxRows; }
+
+extern "C" int tnx_logp_drift_static(void* stream, const float* rollout_logp, const float* trainer_logp,
+                                     const float* mask, int64_t B, int64_t T, float* out5) {
+  TNX_REQUIRE(rollout_logp && trainer_logp && mask && out5, "logp_drift_static: null pointer");
+  TNX_REQUIRE(B > 0 && T > 0, "logp_drift_static: bad shape");
+  TNX_REQUIRE(B <= kDriftStaticMaxRows,
+              "logp_drift_static: %lld rows exceed the built-in scratch of %lld rows; use tnx_logp_drift "
+              "with a workspace", (long long)B, (long long)kDriftStaticMaxRows);
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    tnx_set_error("logp_drift_static: no current device (or its ordinal is above %d)", kMaxDevices - 1);
+    return TNX_EINVAL;
+  }
+  double* ws = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_drift_scratch_mu);
+    if (!g_drift_scratch_ptr[dev]) {   // first call on this device: look its copy of the array up
+      void* p = nullptr;
+      const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(drift_scratch));
+      if (e != hipSuccess || !p) {
+        tnx_set_error("logp_drift_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+        return TNX_ELAUNCH;
+      }
+      g_drift_scratch_ptr[dev] = (double*)p;
+    }
+    ws = g_drift_scratch_ptr[dev];
+  }
+  // every row slot the finishing kernel reads is written by the row kernel of this call: nothing
+  // has to be cleared between calls
+  hipLaunchKernelGGL(drift_rows_kernel, dim3((unsigned)B), dim3(256), 0, as_stream(stream), rollout_logp,
+                     trainer_logp, mask, T, ws);
+  TNX_CHECK_LAUNCH("logp_drift_static rows");
+  hipLaunchKernelGGL(drift_finish_kernel, dim3(1), dim3(256), 0, as_stream(stream), (const double*)ws, B, out5);
+  TNX_CHECK_LAUNCH("logp_drift_static finish");
   return TNX_OK;
 }
 

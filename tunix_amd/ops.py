@@ -233,6 +233,13 @@ def logp_drift(rollout_logp, trainer_logp, mask, out5):
                                  _ptr(ws), _ptr(out5)), "tnx_logp_drift")
 
 
+def logp_drift_static(rollout_logp, trainer_logp, mask, out5):
+  """tnx_logp_drift with the library's built-in scratch: no workspace, nothing allocated."""
+  B, T = rollout_logp.shape
+  L.check(L.lib().tnx_logp_drift_static(_stream(), _ptr(rollout_logp), _ptr(trainer_logp), _ptr(mask), B, T,
+                                        _ptr(out5)), "tnx_logp_drift_static")
+
+
 def fill_u32(t: torch.Tensor, value: int = 0):
   assert t.element_size() == 4
   L.check(L.lib().tnx_fill_u32(_stream(), _ptr(t), t.numel(), value), "tnx_fill_u32")
