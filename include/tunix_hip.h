@@ -236,6 +236,9 @@ int tnx_rope_table(void* stream, const int32_t* positions, int64_t pos_ld, const
  * output rounded to bf16 (llama3/model.py:379-396, qwen3/model.py:674-686,
  * gemma3/model.py:618-660).
  *   q: bf16 [B*T, Hq*dh]; out: bf16 [B*T, Hq*dh]; caches bf16 [B,Hkv,S,dh]
+ *   Every slot of both caches must hold finite values, also the slots no token was written to
+ *   yet (allocate the caches zero-filled): a masked key gets probability exactly 0, but its value
+ *   row still enters the P.V product, and 0 * NaN or 0 * Inf would poison the output.
  *   ws: fp32 workspace of tnx_attn_ws_bytes() bytes (only touched when the key range is split)
  * ------------------------------------------------------------------------------------- */
 typedef struct tnx_attn_desc {
@@ -356,7 +359,8 @@ int tnx_sample_commit(void* stream, const int32_t* ids, const float* logp, int64
  * int4/NF4 grouped GEMM over routed tokens (operator shape of megablox.gmm, :975-995).
  * ------------------------------------------------------------------------------------- */
 /* scores: bf16 [M,E] router outputs.  topk_w: bf16 [M,k]; topk_id: int32 [M,k] (descending
- * probability, lower expert id first among equals). */
+ * probability, lower expert id first among equals).  A row with a NaN score still gets k distinct
+ * ids inside [0,E) (so that the sort and the grouped GEMM stay in bounds) and NaN weights. */
 int tnx_moe_route_topk(void* stream, const uint16_t* scores, int64_t M, int E, int k,
                        uint16_t* topk_w, int32_t* topk_id);
 /* Builds the expert-sorted route list: counts[E], offsets[E+1], sorted_route[M*k] (route =

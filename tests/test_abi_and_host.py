@@ -75,11 +75,26 @@ def test_version_and_argument_errors_without_gpu():
   assert lib.tnx_lmhead_nblocks(128256) > 0
 
 
-def test_struct_layouts_are_stable():
-  # the descriptor structs cross the C ABI by pointer: their sizes are part of the contract
-  assert ctypes.sizeof(L.QLinearDesc) == 200
-  for cls in (L.RopeDesc, L.AttnDesc, L.LmHeadDesc, L.MoeGmmDesc):
-    assert ctypes.sizeof(cls) % 8 == 0
+def test_struct_layouts_match_the_header(tmp_path):
+  # the descriptor structs cross the C ABI by pointer: the ctypes mirrors must have the sizes and
+  # the field offsets a C compiler gives the header's structs
+  pairs = {"tnx_qlinear_desc": L.QLinearDesc, "tnx_rope_desc": L.RopeDesc,
+           "tnx_attn_desc": L.AttnDesc, "tnx_lmhead_desc": L.LmHeadDesc, "tnx_moe_gmm_desc": L.MoeGmmDesc}
+  lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "tunix_hip.h"', 'int main(void) {']
+  for cname, cls in pairs.items():
+    lines.append(f'  printf("{cname} %zu\\n", sizeof({cname}));')
+    for fname, _ in cls._fields_:
+      lines.append(f'  printf("{cname}.{fname} %zu\\n", offsetof({cname}, {fname}));')
+  lines += ['  return 0;', '}']
+  src = tmp_path / "layout.c"
+  src.write_text("\n".join(lines))
+  exe = tmp_path / "layout"
+  subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+  got = dict(ln.split() for ln in subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.splitlines())
+  for cname, cls in pairs.items():
+    assert int(got[cname]) == ctypes.sizeof(cls), cname
+    for fname, _ in cls._fields_:
+      assert int(got[f"{cname}.{fname}"]) == getattr(cls, fname).offset, f"{cname}.{fname}"
 
 
 def test_host_utils_match_oracle_and_reference_vectors():
@@ -139,3 +154,35 @@ def test_missing_library_fails_loudly(monkeypatch):
   monkeypatch.setattr(L, "LIB_PATH", "/nonexistent/libtunix_hip.so")
   with pytest.raises(ImportError, match="no CPU fallback"):
     L.lib()
+
+
+def test_sampling_plan_uses_one_predicate_for_path_and_workspace():
+  """top_k None / <= 0 / >= V all mean "no top-k" -- for the path AND for the workspace size, as
+  the library itself reads k: a top_k equal to the vocabulary with top_p < 1 must get the
+  full-row sort's workspace, not the (much smaller) segmented top-k one."""
+  from tunix_amd.generate.sampler import sampling_plan
+  V = 1000
+  assert sampling_plan(None, 1.0, V) == (0, "head_draw")
+  assert sampling_plan(0, 1.0, V) == (0, "head_draw")
+  assert sampling_plan(V, 1.0, V) == (0, "head_draw")
+  assert sampling_plan(V + 5, 0.9, V) == (0, "fullsort")
+  assert sampling_plan(V, 0.9, V) == (0, "fullsort")
+  assert sampling_plan(None, 0.9, V) == (0, "fullsort")
+  assert sampling_plan(50, 0.9, V) == (50, "topk")
+  assert sampling_plan(V - 1, 1.0, V) == (V - 1, "topk")
+  lib = L.lib()
+  # the library treats k >= V like k = 0 when it sizes the segmented workspace: that size is far
+  # below what the full sort needs, which is why the host must not pair it with top_p < 1
+  B, Vbig = 128, 128256
+  small = lib.tnx_sample_topk_ws_bytes(B, Vbig, Vbig)
+  assert small == lib.tnx_sample_topk_ws_bytes(B, Vbig, 0)
+  assert small < 4 * B * Vbig
+
+
+def test_threefry_seed_mirrors_jax_with_32_bit_integers():
+  from tunix_amd.generate.sampler import _threefry_seed
+  assert _threefry_seed(0) == (0, 0)
+  assert _threefry_seed(7) == (0, 7)
+  assert _threefry_seed(-1) == (0, 0xFFFFFFFF)
+  assert _threefry_seed(-2 ** 31) == (0, 0x80000000)
+  assert _threefry_seed(2 ** 32 + 5) == (0, 5)

@@ -254,7 +254,18 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const uint16_t* scores, i
   }
   sum = wave_sum(sum);
   __syncthreads();
-  for (int e = lane; e < E; e += 64) prob[e] = prob[e] / sum;
+  // A NaN score makes every probability of the row NaN.  The selection below must still pick k
+  // distinct experts inside [0, E) (the route sort and the grouped GEMM index memory with them), so
+  // NaNs are ranked as -0.5: below every real probability, above the -1 that marks a taken
+  // expert.  The row's weights are then written as NaN, and the NaN reaches the layer's output.
+  bool bad = false;
+  for (int e = lane; e < E; e += 64) {
+    const float p = prob[e] / sum;
+    const bool ok = p >= 0.f;
+    bad |= !ok;
+    prob[e] = ok ? p : -0.5f;
+  }
+  bad = __any(bad);
   __syncthreads();
   float wsum = 0.f;
   float sel_w = 0.f;   // lane j keeps the j-th selected weight (k <= 64)
@@ -278,7 +289,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const uint16_t* scores, i
     __syncthreads();
   }
   if (lane < k) {
-    topk_w[m * k + lane] = f2bf(sel_w / wsum);
+    topk_w[m * k + lane] = bad ? (uint16_t)0x7fc0 : f2bf(sel_w / wsum);
     topk_id[m * k + lane] = sel_id;
   }
 }

@@ -461,12 +461,30 @@ int raise_lds_limit(Kern kern, size_t bytes) {
   return TNX_OK;
 }
 
+// qgemm128_kernel addresses LDS absolutely (its table sits at LDS address 0), which holds as long
+// as it has no static LDS: checked here, once per instantiation, before the first launch.
+template <class Kern>
+int prepare_qgemm128(Kern kern, size_t bytes) {
+  hipFuncAttributes attr;
+  hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(kern));
+  if (e != hipSuccess) {
+    tnx_set_error("qgemm128: cannot read the kernel's attributes: %s", hipGetErrorString(e));
+    return TNX_ELAUNCH;
+  }
+  if (attr.sharedSizeBytes != 0) {
+    tnx_set_error("qgemm128: built with %zu bytes of static LDS; its absolute LDS addressing needs none",
+                  (size_t)attr.sharedSizeBytes);
+    return TNX_ENOSYS;
+  }
+  return raise_lds_limit(kern, bytes);
+}
+
 template <int NT, int SPT, int MT>
 int launch_qgemm128(hipStream_t st, const QLArgs& a) {
   static std::once_flag once;
   static int attr_rc = TNX_OK;
   constexpr size_t kSmem = big_smem_bytes(NT, MT);
-  std::call_once(once, [] { attr_rc = raise_lds_limit(&qgemm128_kernel<NT, SPT, MT>, kSmem); });
+  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm128_kernel<NT, SPT, MT>, kSmem); });
   if (attr_rc) return attr_rc;
   dim3 grid((unsigned)cdiv(a.M, 16 * MT), (unsigned)cdiv(a.N, 64 * NT), (unsigned)a.split_k);
   hipLaunchKernelGGL((qgemm128_kernel<NT, SPT, MT>), grid, dim3(512), kSmem, st, a);

@@ -32,9 +32,23 @@ class CacheConfig:
 
 
 def _threefry_seed(seed: int) -> tuple[int, int]:
-  """jax.random.PRNGKey(seed) for the threefry2x32 implementation: (high word, low word)."""
-  seed = int(seed) & 0xFFFFFFFFFFFFFFFF
-  return (seed >> 32) & 0xFFFFFFFF, seed & 0xFFFFFFFF
+  """jax.random.PRNGKey(seed) for the threefry2x32 implementation: (high word, low word).  With
+  jax's default 32-bit integers the seed is an int32 (wider Python ints wrap), its logical shift
+  right by 32 gives 0, and the low word is the seed's two's-complement bit pattern: PRNGKey(-1)
+  is (0, 0xFFFFFFFF)."""
+  return 0, int(seed) & 0xFFFFFFFF
+
+
+def sampling_plan(top_k: int | None, top_p: float, vocab_size: int) -> tuple[int, str]:
+  """(k passed to tnx_sample_topk, which path it takes there) for a top_p-mode call
+  (sampler.py:105-148).  top_k None, <= 0 or >= vocab_size all mean "no top-k", exactly as the
+  library reads k (k <= 0 or k >= V): then top_p >= 1 is the categorical draw inside the head
+  ("head_draw") and top_p < 1 sorts whole rows ("fullsort", workspace of
+  tnx_sample_fullsort_ws_bytes); a real top-k uses the segmented selection ("topk", workspace of
+  tnx_sample_topk_ws_bytes).  One predicate decides both the path and the workspace size."""
+  if top_k is None or top_k <= 0 or top_k >= vocab_size:
+    return 0, ("head_draw" if top_p >= 1.0 else "fullsort")
+  return int(top_k), "topk"
 
 
 class _SamplingState:
@@ -221,13 +235,14 @@ class Sampler:
     if forbidden:
       mode["forbidden"] = torch.tensor(forbidden, dtype=torch.int32, device=dev)
     if top_p is not None:
-      no_topk = top_k is None or top_k <= 0
-      k = 0 if no_topk else int(min(top_k, cfg.vocab_size))
+      k, path = sampling_plan(top_k, float(top_p), cfg.vocab_size)
+      ws_bytes = (ops.sample_fullsort_ws_bytes(B, cfg.vocab_size) if path == "fullsort"
+                  else ops.sample_topk_ws_bytes(B, cfg.vocab_size, k))
+      if path == "fullsort" and ws_bytes == 0:
+        raise ValueError("top_p < 1 without top_k sorts whole rows: batch x vocabulary must stay below 2^31")
       mode.update(name="top_p", temperature=float(temperature), top_p=float(top_p), top_k=k,
                   key=key,
-                  ws=torch.empty(max((ops.sample_fullsort_ws_bytes(B, cfg.vocab_size) if (no_topk and top_p < 1.0)
-                                      else ops.sample_topk_ws_bytes(B, cfg.vocab_size, k)) // 4, 1),
-                                 dtype=torch.float32, device=dev),
+                  ws=torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device=dev),
                   ids=torch.empty(B, dtype=torch.int32, device=dev),
                   logp=torch.empty(B, dtype=torch.float32, device=dev))
       if k == 0 and top_p >= 1.0:

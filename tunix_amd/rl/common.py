@@ -65,7 +65,8 @@ def compute_per_token_logps(model: QLoRAModel, prompt_tokens, completion_tokens,
   ids, positions = process_ids(pt, ct, pad_id)
   Ltot = ids.shape[1]
   if T == 0:
-    return torch.zeros(B, 0, dtype=torch.float32, device=dev)
+    empty = torch.zeros(B, 0, dtype=torch.float32, device=dev)
+    return (empty, torch.zeros_like(empty)) if return_entropy else empty
   if Ltot < T + 1:
     raise ValueError("the first completion token needs at least one token before it")
   cfg = model.cfg
