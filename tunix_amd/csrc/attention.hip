@@ -237,29 +237,77 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
       // a group in flight together), summed in split order, rounded to bf16 and staged in LDS,
       // from where every lane picks the elements of its fragments.
       __shared__ float xs[18 * DH];
+      // sine / cosine of this row's position: a per-step table (tnx_rope_table), computed with
+      // the arithmetic of the stand-alone kernel; fetched together with the planes
+      float sn[KS / 2][8], cs[KS / 2][8];
       {
+        f32x4 s0[KS / 2], s1[KS / 2], c0[KS / 2], c1[KS / 2];
+#pragma unroll
+        for (int j = 0; j < KS / 2; ++j) {
+          const int64_t o = b * (DH / 2) + j * 32 + lq * 8;
+          s0[j] = *reinterpret_cast<const f32x4*>(a.rope_sin + o);
+          s1[j] = *reinterpret_cast<const f32x4*>(a.rope_sin + o + 4);
+          c0[j] = *reinterpret_cast<const f32x4*>(a.rope_cos + o);
+          c1[j] = *reinterpret_cast<const f32x4*>(a.rope_cos + o + 4);
+        }
+        // three turns of 64 lanes x 16 bytes at a time (one turn set covers G = 4), every load of
+        // the set issued before the first sum: a set costs one memory round trip, not one per turn
         const int n4 = (a.G + 2) * (DH / 4);
-        for (int i4 = lane; i4 < n4; i4 += 64) {
-          const int hsel = i4 / (DH / 4), d = (i4 % (DH / 4)) * 4;
-          const int head = hsel < a.G ? hkv * a.G + hsel : (hsel == a.G ? a.Hq + hkv : a.Hq + a.Hkv + hkv);
-          const int64_t o = rowoff + (int64_t)head * DH + d;
-          f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-          if (a.qkv_ws) {
-            for (int z0 = 0; z0 < a.qkv_split; z0 += 8) {
-              f32x4 p[8];
+        for (int base = 0; base < n4; base += 192) {
+          if (a.qkv_ws && a.qkv_split <= 8) {
+            f32x4 p[3][8];
+#pragma unroll
+            for (int tsel = 0; tsel < 3; ++tsel) {
+              const int i4 = min(base + tsel * 64 + lane, n4 - 1);
+              const int hsel = i4 / (DH / 4), d = (i4 % (DH / 4)) * 4;
+              const int head = hsel < a.G ? hkv * a.G + hsel : (hsel == a.G ? a.Hq + hkv : a.Hq + a.Hkv + hkv);
+              const int64_t o = rowoff + (int64_t)head * DH + d;
 #pragma unroll
               for (int u = 0; u < 8; ++u)
-                p[u] = *reinterpret_cast<const f32x4*>(a.qkv_ws + (int64_t)min(z0 + u, a.qkv_split - 1) * plane + o);
+                p[tsel][u] = *reinterpret_cast<const f32x4*>(a.qkv_ws + (int64_t)min(u, a.qkv_split - 1) * plane + o);
+            }
 #pragma unroll
-              for (int u = 0; u < 8; ++u)
-                if (z0 + u < a.qkv_split) acc += p[u];
+            for (int tsel = 0; tsel < 3; ++tsel) {
+              const int i4 = base + tsel * 64 + lane;
+              if (i4 < n4) {
+                f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                  if (u < a.qkv_split) acc += p[tsel][u];
+                *reinterpret_cast<f32x4*>(&xs[i4 * 4]) = f32x4{rbf(acc[0]), rbf(acc[1]), rbf(acc[2]), rbf(acc[3])};
+              }
             }
           } else {
-            const u32x2 q = *reinterpret_cast<const u32x2*>(a.qkv + o);
-            acc = f32x4{bflo(q[0]), bfhi(q[0]), bflo(q[1]), bfhi(q[1])};
+            for (int i4 = base + lane; i4 < min(n4, base + 192); i4 += 64) {
+              const int hsel = i4 / (DH / 4), d = (i4 % (DH / 4)) * 4;
+              const int head = hsel < a.G ? hkv * a.G + hsel : (hsel == a.G ? a.Hq + hkv : a.Hq + a.Hkv + hkv);
+              const int64_t o = rowoff + (int64_t)head * DH + d;
+              f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+              if (a.qkv_ws) {
+                for (int z0 = 0; z0 < a.qkv_split; z0 += 8) {
+                  f32x4 p[8];
+#pragma unroll
+                  for (int u = 0; u < 8; ++u)
+                    p[u] = *reinterpret_cast<const f32x4*>(a.qkv_ws + (int64_t)min(z0 + u, a.qkv_split - 1) * plane + o);
+#pragma unroll
+                  for (int u = 0; u < 8; ++u)
+                    if (z0 + u < a.qkv_split) acc += p[u];
+                }
+              } else {
+                const u32x2 q = *reinterpret_cast<const u32x2*>(a.qkv + o);
+                acc = f32x4{bflo(q[0]), bfhi(q[0]), bflo(q[1]), bfhi(q[1])};
+              }
+              *reinterpret_cast<f32x4*>(&xs[i4 * 4]) = f32x4{rbf(acc[0]), rbf(acc[1]), rbf(acc[2]), rbf(acc[3])};
+            }
           }
-          *reinterpret_cast<f32x4*>(&xs[i4 * 4]) = f32x4{rbf(acc[0]), rbf(acc[1]), rbf(acc[2]), rbf(acc[3])};
         }
+#pragma unroll
+        for (int j = 0; j < KS / 2; ++j)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            sn[j][e] = s0[j][e]; sn[j][4 + e] = s1[j][e];
+            cs[j][e] = c0[j][e]; cs[j][4 + e] = c1[j][e];
+          }
         __syncthreads();
       }
       auto fetch8 = [&](int hsel, int d, float (&x)[8]) {
@@ -271,20 +319,6 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
           x[4 + e] = v1[e];
         }
       };
-      // sine / cosine of this row's position: a per-step table (tnx_rope_table), computed with
-      // the arithmetic of the stand-alone kernel
-      float sn[KS / 2][8], cs[KS / 2][8];
-#pragma unroll
-      for (int j = 0; j < KS / 2; ++j) {
-        const int64_t o = b * (DH / 2) + j * 32 + lq * 8;
-        const f32x4 s0 = *reinterpret_cast<const f32x4*>(a.rope_sin + o), s1 = *reinterpret_cast<const f32x4*>(a.rope_sin + o + 4);
-        const f32x4 c0 = *reinterpret_cast<const f32x4*>(a.rope_cos + o), c1 = *reinterpret_cast<const f32x4*>(a.rope_cos + o + 4);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          sn[j][e] = s0[e]; sn[j][4 + e] = s1[e];
-          cs[j][e] = c0[e]; cs[j][4 + e] = c1[e];
-        }
-      }
       // rotate the head whose first column is `col`: pairs (d, d + DH/2) sit in k-steps j, j + KS/2
       auto rotated = [&](int hsel, u32x4 (&dst)[KS]) {
         float x[KS][8];

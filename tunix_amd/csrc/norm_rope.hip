@@ -93,53 +93,98 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
   const int nchunks = (int)(D / 8);
   float h[kNormMaxChunks][8];
   float ss = 0.f;
+  // Chunks are taken two at a time with every load of the pair issued before the first sum (up
+  // to eight planes per chunk at once, further planes in groups of eight): the kernel is a few
+  // dependent memory round trips long, and each group of loads that waits for the previous sum
+  // adds one.  The sum itself stays in split order.
+#pragma unroll
+  for (int c0 = 0; c0 < kNormMaxChunks; c0 += 2) {
+    if (c0 * 256 >= nchunks) break;   // uniform
+    f32x4 p0[2][8], p1[2][8];
+    u32x4 xin[2], rin[2];
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      const int ch = (c0 + cc) * 256 + threadIdx.x;
+      const int64_t o = row * D + (int64_t)min(ch, nchunks - 1) * 8;
+      if (ws) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int64_t zo = (int64_t)min(u, split_k - 1) * plane + o;
+          p0[cc][u] = *reinterpret_cast<const f32x4*>(ws + zo);
+          p1[cc][u] = *reinterpret_cast<const f32x4*>(ws + zo + 4);
+        }
+      } else {
+        xin[cc] = *reinterpret_cast<const u32x4*>(x + o);
+      }
+      if (res_pre) rin[cc] = *reinterpret_cast<const u32x4*>(res_pre + o);
+    }
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      const int c = c0 + cc;
+      const int ch = c * 256 + threadIdx.x;
+      if (ch < nchunks) {
+        const int64_t o = row * D + (int64_t)ch * 8;
+        if (ws) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) h[c][j] = 0.f;
+#pragma unroll
+          for (int u = 0; u < 8; ++u)
+            if (u < split_k) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                h[c][j] += p0[cc][u][j];
+                h[c][4 + j] += p1[cc][u][j];
+              }
+            }
+          for (int z0 = 8; z0 < split_k; z0 += 8) {   // more than eight planes: the rest in groups
+            f32x4 q0[8], q1[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+              const int64_t zo = (int64_t)min(z0 + u, split_k - 1) * plane + o;
+              q0[u] = *reinterpret_cast<const f32x4*>(ws + zo);
+              q1[u] = *reinterpret_cast<const f32x4*>(ws + zo + 4);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+              if (z0 + u < split_k) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                  h[c][j] += q0[u][j];
+                  h[c][4 + j] += q1[u][j];
+                }
+              }
+          }
+#pragma unroll
+          for (int j = 0; j < 8; ++j) h[c][j] = rbf(h[c][j]);
+        } else {
+          unpack8(xin[cc], h[c]);
+        }
+        if (res_pre) {
+          float r[8];
+          unpack8(rin[cc], r);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) h[c][j] = rbf(h[c][j] + r[j]);
+        }
+        if (h_out) {
+          u32x4 q;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) q[j] = pack2bf(h[c][2 * j], h[c][2 * j + 1]);
+          *reinterpret_cast<u32x4*>(h_out + o) = q;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss += sq_term(h[c][j], flavor);
+      }
+    }
+  }
+  // the norm weights and the post-norm residual do not depend on the row statistics: fetch them
+  // before the reduction instead of behind it
+  u32x4 wpre[kNormMaxChunks], rpost[kNormMaxChunks];
 #pragma unroll
   for (int c = 0; c < kNormMaxChunks; ++c) {
     const int ch = c * 256 + threadIdx.x;
     if (ch < nchunks) {
-      const int64_t o = row * D + (int64_t)ch * 8;
-      if (ws) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) h[c][j] = 0.f;
-        // four planes' loads in flight at a time (planes past the last are clamped and not
-        // added); the sum itself stays in split order
-        for (int z0 = 0; z0 < split_k; z0 += 4) {
-          f32x4 p0[4], p1[4];
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const int64_t zo = (int64_t)min(z0 + u, split_k - 1) * plane + o;
-            p0[u] = *reinterpret_cast<const f32x4*>(ws + zo);
-            p1[u] = *reinterpret_cast<const f32x4*>(ws + zo + 4);
-          }
-#pragma unroll
-          for (int u = 0; u < 4; ++u)
-            if (z0 + u < split_k) {
-#pragma unroll
-              for (int j = 0; j < 4; ++j) {
-                h[c][j] += p0[u][j];
-                h[c][4 + j] += p1[u][j];
-              }
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) h[c][j] = rbf(h[c][j]);
-      } else {
-        unpack8(*reinterpret_cast<const u32x4*>(x + o), h[c]);
-      }
-      if (res_pre) {
-        float r[8];
-        unpack8(*reinterpret_cast<const u32x4*>(res_pre + o), r);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) h[c][j] = rbf(h[c][j] + r[j]);
-      }
-      if (h_out) {
-        u32x4 q;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) q[j] = pack2bf(h[c][2 * j], h[c][2 * j + 1]);
-        *reinterpret_cast<u32x4*>(h_out + o) = q;
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) ss += sq_term(h[c][j], flavor);
+      wpre[c] = *reinterpret_cast<const u32x4*>(w + (int64_t)ch * 8);
+      if (res_post && res_post != h_out) rpost[c] = *reinterpret_cast<const u32x4*>(res_post + row * D + (int64_t)ch * 8);
     }
   }
   ss = block_sum(ss, red);
@@ -151,12 +196,13 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
     if (ch < nchunks) {
       const int64_t o = row * D + (int64_t)ch * 8;
       float wv[8], v[8];
-      unpack8(*reinterpret_cast<const u32x4*>(w + (int64_t)ch * 8), wv);
+      unpack8(wpre[c], wv);
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[j] = norm_elem(h[c][j], wv[j], ms, eps, flavor);
       if (res_post) {
         float r[8];
-        unpack8(*reinterpret_cast<const u32x4*>(res_post + o), r);
+        // (a residual that this launch itself rewrote as h_out is read back here, after the write)
+        unpack8(res_post != h_out ? rpost[c] : *reinterpret_cast<const u32x4*>(res_post + o), r);
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = rbf(v[j] + r[j]);
       }
@@ -203,6 +249,17 @@ __global__ void embed_kernel(const uint16_t* table, int64_t V, int64_t D, const 
   int64_t id = ids[b * ids_ld + col + t];
   if (id < 0 || id >= V) id = 0;  // pad sentinels outside the vocabulary read row 0 (masked later)
   const uint16_t* src = table + id * D;
+  if (D % 8 == 0) {   // 16 bytes per thread and turn
+    for (int64_t i = (int64_t)threadIdx.x * 8; i < D; i += (int64_t)blockDim.x * 8) {
+      u32x4 v = *reinterpret_cast<const u32x4*>(src + i);
+      if (scale_bf != 1.0f) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = pack2bf(bflo(v[q]) * scale_bf, bfhi(v[q]) * scale_bf);
+      }
+      *reinterpret_cast<u32x4*>(out + row * D + i) = v;
+    }
+    return;
+  }
   for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
     uint16_t v = src[i];
     if (scale_bf != 1.0f) v = f2bf(bf2f(v) * scale_bf);

@@ -47,8 +47,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wn = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, lh = lane >> 5;
-  // LDS is addressed absolutely (table at 0)
-  if ((uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem != 0u) return;
+  // LDS is addressed absolutely (table at 0): no static LDS in this kernel, checked by the host
   asm volatile("" ::"s"(a.M), "s"(a.K), "s"(a.N), "s"(a.qtype), "s"(a.x), "s"(a.codes), "s"(a.scales),
                "s"(a.lora_rank), "s"(a.lora_nseg), "s"(a.lora_seg_end[0]), "s"(a.lora_seg_end[1]),
                "s"(a.lora_seg_end[2]), "s"(a.lora_seg_toff[0]), "s"(a.lora_seg_toff[1]),

@@ -224,7 +224,7 @@ __global__ __launch_bounds__(512) void lora_down_kernel(const uint16_t* x, int64
   const uint16_t* ar = a_t + (int64_t)(b_on ? n0 + lm : 0) * K + lq * 16;
   f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
   const int ksteps = (int)((K + 63) / 64);
-#pragma unroll 4
+#pragma unroll 8
   for (int ks = wave; ks < ksteps; ks += 8) {
     u32x4 a0 = u32x4{0, 0, 0, 0}, a1 = a0, b0 = a0, b1 = a0;
     const bool k_on = (int64_t)ks * 64 + lq * 16 < K;
@@ -461,18 +461,19 @@ int raise_lds_limit(Kern kern, size_t bytes) {
   return TNX_OK;
 }
 
-// qgemm128_kernel addresses LDS absolutely (its table sits at LDS address 0), which holds as long
-// as it has no static LDS: checked here, once per instantiation, before the first launch.
+// qgemm128_kernel and qgemm_wide_kernel address LDS absolutely (their table sits at LDS address 0),
+// which holds as long as they have no static LDS: checked here, once per instantiation, before the
+// first launch.
 template <class Kern>
 int prepare_qgemm128(Kern kern, size_t bytes) {
   hipFuncAttributes attr;
   hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(kern));
   if (e != hipSuccess) {
-    tnx_set_error("qgemm128: cannot read the kernel's attributes: %s", hipGetErrorString(e));
+    tnx_set_error("quantised GEMM: cannot read the kernel's attributes: %s", hipGetErrorString(e));
     return TNX_ELAUNCH;
   }
   if (attr.sharedSizeBytes != 0) {
-    tnx_set_error("qgemm128: built with %zu bytes of static LDS; its absolute LDS addressing needs none",
+    tnx_set_error("quantised GEMM: built with %zu bytes of static LDS; its absolute LDS addressing needs none",
                   (size_t)attr.sharedSizeBytes);
     return TNX_ENOSYS;
   }
@@ -496,7 +497,7 @@ template <int SPT>
 int launch_qgemm_wide(hipStream_t st, const QLArgs& a, const WideHead& h = WideHead{nullptr, nullptr, nullptr, 0, 1.0f}) {
   static std::once_flag once;
   static int attr_rc = TNX_OK;
-  std::call_once(once, [] { attr_rc = raise_lds_limit(&qgemm_wide_kernel<SPT>, kWideSmemBytes); });
+  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm_wide_kernel<SPT>, kWideSmemBytes); });
   if (attr_rc) return attr_rc;
   const unsigned wgs = (unsigned)(cdiv(a.M, kWideRows) * cdiv(a.N, kWideCols));
   hipLaunchKernelGGL((qgemm_wide_kernel<SPT>), dim3(wgs), dim3(256), kWideSmemBytes, st, a, h);
