@@ -84,9 +84,14 @@ int tnx_qw_sizes(int64_t K, int64_t N, int group, size_t* codes_bytes, size_t* s
 /* w: bf16 or fp32 [K,N] row-major (w_is_f32 selects).  If `interleave2` != 0 the N columns
  * are the concatenation [gate | up] of two N/2-wide matrices and are stored interleaved in
  * blocks of 16 (gate block, up block, ...) so that TNX_EPI_*_MUL sees matching columns in
- * adjacent tiles.  Replaces qwix's quantizer reached from tunix/cli/utils/model.py:51-68. */
+ * adjacent tiles.  int4_bound: the integer the group's absmax maps to, scale = bf16(absmax /
+ * int4_bound) (ignored for NF4); 7 is this format's definition above, and the parameter is there
+ * so that a quantiser with another symmetric bound (7.5, 8: codes still clamp to [-8, 7]) can be
+ * mirrored without an ABI change; <= 0 selects 7.  Replaces qwix's quantizer reached from
+ * tunix/cli/utils/model.py:51-68. */
 int tnx_quantize_pack(void* stream, const void* w, int w_is_f32, int64_t K, int64_t N,
-                      int group, int qtype, int interleave2, uint32_t* codes, uint16_t* scales);
+                      int group, int qtype, int interleave2, float int4_bound, uint32_t* codes,
+                      uint16_t* scales);
 
 /* Inverse of the packing for tests and export: w_out fp32 [K,N] = w^ (bf16 values). */
 int tnx_qw_dequant(void* stream, const uint32_t* codes, const uint16_t* scales, int64_t K,
@@ -402,7 +407,7 @@ enum { TNX_KL_KL = 0, TNX_KL_MSE = 1, TNX_KL_LOW_VAR = 2 };
 int tnx_kl_divergence(void* stream, const float* logp, const float* ref_logp, int64_t N, int method,
                       float clamp, float* kl);
 
-/* Loss aggregation without packing segments (tunix/rl/common.py:763-854): out[0] = unreduced sum,
+/* Loss aggregation without packing segments (tunix/rl/common.py:763-854, the per-row branch): out[0] = unreduced sum,
  * out[1] = denominator of the mode; the caller divides as WeightedMetric.compute does
  * (tunix/sft/utils.py:201-219).  per_token_loss, mask: fp32 [B, T]; row_ws: [B, 2] fp32 workspace
  * (per-row sum of loss * mask, per-row sum of mask).  norm: the `norm` keyword of the two modes
@@ -417,6 +422,20 @@ enum {
 };
 int tnx_aggregate_loss(void* stream, const float* per_token_loss, const float* mask, int64_t B, int64_t T,
                        int mode, float norm, float* row_ws, float* out);
+
+/* The same over packed batches (the segment branch, tunix/rl/common.py:857-940 with the segment
+ * sums of :704-760): a row holds several sequences, segment_ids int32 [B, T] tells them apart
+ * (0 = padding, ids outside [0, num_segments) belong to no segment), and the per-sequence modes
+ * reduce per segment: a segment counts when it has at least one token with mask != 0, segment 0
+ * never counts, the denominator is the number of counted segments.  "token-mean" and
+ * "sequence-mean-token-sum-norm" sum over all tokens as without packing; norm <= 0 in the latter
+ * selects the reference's default there, the number of counted segments.
+ * "sequence-mean-token-scale" needs an explicit norm > 0.  ws: tnx_aggregate_loss_segmented_ws_bytes
+ * bytes.  Every sum runs in a fixed order. */
+size_t tnx_aggregate_loss_segmented_ws_bytes(int64_t B, int num_segments);
+int tnx_aggregate_loss_segmented(void* stream, const float* per_token_loss, const float* mask,
+                                 const int32_t* segment_ids, int64_t B, int64_t T, int num_segments,
+                                 int mode, float norm, float* ws, float* out);
 
 /* Agreement between the log-probabilities the rollout recorded and the ones the trainer
  * recomputes for the same tokens (tunix/rl/grpo/grpo_learner.py:405-440), over the positions

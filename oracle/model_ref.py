@@ -29,6 +29,9 @@ class RefModel:
     self.cfg = cfg
     self.bf16 = bf16
     self.acc = acc
+    # Gemma-3 softmaxes in the dtype of the scores (gemma3/model.py:647); False gives the fp32
+    # softmax of the other two families, for measuring how far the two flows are apart
+    self.gemma_score_softmax = True
     self.w = {}
     self.q = {}     # name -> (dequantised fp32 [K,N])
     self.lora = {}  # name -> (A [K,r], B [r,N])
@@ -117,12 +120,15 @@ class RefModel:
     return torch.cat([o1, o2], dim=-1)
 
   # ---- attention -----------------------------------------------------------------------------
-  def attention(self, q, k_all, v_all, mask, scale, softmax_bf16_flow=False):
+  def attention(self, q, k_all, v_all, mask, scale, score_dtype_softmax=False):
     """q [B,T,Hq,dh], k_all/v_all [B,S,Hkv,dh], mask [B,T,S] bool.
 
-    llama3/model.py:379-396, qwen3/model.py:674-686, gemma3/model.py:618-660: scores are a
-    bf16 einsum, scaled in bf16 (scale=None: q was pre-scaled), masked with K_MASK, softmaxed
-    in fp32, cast to bf16, then a bf16 einsum with V.
+    llama3/model.py:379-396, qwen3/model.py:674-686: scores are a bf16 einsum, scaled in bf16,
+    masked with K_MASK, softmaxed in fp32 (`attn.astype(jnp.float32)`), cast to bf16, then a bf16
+    einsum with V.  gemma3/model.py:618-660 (scale=None: q was pre-scaled) calls jax.nn.softmax on
+    the bf16 scores themselves (:647, score_dtype_softmax=True): x - max, exp and the division are
+    bf16 operations, the sum is accumulated in fp32 and rounded to bf16 (jnp.sum computes 16-bit
+    floats in fp32 and casts the result back).
     """
     B, T, Hq, dh = q.shape
     Hkv = k_all.shape[2]
@@ -133,8 +139,14 @@ class RefModel:
     if scale is not None:
       s = self.r(s * (self.r(torch.tensor(scale, dtype=torch.float32)) if self.bf16 else scale))
     s = torch.where(mask[:, None, None, :, :], s, torch.tensor(K_MASK))
-    p = torch.softmax(s.to(torch.float32), dim=-1)
-    p = self.r(p)
+    if score_dtype_softmax and self.bf16:
+      mx = s.max(dim=-1, keepdim=True).values
+      e = self.r(torch.exp(self.r(s - mx)))
+      den = self.r(e.to(torch.float32).sum(dim=-1, keepdim=True))
+      p = self.r(e / den)
+    else:
+      p = torch.softmax(s.to(torch.float32), dim=-1)
+      p = self.r(p)
     o = torch.einsum("bhgts,bshd->bthgd", p.to(self.acc), v_all.to(self.acc)).float()
     return self.r(o).reshape(B, T, Hq, dh)
 
@@ -169,7 +181,7 @@ class RefModel:
     m = mask
     if fam == "gemma3" and cfg.is_local_layer(i):
       m = self.sliding_mask(mask, cfg.sliding_window, T)
-    o = self.attention(q, kc, vc, m, scale)
+    o = self.attention(q, kc, vc, m, scale, score_dtype_softmax=(fam == "gemma3" and self.gemma_score_softmax))
     attn_out = self.r(self.linear(o.reshape(B, T, Hq * dh), p + "wo"))
     if fam == "gemma3":
       # gemma3/model.py:875-898: post-norms before each residual add

@@ -43,14 +43,16 @@ def levels(qtype: int) -> np.ndarray:
   return NF4_LEVELS if qtype == NF4 else INT4_LEVELS
 
 
-def quantize(w: np.ndarray, group: int, qtype: int) -> tuple[np.ndarray, np.ndarray]:
-  """w fp32 [K, N] -> (codes uint8 [K, N] in 0..15, scales fp32 [K/group, N] holding bf16 values)."""
+def quantize(w: np.ndarray, group: int, qtype: int, int4_bound: float = 7.0) -> tuple[np.ndarray, np.ndarray]:
+  """w fp32 [K, N] -> (codes uint8 [K, N] in 0..15, scales fp32 [K/group, N] holding bf16 values).
+  int4_bound: the integer a group's absmax maps to (7 in the format's definition; a quantiser
+  with another symmetric bound is mirrored by passing it, codes still clamp to [-8, 7])."""
   w = np.asarray(w, dtype=np.float32)
   K, N = w.shape
   assert K % group == 0
   wg = w.reshape(K // group, group, N)
   amax = np.abs(wg).max(axis=1)
-  scale = rb_np(amax if qtype == NF4 else amax / np.float32(7.0))
+  scale = rb_np(amax if qtype == NF4 else amax / np.float32(int4_bound))
   safe = np.where(scale == 0, np.float32(1.0), scale)
   xn = (wg / safe[:, None, :]).astype(np.float32)
   if qtype == NF4:

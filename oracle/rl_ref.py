@@ -1,7 +1,7 @@
 """Per-token log-probabilities, KL estimators, loss aggregation and the GRPO clipped ratio
 (oracle; tests only).
 
-Follows tunix/rl/common.py:135-203, :234-291, :326-571, :763-854,
+Follows tunix/rl/common.py:135-203, :234-291, :326-571, :704-760 (segment sums), :763-940,
 tunix/rl/algo_core.py:440-489 and tunix/rl/grpo/grpo_learner.py:405-440.
 """
 from __future__ import annotations
@@ -135,6 +135,63 @@ def aggregate_loss(per_token_loss, completion_mask, loss_agg_mode, **kwargs):
   if loss_agg_mode == "sequence-mean-token-sum-norm":
     norm = get_norm(loss.shape[0])
     return (loss * mask).sum(), float(norm), 1e-6
+  raise ValueError(f"Unsupported loss aggregation mode: {loss_agg_mode}.")
+
+
+def segmented_sum(values, segment_ids, num_segments):
+  """tunix/rl/common.py:704-735: per-row sums of `values` grouped by segment id -> [B, S]; ids
+  outside [0, S) are dropped, as jax.ops.segment_sum drops them."""
+  values = np.asarray(values, dtype=np.float64)
+  seg = np.asarray(segment_ids).astype(np.int64)
+  out = np.zeros((values.shape[0], num_segments), dtype=np.float64)
+  for b in range(values.shape[0]):
+    for t in range(values.shape[1]):
+      s = seg[b, t]
+      if 0 <= s < num_segments:
+        out[b, s] += values[b, t]
+  return out
+
+
+def aggregate_loss_segmented(per_token_loss, completion_mask, loss_agg_mode, segment_ids, num_segments,
+                             **kwargs):
+  """tunix/rl/common.py:857-940 (_aggregate_loss_segmented), in float64: per-sequence reductions
+  group by packing segment instead of by row, segment 0 (padding) is excluded, a segment counts
+  when it has at least one scored token.  Returns (unreduced_sum, denominator, min_denom)."""
+  if num_segments is None:
+    raise ValueError("num_segments must be provided when segment_ids is not None.")
+  loss = np.asarray(per_token_loss, dtype=np.float64)
+  mask = np.asarray(completion_mask, dtype=np.float64)
+  masked = loss * mask
+  l_seg = segmented_sum(masked, segment_ids, num_segments)
+  c_seg = segmented_sum(mask, segment_ids, num_segments)
+  a_seg = (c_seg > 0).astype(np.float64)
+  a_seg[:, 0] = 0.0
+  n_act = a_seg.sum()
+
+  def get_norm(default):
+    if "norm" in kwargs:
+      try:
+        norm = float(kwargs["norm"])
+      except (ValueError, TypeError):
+        raise ValueError(f"Invalid 'norm' value: {kwargs['norm']}. Must be a positive number.")
+      if norm <= 0:
+        raise ValueError(f"Invalid 'norm' value: {norm}. Must be a positive number.")
+      return norm
+    return default
+
+  if loss_agg_mode == "token-mean":
+    return masked.sum(), mask.sum(), 1.0
+  if loss_agg_mode == "sequence-mean-token-mean":
+    return ((l_seg / np.clip(c_seg, 1.0, None)) * a_seg).sum(), n_act, 1.0
+  if loss_agg_mode == "sequence-mean-token-scale":
+    if "norm" not in kwargs:
+      raise ValueError("sequence-mean-token-scale under sequence packing requires an explicit 'norm'")
+    norm = get_norm(loss.shape[-1])
+    return ((l_seg / max(norm, 1e-6)) * a_seg).sum(), n_act, 1.0
+  if loss_agg_mode == "seq-mean-token-sum":
+    return (l_seg * a_seg).sum(), n_act, 1e-6
+  if loss_agg_mode == "sequence-mean-token-sum-norm":
+    return masked.sum(), float(get_norm(n_act)), 1e-6
   raise ValueError(f"Unsupported loss aggregation mode: {loss_agg_mode}.")
 
 

@@ -2,7 +2,7 @@
 CPU oracle finishes in seconds (same architecture rules as the full-size configurations:
 Llama-3 NF4 g64 + LoRA, Gemma-3 int4 g128 with sliding-window layers, tied embeddings and
 GeGLU, Qwen3-MoE int4 g128 with top-k routing).  Same bar as test_gpu_sampler.py: greedy ids
-equal the teacher-forced oracle arg-max except at listed near-ties (<= 4 bf16 ulps), and
+equal the teacher-forced oracle arg-max except at listed near-ties (<= 2 bf16 ulps), and
 log-probabilities <= 2e-2."""
 import numpy as np
 import pytest
@@ -35,7 +35,7 @@ def _greedy_case(cfg, gpu, B, P, T, seed, lp_tol=2e-2):
   assert all(len(t) == T for t in out.tokens)
   ref = MR.RefModel(cfg, w)
   logits = _oracle_full_logits(ref, tb, 0)
-  report, n = _check_greedy(tb, logits, P, lps, lp_tol=lp_tol)
+  report, n = _check_greedy(tb, logits, P, lps, lp_tol=lp_tol, label=f"{cfg.family} small shape, greedy")
   print(f"{cfg.family}: {n - len(report)}/{n} greedy ids equal the oracle arg-max; near-ties: {report}")
   assert len(report) <= max(1, n // 20)
 
@@ -88,7 +88,7 @@ def test_qwen3_moe_greedy(gpu):
       if not bool(tainted[b, c - 1]):
         strict += 1
         assert err <= 2e-2, (b, c, err)
-        assert tok == best or float(lg[best] - lg[tok]) <= 4 * ulp, (b, c, tok, best)
+        assert tok == best or float(lg[best] - lg[tok]) <= 2 * ulp, (b, c, tok, best)
       else:
         loose += 1
         assert err <= 0.25, (b, c, err)

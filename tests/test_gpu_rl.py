@@ -313,8 +313,11 @@ def test_aggregate_loss_argument_errors(gpu):
   for bad in (0, -2.0, "x"):
     with pytest.raises(ValueError, match="Invalid 'norm' value"):
       C.aggregate_loss(x, k, "sequence-mean-token-sum-norm", norm=bad)
-  with pytest.raises(NotImplementedError):
-    C.aggregate_loss(x, k, "token-mean", segment_ids=torch.ones(2, 3, dtype=torch.int32, device=gpu), num_segments=2)
+  seg = torch.ones(2, 3, dtype=torch.int32, device=gpu)
+  with pytest.raises(ValueError, match="num_segments must be provided"):
+    C.aggregate_loss(x, k, "token-mean", segment_ids=seg)
+  with pytest.raises(ValueError, match="explicit 'norm'"):
+    C.aggregate_loss(x, k, "sequence-mean-token-scale", segment_ids=seg, num_segments=2)
   with pytest.raises(ValueError):
     C.aggregate_loss(x, k[:, :2], "token-mean")
 
@@ -375,3 +378,48 @@ def test_rollout_and_logps_paths_agree_by_the_drift_monitor(tiny, gpu):
   want = R.sampler_trainer_agreement(rollout_lp.cpu().numpy(), trainer_lp.cpu().numpy(), np.ones((3, T)))
   for k in want:
     np.testing.assert_allclose(m[k], want[k], rtol=1e-4, atol=1e-6, err_msg=k)
+
+
+MODES = ["token-mean", "sequence-mean-token-mean", "sequence-mean-token-scale", "seq-mean-token-sum",
+         "sequence-mean-token-sum-norm"]
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_segmented_aggregate_loss_matches_oracle(gpu, mode):
+  """tnx_aggregate_loss_segmented against the oracle on packed rows (random segment layouts with
+  padding, empty segments, unscored segments, ids beyond num_segments), on the reference's own
+  packed gate case (-2.25), and packed == unpacked; two launches give identical bits."""
+  from tunix_amd.rl import common as C
+  rng = np.random.default_rng(21)
+  for (B, T, S) in ((1, 4, 3), (5, 37, 6), (16, 2500, 300), (3, 1024, 9)):
+    loss = rng.normal(0, 1, size=(B, T)).astype(np.float32)
+    seg = np.zeros((B, T), dtype=np.int32)
+    for b in range(B):   # runs of ascending segment ids, then padding; some ids skipped
+      cuts = np.sort(rng.choice(np.arange(1, T), size=min(S + 1, T - 1), replace=False))
+      ids = np.concatenate([np.arange(1, len(cuts) + 1), [0]])
+      ids[rng.random(len(ids)) < 0.15] = 0
+      seg[b] = np.repeat(ids, np.diff(np.concatenate([[0], cuts, [T]])))[:T]
+    mask = (rng.random((B, T)) < 0.7).astype(np.float32)
+    mask[seg == 2] = 0.0                      # a segment with no scored token is not active
+    kw = {"norm": 17.0} if mode == "sequence-mean-token-scale" else {}
+    want = R.aggregate_loss_segmented(loss, mask, mode, seg, S, **kw)
+    gl, gm, gs = (torch.from_numpy(v).to(gpu) for v in (loss, mask, seg))
+    got = C.aggregate_loss(gl, gm, mode, segment_ids=gs, num_segments=S, **kw)
+    again = C.aggregate_loss(gl, gm, mode, segment_ids=gs, num_segments=S, **kw)
+    np.testing.assert_allclose(got.unreduced_sum.item(), want[0], rtol=2e-5, atol=2e-4)
+    np.testing.assert_allclose(got.denominator.item(), want[1], rtol=1e-6)
+    assert got.min_denom == want[2]
+    assert got.unreduced_sum.item() == again.unreduced_sum.item()
+    if mode == "sequence-mean-token-sum-norm":
+      named = C.aggregate_loss(gl, gm, mode, segment_ids=gs, num_segments=S, norm=5.0)
+      assert named.denominator.item() == 5.0
+  # the reference's packed gate (tests/rl/algo_core_test.py:51-143)
+  loss = -torch.tensor([[1.5, 1.5, 1.5, 3.0]], device=gpu)
+  ones = torch.ones(1, 4, device=gpu)
+  seg = torch.tensor([[1, 1, 1, 2]], dtype=torch.int32, device=gpu)
+  if mode == "sequence-mean-token-mean":
+    packed = C.aggregate_loss(loss, ones, mode, segment_ids=seg, num_segments=3).compute().item()
+    np.testing.assert_allclose(packed, -2.25, rtol=1e-6)
+    unpacked = C.aggregate_loss(-torch.tensor([[1.5, 1.5, 1.5], [3.0, 0.0, 0.0]], device=gpu),
+                                torch.tensor([[1.0, 1, 1], [1, 0, 0]], device=gpu), mode).compute().item()
+    np.testing.assert_allclose(packed, unpacked, rtol=1e-6)

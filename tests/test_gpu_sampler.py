@@ -1,9 +1,9 @@
 """End-to-end parity of the HIP Sampler against the CPU oracle (through the C ABI).
 
 Greedy ids: the oracle is teacher-forced with the ids the GPU produced; at every generated
-position the GPU id must be the oracle's arg-max, or lie within four bf16 ulps of it (the logits
+position the GPU id must be the oracle's arg-max, or lie within two bf16 ulps of it (the logits
 are bf16 values, so near-ties flip with the fp32 accumulation order; every such case is listed
-with its top-2 margin).  Log-probs: <= 2e-2 absolute against the oracle's bf16 flow and against
+with its top-2 margin, and the counts go to a summary file next to the run's other outputs).  Log-probs: <= 2e-2 absolute against the oracle's bf16 flow and against
 the fp32 reference mode (the tolerance north_star states for bf16).
 """
 import numpy as np
@@ -39,7 +39,26 @@ def _oracle_full_logits(ref, token_buffer, pad_id):
              torch.from_numpy(attn), 0)
 
 
-def _check_greedy(tb, logits, P, gpu_logprobs=None, lp_tol=2e-2):
+NEAR_TIES = []   # (label, positions, ids that differ from the oracle arg-max, their margins in ulps)
+
+
+def _write_near_tie_summary():
+  """One line per checked rollout: how many greedy ids were not the oracle's arg-max and how far
+  (in bf16 ulps of the top logit) the chosen logit lay below it."""
+  import json
+  import os
+  root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+  out = os.path.join(root, "gpurun_out")
+  try:
+    os.makedirs(out, exist_ok=True)
+    with open(os.path.join(out, "greedy_near_ties.json"), "w") as f:
+      json.dump([{"case": c, "positions": n, "not_argmax": len(u), "margins_ulp": [round(x, 2) for x in u]}
+                 for c, n, u in NEAR_TIES], f, indent=1)
+  except OSError:
+    pass
+
+
+def _check_greedy(tb, logits, P, gpu_logprobs=None, lp_tol=2e-2, label=None, max_ulps=2.0):
   B, L = tb.shape
   report = []
   n = 0
@@ -53,8 +72,11 @@ def _check_greedy(tb, logits, P, gpu_logprobs=None, lp_tol=2e-2):
         margin = float(lg[best] - lg[tok])
         ulp = 2.0 ** (np.floor(np.log2(max(abs(float(lg[best])), 2.0 ** -120))) - 7)  # bf16 spacing
         report.append((b, c, tok, best, margin, margin / ulp))
+  import inspect
+  NEAR_TIES.append((label or inspect.stack()[1].function, n, [r[5] for r in report]))
+  _write_near_tie_summary()
   for r in report:
-    assert r[5] <= 4.0, f"greedy id differs beyond a near-tie: {r}"
+    assert r[5] <= max_ulps, f"greedy id differs beyond a near-tie: {r}"
   if gpu_logprobs is not None:
     lp = torch.log_softmax(logits.float(), dim=-1)
     ref_lp = np.array([[float(lp[b, c - 1, int(tb[b, c])]) for c in range(P, L)] for b in range(B)])
@@ -266,3 +288,46 @@ def test_lora_update_changes_output_and_checks_structure(tiny, gpu):
   bad.pop(next(iter(bad)))
   with pytest.raises(ValueError, match="same structure"):
     sampler.update_lora(bad)
+
+
+def test_full_state_replacement_requantises_in_place(tiny, gpu):
+  """Full-state replacement (tunix/generate/sampler.py:322-325): new base weights are re-quantised
+  and re-packed into the buffers the model already holds; afterwards the model is bit-identical
+  to one built from the new weights, and a partial state that splits a fused projection, or has
+  another shape, raises."""
+  from tunix_amd import dummy_model
+  from tunix_amd.generate import CacheConfig, Sampler
+  from tunix_amd.generate.utils import IdTokenizer
+  from tunix_amd.model import QLoRAModel
+  cfg, w, _ = tiny
+  model = QLoRAModel(cfg, w, gpu)
+  w2 = dummy_model.create_dummy_weights(cfg, seed=777)
+  fresh = QLoRAModel(cfg, w2, gpu)
+  ptr = model.layers[0]["qkv"].codes.data_ptr()
+  tok = IdTokenizer(cfg.vocab_size, pad_id=0, eos_id=1)
+  cc = CacheConfig(32, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim)
+  sampler = Sampler(model, tok, cc)
+  before = sampler(["3 4 5 6"], 8, return_logprobs=True, eos_tokens=[-1])
+  sampler.update_params(w2)                       # base + LoRA leaves
+  assert model.layers[0]["qkv"].codes.data_ptr() == ptr
+  for a, b in zip(model.layers, fresh.layers):
+    for key in ("qkv", "o", "gu", "down"):
+      assert torch.equal(a[key].codes, b[key].codes) and torch.equal(a[key].scales, b[key].scales)
+      assert torch.equal(a[key].a_t, b[key].a_t) and torch.equal(a[key].b_t, b[key].b_t)
+    assert torch.equal(a["attn_norm"], b["attn_norm"])
+  assert torch.equal(model.embed, fresh.embed) and torch.equal(model.head_w, fresh.head_w)
+  after = sampler(["3 4 5 6"], 8, return_logprobs=True, eos_tokens=[-1])
+  want = Sampler(fresh, tok, cc)(["3 4 5 6"], 8, return_logprobs=True, eos_tokens=[-1])
+  np.testing.assert_array_equal(after.tokens[0], want.tokens[0])
+  np.testing.assert_array_equal(np.asarray(after.logprobs), np.asarray(want.logprobs))
+  assert np.abs(np.asarray(before.logprobs) - np.asarray(after.logprobs)).max() > 0
+  # base weights only: the adapters stay
+  base_only = {k: v for k, v in w.items() if ".lora_" not in k}
+  sampler.update_params(base_only)
+  assert torch.equal(model.layers[0]["qkv"].a_t, fresh.layers[0]["qkv"].a_t)
+  with pytest.raises(ValueError, match="same structure"):
+    sampler.update_params({"l0.wq": w["l0.wq"]})                       # wk / wv of the fused projection missing
+  with pytest.raises(ValueError, match="same shape"):
+    sampler.update_params({"embed": w["embed"][:, :8]})
+  with pytest.raises(ValueError, match="same structure"):
+    sampler.update_params({"no_such_leaf": w["embed"]})

@@ -154,3 +154,26 @@ def test_pack_qw_layout():
     np.testing.assert_array_equal(c2, codes)
     want_bits = torch.from_numpy(s).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
     np.testing.assert_array_equal(s2, want_bits)
+
+
+def test_int4_bound_parameter_closed_forms():
+  """scale = bf16(absmax / bound): with bound 7 the group's extreme element maps to code 7 + 8 (or
+  -7 + 8); with bound 8 a positive extreme would be 8 and clamps to 7 while a negative one uses
+  the full -8; with 7.5 the scale rounds up to bf16(1 / 7.5) = 0.1337890625, so the extreme sits at
+  7.47 and stays 7."""
+  col = np.zeros((32, 1), dtype=np.float32)
+  col[0, 0], col[1, 0], col[2, 0] = 1.0, -1.0, 0.5
+  w = np.repeat(col, 16, axis=1)
+  for bound, want_pos, want_neg, want_half in ((7.0, 7, -7, 4), (8.0, 7, -8, 4), (7.5, 7, -7, 4)):
+    codes, s = Q.quantize(w, 32, Q.INT4, int4_bound=bound)
+    np.testing.assert_array_equal(s, Q.rb_np(np.full((1, 16), 1.0 / bound, dtype=np.float32)))
+    if bound == 7.5:
+      assert float(s[0, 0]) == 0.1337890625
+    q = codes.astype(np.int32) - 8
+    # 0.5 / scale: 3.5 -> 4 (half to even), 4.0 -> 4, 3.75 -> 4 with the scales as rounded to bf16
+    assert (q[0] == want_pos).all() and (q[1] == want_neg).all() and (q[2] == want_half).all(), (bound, q[:3, 0])
+  a, _ = Q.quantize(w, 32, Q.INT4)
+  b, _ = Q.quantize(w, 32, Q.INT4, int4_bound=7.0)
+  np.testing.assert_array_equal(a, b)
+  c_nf4, s_nf4 = Q.quantize(w, 32, Q.NF4, int4_bound=8.0)      # ignored for NF4
+  np.testing.assert_array_equal(s_nf4, np.ones((1, 16), dtype=np.float32))

@@ -181,6 +181,62 @@ def test_aggregate_loss_literal_cases(mode, loss, mask, kwargs, expected):
   np.testing.assert_allclose(got, expected, rtol=1e-6, atol=1e-6)
 
 
+def _pack_rows(loss, mask):
+  """All rows of an unpacked batch laid end to end in ONE packed row: row i becomes segment i + 1,
+  followed by two padding slots of segment 0 whose (non-zero) loss must never count."""
+  loss, mask = np.asarray(loss, dtype=np.float64), np.asarray(mask, dtype=np.float64)
+  B, T = loss.shape
+  pl = np.concatenate([loss.reshape(-1), [7.0, -3.0]])[None, :]
+  pm = np.concatenate([mask.reshape(-1), [1.0, 0.0]])[None, :]
+  seg = np.concatenate([np.repeat(np.arange(1, B + 1), T), [0, 0]])[None, :]
+  return pl, pm, seg, B + 1
+
+
+@pytest.mark.parametrize("mode,loss,mask,kwargs,expected", AGGREGATE_LOSS_CASES)
+def test_segmented_aggregation_of_a_packed_batch_equals_the_literal_unpacked_cases(mode, loss, mask, kwargs, expected):
+  """The property the reference's own packed-vs-unpacked gate asserts
+  (tests/rl/algo_core_test.py:51-143): sequences packed into one row with segment ids aggregate
+  to the same value as one sequence per row.  Run on the thirteen literal cases of
+  tests/rl/common_test.py:457-576; the two modes whose default norm depends on the batch layout
+  get the unpacked default spelled out.  Padding (segment 0) holds a scored, non-zero loss here:
+  the per-sequence modes must drop it (token-mean and sum-norm, segment-agnostic by
+  definition, are given a zero mask there)."""
+  pl, pm, seg, S = _pack_rows(loss, mask)
+  kw = dict(kwargs)
+  if mode == "sequence-mean-token-scale" and "norm" not in kw:
+    kw["norm"] = np.asarray(loss).shape[1]
+  if mode == "sequence-mean-token-sum-norm" and "norm" not in kw:
+    kw["norm"] = np.asarray(loss).shape[0]
+  if mode in ("token-mean", "sequence-mean-token-sum-norm"):
+    pm[0, -2] = 0.0
+  num, den, min_denom = R.aggregate_loss_segmented(pl, pm, mode, seg, S, **kw)
+  got = R.weighted_metric_compute(num, den, min_denom=min_denom)
+  np.testing.assert_allclose(got, expected, rtol=1e-6, atol=1e-6)
+
+
+def test_segmented_aggregation_reference_gate_value():
+  """tests/rl/algo_core_test.py:51-143: with no old log-probabilities the ratio is 1 and the
+  per-token loss is -advantage; sequences A (advantage 1.5, 3 tokens) and B (3.0, 1 token) packed
+  into one row give (-1.5 + -3.0) / 2 = -2.25 under sequence-mean-token-mean, where a per-row
+  aggregation of the packed row would give -1.875."""
+  loss = -np.array([[1.5, 1.5, 1.5, 3.0]])
+  mask = np.ones((1, 4))
+  seg = np.array([[1, 1, 1, 2]])
+  num, den, md = R.aggregate_loss_segmented(loss, mask, "sequence-mean-token-mean", seg, 3)
+  np.testing.assert_allclose(R.weighted_metric_compute(num, den, md), -2.25, rtol=1e-6)
+  num, den, md = R.aggregate_loss(loss, mask, "sequence-mean-token-mean")
+  np.testing.assert_allclose(R.weighted_metric_compute(num, den, md), -1.875, rtol=1e-6)
+  # the default norm of sum-norm is the number of active segments (:926-929)
+  num, den, md = R.aggregate_loss_segmented(loss, mask, "sequence-mean-token-sum-norm", seg, 3)
+  assert den == 2.0 and num == -7.5
+  with pytest.raises(ValueError, match="explicit 'norm'"):
+    R.aggregate_loss_segmented(loss, mask, "sequence-mean-token-scale", seg, 3)
+  with pytest.raises(ValueError, match="num_segments"):
+    R.aggregate_loss_segmented(loss, mask, "token-mean", seg, None)
+  # ids beyond num_segments are dropped, like jax.ops.segment_sum drops them
+  np.testing.assert_array_equal(R.segmented_sum([[1.0, 2.0, 4.0]], [[0, 5, 1]], 2), [[1.0, 4.0]])
+
+
 def test_aggregate_loss_bad_arguments():
   with pytest.raises(ValueError, match="Unsupported loss aggregation mode"):
     R.aggregate_loss([[0.1]], [[1]], "mean")

@@ -90,7 +90,7 @@ SIGNATURES = {
     "tnx_last_error": (C.c_char_p, []),
     "tnx_version": (_i32, []),
     "tnx_qw_sizes": (_i32, [_i64, _i64, _i32, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
-    "tnx_quantize_pack": (_i32, [_p, _p, _i32, _i64, _i64, _i32, _i32, _i32, _p, _p]),
+    "tnx_quantize_pack": (_i32, [_p, _p, _i32, _i64, _i64, _i32, _i32, _i32, _f32, _p, _p]),
     "tnx_qw_dequant": (_i32, [_p, _p, _p, _i64, _i64, _i32, _i32, _i32, _p]),
     "tnx_qlinear_lora": (_i32, [_p, C.POINTER(QLinearDesc)]),
     "tnx_splitk_finish": (_i32, [_p, C.POINTER(QLinearDesc)]),
@@ -118,6 +118,8 @@ SIGNATURES = {
     "tnx_grpo_ratio": (_i32, [_p, _p, _p, _p, _i64, _i64, _f32, _f32, _p, _p, _p]),
     "tnx_kl_divergence": (_i32, [_p, _p, _p, _i64, _i32, _f32, _p]),
     "tnx_aggregate_loss": (_i32, [_p, _p, _p, _i64, _i64, _i32, _f32, _p, _p]),
+    "tnx_aggregate_loss_segmented_ws_bytes": (C.c_size_t, [_i64, _i32]),
+    "tnx_aggregate_loss_segmented": (_i32, [_p, _p, _p, _p, _i64, _i64, _i32, _i32, _f32, _p, _p]),
     "tnx_logp_drift_ws_bytes": (C.c_size_t, [_i64]),
     "tnx_logp_drift": (_i32, [_p, _p, _p, _p, _i64, _i64, _p, _p]),
     "tnx_logp_drift_static_max_rows": (_i64, []),

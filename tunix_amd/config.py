@@ -35,6 +35,7 @@ class ModelConfig:
   # quantisation of the linears (None: dense bf16, not built)
   qtype: int = Q_INT4
   group: int = 64
+  int4_bound: float = 7.0          # int4 scale = group absmax / this bound (codes clamp to [-8, 7])
   quantize_head: bool = False      # lm_head stays bf16 unless set (module_path never matches it)
   # LoRA
   lora_rank: int = 0

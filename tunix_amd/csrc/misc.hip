@@ -146,6 +146,85 @@ __global__ __launch_bounds__(256) void agg_finish_kernel(const float* row_ws, in
   }
 }
 
+// Packed batches: row b holds several sequences told apart by segment_ids[b][t] (0 = padding).
+// Per row and segment s: (sum of loss * mask, sum of mask) -> seg_ws[b][s][0..1], each sum taken
+// over the row's tokens in order by ONE thread (thread s % 256 handles segment s), so the result
+// does not depend on the launch.  The row is staged through LDS 1024 tokens at a time; ids outside
+// [0, S) belong to no segment.
+__global__ __launch_bounds__(256) void agg_segments_kernel(const float* loss, const float* mask,
+                                                           const int32_t* seg, int64_t T, int S, float* seg_ws) {
+  __shared__ float s_lm[1024], s_m[1024];
+  __shared__ int32_t s_seg[1024];
+  const int64_t b = blockIdx.x;
+  for (int s0 = 0; s0 < S; s0 += 256) {
+    const int sid = s0 + threadIdx.x;
+    float l = 0.f, c = 0.f;
+    for (int64_t t0 = 0; t0 < T; t0 += 1024) {
+      __syncthreads();   // the stage may still be read from the turn before
+      for (int i = threadIdx.x; i < 1024; i += 256) {
+        const int64_t t = t0 + i;
+        const float m = t < T ? mask[b * T + t] : 0.f;
+        s_m[i] = m;
+        s_lm[i] = t < T ? loss[b * T + t] * m : 0.f;
+        s_seg[i] = t < T ? seg[b * T + t] : -1;
+      }
+      __syncthreads();
+      const int n = (int)min((int64_t)1024, T - t0);
+      if (sid < S) {
+        for (int i = 0; i < n; ++i)
+          if (s_seg[i] == sid) {
+            l += s_lm[i];
+            c += s_m[i];
+          }
+      }
+    }
+    if (sid < S) {
+      seg_ws[(b * S + sid) * 2] = l;
+      seg_ws[(b * S + sid) * 2 + 1] = c;
+    }
+  }
+}
+
+// (unreduced sum, denominator) of the mode from the per-segment sums (segment 0 excluded, a
+// segment counts when it has a scored token) and, for the two modes that ignore segments, from
+// the per-row sums.  norm <= 0 in the sum-norm mode means the reference's default there: the
+// number of active segments.
+__global__ __launch_bounds__(256) void agg_segments_finish_kernel(const float* seg_ws, const float* row_ws, int64_t B,
+                                                                  int S, int mode, float norm, float* out) {
+  __shared__ float red[4];
+  float num = 0.f, act = 0.f, tot = 0.f, cnt = 0.f;
+  for (int64_t i = threadIdx.x; i < B * S; i += 256) {
+    if (i % S == 0) continue;   // the padding bucket
+    const float l = seg_ws[2 * i], c = seg_ws[2 * i + 1];
+    if (c > 0.f) {
+      act += 1.f;
+      if (mode == TNX_AGG_SEQ_MEAN_TOKEN_MEAN) num += l / fmaxf(c, 1.0f);
+      else if (mode == TNX_AGG_SEQ_MEAN_TOKEN_SCALE) num += l / fmaxf(norm, 1e-6f);
+      else if (mode == TNX_AGG_SEQ_MEAN_TOKEN_SUM) num += l;
+    }
+  }
+  for (int64_t b = threadIdx.x; b < B; b += 256) {
+    tot += row_ws[2 * b];
+    cnt += row_ws[2 * b + 1];
+  }
+  num = block_sum256(num, red);
+  act = block_sum256(act, red);
+  tot = block_sum256(tot, red);
+  cnt = block_sum256(cnt, red);
+  if (threadIdx.x == 0) {
+    if (mode == TNX_AGG_TOKEN_MEAN) {
+      out[0] = tot;
+      out[1] = cnt;
+    } else if (mode == TNX_AGG_SEQ_MEAN_TOKEN_SUM_NORM) {
+      out[0] = tot;
+      out[1] = norm > 0.f ? norm : act;
+    } else {
+      out[0] = num;
+      out[1] = act;
+    }
+  }
+}
+
 // Agreement of two sets of per-token log-probabilities under a mask.  Row pass: eight masked
 // sums in double (count, |dlogp|, |dp|, p_r, p_t, p_r^2, p_t^2, p_r * p_t) and two maxima per
 // row; the finishing work-group adds the rows in order and forms the five figures.
@@ -500,6 +579,33 @@ extern "C" int tnx_aggregate_loss(void* stream, const float* per_token_loss, con
   TNX_CHECK_LAUNCH("aggregate_loss rows");
   hipLaunchKernelGGL(agg_finish_kernel, dim3(1), dim3(256), 0, as_stream(stream), row_ws, B, mode, norm, out);
   TNX_CHECK_LAUNCH("aggregate_loss finish");
+  return TNX_OK;
+}
+
+extern "C" size_t tnx_aggregate_loss_segmented_ws_bytes(int64_t B, int num_segments) {
+  return B > 0 && num_segments > 0 ? (size_t)B * ((size_t)num_segments + 1) * 2 * sizeof(float) : 0;
+}
+
+extern "C" int tnx_aggregate_loss_segmented(void* stream, const float* per_token_loss, const float* mask,
+                                            const int32_t* segment_ids, int64_t B, int64_t T, int num_segments,
+                                            int mode, float norm, float* ws, float* out) {
+  TNX_REQUIRE(per_token_loss && mask && segment_ids && ws && out, "aggregate_loss_segmented: null pointer");
+  TNX_REQUIRE(B > 0 && T > 0 && B <= 0x7fffffffLL, "aggregate_loss_segmented: bad shape");
+  TNX_REQUIRE(num_segments >= 1 && num_segments <= (1 << 20), "aggregate_loss_segmented: num_segments=%d out of range", num_segments);
+  TNX_REQUIRE(mode >= TNX_AGG_TOKEN_MEAN && mode <= TNX_AGG_SEQ_MEAN_TOKEN_SUM_NORM, "aggregate_loss_segmented: bad mode %d", mode);
+  if (mode == TNX_AGG_SEQ_MEAN_TOKEN_SCALE)
+    TNX_REQUIRE(norm > 0.f, "aggregate_loss_segmented: sequence-mean-token-scale needs an explicit positive norm");
+  float* seg_ws = ws;
+  float* row_ws = ws + (size_t)B * num_segments * 2;
+  hipStream_t st = as_stream(stream);
+  hipLaunchKernelGGL(agg_rows_kernel, dim3((unsigned)B), dim3(256), 0, st, per_token_loss, mask, T, row_ws);
+  TNX_CHECK_LAUNCH("aggregate_loss_segmented rows");
+  hipLaunchKernelGGL(agg_segments_kernel, dim3((unsigned)B), dim3(256), 0, st, per_token_loss, mask, segment_ids, T,
+                     num_segments, seg_ws);
+  TNX_CHECK_LAUNCH("aggregate_loss_segmented segments");
+  hipLaunchKernelGGL(agg_segments_finish_kernel, dim3(1), dim3(256), 0, st, seg_ws, row_ws, B, num_segments, mode,
+                     norm, out);
+  TNX_CHECK_LAUNCH("aggregate_loss_segmented finish");
   return TNX_OK;
 }
 

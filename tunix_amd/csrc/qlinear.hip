@@ -292,7 +292,7 @@ __device__ __forceinline__ int64_t packed_col(int64_t c, int64_t N, int interlea
 
 // One thread per (group of `group` consecutive k, source column).
 __global__ void quantize_pack_kernel(const void* w, int w_is_f32, int64_t K, int64_t N, int group,
-                                     int qtype, int interleave2, uint32_t* codes,
+                                     int qtype, int interleave2, float int4_bound, uint32_t* codes,
                                      uint16_t* scales) {
   const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t g = blockIdx.y;
@@ -304,7 +304,7 @@ __global__ void quantize_pack_kernel(const void* w, int w_is_f32, int64_t K, int
   };
   float amax = 0.f;
   for (int i = 0; i < group; ++i) amax = fmaxf(amax, fabsf(ld(k0 + i)));
-  const uint16_t sbits = f2bf(qtype == TNX_Q_NF4 ? amax : amax / 7.0f);
+  const uint16_t sbits = f2bf(qtype == TNX_Q_NF4 ? amax : amax / int4_bound);
   const float s = bf2f(sbits);
   const int64_t pc = packed_col(c, N, interleave2);
   const int64_t nt = pc / 16, lm = pc % 16;
@@ -561,7 +561,7 @@ extern "C" int tnx_qw_sizes(int64_t K, int64_t N, int group, size_t* codes_bytes
 }
 
 extern "C" int tnx_quantize_pack(void* stream, const void* w, int w_is_f32, int64_t K, int64_t N,
-                                 int group, int qtype, int interleave2, uint32_t* codes,
+                                 int group, int qtype, int interleave2, float int4_bound, uint32_t* codes,
                                  uint16_t* scales) {
   int rc = tnx_qw_sizes(K, N, group, nullptr, nullptr);
   if (rc) return rc;
@@ -569,8 +569,9 @@ extern "C" int tnx_quantize_pack(void* stream, const void* w, int w_is_f32, int6
   TNX_REQUIRE(qtype == TNX_Q_INT4 || qtype == TNX_Q_NF4, "quantize_pack: bad qtype %d", qtype);
   if (interleave2) TNX_REQUIRE(N % 32 == 0, "quantize_pack: interleave2 needs N %% 32 == 0");
   dim3 grid((unsigned)cdiv(N, 128), (unsigned)(K / group));
+  if (!(int4_bound > 0.f)) int4_bound = 7.0f;
   hipLaunchKernelGGL(quantize_pack_kernel, grid, dim3(128), 0, as_stream(stream), w, w_is_f32, K, N,
-                     group, qtype, interleave2, codes, scales);
+                     group, qtype, interleave2, int4_bound, codes, scales);
   TNX_CHECK_LAUNCH("quantize_pack");
   return TNX_OK;
 }

@@ -72,7 +72,11 @@ def from_reference_tree(cfg: ModelConfig, tree: dict) -> dict:
   attn.o_proj.w [H,dh,D], mlp.{gate,up,down}_proj.kernel; LoRA w_lora_a/w_lora_b and
   kernel_lora_a/kernel_lora_b (tunix/models/llama3/mapping_sglang_jax.py:64-145).
   gemma3 (gemma3/model.py:527-565): attn.q_einsum.w [H,D,dh], attn.kv_einsum.w [2,K,D,dh],
-  attn.attn_vec_einsum.w [H,dh,D].
+  attn.attn_vec_einsum.w [H,dh,D]; its LoRA leaves (gemma3/params.py:301-318 and the merge at
+  safetensors_saver.py:88-107): q_einsum.w_lora_a [D,r] / w_lora_b [r,H,dh]; kv_einsum.w_lora_a
+  [D,r], shared by k and v, / w_lora_b [r,2,K,dh]; attn_vec_einsum.w_lora_a [H,dh,r] / w_lora_b
+  [r,D]; mlp.*_proj.kernel_lora_a / kernel_lora_b.  MoE models carry LoRA on the attention
+  projections only.
   """
   def arr(x):
     return x if isinstance(x, torch.Tensor) else torch.as_tensor(np.asarray(x))
@@ -99,6 +103,19 @@ def from_reference_tree(cfg: ModelConfig, tree: dict) -> dict:
       out[p + "wk"] = kv[0].permute(1, 0, 2).reshape(D, -1)
       out[p + "wv"] = kv[1].permute(1, 0, 2).reshape(D, -1)
       out[p + "wo"] = arr(tree[s + "attn.attn_vec_einsum.w"]).reshape(-1, D)
+      r = cfg.lora_rank
+      if s + "attn.q_einsum.w_lora_a" in tree:
+        out[p + "wq.lora_a"] = arr(tree[s + "attn.q_einsum.w_lora_a"])
+        out[p + "wq.lora_b"] = arr(tree[s + "attn.q_einsum.w_lora_b"]).reshape(r, -1)
+      if s + "attn.kv_einsum.w_lora_a" in tree:
+        a = arr(tree[s + "attn.kv_einsum.w_lora_a"])               # [D,r]: one A for k and v
+        b = arr(tree[s + "attn.kv_einsum.w_lora_b"])               # [r,2,K,dh]
+        out[p + "wk.lora_a"], out[p + "wv.lora_a"] = a, a.clone()
+        out[p + "wk.lora_b"] = b[:, 0].reshape(r, -1)
+        out[p + "wv.lora_b"] = b[:, 1].reshape(r, -1)
+      if s + "attn.attn_vec_einsum.w_lora_a" in tree:
+        out[p + "wo.lora_a"] = arr(tree[s + "attn.attn_vec_einsum.w_lora_a"]).reshape(-1, r)
+        out[p + "wo.lora_b"] = arr(tree[s + "attn.attn_vec_einsum.w_lora_b"])
     else:
       out[p + "attn_norm"] = arr(tree[s + "input_layernorm.w"])
       out[p + "mlp_norm"] = arr(tree[s + "post_attention_layernorm.w"])

@@ -104,6 +104,10 @@ class Sampler:
     """LoRA-only state replacement (sampler.py:333-352)."""
     self._transformer.update_lora(lora_state)
 
+  def update_params(self, state: dict) -> None:
+    """Full or LoRA-only state replacement (sampler.py:265-352), by flat parameter name."""
+    self._transformer.update_params(state)
+
   @property
   def dtype(self):
     return torch.bfloat16

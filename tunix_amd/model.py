@@ -40,16 +40,15 @@ class FusedLinear:
 
   def __init__(self, cfg: ModelConfig, weights: dict, names: list[str], device,
                interleave2: bool = False):
-    ws = [weights[n].to(device=device, dtype=torch.bfloat16) for n in names]
     self.names = names
-    self.K = ws[0].shape[0]
-    self.widths = [w.shape[1] for w in ws]
+    self.K = weights[names[0]].shape[0]
+    self.widths = [weights[n].shape[1] for n in names]
     self.N = sum(self.widths)
     self.interleave2 = interleave2
-    self.group, self.qtype = cfg.group, cfg.qtype
-    w = torch.cat(ws, dim=1).contiguous() if len(ws) > 1 else ws[0].contiguous()
-    self.codes, self.scales = ops.quantize_pack(w, cfg.group, cfg.qtype, interleave2)
-    del w
+    self.group, self.qtype, self.int4_bound = cfg.group, cfg.qtype, cfg.int4_bound
+    self.device = device
+    self.codes = self.scales = None
+    self.load_base(weights)
     r = cfg.lora_rank
     self.has_lora = any((n + ".lora_a") in weights for n in names)
     self.rp = _pad32(r) if self.has_lora else 0
@@ -71,6 +70,26 @@ class FusedLinear:
         h, cc = c // half, c % half
         self._row_perm = (cc // 16) * 32 + h * 16 + (cc % 16)
       self.load_lora(weights)
+
+  def load_base(self, weights: dict):
+    """(Re-)quantises and packs the base kernels of every member from `weights` (all members of a
+    fused projection must be present, with the shapes the linear was built with)."""
+    ws = []
+    for n, wd in zip(self.names, self.widths):
+      if n not in weights:
+        raise ValueError(f"New state must have the same structure as the old state: {n} is missing")
+      w = weights[n]
+      if tuple(w.shape) != (self.K, wd):
+        raise ValueError(f"New state must have the same shape as the old state: {n} {tuple(w.shape)} "
+                         f"vs {(self.K, wd)}")
+      ws.append(w.to(device=self.device, dtype=torch.bfloat16))
+    w = torch.cat(ws, dim=1).contiguous() if len(ws) > 1 else ws[0].contiguous()
+    codes, scales = ops.quantize_pack(w, self.group, self.qtype, self.interleave2, self.int4_bound)
+    if self.codes is None:
+      self.codes, self.scales = codes, scales
+    else:   # in place: captured graphs and descriptors keep their pointers
+      self.codes.copy_(codes)
+      self.scales.copy_(scales)
 
   def load_lora(self, weights: dict):
     """Copies lora_a [K,r] / lora_b [r,N_i] of every member into the kernel layout."""
@@ -103,8 +122,9 @@ class ExpertBank:
   """Per-expert QW weights of one MoE layer: fused gate|up (interleaved) and down."""
 
   def __init__(self, cfg: ModelConfig, weights: dict, prefix: str, device):
-    g, u, d = weights[prefix + "e_gate"], weights[prefix + "e_up"], weights[prefix + "e_down"]
+    g = weights[prefix + "e_gate"]
     E = g.shape[0]
+    self.cfg, self.prefix, self.device = cfg, prefix, device
     self.E, self.D, self.F = E, g.shape[1], g.shape[2]
     cb, sb = ops.qw_sizes(self.D, 2 * self.F, cfg.group)
     self.gu_codes = torch.empty(E * cb // 4, dtype=torch.int32, device=device)
@@ -112,15 +132,31 @@ class ExpertBank:
     cb2, sb2 = ops.qw_sizes(self.F, self.D, cfg.group)
     self.dn_codes = torch.empty(E * cb2 // 4, dtype=torch.int32, device=device)
     self.dn_scales = torch.empty(E * sb2 // 2, dtype=torch.bfloat16, device=device)
+    self.router_t = torch.empty(E, self.D, dtype=torch.bfloat16, device=device)
+    self.load_base(weights)
+
+  def load_base(self, weights: dict):
+    """(Re-)quantises the experts and copies the router from `weights`, in place."""
+    cfg, prefix, device, E = self.cfg, self.prefix, self.device, self.E
+    for n, shape in ((prefix + "e_gate", (E, self.D, self.F)), (prefix + "e_up", (E, self.D, self.F)),
+                     (prefix + "e_down", (E, self.F, self.D)), (prefix + "router", (self.D, E))):
+      if n not in weights:
+        raise ValueError(f"New state must have the same structure as the old state: {n} is missing")
+      if tuple(weights[n].shape) != shape:
+        raise ValueError(f"New state must have the same shape as the old state: {n} {tuple(weights[n].shape)} vs {shape}")
+    g, u, d = weights[prefix + "e_gate"], weights[prefix + "e_up"], weights[prefix + "e_down"]
+    cb, sb = ops.qw_sizes(self.D, 2 * self.F, cfg.group)
+    cb2, sb2 = ops.qw_sizes(self.F, self.D, cfg.group)
     for e in range(E):
       w = torch.cat([g[e], u[e]], dim=1).to(device, torch.bfloat16).contiguous()
-      c, s = ops.quantize_pack(w, cfg.group, cfg.qtype, True)
+      c, s = ops.quantize_pack(w, cfg.group, cfg.qtype, True, cfg.int4_bound)
       self.gu_codes[e * cb // 4:(e + 1) * cb // 4].copy_(c)
       self.gu_scales[e * sb // 2:(e + 1) * sb // 2].copy_(s)
-      c, s = ops.quantize_pack(d[e].to(device, torch.bfloat16).contiguous(), cfg.group, cfg.qtype)
+      c, s = ops.quantize_pack(d[e].to(device, torch.bfloat16).contiguous(), cfg.group, cfg.qtype, False,
+                               cfg.int4_bound)
       self.dn_codes[e * cb2 // 4:(e + 1) * cb2 // 4].copy_(c)
       self.dn_scales[e * sb2 // 2:(e + 1) * sb2 // 2].copy_(s)
-    self.router_t = weights[prefix + "router"].to(device, torch.bfloat16).t().contiguous()
+    self.router_t.copy_(weights[prefix + "router"].to(device, torch.bfloat16).t())
 
 
 class QLoRAModel:
@@ -179,6 +215,67 @@ class QLoRAModel:
           ly[key].load_lora(new_lora)
     if self.head is not None:
       self.head.load_lora(new_lora)
+    torch.cuda.synchronize(self.device)
+
+  # full state replacement (tunix/generate/sampler.py:265-332; VanillaRollout.update_params,
+  # tunix/rl/rollout/vanilla_rollout.py:92-121, merges a partial state into the old one first)
+  def update_params(self, new_state: dict):
+    """Replaces parameters by name.  A state holding only LoRA leaves (`*.lora_a` / `*.lora_b`)
+    is the LoRA-only swap and must name every adapter (`update_lora`).  A state with base
+    parameters replaces those -- embedding, norms, head, and linears, which are re-quantised and
+    re-packed in place; the members of a fused projection (q|k|v, gate|up, an expert bank)
+    come together -- and may carry LoRA leaves as well.  Shapes must match the old state's."""
+    base = {k: v for k, v in new_state.items() if not k.endswith((".lora_a", ".lora_b"))}
+    lora = {k: v for k, v in new_state.items() if k.endswith((".lora_a", ".lora_b"))}
+    if not base:
+      self.update_lora(lora)
+      return
+    dev, bf = self.device, torch.bfloat16
+    known = {"embed", "final_norm"} | ({"lm_head"} if not self.cfg.tied_embedding else set())
+    for i in range(self.cfg.num_layers):
+      p = f"l{i}."
+      known |= {p + n for n in ("attn_norm", "mlp_norm", "q_norm", "k_norm", "post_attn_norm", "post_ffw_norm",
+                                "wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down", "router", "e_gate", "e_up",
+                                "e_down")}
+    extra = sorted(set(base) - known)
+    if extra:
+      raise ValueError(f"New state must have the same structure as the old state. extra={extra}")
+
+    def copy_into(dst: torch.Tensor, name: str, transpose: bool = False):
+      src = base[name].to(dev, bf)
+      src = src.t() if transpose else src
+      if tuple(src.shape) != tuple(dst.shape):
+        raise ValueError(f"New state must have the same shape as the old state: {name} {tuple(base[name].shape)}")
+      dst.copy_(src)
+
+    if "embed" in base:
+      copy_into(self.embed, "embed")
+    if "final_norm" in base:
+      copy_into(self.final_norm, "final_norm")
+    if "lm_head" in base:
+      if self.head is not None:
+        self.head.load_base(base)
+      elif self.head_w is not None:
+        copy_into(self.head_w, "lm_head", transpose=True)
+    for i, ly in enumerate(self.layers):
+      p = f"l{i}."
+      for n in ("attn_norm", "mlp_norm", "q_norm", "k_norm", "post_attn_norm", "post_ffw_norm"):
+        if p + n in base:
+          if n not in ly:
+            raise ValueError(f"New state must have the same structure as the old state. extra={[p + n]}")
+          copy_into(ly[n], p + n)
+      for key in ("qkv", "o", "gu", "down"):
+        if key in ly and any(n in base for n in ly[key].names):
+          ly[key].load_base(base)
+      if "experts" in ly and any(p + n in base for n in ("router", "e_gate", "e_up", "e_down")):
+        ly["experts"].load_base(base)
+    if lora:
+      for ly in self.layers:
+        for key in ("qkv", "o", "gu", "down"):
+          if key in ly:
+            ly[key].load_lora(lora)
+      if self.head is not None:
+        self.head.load_lora(lora)
     torch.cuda.synchronize(self.device)
 
   def weight_bytes(self) -> dict:

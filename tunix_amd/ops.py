@@ -36,17 +36,19 @@ def qw_sizes(K: int, N: int, group: int) -> tuple[int, int]:
   return cb.value, sb.value
 
 
-def quantize_pack(w: torch.Tensor, group: int, qtype: int, interleave2: bool = False):
-  """w [K,N] bf16 or fp32 on the GPU -> (codes int32 [K*N/8], scales bf16 [...])."""
+def quantize_pack(w: torch.Tensor, group: int, qtype: int, interleave2: bool = False, int4_bound: float = 7.0):
+  """w [K,N] bf16 or fp32 on the GPU -> (codes int32 [K*N/8], scales bf16 [...]).  int4_bound: the
+  integer a group's absmax maps to (scale = absmax / bound; ignored for NF4)."""
   K, N = w.shape
   cb, sb = qw_sizes(K, N, group)
   codes = torch.empty(cb // 4, dtype=torch.int32, device=w.device)
   scales = torch.empty(sb // 2, dtype=torch.bfloat16, device=w.device)
+  scales[-8:] = 0   # the 16 bytes of tail padding the packer does not write
   is_f32 = 1 if w.dtype == torch.float32 else 0
   if not is_f32:
     _expect(w, torch.bfloat16, "quantize_pack")
   L.check(L.lib().tnx_quantize_pack(_stream(), _ptr(w), is_f32, K, N, group, qtype,
-                                    1 if interleave2 else 0, _ptr(codes), _ptr(scales)),
+                                    1 if interleave2 else 0, float(int4_bound), _ptr(codes), _ptr(scales)),
           "tnx_quantize_pack")
   return codes, scales
 
@@ -224,6 +226,15 @@ def aggregate_loss(per_token_loss, mask, mode: int, norm: float, row_ws, out):
   B, T = per_token_loss.shape
   L.check(L.lib().tnx_aggregate_loss(_stream(), _ptr(per_token_loss), _ptr(mask), B, T, mode,
                                      float(norm), _ptr(row_ws), _ptr(out)), "tnx_aggregate_loss")
+
+
+def aggregate_loss_segmented(per_token_loss, mask, segment_ids, num_segments: int, mode: int, norm: float, out):
+  B, T = per_token_loss.shape
+  nb = int(L.lib().tnx_aggregate_loss_segmented_ws_bytes(B, num_segments))
+  ws = torch.empty(nb // 4, dtype=torch.float32, device=out.device)
+  L.check(L.lib().tnx_aggregate_loss_segmented(_stream(), _ptr(per_token_loss), _ptr(mask), _ptr(segment_ids), B, T,
+                                               int(num_segments), mode, float(norm), _ptr(ws), _ptr(out)),
+          "tnx_aggregate_loss_segmented")
 
 
 def logp_drift(rollout_logp, trainer_logp, mask, out5):

@@ -179,11 +179,9 @@ def _check_get_norm(arguments: dict[str, Any], default: float) -> float:
 
 def aggregate_loss(per_token_loss: torch.Tensor, completion_mask: torch.Tensor, loss_agg_mode: str,
                    segment_ids=None, num_segments=None, **kwargs: Any) -> WeightedMetric:
-  """Aggregates a [B, T] per-token loss under its completion mask (tunix/rl/common.py:763-854).
-  Packing segments (`segment_ids`) belong to the trainer's packed batches and are not part of
-  this build."""
-  if segment_ids is not None:
-    raise NotImplementedError("aggregate_loss over packing segments is outside this build")
+  """Aggregates a [B, T] per-token loss under its completion mask (tunix/rl/common.py:763-940).
+  With `segment_ids` ([B, T], 0 = padding) the batch is packed: the per-sequence modes reduce per
+  segment instead of per row (the segment branch, :857-940); `num_segments` bounds the ids."""
   if loss_agg_mode not in ops.AGG_MODES:
     raise ValueError(
         f"Unsupported loss aggregation mode: {loss_agg_mode}. Supported modes:"
@@ -193,15 +191,36 @@ def aggregate_loss(per_token_loss: torch.Tensor, completion_mask: torch.Tensor, 
   if per_token_loss.dim() != 2 or per_token_loss.shape != completion_mask.shape:
     raise ValueError("per_token_loss and completion_mask must both be [batch_size, sequence_len]")
   B, T = per_token_loss.shape
+  min_denom = 1e-6 if loss_agg_mode in ("seq-mean-token-sum", "sequence-mean-token-sum-norm") else 1.0
+  loss = per_token_loss.to(torch.float32).contiguous()
+  mask = completion_mask.to(torch.float32).contiguous()
+  out = torch.zeros(2, dtype=torch.float32, device=loss.device)
+  if segment_ids is not None:
+    if num_segments is None:
+      raise ValueError("num_segments must be provided when segment_ids is not None.")
+    if tuple(segment_ids.shape) != (B, T):
+      raise ValueError("segment_ids must be [batch_size, sequence_len]")
+    norm = -1.0   # sum-norm: the number of active segments unless the caller names a norm
+    if loss_agg_mode == "sequence-mean-token-scale":
+      if "norm" not in kwargs:
+        raise ValueError(
+            "sequence-mean-token-scale under sequence packing requires an"
+            " explicit 'norm' (e.g. max_response_length); the default row-width"
+            " norm is the pack budget, which dilutes every sequence.")
+      norm = _check_get_norm(kwargs, T)
+    elif loss_agg_mode == "sequence-mean-token-sum-norm" and "norm" in kwargs:
+      norm = _check_get_norm(kwargs, 1.0)
+    if B and T:
+      seg = segment_ids.to(device=loss.device, dtype=torch.int32).contiguous()
+      ops.aggregate_loss_segmented(loss, mask, seg, int(num_segments), ops.AGG_MODES[loss_agg_mode], norm, out)
+    elif loss_agg_mode == "sequence-mean-token-sum-norm" and norm > 0:
+      out[1] = norm
+    return WeightedMetric(out[0], out[1], min_denom=min_denom)
   norm = 1.0
   if loss_agg_mode == "sequence-mean-token-scale":
     norm = _check_get_norm(kwargs, T)
   elif loss_agg_mode == "sequence-mean-token-sum-norm":
     norm = _check_get_norm(kwargs, B)
-  min_denom = 1e-6 if loss_agg_mode in ("seq-mean-token-sum", "sequence-mean-token-sum-norm") else 1.0
-  loss = per_token_loss.to(torch.float32).contiguous()
-  mask = completion_mask.to(torch.float32).contiguous()
-  out = torch.zeros(2, dtype=torch.float32, device=loss.device)
   if B and T:
     row_ws = torch.empty(B, 2, dtype=torch.float32, device=loss.device)
     ops.aggregate_loss(loss, mask, ops.AGG_MODES[loss_agg_mode], norm, row_ws, out)

@@ -74,10 +74,12 @@ class HipRollout:
                                           temperature=temperature, chunk_size=chunk_size)
 
   def update_params(self, params: dict, filter_types: Any = None) -> None:
-    """LoRA factors only (the base weights are frozen and quantized): `params` maps
-    '<linear>.lora_a' / '<linear>.lora_b' to new tensors, every adapter present
-    (tunix/generate/sampler.py:333-352 requires the same structure as the old state)."""
-    self._sampler.update_lora(params)
+    """Weight sync between steps (tunix/rl/rollout/vanilla_rollout.py:92-121).  `params` maps flat
+    names to new tensors.  Only '<linear>.lora_a' / '<linear>.lora_b' leaves: the LoRA-only swap,
+    every adapter present (tunix/generate/sampler.py:333-352 requires the same structure as the
+    old state).  With base parameters in it: those are replaced too, the linears re-quantised
+    and re-packed in place (the full-state branch, sampler.py:322-325)."""
+    self._sampler.update_params(params)
 
   def pad_id(self) -> int:
     return self._sampler.tokenizer.pad_id()
