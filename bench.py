@@ -4,15 +4,24 @@
 (random-init weights, synthetic prompts), prefills batch 128 x prompt 512, runs W untimed decode
 steps and times exactly K decode steps (one captured HIP graph replayed K times), then prints ONE
 JSON line.  A "step" is one decode step of the whole batch: embedding -> 32 layers -> lm_head ->
-greedy sampling -> token commit.
+greedy sampling -> token commit.  The workload is a 512-step rollout whose context grows from
+512 to 1024: when K is smaller than the rollout, the K steps are taken in equal groups spread
+evenly over that range (the device step counter is moved between groups, over a cache filled
+beforehand; each group is bracketed by a synchronisation and only the groups are timed), so
+that `value` speaks for the whole rollout (mean context 768) whatever K is; the figure over the
+first K steps alone is reported beside it (`first_steps`).
 
 Extra objects on the line:
   roofline      the kernel with the largest share of a step (the quantised GEMM), timed in
                 isolation with events on its launch stream; roofline_hbm prices the same
                 launches against the HBM roof
   kernels       the same measurement for every kernel family of the step
+  fused_logps   the standalone per-token log-probability workload at training scale
   cpu_baseline  the CPU oracle (a port of the reference's JAX path) timed on this host on a
                 bounded sample and scaled linearly
+
+`--config c1|c2|c4` measures the other rollout workloads through the public Sampler call
+(their own JSON line), `--fused-logps` the standalone log-probability workload alone.
 """
 from __future__ import annotations
 
@@ -165,10 +174,35 @@ def many_rows_breakdown(model, rows, iters):
           "linears": out}
 
 
-# HBM bytes of one qgemm128 launch on the default workload (batch 128, Llama-3.1-8B shapes, mean
-# over the four linears): rocprofv3 FETCH_SIZE + WRITE_SIZE, (22190 + 12947) KiB, both counters
-# scaled by 1.000 against a plain copy of known size (profiles/qgemm128_kernel_llama8b_decode_b128.md).
-QGEMM128_TRAFFIC_BYTES_B128 = 35_980_288
+# HBM bytes of one qgemm128 launch on the default workload come from counter runs of this script
+# (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over `--kernels-only`), kept in a tracked summary next
+# to a hash of the kernel's sources: the figure is reported only while the sources are the ones it
+# was measured on.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "qgemm128_kernel_llama8b_decode_b128.json")
+KERNEL_SOURCES = ("qgemm128.h", "gemm_tile.h")
+
+
+def kernel_source_hash():
+  import hashlib
+  h = hashlib.sha256()
+  for name in KERNEL_SOURCES:
+    with open(os.path.join(ROOT, "tunix_amd", "csrc", name), "rb") as f:
+      h.update(f.read())
+  return h.hexdigest()[:16]
+
+
+def measured_traffic():
+  """{"traffic": bytes per launch, "read": ..., "write": ...} from the tracked counter summary, or
+  None when there is none for the current kernel sources."""
+  try:
+    with open(TRAFFIC_PROFILE) as f:
+      prof = json.load(f)
+  except (OSError, ValueError):
+    return None
+  if prof.get("kernel_source_sha256_16") != kernel_source_hash():
+    return None
+  return {"traffic": int(prof["read_bytes_per_launch"] + prof["write_bytes_per_launch"]),
+          "read": int(prof["read_bytes_per_launch"]), "write": int(prof["write_bytes_per_launch"])}
 
 
 def rooflines(kern, default_workload=False):
@@ -183,9 +217,11 @@ def rooflines(kern, default_workload=False):
   us = sum(kern[k]["kernel_ms"] for k in names) / len(names) * 1e3
   tf = flops / (us * 1e-6) / 1e12
   gbs = nbytes / (us * 1e-6) / 1e9
+  meas = measured_traffic() if default_workload else None
   roofline = {"kernel": "qgemm128_kernel", "bound": "mfma", "achieved": round(tf, 1),
               "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-              "traffic": QGEMM128_TRAFFIC_BYTES_B128 if default_workload else None,
+              "traffic": meas["traffic"] if meas else None,
+              "traffic_read": meas["read"] if meas else None, "traffic_write": meas["write"] if meas else None,
               "us_per_launch": round(us, 2), "algorithmic_flops": flops,
               "algorithmic_bytes": nbytes,
               "launch_shapes_us": {k: round(kern[k]["kernel_ms"] * 1e3, 2) for k in names}}
@@ -317,7 +353,9 @@ def fused_logps_workload(rows, chunk, iters):
   ms = e0.elapsed_time(e1) / iters
   flops = 2.0 * rows * D * V + 2.0 * rows * r * (D + V)
   assert bool(torch.isfinite(logp).all()) and bool(torch.isfinite(loss).all())
-  print(json.dumps({
+  del x, codes, scales, b_t, part
+  torch.cuda.empty_cache()
+  return {
       "metric": "fused per-token logps rows/sec @1 MI355X (int4 g128 + LoRA r64 head, 4096 x 128256)",
       "value": round(rows / (ms * 1e-3), 1), "unit": "rows/s", "n_gpus": 1, "steps": iters, "warmup": 1,
       "ms_per_step": round(ms, 3), "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
@@ -325,7 +363,65 @@ def fused_logps_workload(rows, chunk, iters):
                  "rows_per_launch": chunk},
       "roofline": {"kernel": "qgemm_wide_kernel (statistics epilogue)", "bound": "mfma",
                    "achieved": round(flops / (ms * 1e-3) / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                   "frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}}), flush=True)
+                   "frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}}
+
+
+def config_workload(name, steps):
+  """The other rollout workloads, through the public Sampler call: two rollouts of different
+  length, so that prefill, graph capture and host work cancel; ms per decode step from the
+  difference.  c1: tiny Qwen3-style decoder, batch 8, prompt 64, greedy.  c2: Gemma3-1B shape,
+  batch 64, prompt 256, temperature 1.0 / top-k 50.  c4: Qwen3-30B-A3B shape (128 experts, top-8),
+  batch 64, prompt 1024, greedy."""
+  import numpy as np
+  import torch
+
+  from tunix_amd import config, dummy_model
+  from tunix_amd.generate import CacheConfig, Sampler
+  from tunix_amd.generate.utils import IdTokenizer
+  from tunix_amd.model import QLoRAModel
+  dev = torch.device("cuda:0")
+  spec = {
+      "c1": (config.tiny_qwen3(), 8, 64, 64, dict(), "tiny Qwen3-style decoder (2 layers, D512, V32000, int4 g64 + LoRA r8), greedy"),
+      "c2": (config.gemma3_1b(), 64, 256, 256, dict(temperature=1.0, top_p=1.0, top_k=50, seed=7),
+             "Gemma3-1B-shaped (26 layers, V262144 tied head, int4 g128 + LoRA r16), temperature 1.0 top-k 50"),
+      "c4": (config.qwen3_30b_a3b(), 64, 1024, 256, dict(),
+             "Qwen3-30B-A3B-shaped MoE (48 layers, 128 experts top-8, int4 g128, LoRA r16 on attention), greedy"),
+  }[name]
+  cfg, B, P, T, kw, label = spec
+  t0 = time.time()
+  model = QLoRAModel(cfg, dummy_model.create_dummy_weights(cfg, seed=20250 + int(name[1]), device=dev), dev)
+  torch.cuda.empty_cache()
+  log(f"{name}: model built in {time.time() - t0:.1f}s; bytes per step {model.weight_bytes()}")
+  tok = IdTokenizer(cfg.vocab_size, pad_id=0, eos_id=1)
+  sampler = Sampler(model, tok, CacheConfig(P + T, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim))
+  ids = np.random.Generator(np.random.PCG64(20250)).integers(1, cfg.vocab_size, size=(B, P)).astype(np.int32)
+  prompts = [ids[b] for b in range(B)]
+  steps = max(1, min(steps, T - 8))
+  times, stats = [], []
+  for n in (4, 4, 4 + steps):     # the first call also pays the lazy module loads
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    sampler(prompts, n, max_prompt_length=P, return_logprobs=True, eos_tokens=[-1], **kw)
+    torch.cuda.synchronize()
+    times.append(time.perf_counter() - t0)
+    stats.append(dict(sampler.last_stats))
+  ms = (times[2] - times[1]) / steps * 1e3
+  wb = model.weight_bytes()
+  mean_ctx = P + 4 + steps / 2.0
+  window = cfg.sliding_window or 0
+  kv = 0
+  for i in range(cfg.num_layers):
+    ctx = min(mean_ctx, window) if (window and cfg.is_local_layer(i)) else mean_ctx
+    kv += B * cfg.num_kv_heads * ctx * cfg.head_dim * 4
+  step_bytes = wb["quantized"] + wb["lora"] + wb["head"] + kv
+  return {
+      "metric": f"decode tokens/sec @1 MI355X ({name})", "value": round(B / (ms * 1e-3), 1), "unit": "tokens/s",
+      "n_gpus": 1, "steps": steps, "warmup": 4, "ms_per_step": round(ms, 4), "higher_is_better": True,
+      "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+      "config": {"workload": label, "layers": cfg.num_layers, "global_batch": B, "prompt_len": P, "gen_len": T,
+                 "context_range": [P + 4, P + 4 + steps], "parallelism": "single GPU"},
+      "prefill_s": round(stats[2]["prefill_ms"] * 1e-3, 3),
+      "hbm_roofline_frac_step": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "step_bytes": int(step_bytes)}
 
 
 def main():
@@ -348,13 +444,21 @@ def main():
                   help="instead of the decode benchmark: the standalone fused per-token log-probability "
                        "workload (32 x 4096 rows, quantised 128256-column head), its own JSON line")
   ap.add_argument("--fused-logps-rows", type=int, default=131072)
+  ap.add_argument("--no-fused-logps", action="store_true",
+                  help="leave the standalone log-probability workload out of the default run's line")
+  ap.add_argument("--config", choices=["c1", "c2", "c3", "c4"], default="c3",
+                  help="c3 (default): the headline workload; c1 / c2 / c4: the other rollout workloads through "
+                       "the public Sampler call, their own JSON line")
+  ap.add_argument("--contiguous", action="store_true",
+                  help="time the K steps that follow the prefill directly instead of K steps spread over the "
+                       "rollout's context range")
   ap.add_argument("--summarize-trace", metavar="CSV", default=None,
                   help="no GPU work: tabulate one decode step of a rocprofv3 kernel-trace csv of this script")
   args = ap.parse_args()
   if args.fused_logps:
     if args.gpus != 1:
       sys.exit("bench.py measures one GPU; --gpus must be 1")
-    fused_logps_workload(args.fused_logps_rows, 16384, max(1, args.kernel_iters // 10))
+    print(json.dumps(fused_logps_workload(args.fused_logps_rows, 16384, max(1, args.kernel_iters // 10))), flush=True)
     return
   if args.summarize_trace:
     summarize_step_trace(args.summarize_trace)
@@ -363,6 +467,10 @@ def main():
     print("bench.py measures one GPU: this build has no multi-GPU path (the decode path shards "
           "by batch rows with no exchange); run with --gpus 1", file=sys.stderr)
     sys.exit(2)
+
+  if args.config != "c3":
+    print(json.dumps(config_workload(args.config, args.steps if args.steps != 508 else 200)), flush=True)
+    return
 
   import numpy as np
   import torch
@@ -400,7 +508,15 @@ def main():
     dst = torch.empty_like(src)
     for _ in range(3):
       dst.copy_(src)
+    # and a second yardstick for reads: 1 GiB fetched once with the 16-byte-per-lane buffer loads
+    # the GEMM, attention and head kernels stream their operands with (stream_read_kernel)
+    from tunix_amd import ops as _ops
+    big = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+    sink = torch.zeros(64, dtype=torch.int32, device=dev)
+    for width in (16, 8, 16, 8):      # 8 bytes per lane: the GEMM's packed-code loads
+      _ops.stream_read(big, sink, width)
     torch.cuda.synchronize()
+    del big
     many = many_rows_breakdown(model, 8192, max(2, args.kernel_iters // 5))
     print(json.dumps({"kernels_only": True, "context": P + T // 2, "roofline": roofline,
                       "roofline_hbm": roofline_hbm, "roofline_many_rows": many,
@@ -447,17 +563,55 @@ def main():
   torch.cuda.current_stream().wait_stream(side)
   torch.cuda.synchronize()
   step_first = int(st.step.item())
-  t0 = time.perf_counter()
-  for _ in range(K):
-    graph.replay()
-  torch.cuda.synchronize()
-  dt = time.perf_counter() - t0
-  step_last = int(st.step.item())
-  assert step_last - step_first == K, (step_first, step_last, K)
+  last_step = P + T - 2          # the step counter's value before the rollout's last decode step
+
+  def timed(n):
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n):
+      graph.replay()
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+  first_steps = None
+  if args.contiguous or K >= last_step - step_first:
+    dt = timed(K)
+    step_last = int(st.step.item())
+    assert step_last - step_first == K, (step_first, step_last, K)
+    contexts = [step_first + 1 + i for i in range(K)]
+    groups = 1
+  else:
+    # K steps in `groups` equal groups whose starting points are spread evenly from the step after
+    # the warm-up to the end of the rollout.  The part of the rollout that is skipped must look
+    # like a rollout to the kernels: the cache slots and token columns between the groups are
+    # filled with values of the kind a decode step writes (no pad ids: every key is attended).
+    groups = max(g for g in (8, 5, 4, 2, 1) if K % g == 0 and K // g >= 1)
+    per = K // groups
+    gen = torch.Generator(device=dev).manual_seed(20253)
+    st.token_buffer[:, step_first + 1:] = torch.randint(1, cfg.vocab_size, (B, S - step_first - 1), generator=gen,
+                                                        device=dev, dtype=torch.int32)
+    for kc, vc in zip(st.kcache, st.vcache):
+      kc[:, :, step_first + 1:].normal_(generator=gen)
+      vc[:, :, step_first + 1:].normal_(generator=gen)
+    starts = [step_first + round(g * (last_step + 1 - per - step_first) / max(groups - 1, 1)) for g in range(groups)]
+    dt, contexts = 0.0, []
+    first_dt = None
+    for s0 in starts:
+      st.step.fill_(s0)
+      dt_g = timed(per)
+      assert int(st.step.item()) == s0 + per
+      contexts += [s0 + 1 + i for i in range(per)]
+      dt += dt_g
+      if first_dt is None:
+        first_dt = dt_g
+    first_steps = {"steps": per, "ms_per_step": round(first_dt / per * 1e3, 4),
+                   "tokens_per_s": round(B * per / first_dt, 1), "context_range": [starts[0] + 1, starts[0] + per]}
+    step_last = starts[-1] + per
   ms_per_step = dt / K * 1e3
   value = B * K / dt
-  mean_ctx = (step_first + 1 + step_last) / 2.0 + 0.5
-  log(f"decode: {K} steps, {ms_per_step:.3f} ms/step, {value:.0f} tokens/s, mean context {mean_ctx:.1f}")
+  mean_ctx = sum(contexts) / len(contexts) + 0.5
+  log(f"decode: {K} steps in {groups} group(s), {ms_per_step:.3f} ms/step, {value:.0f} tokens/s, "
+      f"mean context {mean_ctx:.1f} (contexts {contexts[0]}..{contexts[-1]})")
 
   # The workload's other variant: temperature 1.0, top_p 1.0, no top-k (the reference's default
   # rollout sampling: one categorical draw over the whole vocabulary per row and step), through
@@ -497,7 +651,8 @@ def main():
       "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
       "config": {"workload": "Llama-3.1-8B-shaped NF4(g64)+LoRA r64 greedy rollout decode",
                  "layers": cfg.num_layers, "global_batch": B, "prompt_len": P, "gen_len": T,
-                 "context_range": [step_first + 1, step_last + 1], "parallelism": "single GPU"},
+                 "context_range": [contexts[0], contexts[-1]], "mean_context": round(mean_ctx, 1),
+                 "timed_groups": groups, "parallelism": "single GPU"},
       "hbm_roofline_frac_step": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
       "step_bytes": int(step_bytes), "prefill_s": round(prefill_s, 3),
       "roofline": roofline, "roofline_hbm": roofline_linears, "roofline_many_rows": many,
@@ -505,8 +660,16 @@ def main():
                       "TFLOPs": round(v["tflops"], 1), "ms_per_step": round(v["step_ms"], 4)}
                   for k, v in kern.items()},
   }
+  if first_steps is not None:
+    result["first_steps"] = first_steps
   if sampling is not None:
     result["sampling_variant"] = sampling
+  if not args.no_fused_logps:
+    del sampler, st, runner, graph
+    torch.cuda.empty_cache()
+    fl = fused_logps_workload(args.fused_logps_rows, 16384, 2)
+    result["fused_logps"] = {k: fl[k] for k in ("metric", "value", "unit", "ms_per_step", "config", "roofline")}
+    log(f"fused logps: {fl['ms_per_step']} ms per pass over {args.fused_logps_rows} rows, {fl['roofline']['achieved']} TFLOP/s")
   if not args.no_cpu_baseline:
     threads = min(16, os.cpu_count() or 1)
     t0 = time.time()

@@ -459,6 +459,13 @@ int64_t tnx_logp_drift_static_max_rows(void);
 int tnx_logp_drift_static(void* stream, const float* rollout_logp, const float* trainer_logp,
                           const float* mask, int64_t B, int64_t T, float* out5);
 
+/* Measurement aid, no counterpart in the reference: reads `bytes` bytes at `src` exactly once with
+ * the access pattern of this library's streaming kernels (buffer loads of bytes_per_lane = 16 or
+ * 8 bytes per lane) and xors them into sink64[0..63] (64 device words).  A read of known size:
+ * run it under a hardware fetch counter next to the kernels of interest to learn what the counter
+ * reports per byte for this kind of load. */
+int tnx_stream_read(void* stream, const void* src, uint64_t bytes, int bytes_per_lane, uint32_t* sink64);
+
 /* Fill n 32-bit words with `value` (graph-capturable replacement for hipMemsetAsync). */
 int tnx_fill_u32(void* stream, uint32_t* p, int64_t n, uint32_t value);
 

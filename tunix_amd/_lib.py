@@ -124,6 +124,7 @@ SIGNATURES = {
     "tnx_logp_drift": (_i32, [_p, _p, _p, _p, _i64, _i64, _p, _p]),
     "tnx_logp_drift_static_max_rows": (_i64, []),
     "tnx_logp_drift_static": (_i32, [_p, _p, _p, _p, _i64, _i64, _p]),
+    "tnx_stream_read": (_i32, [_p, _p, C.c_uint64, _i32, _p]),
     "tnx_fill_u32": (_i32, [_p, _p, _i64, C.c_uint32]),
 }
 
