@@ -326,6 +326,13 @@ typedef struct tnx_lmhead_desc {
   const int32_t* draw_step_ptr;
   int32_t* draw_id;           /* int32 [M]                                                   */
   float* draw_logp;           /* fp32 [M]: log-softmax at the drawn id, or NULL              */
+  /* fp32-accumulate reference mode: != 0 keeps the fp32 accumulator as the logit instead of
+   * rounding it to bf16 first (the reference's head is a bf16 einsum cast to fp32,
+   * llama3/model.py:688-697; this mode is what that einsum would give with an fp32 result).
+   * Inputs are what they are in the normal mode (bf16 x, weights dequantised to bf16, bf16 t);
+   * every sum and the log-softmax run in fp32.  Log-probabilities then agree with an fp64
+   * evaluation of the same bf16 operands to 1e-4 instead of to bf16 resolution. */
+  int logits_fp32;
 } tnx_lmhead_desc;
 int64_t tnx_lmhead_nblocks(int64_t V);
 int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* h_desc);

@@ -624,6 +624,77 @@ def test_lmhead_many_rows_quantized_head(gpu, M, D, V, group, qtype, r, entropy)
   assert (tlp.cpu() - ref_t).abs().max().item() < 2e-2
 
 
+@pytest.mark.parametrize("M,D,V,dense,r", [(300, 512, 8208, False, 64), (128, 512, 4096, True, 0), (1030, 256, 8192, False, 32)])
+def test_lmhead_fp32_accumulate_reference_mode(gpu, M, D, V, dense, r):
+  """logits_fp32: the fp32 accumulators are the logits (no rounding to bf16).  Against an fp64
+  evaluation of the same operands -- bf16 hidden states, weights dequantised to bf16, bf16
+  adapter intermediate t -- the per-token log-probabilities, logsumexp and entropy agree to 1e-4
+  (the tolerance the fp32-accumulate reference mode is held to), where the normal mode, whose
+  logits are bf16 values, is only good to bf16 resolution; the arg-max is that of the fp64 logits
+  except at margins below 1e-4.  The many-row shape, which the bf16 mode sends through the
+  128 x 256 kernel, takes the 128 x 128 head kernel here (that one stages its tile in bf16)."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  x = rnd((M, D), 160)
+  w = rnd((D, V), 161, 0.05)
+  g = torch.Generator().manual_seed(162)
+  targets = torch.randint(0, V, (M,), generator=g, dtype=torch.int32)
+  gx = bf(x).to(gpu)
+  d = L.LmHeadDesc()
+  d.M, d.D, d.V, d.x = M, D, V, gx.data_ptr()
+  if dense:
+    gw = bf(w).t().contiguous().to(gpu)
+    d.w_bf16 = gw.data_ptr()
+    ref_lg = x.double() @ Q.rb(w).double()
+  else:
+    c, s = ops.quantize_pack(bf(w).to(gpu), 128, Q.INT4)
+    d.codes, d.scales, d.group, d.qtype = c.data_ptr(), s.data_ptr(), 128, Q.INT4
+    codes, scale = Q.quantize(w.numpy(), 128, Q.INT4)
+    wd = torch.from_numpy(Q.dequantize(codes, scale, 128, Q.INT4)).double()
+    ref_lg = x.double() @ wd
+  if r:
+    a, b = _lora(D, V, r, 163)
+    a_t, b_t = _pad_lora(a, b, r)
+    t = torch.zeros(M, r, dtype=torch.bfloat16, device=gpu)
+    ops.lora_down(gx, bf(a_t).to(gpu), t)
+    gb = bf(b_t).to(gpu)
+    d.lora_rank, d.t, d.t_ld, d.lora_b, d.lora_scale = r, t.data_ptr(), r, gb.data_ptr(), 2.0
+    ref_lg = ref_lg + 2.0 * (t.cpu().double() @ b.double())       # the kernel's own bf16 t
+    assert_bf16_close(t, Q.rb((x.double() @ a.double()).float()), what="t")
+  temperature = 0.9
+  d.temperature = temperature
+  nvb = ops.lmhead_nblocks(V)
+  part = torch.empty(M * nvb * 4, dtype=torch.float32, device=gpu)
+  pent = torch.empty(M * nvb, dtype=torch.float32, device=gpu)
+  best = torch.empty(M, dtype=torch.int32, device=gpu)
+  gt = targets.to(gpu)
+  d.targets, d.part, d.best_id = gt.data_ptr(), part.data_ptr(), best.data_ptr()
+  d.part_entropy = pent.data_ptr()
+  ref = ref_lg / temperature
+  ref_lp = torch.log_softmax(ref, -1)
+  want_t = torch.gather(ref_lp, -1, targets.long()[:, None])[:, 0]
+  want_ent = -(ref_lp.exp() * ref_lp).sum(-1)
+  errs = {}
+  for mode in (1, 0):
+    tlp, lse, ent, blp = (torch.empty(M, dtype=torch.float32, device=gpu) for _ in range(4))
+    d.target_logp, d.lse, d.entropy, d.best_logp = tlp.data_ptr(), lse.data_ptr(), ent.data_ptr(), blp.data_ptr()
+    d.logits_fp32 = mode
+    ops.lmhead(d)
+    torch.cuda.synchronize()
+    errs[mode] = (tlp.cpu().double() - want_t).abs().max().item()
+    if mode == 1:
+      assert errs[1] <= 1e-4, errs[1]
+      assert (lse.cpu().double() - torch.logsumexp(ref, -1)).abs().max().item() <= 1e-4
+      assert (ent.cpu().double() - want_ent).abs().max().item() <= 1e-4
+      top = ref.max(-1)
+      differs = best.cpu().long() != top.indices
+      gap = top.values - torch.gather(ref, -1, best.cpu().long()[:, None])[:, 0]
+      assert (gap[differs] <= 1e-4).all()
+      assert (blp.cpu().double() - (top.values - torch.logsumexp(ref, -1))).abs().max().item() <= 1e-4
+  assert errs[0] > 10 * errs[1]        # the bf16 logits of the normal mode are visibly coarser
+  assert errs[0] <= 2e-2
+
+
 def test_lmhead_forbidden_and_ties(gpu):
   """Equal maxima resolve to the lowest index; forbidden ids are never chosen."""
   from tunix_amd import _lib as L

@@ -72,7 +72,7 @@ class LmHeadDesc(C.Structure):
       ("target_logp", _p), ("lse", _p), ("logits_out", _p),
       ("part_entropy", _p), ("entropy", _p),
       ("part_draw", _p), ("draw_key0", C.c_uint32), ("draw_key1", C.c_uint32), ("draw_rng_variant", _i32),
-      ("draw_step_ptr", _p), ("draw_id", _p), ("draw_logp", _p),
+      ("draw_step_ptr", _p), ("draw_id", _p), ("draw_logp", _p), ("logits_fp32", _i32),
   ]
 
 

@@ -41,6 +41,7 @@ struct LHArgs {
   uint32_t key0, key1;
   int variant;
   const int32_t* step_ptr;
+  int logits_fp32;   // keep the fp32 accumulator as the logit (reference mode)
 };
 
 constexpr float kNegInf = -__builtin_inff();
@@ -133,7 +134,8 @@ __global__ __launch_bounds__(DENSE ? 512 : 256) void lmhead_kernel(const LHArgs 
       const int64_t row = m0 + rl;
       const bool rok = row < a.M;
       // logits are the bf16 einsum output cast to fp32, then divided by the temperature
-      const float ra = rbf(acc[mt][0][i]), rb_ = rbf(acc[mt][1][i]);
+      const float ra = a.logits_fp32 ? acc[mt][0][i] : rbf(acc[mt][0][i]);
+      const float rb_ = a.logits_fp32 ? acc[mt][1][i] : rbf(acc[mt][1][i]);
       const float la = okA ? __fdiv_rn(ra, a.temperature) : kNegInf;
       const float lb = okB ? __fdiv_rn(rb_, a.temperature) : kNegInf;
       if (a.logits_out && rok) {  // raw model logits: no temperature, no forbidden mask
@@ -329,6 +331,7 @@ extern "C" int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* d) {
   TNX_REQUIRE(!d->entropy || d->part_entropy, "lmhead: entropy needs the part_entropy workspace [M, n_vblocks]");
   a.part_ent = d->entropy ? d->part_entropy : nullptr;
   a.part_draw = nullptr; a.key0 = a.key1 = 0; a.variant = 0; a.step_ptr = nullptr;
+  a.logits_fp32 = d->logits_fp32 != 0;
   if (d->draw_id) {
     TNX_REQUIRE(d->part_draw && d->draw_step_ptr, "lmhead: the draw needs the part_draw workspace [M, n_vblocks, 3] and a step pointer");
     TNX_REQUIRE(d->draw_rng_variant == 0 || d->draw_rng_variant == 1, "lmhead: rng_variant must be 0 or 1");

@@ -612,7 +612,7 @@ extern "C" int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* d) {
 // the shape is not one the kernel takes (the caller then uses its own kernel), 0 when launched.
 int tnx_internal_wide_head(hipStream_t st, const tnx_lmhead_desc* d, float temperature, int64_t nvb,
                            float* part_ent) {
-  if (d->w_bf16 || d->logits_out || d->forbidden || d->draw_id) return 1;
+  if (d->w_bf16 || d->logits_out || d->forbidden || d->draw_id || d->logits_fp32) return 1;   // (its tile is staged in bf16)
   if (d->group < 32 || d->group % 32 != 0 || (d->group <= KTILE ? KTILE % d->group != 0 : d->group % KTILE != 0) ||
       d->D % d->group != 0)
     return 1;

@@ -564,7 +564,7 @@ class Runner:
 
   def head_desc(self, x, rows, part, temperature=1.0, targets=None, best_id=None, best_logp=None,
                 target_logp=None, lse=None, logits_out=None, forbidden=None, entropy=None,
-                part_entropy=None, draw=None) -> L.LmHeadDesc:
+                part_entropy=None, draw=None, logits_fp32=False) -> L.LmHeadDesc:
     cfg, m = self.cfg, self.model
     d = L.LmHeadDesc()
     d.M, d.D, d.V = rows, cfg.embed_dim, cfg.vocab_size
@@ -578,6 +578,7 @@ class Runner:
     else:
       d.w_bf16 = (m.head_w if m.head_w is not None else m.embed).data_ptr()
     d.temperature = float(temperature)
+    d.logits_fp32 = 1 if logits_fp32 else 0
     if forbidden is not None:
       d.forbidden, d.n_forbidden = forbidden.data_ptr(), forbidden.numel()
     for name, tns in (("targets", targets), ("best_id", best_id), ("best_logp", best_logp),

@@ -44,14 +44,16 @@ def process_ids(prompt_tokens: torch.Tensor, completion_tokens: torch.Tensor, pa
 def compute_per_token_logps(model: QLoRAModel, prompt_tokens, completion_tokens, pad_id: int,
                             eos_id: int | None = None, *, temperature: float = 1.0,
                             chunk_size: int = 0, return_entropy: bool = False,
-                            max_rows: int = 16384) -> torch.Tensor:
+                            max_rows: int = 16384, logits_fp32: bool = False) -> torch.Tensor:
   """fp32 [B, completion_len]: log p(completion token | everything before it).
 
   prompt_tokens [B, P] (left padded) and completion_tokens [B, T] (right padded) are integer
   arrays or tensors.  `temperature` divides the logits as in the reference (:431-436: ignored
   when 0 or 1).  `max_rows` bounds the token rows of one forward pass.  With return_entropy the
   result is (logps, entropy), entropy = -sum p log p of the same (temperature-scaled) logits
-  (compute_entropy_from_logits, :1136-1148), also from the fused head kernel.
+  (compute_entropy_from_logits, :1136-1148), also from the fused head kernel.  logits_fp32: the
+  head's fp32-accumulate reference mode (the logits keep their fp32 accumulators instead of being
+  rounded to bf16 as the reference's bf16 einsum output is).
   """
   dev = model.device
   pt = torch.as_tensor(np.asarray(prompt_tokens) if not isinstance(prompt_tokens, torch.Tensor)
@@ -100,7 +102,7 @@ def compute_per_token_logps(model: QLoRAModel, prompt_tokens, completion_tokens,
       if return_entropy:  # entropy of the temperature-scaled distribution (:479-481)
         kw = dict(entropy=ent[b0:b0 + nb].view(-1)[r0:r0 + nr], part_entropy=part_ent)
       runner.run_head(xs[r0:r0 + nr], nr, temperature=temp, targets=tg[r0:r0 + nr],
-                      target_logp=lp[r0:r0 + nr], **kw)
+                      target_logp=lp[r0:r0 + nr], logits_fp32=logits_fp32, **kw)
   return (out, ent) if return_entropy else out
 
 
