@@ -584,15 +584,17 @@ def main():
     # K steps in `groups` equal groups whose starting points are spread evenly from the step after
     # the warm-up to the end of the rollout.  The part of the rollout that is skipped must look
     # like a rollout to the kernels: the cache slots and token columns between the groups are
-    # filled with values of the kind a decode step writes (no pad ids: every key is attended).
+    # filled with values of the kind a decode step writes (copies of the prompt's keys and values,
+    # random non-pad token ids: every key is attended).
     groups = max(g for g in (8, 5, 4, 2, 1) if K % g == 0 and K // g >= 1)
     per = K // groups
     gen = torch.Generator(device=dev).manual_seed(20253)
     st.token_buffer[:, step_first + 1:] = torch.randint(1, cfg.vocab_size, (B, S - step_first - 1), generator=gen,
                                                         device=dev, dtype=torch.int32)
-    for kc, vc in zip(st.kcache, st.vcache):
-      kc[:, :, step_first + 1:].normal_(generator=gen)
-      vc[:, :, step_first + 1:].normal_(generator=gen)
+    n_fill = S - step_first - 1
+    for kc, vc in zip(st.kcache, st.vcache):   # keys / values of the kind the model writes: the prompt's own
+      kc[:, :, step_first + 1:] = kc[:, :, :n_fill]
+      vc[:, :, step_first + 1:] = vc[:, :, :n_fill]
     starts = [step_first + round(g * (last_step + 1 - per - step_first) / max(groups - 1, 1)) for g in range(groups)]
     dt, contexts = 0.0, []
     first_dt = None

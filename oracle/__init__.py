@@ -15,6 +15,10 @@ tree).  Pinning status of each part:
                  tests/rl/algo_core_test.py:51-143 (ratio == 1).
                  aggregate_loss (five modes, no packing segments) and WeightedMetric.compute:
                  pinned by the thirteen literal cases of tests/rl/common_test.py:457-576.
+                 aggregate_loss_segmented (packed batches, :857-940): pinned by the packed gate of
+                 tests/rl/algo_core_test.py:51-143 (-2.25, and -1.875 for the per-row form) and by
+                 the property that gate asserts -- packed equals unpacked -- run on the same
+                 thirteen literal cases.
                  sampler_trainer_agreement (grpo_learner.py:405-440; the reference holds no
                  vector for it): pinned by numpy.corrcoef / masked means and maxima over the
                  masked subset, and by the closed forms (equal inputs, a constant log offset,
@@ -22,7 +26,13 @@ tree).  Pinning status of each part:
   model_ref      RMSNorm / RoPE / GQA attention / SwiGLU / full decoder: pinned against
                  transformers' Qwen3 / Llama / Gemma3 / Qwen3Moe random-init models in fp32
                  (tol 1e-3, the equivalence tests/model_alignment/qwen_align_test.py:113-200
-                 asserts for the reference itself) and by brute-force fp64 attention.
+                 asserts for the reference itself) and by brute-force fp64 attention.  Where the
+                 bf16 mode rounds (the r() calls): pinned by tests/test_oracle_rounding.py, which
+                 writes each cited formula out again with real bf16 / fp32 tensors and jax's
+                 promotion rules, so that the dtypes do the rounding, and shows for every site
+                 that a moved or dropped rounding changes the result.  What stays unpinned
+                 there: the precision XLA keeps INSIDE one bf16 op (the accumulation order and
+                 width of a bf16 einsum or reduction), i.e. bit-exact agreement with XLA-CPU.
   quant_ref      int4 / NF4 group quantisation and the QArray arithmetic live in the third-party
                  package qwix (pyproject.toml:43 `qwix>=0.1.6`, not vendored, not installed):
                  PARITY UNPINNED against qwix.  The format is defined by include/tunix_hip.h;

@@ -7,7 +7,7 @@ original layout (counter array split in two halves); uniform / randint / gumbel 
 
 jax is not importable in this build, so this file is pinned by the golden arrays the
 reference's own tests hold for jax.random.PRNGKey(0) inputs (tests/rl/common_test.py:35-108);
-see tests/test_oracle_threefry.py for which layout reproduces them.
+see tests/test_oracle_rl.py (the threefry and golden-array tests) for which layout reproduces them.
 """
 from __future__ import annotations
 

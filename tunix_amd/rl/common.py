@@ -23,8 +23,10 @@ from ..model import QLoRAModel, Runner
 
 def selective_log_softmax(logits: torch.Tensor, input_ids: torch.Tensor) -> torch.Tensor:
   """log_softmax(logits)[..., input_ids] for logits that already exist as a tensor
-  (tunix/rl/common.py:187-203).  A convenience on device tensors; the rollout path itself
-  goes through the fused head kernel and never materialises logits."""
+  (tunix/rl/common.py:187-203).  A convenience for callers that already hold a logits tensor,
+  written with torch tensor methods: it is NOT one of this package's HIP kernels and nothing on
+  the rollout or log-probability path calls it (those go through the fused head kernel,
+  tnx_lmhead_logp, and never materialise logits)."""
   lg = logits.to(torch.float32)
   tgt = torch.gather(lg, -1, input_ids.long().unsqueeze(-1)).squeeze(-1)
   return tgt - torch.logsumexp(lg, dim=-1)
