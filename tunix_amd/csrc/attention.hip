@@ -123,13 +123,13 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
     for (int tt = 0; tt < 2; ++tt) {
       const uint32_t o = koff + kb_bytes + (uint32_t)(tt * 16 * DH * 2);
 #pragma unroll
-      for (int j = 0; j < KS; ++j) sg.kf[tt][j] = __builtin_amdgcn_raw_buffer_load_b128(rk, o + (uint32_t)(j * 64), 0, 0);
+      for (int j = 0; j < KS; ++j) sg.kf[tt][j] = __builtin_amdgcn_raw_buffer_load_b128(rk, o + (uint32_t)(j * 64), 0, kStreamOnce);
     }
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       const uint32_t o = voff + kb_bytes + (uint32_t)(((s < 4 ? s : 12 + s)) * DH * 2);
 #pragma unroll
-      for (int h = 0; h < NH; ++h) sg.vf[h][s] = __builtin_amdgcn_raw_buffer_load_b128(rv, o + (uint32_t)(h * 256), 0, 0);
+      for (int h = 0; h < NH; ++h) sg.vf[h][s] = __builtin_amdgcn_raw_buffer_load_b128(rv, o + (uint32_t)(h * 256), 0, kStreamOnce);
     }
     // token ids of this lane's 8 keys (two runs of 4 consecutive slots), fetched unconditionally
     // together with K and V: a predicated load per key would serialise eight memory latencies
