@@ -135,9 +135,10 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint64_t bytes) {
                                            0x00020000);
 }
 // Cache policy of buffer loads whose data is used exactly once per launch and by one wave (the
-// keys and values of attention, the packed weights of a GEMM): non-temporal, so that the stream
-// does not push what other waves re-read (activations, tables) out of L2.  Measured on the cold
-// KV cache of the 8B workload: 5.4 -> 6.0 TB/s at context 768.
+// keys and values of attention): non-temporal.  A flat read of this part runs at 7.1-7.3 TB/s
+// with it against 6.2-6.4 TB/s without; attention over cold caches 6.0 against 5.4 TB/s at
+// context 768.  (Measured and not adopted for the packed weights of the GEMM, 1 us slower per
+// launch, and for the head's weight rows, neutral.)
 constexpr int kStreamOnce = 2;   // the "nt" bit of the gfx940+ cache-policy operand
 __device__ __forceinline__ u32x4 buf_load128(rsrc_t r, uint32_t byte_off) {
   return __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
