@@ -82,6 +82,7 @@ __device__ __forceinline__ void unpack8(const u32x4& p, float (&f)[8]) {
 }
 // With `ws` the input row is bf16(sum of the split_k fp32 partial planes ws[z][row][:]) of a
 // split-k linear, added in split order: the linear's own finishing pass folded into the norm.
+template <int MAXC>
 __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, const uint16_t* res_pre,
                                                           uint16_t* h_out, const uint16_t* w,
                                                           const uint16_t* res_post, uint16_t* y,
@@ -91,14 +92,14 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
   __shared__ float red[4];
   const int64_t row = blockIdx.x;
   const int nchunks = (int)(D / 8);
-  float h[kNormMaxChunks][8];
+  float h[MAXC][8];
   float ss = 0.f;
   // Chunks are taken two at a time with every load of the pair issued before the first sum (up
   // to eight planes per chunk at once, further planes in groups of eight): the kernel is a few
   // dependent memory round trips long, and each group of loads that waits for the previous sum
   // adds one.  The sum itself stays in split order.
 #pragma unroll
-  for (int c0 = 0; c0 < kNormMaxChunks; c0 += 2) {
+  for (int c0 = 0; c0 < MAXC; c0 += 2) {
     if (c0 * 256 >= nchunks) break;   // uniform
     f32x4 p0[2][8], p1[2][8];
     u32x4 xin[2], rin[2];
@@ -178,9 +179,9 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
   }
   // the norm weights and the post-norm residual do not depend on the row statistics: fetch them
   // before the reduction instead of behind it
-  u32x4 wpre[kNormMaxChunks], rpost[kNormMaxChunks];
+  u32x4 wpre[MAXC], rpost[MAXC];
 #pragma unroll
-  for (int c = 0; c < kNormMaxChunks; ++c) {
+  for (int c = 0; c < MAXC; ++c) {
     const int ch = c * 256 + threadIdx.x;
     if (ch < nchunks) {
       wpre[c] = *reinterpret_cast<const u32x4*>(w + (int64_t)ch * 8);
@@ -191,7 +192,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
   const float ms = finish_ms(ss, (float)D, flavor);
   float ss2 = 0.f;
 #pragma unroll
-  for (int c = 0; c < kNormMaxChunks; ++c) {
+  for (int c = 0; c < MAXC; ++c) {
     const int ch = c * 256 + threadIdx.x;
     if (ch < nchunks) {
       const int64_t o = row * D + (int64_t)ch * 8;
@@ -225,7 +226,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
   ss2 = block_sum(ss2, red);
   const float ms2 = finish_ms(ss2, (float)D, flavor);
 #pragma unroll
-  for (int c = 0; c < kNormMaxChunks; ++c) {
+  for (int c = 0; c < MAXC; ++c) {
     const int ch = c * 256 + threadIdx.x;
     if (ch < nchunks) {
       float wv[8];
@@ -238,6 +239,16 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
       *reinterpret_cast<u32x4*>(y2 + row * D + (int64_t)ch * 8) = q;
     }
   }
+}
+
+// The kernel is unrolled over its chunks (256 threads x 8 elements each): instantiated for 2, 4
+// and 8 chunks per thread so that the common widths (D <= 4096) run the small instance -- the
+// code a wave walks through once is fetched cold at every launch.
+template <class... Args>
+void launch_rmsnorm_vec(hipStream_t st, int64_t M, int64_t D, Args... args) {
+  if (D <= 8 * 256 * 2) hipLaunchKernelGGL(rmsnorm_vec_kernel<2>, dim3((unsigned)M), dim3(256), 0, st, args...);
+  else if (D <= 8 * 256 * 4) hipLaunchKernelGGL(rmsnorm_vec_kernel<4>, dim3((unsigned)M), dim3(256), 0, st, args...);
+  else hipLaunchKernelGGL(rmsnorm_vec_kernel<kNormMaxChunks>, dim3((unsigned)M), dim3(256), 0, st, args...);
 }
 
 __global__ void embed_kernel(const uint16_t* table, int64_t V, int64_t D, const int32_t* ids,
@@ -411,9 +422,8 @@ extern "C" int tnx_rmsnorm(void* stream, const uint16_t* x, const uint16_t* res_
   TNX_REQUIRE(M > 0 && D > 0 && D <= 16384, "rmsnorm: D=%lld out of range (1..16384)", (long long)D);
   TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm: bad flavor %d", flavor);
   if (D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks)
-    hipLaunchKernelGGL(rmsnorm_vec_kernel, dim3((unsigned)M), dim3(256), 0, as_stream(stream), x, res_pre,
-                       h_out, w, res_post, y, D, eps, flavor, (const float*)nullptr, 0, (int64_t)0,
-                       (const uint16_t*)nullptr, (uint16_t*)nullptr);
+    launch_rmsnorm_vec(as_stream(stream), M, D, x, res_pre, h_out, w, res_post, y, D, eps, flavor,
+                       (const float*)nullptr, 0, (int64_t)0, (const uint16_t*)nullptr, (uint16_t*)nullptr);
   else
     hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)M), dim3(256), (size_t)D * sizeof(float),
                        as_stream(stream), x, res_pre, h_out, w, res_post, y, D, eps, flavor);
@@ -429,9 +439,8 @@ extern "C" int tnx_rmsnorm_splitk(void* stream, const float* ws, int split_k, co
   TNX_REQUIRE(M > 0 && D > 0 && D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks,
               "rmsnorm_splitk: D=%lld must be a multiple of 8 and <= 16384", (long long)D);
   TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm_splitk: bad flavor %d", flavor);
-  hipLaunchKernelGGL(rmsnorm_vec_kernel, dim3((unsigned)M), dim3(256), 0, as_stream(stream),
-                     (const uint16_t*)nullptr, res_pre, h_out, w, res_post, y, D, eps, flavor, ws, split_k,
-                     (int64_t)(M * D), (const uint16_t*)nullptr, (uint16_t*)nullptr);
+  launch_rmsnorm_vec(as_stream(stream), M, D, (const uint16_t*)nullptr, res_pre, h_out, w, res_post, y, D, eps,
+                     flavor, ws, split_k, (int64_t)(M * D), (const uint16_t*)nullptr, (uint16_t*)nullptr);
   TNX_CHECK_LAUNCH("rmsnorm_splitk");
   return TNX_OK;
 }
@@ -446,8 +455,8 @@ extern "C" int tnx_rmsnorm_pair(void* stream, const uint16_t* x, const float* ws
   TNX_REQUIRE(M > 0 && D > 0 && D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks,
               "rmsnorm_pair: D=%lld must be a multiple of 8 and <= 16384", (long long)D);
   TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm_pair: bad flavor %d", flavor);
-  hipLaunchKernelGGL(rmsnorm_vec_kernel, dim3((unsigned)M), dim3(256), 0, as_stream(stream), x, res_pre, h_out,
-                     w, res_post, y, D, eps, flavor, ws, ws ? split_k : 0, (int64_t)(M * D), w2, y2);
+  launch_rmsnorm_vec(as_stream(stream), M, D, x, res_pre, h_out, w, res_post, y, D, eps, flavor, ws,
+                     ws ? split_k : 0, (int64_t)(M * D), w2, y2);
   TNX_CHECK_LAUNCH("rmsnorm_pair");
   return TNX_OK;
 }
