@@ -11,6 +11,10 @@
 
 #include "common.h"
 
+#ifndef TNX_ATTN_NS
+#define TNX_ATTN_NS 2
+#endif
+
 namespace {
 
 struct AttnArgs {
@@ -39,11 +43,15 @@ struct AttnArgs {
 
 constexpr float kNegBig = -1.0e30f;
 
-template <int DH, bool FUSE>
+// FUSE: 0 = q comes rotated, keys and values are in the cache; 1 = the fused rotation and cache
+// write of a decode step (below), qkv taken from the finished output or from any number of
+// partial planes; 2 = the same from at most eight partial planes and at most four query heads per
+// kv head (one set of 3 x 64 lanes x 16 bytes per plane), all fetched in one round trip.
+template <int DH, int FUSE, bool TOKVEC>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2 : 1, DH > 128 ? 2 : 1))) void attn_kernel(const AttnArgs a) {
   constexpr int KS = DH / 32;                 // k-steps of the QK product
   constexpr int NH = DH > 128 ? DH / 128 : 1; // 128-column halves of V / O
-  constexpr int NS = DH > 128 ? 1 : 3;        // register stages of the key-block pipeline
+  constexpr int NS = DH > 128 ? 1 : TNX_ATTN_NS;        // register stages of the key-block pipeline
   const int lane = threadIdx.x, lm = lane & 15, lq = lane >> 4;
   const int chunk = blockIdx.x, hkv = blockIdx.y;
   const int PT = 16 / a.Gp;                              // positions per query tile
@@ -68,7 +76,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
     k_hi = min(k_hi, chunk * a.kv_chunk + a.kv_chunk - 1);
   }
 
-  constexpr bool fused = FUSE;                           // T == 1: c_n = col0 for every lane
+  constexpr bool fused = FUSE != 0;                         // T == 1: c_n = col0 for every lane
   u32x4 qf[KS];
 #pragma unroll
   for (int j = 0; j < KS; ++j) {
@@ -92,9 +100,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
   const uint16_t* vbase = a.v + ((b * a.Hkv + hkv) * a.S) * DH;
   const int32_t* tok = a.tokens + b * a.tok_ld;
   const int vcol = (8 * lm) % (DH < 128 ? DH : 128);     // DH=64: upper lanes duplicate
-  // 16-byte token loads need 16-byte aligned rows and whole groups of four slots (keys beyond
-  // the range are masked by the range test anyway)
-  const bool tok_vec = (a.tok_ld % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.tokens) & 15) == 0) && a.S % 4 == 0;
+  // TOKVEC: 16-byte token loads; the host chooses them when rows are 16-byte aligned and hold
+  // whole groups of four slots (keys beyond the range are masked by the range test anyway).  A
+  // compile-time choice: a branch around loads would make every wait behind it assume that the
+  // shorter side was taken.
 
   // A ring of NS register stages: the loads of the next NS-1 key blocks are in flight while a
   // block is computed, so the memory system is never left idle behind a wave's softmax and
@@ -133,7 +142,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
     }
     // token ids of this lane's 8 keys (two runs of 4 consecutive slots), fetched unconditionally
     // together with K and V: a predicated load per key would serialise eight memory latencies
-    if (tok_vec) {
+    if constexpr (TOKVEC) {
       const u32x4 t0 = __builtin_amdgcn_raw_buffer_load_b128(rtok, (uint32_t)(kb + 4 * lq) * 4u, 0, 0);
       const u32x4 t1 = __builtin_amdgcn_raw_buffer_load_b128(rtok, (uint32_t)(kb + 16 + 4 * lq) * 4u, 0, 0);
 #pragma unroll
@@ -219,10 +228,18 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
     const int kb0 = k_lo & ~31;
     const int kb_last = k_hi & ~31;
     const bool any = kb0 <= k_hi;
-    if (any) {
+    // (issued even when the key range is empty: a block outside the slab reads zeros, and an
+    // unconditional load keeps the counted waits behind it exact)
+    auto issue_stage = [&](int u) { load_block(min(kb0 + 32 * u, kb_last), sg[u]); };
+    auto issue_ring = [&]() {
 #pragma unroll
-      for (int u = 0; u < NS - 1; ++u) load_block(min(kb0 + 32 * u, kb_last), sg[u]);
-    }
+      for (int u = 0; u < NS - 1; ++u) issue_stage(u);
+    };
+    // Without the fused rotation the first key blocks are requested right away.  With it the
+    // partial planes of this step's q / k / v go first: a wave's loads return in order, so
+    // planes requested behind 32 KiB of keys and values would only be usable once those have
+    // arrived, and the rotation would start late instead of running while the blocks stream in.
+    if constexpr (!fused) issue_ring();
     // the step's own key / value wait in LDS while the cached keys stream through the registers
     __shared__ u32x4 park[FUSE ? KS + NH : 1][64];
     if constexpr (fused) {
@@ -253,32 +270,62 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
         // three turns of 64 lanes x 16 bytes at a time (one turn set covers G = 4), every load of
         // the set issued before the first sum: a set costs one memory round trip, not one per turn
         const int n4 = (a.G + 2) * (DH / 4);
-        for (int base = 0; base < n4; base += 192) {
-          if (a.qkv_ws && a.qkv_split <= 8) {
-            f32x4 p[3][8];
+        constexpr bool planes_first = FUSE == 2;   // (the host checks qkv_ws, qkv_split <= 8 and G <= 4)
+        // (called inside each of the two paths below, not behind their join: a use of the
+        // oldest loads after a join of paths with different load sequences waits for everything)
+        auto take_sincos = [&]() {
 #pragma unroll
-            for (int tsel = 0; tsel < 3; ++tsel) {
-              const int i4 = min(base + tsel * 64 + lane, n4 - 1);
-              const int hsel = i4 / (DH / 4), d = (i4 % (DH / 4)) * 4;
-              const int head = hsel < a.G ? hkv * a.G + hsel : (hsel == a.G ? a.Hq + hkv : a.Hq + a.Hkv + hkv);
-              const int64_t o = rowoff + (int64_t)head * DH + d;
+          for (int j = 0; j < KS / 2; ++j)
 #pragma unroll
-              for (int u = 0; u < 8; ++u)
-                p[tsel][u] = *reinterpret_cast<const f32x4*>(a.qkv_ws + (int64_t)min(u, a.qkv_split - 1) * plane + o);
+            for (int e = 0; e < 4; ++e) {
+              sn[j][e] = s0[j][e]; sn[j][4 + e] = s1[j][e];
+              cs[j][e] = c0[j][e]; cs[j][4 + e] = c1[j][e];
             }
+        };
+        auto load_planes = [&](int base, f32x4 (&p)[3][8]) {
 #pragma unroll
-            for (int tsel = 0; tsel < 3; ++tsel) {
-              const int i4 = base + tsel * 64 + lane;
-              if (i4 < n4) {
-                f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+          for (int tsel = 0; tsel < 3; ++tsel) {
+            const int i4 = min(base + tsel * 64 + lane, n4 - 1);
+            const int hsel = i4 / (DH / 4), d = (i4 % (DH / 4)) * 4;
+            const int head = hsel < a.G ? hkv * a.G + hsel : (hsel == a.G ? a.Hq + hkv : a.Hq + a.Hkv + hkv);
+            const int64_t o = rowoff + (int64_t)head * DH + d;
 #pragma unroll
-                for (int u = 0; u < 8; ++u)
-                  if (u < a.qkv_split) acc += p[tsel][u];
-                *reinterpret_cast<f32x4*>(&xs[i4 * 4]) = f32x4{rbf(acc[0]), rbf(acc[1]), rbf(acc[2]), rbf(acc[3])};
-              }
-            }
-          } else {
-            for (int i4 = base + lane; i4 < min(n4, base + 192); i4 += 64) {
+            for (int u = 0; u < 8; ++u)
+              p[tsel][u] = *reinterpret_cast<const f32x4*>(a.qkv_ws + (int64_t)min(u, a.qkv_split - 1) * plane + o);
+          }
+        };
+        auto sum_planes = [&](int base, const f32x4 (&p)[3][8]) {
+#pragma unroll
+          for (int tsel = 0; tsel < 3; ++tsel) {
+            const int i4 = base + tsel * 64 + lane;
+            f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+              if (u < a.qkv_split) acc += p[tsel][u];
+            if (i4 < n4) *reinterpret_cast<f32x4*>(&xs[i4 * 4]) = f32x4{rbf(acc[0]), rbf(acc[1]), rbf(acc[2]), rbf(acc[3])};
+          }
+        };
+        if constexpr (planes_first) {
+          // the plane set, then the first block of the key / value ring, then the sums:
+          // straight-line, so that the wait for the planes counts the ring's loads behind them
+          // (the second block of the ring follows once the planes' registers are free: with
+          // both in flight next to 24 plane vectors the ring would not get the registers it keeps
+          // in the loop, and moving a register that is still being loaded waits for the load)
+          f32x4 p[3][8];
+          load_planes(0, p);
+          __builtin_amdgcn_sched_barrier(0);
+          issue_stage(0);
+          __builtin_amdgcn_sched_barrier(0);
+          sum_planes(0, p);
+          take_sincos();
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int u = 1; u < NS - 1; ++u) issue_stage(u);
+          __builtin_amdgcn_sched_barrier(0);
+        } else {
+          issue_ring();
+          take_sincos();
+          for (int i4 = lane; i4 < n4; i4 += 64) {
               const int hsel = i4 / (DH / 4), d = (i4 % (DH / 4)) * 4;
               const int head = hsel < a.G ? hkv * a.G + hsel : (hsel == a.G ? a.Hq + hkv : a.Hq + a.Hkv + hkv);
               const int64_t o = rowoff + (int64_t)head * DH + d;
@@ -298,17 +345,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
                 acc = f32x4{bflo(q[0]), bfhi(q[0]), bflo(q[1]), bfhi(q[1])};
               }
               *reinterpret_cast<f32x4*>(&xs[i4 * 4]) = f32x4{rbf(acc[0]), rbf(acc[1]), rbf(acc[2]), rbf(acc[3])};
-            }
           }
         }
-#pragma unroll
-        for (int j = 0; j < KS / 2; ++j)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            sn[j][e] = s0[j][e]; sn[j][4 + e] = s1[j][e];
-            cs[j][e] = c0[j][e]; cs[j][4 + e] = c1[j][e];
-          }
-        __syncthreads();
+        // the work-group is this one wave: LDS executes a wave's accesses in order, so the staged
+        // values only need the compiler to keep the reads behind the writes (a work-group
+        // barrier would also wait for the key / value loads in flight)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
       }
       auto fetch8 = [&](int hsel, int d, float (&x)[8]) {
         const f32x4 v0 = *reinterpret_cast<const f32x4*>(&xs[hsel * DH + d]);
@@ -370,16 +414,24 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
       for (int h = 0; h < NH; ++h) park[KS + h][lane] = vn[h];
     }
     if (any) {
-      for (int kb = kb0; kb <= k_hi; kb += 32 * NS) {
+      // Whole turns of the ring without a branch inside (an exit in the middle of a turn makes
+      // the compiler merge the stages' registers on the exit edges, and a copy of a register
+      // that is still being loaded waits for everything in flight), then the last one or two
+      // blocks, whose loads were issued by the turn before them.
+      const int nblk = ((kb_last - kb0) >> 5) + 1;
+      int i = 0;
+      for (; i + NS <= nblk; i += NS) {
 #pragma unroll
         for (int u = 0; u < NS; ++u) {
-          const int kbu = kb + 32 * u;
-          if (kbu > k_hi) break;
+          const int kbu = kb0 + 32 * (i + u);
           load_block(min(kbu + 32 * (NS - 1), kb_last), sg[(u + NS - 1) % NS]);
           __builtin_amdgcn_sched_barrier(0);
           compute_block(kbu, sg[u]);
         }
       }
+#pragma unroll
+      for (int u = 0; u < NS - 1; ++u)
+        if (i + u < nblk) compute_block(kb0 + 32 * (i + u), sg[u]);
     }
     if (writer) {
       // the step's own key / value as a block of one key (at position col0) from registers
@@ -527,14 +579,22 @@ extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
   TNX_REQUIRE(d->B * QT <= 65535 * 32, "attn: too many query tiles");
   dim3 grid((unsigned)a.n_chunks, (unsigned)d->Hkv, (unsigned)(d->B * QT));
   hipStream_t st = as_stream(stream);
+  const bool tv = (d->tok_ld % 4 == 0) && ((reinterpret_cast<uintptr_t>(d->tokens) & 15) == 0) && d->S % 4 == 0;
+#define TNX_ATTN_LAUNCH(DH, FUSE)                                                                \
+  do {                                                                                           \
+    if (tv) hipLaunchKernelGGL((attn_kernel<DH, FUSE, true>), grid, dim3(64), 0, st, a);         \
+    else hipLaunchKernelGGL((attn_kernel<DH, FUSE, false>), grid, dim3(64), 0, st, a);           \
+  } while (0)
   switch (d->dh) {
-    case 64: hipLaunchKernelGGL((attn_kernel<64, false>), grid, dim3(64), 0, st, a); break;
+    case 64: TNX_ATTN_LAUNCH(64, 0); break;
     case 128:
-      if (a.rope_sin) hipLaunchKernelGGL((attn_kernel<128, true>), grid, dim3(64), 0, st, a);
-      else hipLaunchKernelGGL((attn_kernel<128, false>), grid, dim3(64), 0, st, a);
+      if (a.rope_sin && a.qkv_ws && a.qkv_split <= 8 && G <= 4) TNX_ATTN_LAUNCH(128, 2);
+      else if (a.rope_sin) TNX_ATTN_LAUNCH(128, 1);
+      else TNX_ATTN_LAUNCH(128, 0);
       break;
-    default: hipLaunchKernelGGL((attn_kernel<256, false>), grid, dim3(64), 0, st, a); break;
+    default: TNX_ATTN_LAUNCH(256, 0); break;
   }
+#undef TNX_ATTN_LAUNCH
   TNX_CHECK_LAUNCH("gqa_attn");
   if (a.n_chunks > 1) {
     const int64_t nq = d->B * d->T * d->Hq;

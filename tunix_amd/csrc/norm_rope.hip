@@ -82,11 +82,11 @@ __device__ __forceinline__ void unpack8(const u32x4& p, float (&f)[8]) {
 }
 // With `ws` the input row is bf16(sum of the split_k fp32 partial planes ws[z][row][:]) of a
 // split-k linear, added in split order: the linear's own finishing pass folded into the norm.
-template <int MAXC>
+template <int MAXC, int FLAVOR, bool PLANES>
 __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, const uint16_t* res_pre,
                                                           uint16_t* h_out, const uint16_t* w,
                                                           const uint16_t* res_post, uint16_t* y,
-                                                          int64_t D, float eps, int flavor,
+                                                          int64_t D, float eps, int /*flavor*/,
                                                           const float* ws, int split_k, int64_t plane,
                                                           const uint16_t* w2, uint16_t* y2) {
   __shared__ float red[4];
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
     for (int cc = 0; cc < 2; ++cc) {
       const int ch = (c0 + cc) * 256 + threadIdx.x;
       const int64_t o = row * D + (int64_t)min(ch, nchunks - 1) * 8;
-      if (ws) {
+      if (PLANES) {
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
           const int64_t zo = (int64_t)min(u, split_k - 1) * plane + o;
@@ -125,7 +125,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
       const int ch = c * 256 + threadIdx.x;
       if (ch < nchunks) {
         const int64_t o = row * D + (int64_t)ch * 8;
-        if (ws) {
+        if (PLANES) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) h[c][j] = 0.f;
 #pragma unroll
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
           *reinterpret_cast<u32x4*>(h_out + o) = q;
         }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) ss += sq_term(h[c][j], flavor);
+        for (int j = 0; j < 8; ++j) ss += sq_term(h[c][j], FLAVOR);
       }
     }
   }
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
     }
   }
   ss = block_sum(ss, red);
-  const float ms = finish_ms(ss, (float)D, flavor);
+  const float ms = finish_ms(ss, (float)D, FLAVOR);
   float ss2 = 0.f;
 #pragma unroll
   for (int c = 0; c < MAXC; ++c) {
@@ -199,7 +199,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
       float wv[8], v[8];
       unpack8(wpre[c], wv);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) v[j] = norm_elem(h[c][j], wv[j], ms, eps, flavor);
+      for (int j = 0; j < 8; ++j) v[j] = norm_elem(h[c][j], wv[j], ms, eps, FLAVOR);
       if (res_post) {
         float r[8];
         // (a residual that this launch itself rewrote as h_out is read back here, after the write)
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           h[c][j] = rbf(v[j]);
-          ss2 += sq_term(h[c][j], flavor);
+          ss2 += sq_term(h[c][j], FLAVOR);
         }
       }
     }
@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
   // y2 = norm(y) with its own weight, the row still in registers (same thread -> chunk map and
   // reduction order as a launch of its own would use: the results are identical)
   ss2 = block_sum(ss2, red);
-  const float ms2 = finish_ms(ss2, (float)D, flavor);
+  const float ms2 = finish_ms(ss2, (float)D, FLAVOR);
 #pragma unroll
   for (int c = 0; c < MAXC; ++c) {
     const int ch = c * 256 + threadIdx.x;
@@ -234,8 +234,8 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
       u32x4 q;
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        q[j] = pack2bf(norm_elem(h[c][2 * j], wv[2 * j], ms2, eps, flavor),
-                       norm_elem(h[c][2 * j + 1], wv[2 * j + 1], ms2, eps, flavor));
+        q[j] = pack2bf(norm_elem(h[c][2 * j], wv[2 * j], ms2, eps, FLAVOR),
+                       norm_elem(h[c][2 * j + 1], wv[2 * j + 1], ms2, eps, FLAVOR));
       *reinterpret_cast<u32x4*>(y2 + row * D + (int64_t)ch * 8) = q;
     }
   }
@@ -244,11 +244,21 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
 // The kernel is unrolled over its chunks (256 threads x 8 elements each): instantiated for 2, 4
 // and 8 chunks per thread so that the common widths (D <= 4096) run the small instance -- the
 // code a wave walks through once is fetched cold at every launch.
+template <int MAXC, class... Args>
+void launch_rmsnorm_vec_c(hipStream_t st, int64_t M, int flavor, bool planes, Args... args) {
+#define TNX_NORM_CASE(F)                                                                                   \
+  if (planes) hipLaunchKernelGGL((rmsnorm_vec_kernel<MAXC, F, true>), dim3((unsigned)M), dim3(256), 0, st, args...); \
+  else hipLaunchKernelGGL((rmsnorm_vec_kernel<MAXC, F, false>), dim3((unsigned)M), dim3(256), 0, st, args...)
+  if (flavor == TNX_NORM_LLAMA) { TNX_NORM_CASE(TNX_NORM_LLAMA); }
+  else if (flavor == TNX_NORM_QWEN3) { TNX_NORM_CASE(TNX_NORM_QWEN3); }
+  else { TNX_NORM_CASE(TNX_NORM_GEMMA3); }
+#undef TNX_NORM_CASE
+}
 template <class... Args>
-void launch_rmsnorm_vec(hipStream_t st, int64_t M, int64_t D, Args... args) {
-  if (D <= 8 * 256 * 2) hipLaunchKernelGGL(rmsnorm_vec_kernel<2>, dim3((unsigned)M), dim3(256), 0, st, args...);
-  else if (D <= 8 * 256 * 4) hipLaunchKernelGGL(rmsnorm_vec_kernel<4>, dim3((unsigned)M), dim3(256), 0, st, args...);
-  else hipLaunchKernelGGL(rmsnorm_vec_kernel<kNormMaxChunks>, dim3((unsigned)M), dim3(256), 0, st, args...);
+void launch_rmsnorm_vec(hipStream_t st, int64_t M, int64_t D, int flavor, bool planes, Args... args) {
+  if (D <= 8 * 256 * 2) launch_rmsnorm_vec_c<2>(st, M, flavor, planes, args...);
+  else if (D <= 8 * 256 * 4) launch_rmsnorm_vec_c<4>(st, M, flavor, planes, args...);
+  else launch_rmsnorm_vec_c<kNormMaxChunks>(st, M, flavor, planes, args...);
 }
 
 __global__ void embed_kernel(const uint16_t* table, int64_t V, int64_t D, const int32_t* ids,
@@ -422,7 +432,7 @@ extern "C" int tnx_rmsnorm(void* stream, const uint16_t* x, const uint16_t* res_
   TNX_REQUIRE(M > 0 && D > 0 && D <= 16384, "rmsnorm: D=%lld out of range (1..16384)", (long long)D);
   TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm: bad flavor %d", flavor);
   if (D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks)
-    launch_rmsnorm_vec(as_stream(stream), M, D, x, res_pre, h_out, w, res_post, y, D, eps, flavor,
+    launch_rmsnorm_vec(as_stream(stream), M, D, flavor, false, x, res_pre, h_out, w, res_post, y, D, eps, flavor,
                        (const float*)nullptr, 0, (int64_t)0, (const uint16_t*)nullptr, (uint16_t*)nullptr);
   else
     hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)M), dim3(256), (size_t)D * sizeof(float),
@@ -439,7 +449,7 @@ extern "C" int tnx_rmsnorm_splitk(void* stream, const float* ws, int split_k, co
   TNX_REQUIRE(M > 0 && D > 0 && D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks,
               "rmsnorm_splitk: D=%lld must be a multiple of 8 and <= 16384", (long long)D);
   TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm_splitk: bad flavor %d", flavor);
-  launch_rmsnorm_vec(as_stream(stream), M, D, (const uint16_t*)nullptr, res_pre, h_out, w, res_post, y, D, eps,
+  launch_rmsnorm_vec(as_stream(stream), M, D, flavor, true, (const uint16_t*)nullptr, res_pre, h_out, w, res_post, y, D, eps,
                      flavor, ws, split_k, (int64_t)(M * D), (const uint16_t*)nullptr, (uint16_t*)nullptr);
   TNX_CHECK_LAUNCH("rmsnorm_splitk");
   return TNX_OK;
@@ -455,7 +465,7 @@ extern "C" int tnx_rmsnorm_pair(void* stream, const uint16_t* x, const float* ws
   TNX_REQUIRE(M > 0 && D > 0 && D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks,
               "rmsnorm_pair: D=%lld must be a multiple of 8 and <= 16384", (long long)D);
   TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm_pair: bad flavor %d", flavor);
-  launch_rmsnorm_vec(as_stream(stream), M, D, x, res_pre, h_out, w, res_post, y, D, eps, flavor, ws,
+  launch_rmsnorm_vec(as_stream(stream), M, D, flavor, ws != nullptr, x, res_pre, h_out, w, res_post, y, D, eps, flavor, ws,
                      ws ? split_k : 0, (int64_t)(M * D), w2, y2);
   TNX_CHECK_LAUNCH("rmsnorm_pair");
   return TNX_OK;
