@@ -303,6 +303,31 @@ def summarize_step_trace(path):
     print(f"| {name:34s} | {n:5d} | {busy / 1e3:8.1f} | {busy / n / 1e3:7.2f} | {span / n / 1e3:22.2f} |")
 
 
+def summarize_counters(path):
+  """Prints, per kernel, the mean of every counter in a `rocprofv3 --pmc ...` counter-collection
+  csv of this script (one row per dispatch and counter), and, where the counters are there, the
+  L1 -> L2 read latency per request and the address-translation miss rate."""
+  import collections
+  import csv
+  import re
+  agg = collections.defaultdict(lambda: collections.defaultdict(list))
+  for row in csv.DictReader(open(path)):
+    name = row["Kernel_Name"].replace("(anonymous namespace)::", "")
+    m = re.search(r"([A-Za-z_0-9]+(<[^(]*>)?)\(", name)
+    agg[(m.group(1) if m else name)[:48]][row["Counter_Name"]].append(float(row["Counter_Value"]))
+  for name, counters in sorted(agg.items()):
+    mean = {c: sum(v) / len(v) for c, v in counters.items()}
+    n = max(len(v) for v in counters.values())
+    line = f"{name:48s} dispatches {n:5d}  " + "  ".join(f"{c} {v:.0f}" for c, v in sorted(mean.items()))
+    req, lat = mean.get("TCP_TCC_READ_REQ_sum"), mean.get("TCP_TCC_READ_REQ_LATENCY_sum")
+    if req and lat is not None:
+      line += f"  | {lat / req:.0f} cycles per read request"
+    hit, miss = mean.get("TCP_UTCL1_TRANSLATION_HIT_sum"), mean.get("TCP_UTCL1_TRANSLATION_MISS_sum")
+    if hit is not None and miss is not None and hit + miss > 0:
+      line += f"  | translation miss rate {miss / (hit + miss):.4%}"
+    print(line)
+
+
 def fused_logps_workload(rows, chunk, iters):
   """The standalone per-token log-probability case at training scale: hidden states
   [rows, 4096] bf16 N(0,1) x an int4 (group 128) + LoRA r64 lm_head of 128256 columns ->
@@ -454,6 +479,8 @@ def main():
                        "rollout's context range")
   ap.add_argument("--summarize-trace", metavar="CSV", default=None,
                   help="no GPU work: tabulate one decode step of a rocprofv3 kernel-trace csv of this script")
+  ap.add_argument("--summarize-counters", metavar="CSV", default=None,
+                  help="no GPU work: per-kernel means of a rocprofv3 --pmc counter-collection csv of this script")
   args = ap.parse_args()
   if args.fused_logps:
     if args.gpus != 1:
@@ -462,6 +489,9 @@ def main():
     return
   if args.summarize_trace:
     summarize_step_trace(args.summarize_trace)
+    return
+  if args.summarize_counters:
+    summarize_counters(args.summarize_counters)
     return
   if args.gpus != 1:
     print("bench.py measures one GPU: this build has no multi-GPU path (the decode path shards "
