@@ -73,12 +73,17 @@ __device__ __forceinline__ Stat merge(const Stat& a, const Stat& b) {
   return r;
 }
 
-// The dense (bf16 weight) flavour is latency bound on its weight stream: it needs no code-book
-// table, so its LDS footprint lets two work-groups share a compute unit, and the launch bound
-// (a register budget, the work-group size is always 256) keeps it within half the register file.
-template <int MT, bool DENSE>
-__global__ __launch_bounds__(DENSE ? 512 : 256) void lmhead_kernel(const LHArgs a) {
-  constexpr int NT = 2;
+// A work-group covers 16 * MT rows x 64 * NT columns = NT / 2 statistics blocks of 128 columns.
+// NT = 2 everywhere today.  The dense (bf16 weight) flavour is bound by what a compute unit can
+// fetch; it needs no code-book table, so its LDS footprint lets two work-groups share a compute
+// unit, and the launch bound (a register budget, the work-group size is always 256) keeps it
+// within half the register file.  NT = 4 for the dense flavour (256 columns: half the activation
+// re-reads per weight byte, one work-group of four waves per unit with its accumulators in AGPRs)
+// was measured at 376 us against 312 us for the Llama-3.1-8B head at 128 rows: two independent
+// four-wave groups hide each other's barrier and load waits, one group waits together.
+template <int MT, int NT, bool DENSE>
+__global__ __launch_bounds__(DENSE && NT == 2 ? 512 : 256) void lmhead_kernel(const LHArgs a) {
+  static_assert(NT == 2 || NT == 4, "one or two 128-column statistics blocks per work-group");
   extern __shared__ __align__(16) unsigned char smem[];
   uint16_t* sA = reinterpret_cast<uint16_t*>(smem);
   uint32_t* sLut = tile_lut(smem, MT);
@@ -107,18 +112,27 @@ __global__ __launch_bounds__(DENSE ? 512 : 256) void lmhead_kernel(const LHArgs 
     for (int nt = 0; nt < NT; ++nt) zero_acc(acc[mt][nt]);
   tile_mainloop<MT, NT, DENSE>(s, m0, ntile0, 0, (int)(a.D / KTILE), sA, lut_lane, acc);
   if (a.lora_rank > 0) {
-    int toff[NT] = {0, 0};
+    int toff[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) toff[nt] = 0;
     tile_lora<MT, NT>(s, m0, ntile0, toff, acc);
   }
 
   __syncthreads();  // sA is reused for the cross-wave reduction
   Stat* sRed = reinterpret_cast<Stat*>(smem);  // [4 waves][16*MT rows]
-  const int64_t colA = (ntile0 + 0) * 16 + lm, colB = (ntile0 + 1) * 16 + lm;
-  bool okA = (ntile0 + 0) < s.ntiles, okB = (ntile0 + 1) < s.ntiles;
+  int64_t col[NT];
+  bool ok[NT], in_v[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    col[nt] = (ntile0 + nt) * 16 + lm;
+    in_v[nt] = (ntile0 + nt) < s.ntiles;
+    ok[nt] = in_v[nt];
+  }
   for (int f = 0; f < a.n_forbidden; ++f) {
     const int64_t fid = a.forbidden[f];
-    if (fid == colA) okA = false;
-    if (fid == colB) okB = false;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+      if (fid == col[nt]) ok[nt] = false;
   }
   // fold_in(key, step) for the draw: threefry of the key over the counter pair (0, step)
   uint32_t ks0 = 0u, ks1 = 0u;
@@ -134,22 +148,30 @@ __global__ __launch_bounds__(DENSE ? 512 : 256) void lmhead_kernel(const LHArgs 
       const int64_t row = m0 + rl;
       const bool rok = row < a.M;
       // logits are the bf16 einsum output cast to fp32, then divided by the temperature
-      const float ra = a.logits_fp32 ? acc[mt][0][i] : rbf(acc[mt][0][i]);
-      const float rb_ = a.logits_fp32 ? acc[mt][1][i] : rbf(acc[mt][1][i]);
-      const float la = okA ? __fdiv_rn(ra, a.temperature) : kNegInf;
-      const float lb = okB ? __fdiv_rn(rb_, a.temperature) : kNegInf;
-      if (a.logits_out && rok) {  // raw model logits: no temperature, no forbidden mask
-        if ((ntile0 + 0) < s.ntiles) a.logits_out[row * a.V + colA] = ra;
-        if ((ntile0 + 1) < s.ntiles) a.logits_out[row * a.V + colB] = rb_;
+      float raw[NT], l[NT];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        raw[nt] = a.logits_fp32 ? acc[mt][nt][i] : rbf(acc[mt][nt][i]);
+        l[nt] = ok[nt] ? __fdiv_rn(raw[nt], a.temperature) : kNegInf;
       }
-      Stat st;
-      st.mx = fmaxf(la, lb);
-      st.idx = (lb > la) ? (int)colB : (int)colA;
+      if (a.logits_out && rok) {  // raw model logits: no temperature, no forbidden mask
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          if (in_v[nt]) a.logits_out[row * a.V + col[nt]] = raw[nt];
+      }
       const int tg = (a.targets && rok) ? a.targets[row] : -1;
-      st.tgt = tg == (int)colA ? la : (tg == (int)colB ? lb : kNegInf);
+      // this lane's columns grow with nt: the first maximum wins
+      float mx = l[0], tgt = tg == (int)col[0] ? l[0] : kNegInf;
+      int idx = (int)col[0];
+#pragma unroll
+      for (int nt = 1; nt < NT; ++nt) {
+        if (l[nt] > mx) {
+          mx = l[nt];
+          idx = (int)col[nt];
+        }
+        if (tg == (int)col[nt]) tgt = l[nt];
+      }
       // arg-max over the 16 lanes of the row (columns grow with lm)
-      float mx = st.mx;
-      int idx = st.idx;
 #pragma unroll
       for (int o = 1; o < 16; o <<= 1) {
         const float omx = __shfl_xor(mx, o, 64);
@@ -158,33 +180,38 @@ __global__ __launch_bounds__(DENSE ? 512 : 256) void lmhead_kernel(const LHArgs 
           mx = omx;
           idx = oidx;
         }
-        st.tgt = fmaxf(st.tgt, __shfl_xor(st.tgt, o, 64));
+        tgt = fmaxf(tgt, __shfl_xor(tgt, o, 64));
       }
       float se = 0.f, we = 0.f;
       if (mx != kNegInf) {
-        const float ea = la == kNegInf ? 0.f : __expf(la - mx), eb = lb == kNegInf ? 0.f : __expf(lb - mx);
-        se = ea + eb;
-        we = (la == kNegInf ? 0.f : ea * la) + (lb == kNegInf ? 0.f : eb * lb);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          const float e = l[nt] == kNegInf ? 0.f : __expf(l[nt] - mx);
+          se += e;
+          we += l[nt] == kNegInf ? 0.f : e * l[nt];
+        }
       }
 #pragma unroll
       for (int o = 1; o < 16; o <<= 1) {
         se += __shfl_xor(se, o, 64);
         we += __shfl_xor(we, o, 64);
       }
-      // the draw: arg-max of logit + gumbel noise over the 32 columns of this row in the wave
+      // the draw: arg-max of logit + gumbel noise over this row's columns in the wave
       // (noise of element (row, v): counter row * V + v of M * V, one draw over [M, V])
       float gv = kNegInf, gl = kNegInf;
       int gi = 0x7fffffff;
       if (a.part_draw && rok) {
         const uint64_t tot = (uint64_t)a.M * (uint64_t)a.V;
-        const float na = la == kNegInf ? kNegInf
-            : la + gumbel_from_bits(random_bits(ks0, ks1, (uint64_t)row * a.V + colA, tot, a.variant));
-        const float nb = lb == kNegInf ? kNegInf
-            : lb + gumbel_from_bits(random_bits(ks0, ks1, (uint64_t)row * a.V + colB, tot, a.variant));
-        const bool tb = nb > na;   // colA < colB: ties keep the lower column
-        gv = tb ? nb : na;
-        gi = tb ? (int)colB : (int)colA;
-        gl = tb ? lb : la;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          const float n = l[nt] == kNegInf ? kNegInf
+              : l[nt] + gumbel_from_bits(random_bits(ks0, ks1, (uint64_t)row * a.V + col[nt], tot, a.variant));
+          if (n > gv) {   // columns grow with nt: ties keep the lower column
+            gv = n;
+            gi = (int)col[nt];
+            gl = l[nt];
+          }
+        }
 #pragma unroll
         for (int o = 1; o < 16; o <<= 1) {
           const float ov = __shfl_xor(gv, o, 64), ol = __shfl_xor(gl, o, 64);
@@ -198,7 +225,7 @@ __global__ __launch_bounds__(DENSE ? 512 : 256) void lmhead_kernel(const LHArgs 
       }
       if (lm == 0) {
         Stat r;
-        r.mx = mx; r.idx = idx; r.sum = se; r.tgt = st.tgt; r.wsum = we;
+        r.mx = mx; r.idx = idx; r.sum = se; r.tgt = tgt; r.wsum = we;
         r.gv = gv; r.gi = gi; r.gl = gl;
         sRed[wave * (MT * 16) + rl] = r;
       }
@@ -208,17 +235,29 @@ __global__ __launch_bounds__(DENSE ? 512 : 256) void lmhead_kernel(const LHArgs 
     Stat r = sRed[tid];
 #pragma unroll
     for (int w = 1; w < 4; ++w) r = merge(r, sRed[w * (MT * 16) + tid]);
-    float* p = a.part + ((m0 + tid) * a.nvb + vb) * 4;
-    p[0] = r.mx;
-    p[1] = __int_as_float(r.idx);
-    p[2] = r.sum;
-    p[3] = r.tgt;
-    if (a.part_ent) a.part_ent[(m0 + tid) * a.nvb + vb] = r.wsum;
-    if (a.part_draw) {
-      float* q = a.part_draw + ((m0 + tid) * a.nvb + vb) * 3;
-      q[0] = r.gv;
-      q[1] = __int_as_float(r.gi);
-      q[2] = r.gl;
+    // the work-group's statistics go to its first 128-column block; its other blocks (NT = 4)
+    // get the neutral element, so the merging pass and the workspace layout do not change
+    constexpr int BPW = NT / 2;
+#pragma unroll
+    for (int k = 0; k < BPW; ++k) {
+      const int64_t pb = vb * BPW + k;
+      if (pb >= a.nvb) break;
+      if (k == 1) {
+        r.mx = kNegInf; r.idx = 0x7fffffff; r.sum = 0.f; r.tgt = kNegInf; r.wsum = 0.f;
+        r.gv = kNegInf; r.gi = 0x7fffffff; r.gl = kNegInf;
+      }
+      float* p = a.part + ((m0 + tid) * a.nvb + pb) * 4;
+      p[0] = r.mx;
+      p[1] = __int_as_float(r.idx);
+      p[2] = r.sum;
+      p[3] = r.tgt;
+      if (a.part_ent) a.part_ent[(m0 + tid) * a.nvb + pb] = r.wsum;
+      if (a.part_draw) {
+        float* q = a.part_draw + ((m0 + tid) * a.nvb + pb) * 3;
+        q[0] = r.gv;
+        q[1] = __int_as_float(r.gi);
+        q[2] = r.gl;
+      }
     }
   }
 }
@@ -287,13 +326,15 @@ int raise_lds_limit(Kern kern, size_t bytes) {
 
 template <int MT, bool DENSE>
 int launch_lmhead(hipStream_t st, const LHArgs& a) {
+  constexpr int NT = 2;
   static std::once_flag once;
   static int attr_rc = TNX_OK;
   constexpr size_t kLds = DENSE ? 2 * (size_t)MT * 16 * A_LD * sizeof(uint16_t) : tile_smem_bytes(MT);
-  std::call_once(once, [] { attr_rc = raise_lds_limit(&lmhead_kernel<MT, DENSE>, kLds); });
+  static_assert(kLds >= 4 * (size_t)MT * 16 * sizeof(Stat), "the statistics exchange reuses the activation buffers");
+  std::call_once(once, [] { attr_rc = raise_lds_limit(&lmhead_kernel<MT, NT, DENSE>, kLds); });
   if (attr_rc) return attr_rc;
-  dim3 grid((unsigned)a.nvb, (unsigned)cdiv(a.M, MT * 16));
-  hipLaunchKernelGGL((lmhead_kernel<MT, DENSE>), grid, dim3(256), kLds, st, a);
+  dim3 grid((unsigned)cdiv(a.nvb, NT / 2), (unsigned)cdiv(a.M, MT * 16));
+  hipLaunchKernelGGL((lmhead_kernel<MT, NT, DENSE>), grid, dim3(256), kLds, st, a);
   TNX_CHECK_LAUNCH("lmhead");
   return TNX_OK;
 }
