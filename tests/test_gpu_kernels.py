@@ -374,6 +374,39 @@ def test_rmsnorm_flavours(gpu, family):
   assert_bf16_close(y2, ref2, min_equal=0.95, what=f"rmsnorm+residual {family}")
 
 
+@pytest.mark.parametrize("family,D,split", [("llama3", 5120, 3), ("qwen3", 9216, 2), ("gemma3", 16384, 1),
+                                            ("llama3", 4096, 11), ("gemma3", 1152, 9)])
+def test_rmsnorm_wide_rows_and_many_planes(gpu, family, D, split):
+  """The instances of the vector norm for 4 and 8 chunks per thread (rows wider than 4096) and
+  the path for more than eight partial planes: a bf16 row against the oracle, and the same row
+  handed over as `split` fp32 planes (summed in split order, rounded to bf16) bit-equal to it."""
+  from tunix_amd import ops
+  from tunix_amd.model import _NORM
+  M = 5
+  eps = 1e-6 if family == "gemma3" else 1e-5
+  g = torch.Generator().manual_seed(300 + D + split)
+  planes = torch.randn(split, M, D, generator=g) * (1.5 / split ** 0.5)
+  acc = torch.zeros(M, D)
+  for z in range(split):
+    acc = acc + planes[z]
+  x = Q.rb(acc)
+  res = rnd((M, D), 301)
+  w = Q.rb(rnd((D,), 302, 0.5) + (0.0 if family == "gemma3" else 1.0))
+  ref_m = MR.RefModel.__new__(MR.RefModel)
+  ref_m.cfg, ref_m.bf16 = _Cfg(family, eps), True
+  h = Q.rb(x + res)
+  ref = ref_m.rmsnorm(h, w)
+  y1, h1 = (torch.empty(M, D, dtype=torch.bfloat16, device=gpu) for _ in range(2))
+  ops.rmsnorm(bf(x).to(gpu), bf(w).to(gpu), y1, eps, _NORM[family], res_pre=bf(res).to(gpu), h_out=h1)
+  assert torch.equal(h1.float().cpu(), h)
+  assert_bf16_close(y1, ref, min_equal=0.95, what=f"rmsnorm {family} D={D}")
+  y2, h2 = torch.empty_like(y1), bf(res).to(gpu)
+  ops.rmsnorm_splitk(planes.to(gpu).contiguous().view(-1), split, bf(w).to(gpu), y2, eps, _NORM[family], M, D,
+                     res_pre=h2, h_out=h2)
+  torch.cuda.synchronize()
+  assert torch.equal(h1, h2) and torch.equal(y1, y2)
+
+
 @pytest.mark.parametrize("family,dh,Hq,Hkv", [("llama3", 128, 8, 2), ("qwen3", 64, 8, 2),
                                                ("gemma3", 256, 4, 1)])
 def test_rope_kvwrite(gpu, family, dh, Hq, Hkv):
