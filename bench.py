@@ -205,6 +205,66 @@ def measured_traffic():
           "read": int(prof["read_bytes_per_launch"]), "write": int(prof["write_bytes_per_launch"])}
 
 
+def write_traffic_profile(fetch_csv, write_csv):
+  """Rebuilds the tracked traffic record from two `rocprofv3 --pmc` runs of
+  `bench.py --kernels-only` (FETCH_SIZE in one, WRITE_SIZE in the other; KiB per dispatch).  The
+  GEMM's dispatches come in four runs, in the order the breakdown launches them (qkv, o, gate|up,
+  down); the 1 GiB `stream_read_kernel` launches of the same runs give the scale of FETCH_SIZE
+  for the 8- / 16-byte-per-lane buffer loads every streaming kernel here uses, a 1002 MiB torch
+  copy the scale of both counters for plain copies."""
+  import csv
+
+  def runs(path, counter):
+    rows = [r for r in csv.DictReader(open(path)) if r["Counter_Name"] == counter]
+    rows.sort(key=lambda r: int(r["Dispatch_Id"]))
+    gemm, stream, copy = [], {}, []
+    for r in rows:
+      name, grid, val = r["Kernel_Name"], r.get("Grid_Size", "?"), float(r["Counter_Value"])
+      if "qgemm128_kernel" in name:
+        if gemm and gemm[-1][0] == grid:
+          gemm[-1][1].append(val)
+        else:
+          gemm.append((grid, [val]))
+      elif "stream_read_kernel" in name:
+        stream.setdefault("stream_read_kernel<16>" if "<16>" in name else "stream_read_kernel<8>", []).append(val)
+      elif "copy" in name.lower() and val > 1000000:
+        copy.append(val)
+    gemm = [(g, v) for g, v in gemm if len(v) >= 5]
+    if len(gemm) != 4:
+      raise SystemExit(f"expected four runs of qgemm128 dispatches in {path}, found {len(gemm)}")
+    return [sum(v) / len(v) for _, v in gemm], {k: sum(v) / len(v) for k, v in stream.items()}, copy
+
+  f_shapes, f_stream, f_copy = runs(fetch_csv, "FETCH_SIZE")
+  w_shapes, _, w_copy = runs(write_csv, "WRITE_SIZE")
+  true_kib = (1 << 30) / 1024.0
+  factors = [true_kib / v for v in f_stream.values()]
+  if not factors or max(factors) - min(factors) > 0.02 * max(factors):
+    raise SystemExit(f"no consistent stream_read yardstick in {fetch_csv}: {f_stream}")
+  fetch_factor = round(sum(factors) / len(factors), 3)
+  names = ["qkv", "o", "gate_up", "down"]
+  rec = {
+      "kernel": "qgemm128_kernel<2,2,8>",
+      "workload": "Llama-3.1-8B NF4(g64)+LoRA r64 decode, batch 128: mean over the qkv / o / gate|up / down "
+                  "launches of a layer",
+      "kernel_source_sha256_16": kernel_source_hash(),
+      "kernel_sources": list(KERNEL_SOURCES),
+      "fetch_counter_factor": fetch_factor,
+      "write_counter_factor": 1.0,
+      "yardsticks": {**{f"{k} over 1 GiB": {"FETCH_SIZE_kib": round(v, 1), "true_kib": int(true_kib)}
+                        for k, v in f_stream.items()},
+                     "largest torch copies": {"FETCH_SIZE_kib": [round(v) for v in f_copy[:3]],
+                                              "WRITE_SIZE_kib": [round(v) for v in w_copy[:3]]}},
+      "per_shape_counter_kib": {n: {"fetch_kib": round(f, 1), "write_kib": round(w, 1)}
+                                for n, f, w in zip(names, f_shapes, w_shapes)},
+      "read_bytes_per_launch": int(sum(f_shapes) / 4 * 1024 * fetch_factor),
+      "write_bytes_per_launch": int(sum(w_shapes) / 4 * 1024),
+  }
+  with open(TRAFFIC_PROFILE, "w") as f:
+    json.dump(rec, f, indent=1)
+    f.write("\n")
+  print(json.dumps(rec, indent=1))
+
+
 def rooflines(kern, default_workload=False):
   """The dominant kernel of a step is the quantised GEMM (one kernel, launched for the four
   linears of every layer).  One launch = the mean over those four shapes.  At 128 rows its
@@ -479,6 +539,9 @@ def main():
                        "rollout's context range")
   ap.add_argument("--summarize-trace", metavar="CSV", default=None,
                   help="no GPU work: tabulate one decode step of a rocprofv3 kernel-trace csv of this script")
+  ap.add_argument("--write-traffic-profile", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"), default=None,
+                  help="no GPU work: rebuild profiles/qgemm128_kernel_llama8b_decode_b128.json from the counter csvs "
+                       "of two `rocprofv3 --pmc FETCH_SIZE | WRITE_SIZE -- python3 bench.py --kernels-only` runs")
   ap.add_argument("--summarize-counters", metavar="CSV", default=None,
                   help="no GPU work: per-kernel means of a rocprofv3 --pmc counter-collection csv of this script")
   args = ap.parse_args()
@@ -492,6 +555,9 @@ def main():
     return
   if args.summarize_counters:
     summarize_counters(args.summarize_counters)
+    return
+  if args.write_traffic_profile:
+    write_traffic_profile(*args.write_traffic_profile)
     return
   if args.gpus != 1:
     print("bench.py measures one GPU: this build has no multi-GPU path (the decode path shards "

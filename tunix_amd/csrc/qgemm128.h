@@ -574,6 +574,40 @@ void qgemm128_kernel(const QLArgs a) {
         }
       }
     }
+  } else if (NT == 2 && MT >= 4 && a.split_k > 1 && has_rows && ntile0 + NT <= ntiles &&
+             (uint64_t)a.M * (uint64_t)a.N * 4 < (1ull << 32)) {
+    // fp32 partial plane of this k split.  A lane's accumulators are four rows of one column;
+    // stored as they are, a wave would issue 32 four-byte stores of 64-byte runs.  Each 16 x 32
+    // row tile goes through a wave-private corner of the activation buffers instead (idle since
+    // the barriers of the exchange above) and leaves as two 16-byte stores per lane, 128-byte
+    // runs (rows past M fall outside the plane's buffer and are dropped).
+    constexpr int T_LD = 36;   // floats per LDS row: 32 + 4, conflict-free for both passes
+    const uint32_t scr = kBigLutBytes + (uint32_t)wv * (16u * T_LD * 4u);
+    static_assert(MT < 4 || 8 * 16 * T_LD * 4 <= 2 * (int)ABYTES, "transposition scratch fits the activation buffers");
+    const rsrc_t rp = make_rsrc(a.ws + (int64_t)blockIdx.z * a.M * a.N, (uint64_t)a.M * a.N * 4);
+    const uint32_t col0 = (uint32_t)ntile0 * 16u;
+#pragma unroll
+    for (int mt = 0; mt < HM; ++mt) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float v = out[mt][nt][i];   // (a bit cast applied to the vector element itself reads element 0)
+          *reinterpret_cast<lds_u32*>(static_cast<uintptr_t>(scr + (uint32_t)(((lq * 4 + i) * T_LD + nt * 16 + lm) * 4))) =
+              __float_as_uint(v);
+        }
+      // (the reads below are of another type than the writes above: keep the compiler from
+      // moving them across; LDS itself executes a wave's accesses in order)
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int r = (lane >> 3) + 8 * j, c4 = (lane & 7) * 4;
+        const u32x4 v = lds_ld128(scr + (uint32_t)((r * T_LD + c4) * 4));
+        const uint32_t off = ((uint32_t)(m0w + mt * 16 + r) * (uint32_t)a.N + col0 + (uint32_t)c4) * 4u;
+        __builtin_amdgcn_raw_buffer_store_b128(v, rp, off, 0, 0);
+      }
+      asm volatile("" ::: "memory");
+    }
   } else {
     if (has_rows) store_tile<HM, NT>(a, m0w, a.M, ntile0, ntiles, out, [](int64_t r) { return r; });
   }
