@@ -394,10 +394,7 @@ void qgemm128_kernel(const QLArgs a) {
 #pragma unroll
     for (int c = 0; c < AP; ++c) a_first[c] = a_next[c];
     load_w(ic<0>{}, kt_begin);
-    load_w(ic<1>{}, kt_begin + 1);
-    load_a(kt_begin + 1);
-    load_w(ic<2>{}, kt_begin + 2);
-    if (lora_fast) load_adapter_b();
+    __builtin_amdgcn_sched_barrier(0);
     TNX_STAMP(7);
     {  // table entry e = f16 pair (level[e & 15], level[e >> 4]); copies rotated over banks,
        // half of them per thread; built while the first loads are in flight
@@ -408,6 +405,15 @@ void qgemm128_kernel(const QLArgs a) {
 #pragma unroll
       for (int c = 0; c < 32; ++c) lut[e * 64 + ((c0 + c + lane) & 63)] = v;
     }
+    // The rest of the first loads go out behind the table: what the first k-tile needs (its
+    // activations and weights, requested above by every wave) is then at the head of the unit's
+    // memory queue, and the first tile is multiplied while the second one's data arrives.
+    __builtin_amdgcn_sched_barrier(0);
+    load_w(ic<1>{}, kt_begin + 1);
+    load_a(kt_begin + 1);
+    load_w(ic<2>{}, kt_begin + 2);
+    if (lora_fast) load_adapter_b();
+    __builtin_amdgcn_sched_barrier(0);
     TNX_STAMP(1);
 #pragma unroll
     for (int c = 0; c < AP; ++c) lds_st128(a_wr + (uint32_t)(c * 32 * A_LD * 2), a_first[c]);
