@@ -133,6 +133,27 @@ void qgemm128_kernel(const QLArgs a) {
   u32x4 bfr[2][NT];       // weight fragments of the two k-steps
   uint32_t lp[2][NT][4];  // table entries (f16 level pairs): [s] is read by the steps of parity s, written by the others
 
+  auto load_w = [&](auto Dc, int kt) {
+    constexpr int D = decltype(Dc)::value;
+    const int ktc = min(kt, ktiles - 1);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      ring_c[D][nt] = __builtin_amdgcn_raw_buffer_load_b64(rc, coff[nt], ktc * 1024, 0);
+      ring_s[D][nt] = __builtin_amdgcn_raw_buffer_load_b32(rs, soff[nt], ktc * (16 * SPT * 2), 0);
+    }
+  };
+  // What the first k-tile needs is requested here, ahead of the adapter bookkeeping below (a
+  // few hundred scalar and vector instructions that touch no memory).  The first activation
+  // tile has registers of its own (live only up to its store).
+  u32x4 a_first[AP];
+  if (kt_begin < kt_end) {
+#pragma unroll
+    for (int c = 0; c < AP; ++c)
+      a_first[c] = __builtin_amdgcn_raw_buffer_load_b128(rx, xbase + (uint32_t)c * xstride, kt_begin * (KTILE * 2), 0);
+    load_w(ic<0>{}, kt_begin);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
   // LoRA delta through the activation pipeline: the "k-tile" after the last real one is the
   // 128-row block of t = bf16(x . A), columns [toff_a, +64) | [toff_b, +64) (the one or two
   // adapter segments this work-group's columns belong to), so that it is in LDS when the main
@@ -218,15 +239,6 @@ void qgemm128_kernel(const QLArgs a) {
 #pragma unroll
     for (int c = 0; c < AP; ++c)
       a_next[c] = __builtin_amdgcn_raw_buffer_load_b128(r, base + (uint32_t)c * stride, s, 0);
-  };
-  auto load_w = [&](auto Dc, int kt) {
-    constexpr int D = decltype(Dc)::value;
-    const int ktc = min(kt, ktiles - 1);
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      ring_c[D][nt] = __builtin_amdgcn_raw_buffer_load_b64(rc, coff[nt], ktc * 1024, 0);
-      ring_s[D][nt] = __builtin_amdgcn_raw_buffer_load_b32(rs, soff[nt], ktc * (16 * SPT * 2), 0);
-    }
   };
   // scales of ring stage D -> fp32; a k-tile past the end gets zero scales, which turns its
   // weights into zeros
@@ -389,12 +401,6 @@ void qgemm128_kernel(const QLArgs a) {
     // in the steady state of the loop, so the counted waits of the loop body need not fall back
     // to "everything outstanding" for the sake of the path that enters from here.  The first
     // activation tile has registers of its own for that (live only up to its store).
-    u32x4 a_first[AP];
-    load_a(kt_begin);
-#pragma unroll
-    for (int c = 0; c < AP; ++c) a_first[c] = a_next[c];
-    load_w(ic<0>{}, kt_begin);
-    __builtin_amdgcn_sched_barrier(0);
     TNX_STAMP(7);
     {  // table entry e = f16 pair (level[e & 15], level[e >> 4]); copies rotated over banks,
        // half of them per thread; built while the first loads are in flight
