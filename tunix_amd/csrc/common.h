@@ -134,11 +134,12 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint64_t bytes) {
                                            (uint32_t)(bytes > 0xffffffffull ? 0xffffffffull : bytes),
                                            0x00020000);
 }
-// Cache policy of buffer loads whose data is used exactly once per launch and by one wave (the
-// keys and values of attention): non-temporal.  A flat read of this part runs at 7.1-7.3 TB/s
-// with it against 6.2-6.4 TB/s without; attention over cold caches 6.0 against 5.4 TB/s at
-// context 768.  (Measured and not adopted for the packed weights of the GEMM, 1 us slower per
-// launch, and for the head's weight rows, neutral.)
+// Cache policy of buffer accesses whose data is used exactly once and by one wave (the keys and
+// values of attention; the fp32 partial planes a split-k GEMM leaves for the next kernel):
+// non-temporal.  A flat read of this part runs at 7.1-7.3 TB/s with it against 6.2-6.4 TB/s
+// without; attention over cold caches 6.0 against 5.4 TB/s at context 768.  (Measured and not
+// adopted for the packed weights of the GEMM, 1 us slower per launch, for the head's weight rows,
+// neutral, and for the norm's reads of the partial planes, slower.)
 constexpr int kStreamOnce = 2;   // the "nt" bit of the gfx940+ cache-policy operand
 __device__ __forceinline__ u32x4 buf_load128(rsrc_t r, uint32_t byte_off) {
   return __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
