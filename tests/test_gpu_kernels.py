@@ -1039,6 +1039,71 @@ def test_moe_route_sort_gmm_combine(gpu, M, E, k, D, F):
   assert_bf16_close(out, ref, atol=1e-5, min_equal=0.85, what="moe", mag=ref_mag.float())
 
 
+@pytest.mark.parametrize("E,n_tok,k,K,N,group,qtype,mul", [
+    (16, 48, 2, 512, 256, 128, Q.INT4, True),     # experts of 40 and 17 rows: several 16-row blocks
+    (16, 48, 2, 512, 256, 64, Q.NF4, False),
+    (16, 48, 2, 256, 96, 32, Q.INT4, False),      # four scale slots per k-tile
+    (256, 256, 4, 256, 288, 128, Q.INT4, False),  # 9 tile pairs per block, 2 per wave: runs span two blocks
+    (256, 256, 4, 256, 576, 128, Q.NF4, True),
+    (16, 48, 2, 384, 80, 128, Q.INT4, False),     # 5 column tiles: no pairs, the general kernel
+])
+def test_moe_gmm_skewed_routes(gpu, E, n_tok, k, K, N, group, qtype, mul):
+  """The grouped GEMM alone, on routes built by hand: experts with no rows, with one row, with
+  exactly 16 and with more than 16 rows (several row blocks of one expert), gathered through a
+  shuffled route order; k-tile counts below the kernel's ring depth; both code books, two and
+  four scale slots, the plain and the SiLU-mul epilogue."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  rng = np.random.Generator(np.random.PCG64(2000 + E + N))
+  n_routes = n_tok * k
+  if E == 16:
+    cnt = np.zeros(E, dtype=np.int64)
+    cnt[[0, 2, 3, 5, 6, 7]] = [40, 3, 17, 1, 16, n_routes - 77]
+  else:
+    ids = rng.integers(0, E - 3, size=n_routes)
+    ids[:40] = 7                                    # one expert far above the average
+    cnt = np.bincount(ids, minlength=E)
+  assert cnt.sum() == n_routes and cnt.min() == 0 and cnt.max() > 16
+  expert_of = np.repeat(np.arange(E), cnt)          # expert of each sorted position
+  sorted_route = rng.permutation(n_routes).astype(np.int32)   # position -> route (= output row)
+  offs = np.concatenate([[0], np.cumsum(cnt)]).astype(np.int32)
+  x_div = k if mul else 1
+  x = rnd((n_routes // x_div, K), 90)
+  w = rnd((E, K, N), 91, 0.05)
+  cb, sb = ops.qw_sizes(K, N, group)
+  gc = torch.empty(E * cb // 4, dtype=torch.int32, device=gpu)
+  gs = torch.empty(E * sb // 2, dtype=torch.bfloat16, device=gpu)
+  ncol = N // 2 if mul else N
+  ref = torch.full((n_routes, ncol), 7.0)
+  for e in range(E):
+    c, s = ops.quantize_pack(bf(w[e]).to(gpu), group, qtype, mul)
+    gc[e * cb // 4:(e + 1) * cb // 4] = c
+    gs[e * sb // 2:(e + 1) * sb // 2] = s
+    if cnt[e] == 0:
+      continue
+    dq = torch.from_numpy(Q.dequantize(*Q.quantize(w[e].numpy(), group, qtype), group, qtype)).double()
+    routes = torch.from_numpy(sorted_route[offs[e]:offs[e + 1]].astype(np.int64))
+    yy = Q.rb((x[routes // x_div].double() @ dq).float())
+    if mul:
+      gg, uu = yy[:, :N // 2], yy[:, N // 2:]
+      yy = Q.rb(Q.rb(gg * Q.rb(torch.sigmoid(gg))) * uu)
+    ref[routes] = yy
+  y = torch.full((n_routes, ncol), 7.0, dtype=torch.bfloat16, device=gpu)
+  d = L.MoeGmmDesc()
+  d.n_routes, d.E, d.k, d.K, d.N, d.group, d.qtype = n_routes, E, k, K, N, group, qtype
+  gx = bf(x).to(gpu)
+  d.x, d.x_div, d.codes, d.scales = gx.data_ptr(), x_div, gc.data_ptr(), gs.data_ptr()
+  go, gr = torch.from_numpy(offs).to(gpu), torch.from_numpy(sorted_route).to(gpu)
+  d.offsets, d.sorted_route = go.data_ptr(), gr.data_ptr()
+  d.epilogue, d.y = (L.TNX_EPI_SILU_MUL if mul else L.TNX_EPI_STORE), y.data_ptr()
+  for _ in range(2):
+    ops.moe_gmm(d)
+  torch.cuda.synchronize()
+  # (the activation is computed from two rounded tiles and rounded three more times: one ulp on
+  # the gate and one on the up value can add up to three on the product)
+  assert_bf16_close(y, ref, atol=1e-5, min_equal=0.9 if mul else 0.97, what="moe gmm", ulps=3 if mul else 1)
+
+
 def test_argument_errors_raise(gpu):
   from tunix_amd import ops
   with pytest.raises(ValueError, match="K % 128"):

@@ -167,6 +167,7 @@ __global__ __launch_bounds__(256) void moe_gmm_kernel(const QLArgs a) {
 }  // namespace
 #include "qgemm128.h"
 #include "qgemm_wide.h"
+#include "moe_gmm16.h"
 namespace {
 
 // y = epi(sum of the split_k partial tiles, added in split order).  One thread per output
@@ -544,6 +545,49 @@ int launch_moe(hipStream_t st, const QLArgs& a, int E, int64_t max_rows) {
   return TNX_OK;
 }
 
+// The streaming kernel for expert batches of at most 16 rows per block: one persistent
+// work-group per compute unit.  It addresses an expert bank and the output with 32-bit offsets,
+// pairs adjacent column tiles, needs at most as many (expert, row block) pairs as it has waves
+// and parks at most kMoeMaxRun finished tile pairs per wave in LDS.
+bool moe16_shape(const QLArgs& a, int E, size_t codes_bytes, size_t scales_bytes, int cus) {
+  if (a.N % 32 != 0 || cus <= 0) return false;
+  if ((uint64_t)E * codes_bytes >= (1ull << 32) || (uint64_t)E * scales_bytes >= (1ull << 32)) return false;
+  const int64_t max_blocks = (int64_t)E + a.M / 16;
+  const int64_t waves = (int64_t)cus * kMoeWaves;
+  if (max_blocks > waves || max_blocks * (a.N / 32) > waves * kMoeMaxRun) return false;
+  const bool mul = a.epilogue == TNX_EPI_SILU_MUL;
+  if ((uint64_t)a.M * (uint64_t)(mul ? a.N / 2 : a.N) * 2 >= (1ull << 32) || ((uintptr_t)a.y & 15) != 0) return false;
+  return moe16_smem_bytes(E, a.M) <= 160 * 1024;
+}
+
+template <bool MUL, int SPT>
+int launch_moe16_t(hipStream_t st, const QLArgs& a, int E, int cus) {
+  static std::once_flag once;
+  static int attr_rc = TNX_OK;
+  std::call_once(once, [] { attr_rc = prepare_qgemm128(&moe_gmm16_kernel<MUL, SPT>, 160 * 1024); });
+  if (attr_rc) return attr_rc;
+  hipLaunchKernelGGL((moe_gmm16_kernel<MUL, SPT>), dim3((unsigned)cus), dim3(kMoeWaves * 64), moe16_smem_bytes(E, a.M), st, a, E);
+  TNX_CHECK_LAUNCH("moe_gmm16");
+  return TNX_OK;
+}
+
+int launch_moe16(hipStream_t st, const QLArgs& a, int E, int cus) {
+  const bool mul = a.epilogue == TNX_EPI_SILU_MUL;
+  if (scales_per_tile(a.group) == 2)
+    return mul ? launch_moe16_t<true, 2>(st, a, E, cus) : launch_moe16_t<false, 2>(st, a, E, cus);
+  return mul ? launch_moe16_t<true, 4>(st, a, E, cus) : launch_moe16_t<false, 4>(st, a, E, cus);
+}
+
+int device_cus() {
+  static int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    return n;
+  }();
+  return cus;
+}
+
 }  // namespace
 
 extern "C" int tnx_qw_sizes(int64_t K, int64_t N, int group, size_t* codes_bytes,
@@ -727,7 +771,11 @@ extern "C" int tnx_moe_int4_gmm(void* stream, const tnx_moe_gmm_desc* d) {
   const int64_t max_rows = d->n_routes / d->k;
   const int64_t avg_rows = cdiv(d->n_routes, (int64_t)d->E);
   hipStream_t st = as_stream(stream);
-  if (max_rows <= 16 || avg_rows <= 8) return launch_moe<1, 2>(st, a, d->E, max_rows);
+  if (max_rows <= 16 || avg_rows <= 8) {
+    const int cus = device_cus();
+    if (moe16_shape(a, d->E, cb, sb, cus)) return launch_moe16(st, a, d->E, cus);
+    return launch_moe<1, 2>(st, a, d->E, max_rows);
+  }
   if (max_rows <= 32 || avg_rows <= 24) return launch_moe<2, 2>(st, a, d->E, max_rows);
   return launch_moe<4, 2>(st, a, d->E, max_rows);
 }
