@@ -20,11 +20,11 @@
 //   * activation fragments come straight from global memory in MFMA layout (the eight waves of a
 //     work-group work on the same expert's rows, the requests meet in L1); rows the block does
 //     not have are out-of-range buffer offsets, which read zeros and move no data;
-//   * the loop has no barrier, no load behind a branch and no store: stores complete out of order
-//     with respect to loads, so one store in flight turns every counted wait on the ring into
-//     "everything outstanding".  Finished tiles are parked in LDS and written out after the loop.
-//     The first loads are issued in the order of the loop's, for the same reason as in
-//     qgemm128.h: the waits of the loop body are the minimum over the paths that reach them;
+//   * the loop has no barrier and no memory instruction behind a branch: the counted waits on
+//     the ring are the minimum over the paths that reach them, so a tile stored only in the step
+//     that finishes it would make the waits of the steps behind it stricter than the ring needs.
+//     Finished tiles are parked in LDS and written out after the loop.  For the same reason the
+//     first loads are issued in the order of the loop's (as in qgemm128.h);
 //   * a k-tile is eight groups (k-step x column tile) of four look-ups, twelve conversion
 //     instructions and one MFMA, software-pipelined by hand: the look-ups run two groups ahead of
 //     the MFMA, the conversions one.
