@@ -177,6 +177,14 @@ int tnx_rmsnorm(void* stream, const uint16_t* x, const uint16_t* res_pre, uint16
 int tnx_rmsnorm_splitk(void* stream, const float* ws, int split_k, const uint16_t* res_pre,
                        uint16_t* h_out, const uint16_t* w, const uint16_t* res_post, uint16_t* y,
                        int64_t M, int64_t D, float eps, int flavor);
+/* The same, with the input row taken from the k routed rows of a token: x = bf16(sum_j topk_w[m,j]
+ * * y_route[m*k + j]), j ascending (tnx_moe_combine's arithmetic).  It replaces tnx_moe_combine +
+ * tnx_rmsnorm where an MoE layer's output feeds the residual add and the next norm
+ * (qwen3/model.py:826-832 into :450-456).  D % 8 == 0. */
+int tnx_rmsnorm_moe_combine(void* stream, const uint16_t* y_route, const uint16_t* topk_w, int k,
+                            const uint16_t* res_pre, uint16_t* h_out, const uint16_t* w,
+                            const uint16_t* res_post, uint16_t* y, int64_t M, int64_t D, float eps,
+                            int flavor);
 /* Two norms in a row in one launch: y as above (input x, or the partial planes ws of a split-k
  * linear when x is NULL), then y2 = norm(y) with weight w2.  Gemma-3's block applies
  * post_attention_norm, adds the residual and applies pre_ffw_norm to the sum, and likewise

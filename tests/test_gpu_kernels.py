@@ -1113,6 +1113,29 @@ def test_argument_errors_raise(gpu):
     ops.quantize_pack(x.t().contiguous(), 48, 0)
 
 
+@pytest.mark.parametrize("family,M,k,D", [("qwen3", 64, 8, 2048), ("llama3", 5, 11, 512), ("gemma3", 3, 1, 4104)])
+def test_rmsnorm_moe_combine_equals_combine_then_norm(gpu, family, M, k, D):
+  """The folded pass (weighted combine of a token's k routed rows + residual + norm) against the
+  two separate kernels it replaces: the new residual stream and the normed row bit for bit; more
+  routes per token than one group of loads takes, a width that is not a multiple of 2048."""
+  from tunix_amd import ops
+  from tunix_amd.model import _NORM
+  yr = bf(rnd((M * k, D), 310)).to(gpu)
+  tw = bf(torch.softmax(rnd((M, k), 311), -1)).to(gpu)
+  res = bf(rnd((M, D), 312)).to(gpu)
+  nw = bf(rnd((D,), 313, 0.3) + 1.0).to(gpu)
+  h1 = res.clone()
+  ops.moe_combine(yr, tw, M, k, D, h1, h1)
+  y1 = torch.empty_like(h1)
+  ops.rmsnorm(h1, nw, y1, 1e-6, _NORM[family])
+  h2 = res.clone()
+  y2 = torch.empty_like(h1)
+  ops.rmsnorm_moe_combine(yr, tw, k, nw, y2, 1e-6, _NORM[family], M, D, res_pre=h2, h_out=h2)
+  torch.cuda.synchronize()
+  assert torch.equal(h1, h2) and torch.equal(y1, y2)
+  assert not torch.equal(h1, res)
+
+
 @pytest.mark.parametrize("family", ["llama3", "qwen3"])
 def test_rmsnorm_splitk_equals_finish_then_norm(gpu, family):
   """The folded pass (sum of split-k planes + residual + norm) against the two separate

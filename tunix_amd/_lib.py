@@ -99,6 +99,7 @@ SIGNATURES = {
     "tnx_embed": (_i32, [_p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _f32, _p]),
     "tnx_rmsnorm": (_i32, [_p, _p, _p, _p, _p, _p, _p, _i64, _i64, _f32, _i32]),
     "tnx_rmsnorm_splitk": (_i32, [_p, _p, _i32, _p, _p, _p, _p, _p, _i64, _i64, _f32, _i32]),
+    "tnx_rmsnorm_moe_combine": (_i32, [_p, _p, _p, _i32, _p, _p, _p, _p, _p, _i64, _i64, _f32, _i32]),
     "tnx_rmsnorm_pair": (_i32, [_p, _p, _p, _i32, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _f32, _i32]),
     "tnx_qknorm_rope_kvwrite": (_i32, [_p, C.POINTER(RopeDesc)]),
     "tnx_rope_table": (_i32, [_p, _p, _i64, _p, _i64, _p, _i32, _p, _p]),

@@ -80,15 +80,20 @@ __device__ __forceinline__ void unpack8(const u32x4& p, float (&f)[8]) {
     f[2 * j + 1] = bfhi(p[j]);
   }
 }
-// With `ws` the input row is bf16(sum of the split_k fp32 partial planes ws[z][row][:]) of a
-// split-k linear, added in split order: the linear's own finishing pass folded into the norm.
-template <int MAXC, int FLAVOR, bool PLANES>
+// The input row, by IN: kNormInRow -- x[row]; kNormInPlanes -- bf16(sum of the split_k fp32 partial
+// planes ws[z][row][:]) of a split-k linear, added in split order: the linear's own finishing
+// pass folded into the norm; kNormInRoutes -- bf16(sum_j cw[row, j] * x[row * split_k + j]) over
+// the split_k routed rows of a token, j ascending: the weighted combine of an MoE layer folded
+// into the norm (same arithmetic as moe_combine_vec_kernel).
+constexpr int kNormInRow = 0, kNormInPlanes = 1, kNormInRoutes = 2;
+template <int MAXC, int FLAVOR, int IN>
 __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, const uint16_t* res_pre,
                                                           uint16_t* h_out, const uint16_t* w,
                                                           const uint16_t* res_post, uint16_t* y,
                                                           int64_t D, float eps, int /*flavor*/,
                                                           const float* ws, int split_k, int64_t plane,
-                                                          const uint16_t* w2, uint16_t* y2) {
+                                                          const uint16_t* w2, uint16_t* y2, const uint16_t* cw) {
+  constexpr bool PLANES = IN == kNormInPlanes, ROUTES = IN == kNormInRoutes;
   __shared__ float red[4];
   const int64_t row = blockIdx.x;
   const int nchunks = (int)(D / 8);
@@ -102,7 +107,7 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
   for (int c0 = 0; c0 < MAXC; c0 += 2) {
     if (c0 * 256 >= nchunks) break;   // uniform
     f32x4 p0[2][8], p1[2][8];
-    u32x4 xin[2], rin[2];
+    u32x4 xin[2], rin[2], yin[2][8];
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
       const int ch = (c0 + cc) * 256 + threadIdx.x;
@@ -114,6 +119,11 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
           p0[cc][u] = *reinterpret_cast<const f32x4*>(ws + zo);
           p1[cc][u] = *reinterpret_cast<const f32x4*>(ws + zo + 4);
         }
+      } else if (ROUTES) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          yin[cc][u] = *reinterpret_cast<const u32x4*>(
+              x + (row * split_k + min(u, split_k - 1)) * D + (int64_t)min(ch, nchunks - 1) * 8);
       } else {
         xin[cc] = *reinterpret_cast<const u32x4*>(x + o);
       }
@@ -152,6 +162,37 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
                 for (int j = 0; j < 4; ++j) {
                   h[c][j] += q0[u][j];
                   h[c][4 + j] += q1[u][j];
+                }
+              }
+          }
+#pragma unroll
+          for (int j = 0; j < 8; ++j) h[c][j] = rbf(h[c][j]);
+        } else if (ROUTES) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) h[c][j] = 0.f;
+#pragma unroll
+          for (int u = 0; u < 8; ++u)
+            if (u < split_k) {
+              const float wt = bf2f(cw[row * split_k + u]);
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                h[c][2 * q] += wt * bflo(yin[cc][u][q]);
+                h[c][2 * q + 1] += wt * bfhi(yin[cc][u][q]);
+              }
+            }
+          for (int z0 = 8; z0 < split_k; z0 += 8) {   // more than eight routes per token: the rest in groups
+            u32x4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+              v[u] = *reinterpret_cast<const u32x4*>(x + (row * split_k + min(z0 + u, split_k - 1)) * D + (int64_t)ch * 8);
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+              if (z0 + u < split_k) {
+                const float wt = bf2f(cw[row * split_k + z0 + u]);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                  h[c][2 * q] += wt * bflo(v[u][q]);
+                  h[c][2 * q + 1] += wt * bfhi(v[u][q]);
                 }
               }
           }
@@ -245,20 +286,21 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const uint16_t* x, con
 // and 8 chunks per thread so that the common widths (D <= 4096) run the small instance -- the
 // code a wave walks through once is fetched cold at every launch.
 template <int MAXC, class... Args>
-void launch_rmsnorm_vec_c(hipStream_t st, int64_t M, int flavor, bool planes, Args... args) {
+void launch_rmsnorm_vec_c(hipStream_t st, int64_t M, int flavor, int in, Args... args) {
 #define TNX_NORM_CASE(F)                                                                                   \
-  if (planes) hipLaunchKernelGGL((rmsnorm_vec_kernel<MAXC, F, true>), dim3((unsigned)M), dim3(256), 0, st, args...); \
-  else hipLaunchKernelGGL((rmsnorm_vec_kernel<MAXC, F, false>), dim3((unsigned)M), dim3(256), 0, st, args...)
+  if (in == kNormInPlanes) hipLaunchKernelGGL((rmsnorm_vec_kernel<MAXC, F, kNormInPlanes>), dim3((unsigned)M), dim3(256), 0, st, args...); \
+  else if (in == kNormInRoutes) hipLaunchKernelGGL((rmsnorm_vec_kernel<MAXC, F, kNormInRoutes>), dim3((unsigned)M), dim3(256), 0, st, args...); \
+  else hipLaunchKernelGGL((rmsnorm_vec_kernel<MAXC, F, kNormInRow>), dim3((unsigned)M), dim3(256), 0, st, args...)
   if (flavor == TNX_NORM_LLAMA) { TNX_NORM_CASE(TNX_NORM_LLAMA); }
   else if (flavor == TNX_NORM_QWEN3) { TNX_NORM_CASE(TNX_NORM_QWEN3); }
   else { TNX_NORM_CASE(TNX_NORM_GEMMA3); }
 #undef TNX_NORM_CASE
 }
 template <class... Args>
-void launch_rmsnorm_vec(hipStream_t st, int64_t M, int64_t D, int flavor, bool planes, Args... args) {
-  if (D <= 8 * 256 * 2) launch_rmsnorm_vec_c<2>(st, M, flavor, planes, args...);
-  else if (D <= 8 * 256 * 4) launch_rmsnorm_vec_c<4>(st, M, flavor, planes, args...);
-  else launch_rmsnorm_vec_c<kNormMaxChunks>(st, M, flavor, planes, args...);
+void launch_rmsnorm_vec(hipStream_t st, int64_t M, int64_t D, int flavor, int in, Args... args) {
+  if (D <= 8 * 256 * 2) launch_rmsnorm_vec_c<2>(st, M, flavor, in, args...);
+  else if (D <= 8 * 256 * 4) launch_rmsnorm_vec_c<4>(st, M, flavor, in, args...);
+  else launch_rmsnorm_vec_c<kNormMaxChunks>(st, M, flavor, in, args...);
 }
 
 __global__ void embed_kernel(const uint16_t* table, int64_t V, int64_t D, const int32_t* ids,
@@ -432,8 +474,9 @@ extern "C" int tnx_rmsnorm(void* stream, const uint16_t* x, const uint16_t* res_
   TNX_REQUIRE(M > 0 && D > 0 && D <= 16384, "rmsnorm: D=%lld out of range (1..16384)", (long long)D);
   TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm: bad flavor %d", flavor);
   if (D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks)
-    launch_rmsnorm_vec(as_stream(stream), M, D, flavor, false, x, res_pre, h_out, w, res_post, y, D, eps, flavor,
-                       (const float*)nullptr, 0, (int64_t)0, (const uint16_t*)nullptr, (uint16_t*)nullptr);
+    launch_rmsnorm_vec(as_stream(stream), M, D, flavor, kNormInRow, x, res_pre, h_out, w, res_post, y, D, eps, flavor,
+                       (const float*)nullptr, 0, (int64_t)0, (const uint16_t*)nullptr, (uint16_t*)nullptr,
+                       (const uint16_t*)nullptr);
   else
     hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)M), dim3(256), (size_t)D * sizeof(float),
                        as_stream(stream), x, res_pre, h_out, w, res_post, y, D, eps, flavor);
@@ -449,9 +492,25 @@ extern "C" int tnx_rmsnorm_splitk(void* stream, const float* ws, int split_k, co
   TNX_REQUIRE(M > 0 && D > 0 && D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks,
               "rmsnorm_splitk: D=%lld must be a multiple of 8 and <= 16384", (long long)D);
   TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm_splitk: bad flavor %d", flavor);
-  launch_rmsnorm_vec(as_stream(stream), M, D, flavor, true, (const uint16_t*)nullptr, res_pre, h_out, w, res_post, y, D, eps,
-                     flavor, ws, split_k, (int64_t)(M * D), (const uint16_t*)nullptr, (uint16_t*)nullptr);
+  launch_rmsnorm_vec(as_stream(stream), M, D, flavor, kNormInPlanes, (const uint16_t*)nullptr, res_pre, h_out, w, res_post, y,
+                     D, eps, flavor, ws, split_k, (int64_t)(M * D), (const uint16_t*)nullptr, (uint16_t*)nullptr,
+                     (const uint16_t*)nullptr);
   TNX_CHECK_LAUNCH("rmsnorm_splitk");
+  return TNX_OK;
+}
+
+extern "C" int tnx_rmsnorm_moe_combine(void* stream, const uint16_t* y_route, const uint16_t* topk_w, int k,
+                                       const uint16_t* res_pre, uint16_t* h_out, const uint16_t* w,
+                                       const uint16_t* res_post, uint16_t* y, int64_t M, int64_t D, float eps,
+                                       int flavor) {
+  TNX_REQUIRE(y_route && topk_w && w && y, "rmsnorm_moe_combine: null pointer");
+  TNX_REQUIRE(k >= 1, "rmsnorm_moe_combine: k must be >= 1");
+  TNX_REQUIRE(M > 0 && D > 0 && D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks,
+              "rmsnorm_moe_combine: D=%lld must be a multiple of 8 and <= 16384", (long long)D);
+  TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm_moe_combine: bad flavor %d", flavor);
+  launch_rmsnorm_vec(as_stream(stream), M, D, flavor, kNormInRoutes, y_route, res_pre, h_out, w, res_post, y, D, eps, flavor,
+                     (const float*)nullptr, k, (int64_t)0, (const uint16_t*)nullptr, (uint16_t*)nullptr, topk_w);
+  TNX_CHECK_LAUNCH("rmsnorm_moe_combine");
   return TNX_OK;
 }
 
@@ -465,8 +524,8 @@ extern "C" int tnx_rmsnorm_pair(void* stream, const uint16_t* x, const float* ws
   TNX_REQUIRE(M > 0 && D > 0 && D % 8 == 0 && D <= 8 * 256 * kNormMaxChunks,
               "rmsnorm_pair: D=%lld must be a multiple of 8 and <= 16384", (long long)D);
   TNX_REQUIRE(flavor >= TNX_NORM_LLAMA && flavor <= TNX_NORM_GEMMA3, "rmsnorm_pair: bad flavor %d", flavor);
-  launch_rmsnorm_vec(as_stream(stream), M, D, flavor, ws != nullptr, x, res_pre, h_out, w, res_post, y, D, eps, flavor, ws,
-                     ws ? split_k : 0, (int64_t)(M * D), w2, y2);
+  launch_rmsnorm_vec(as_stream(stream), M, D, flavor, ws ? kNormInPlanes : kNormInRow, x, res_pre, h_out, w, res_post, y, D,
+                     eps, flavor, ws, ws ? split_k : 0, (int64_t)(M * D), w2, y2, (const uint16_t*)nullptr);
   TNX_CHECK_LAUNCH("rmsnorm_pair");
   return TNX_OK;
 }

@@ -20,6 +20,7 @@ from . import ops
 from .config import ModelConfig
 
 _NORM = {"llama3": L.TNX_NORM_LLAMA, "qwen3": L.TNX_NORM_QWEN3, "gemma3": L.TNX_NORM_GEMMA3}
+_MOE_PENDING = -1   # norm_after: the weighted combine of an MoE layer still awaits its sum
 _ROPE = {"llama3": L.TNX_ROPE_LLAMA, "qwen3": L.TNX_ROPE_QWEN3, "gemma3": L.TNX_ROPE_GEMMA3}
 
 
@@ -435,7 +436,10 @@ class Runner:
     self.h += bf16(sum of planes) first (the linear's residual epilogue) in the same kernel."""
     cfg = self.cfg
     flavor = _NORM[cfg.family]
-    if pending > 1:
+    if pending == _MOE_PENDING:   # h += the weighted combine of the routed rows, in the same kernel
+      ops.rmsnorm_moe_combine(self.y_route, self.topk_w, cfg.num_experts_per_tok, w, self.xn, cfg.norm_eps,
+                              flavor, M, cfg.embed_dim, res_pre=self.h, h_out=self.h)
+    elif pending > 1:
       ops.rmsnorm_splitk(self.splitk_ws, pending, w, self.xn, cfg.norm_eps, flavor, M, cfg.embed_dim,
                          res_pre=self.h, h_out=self.h)
     else:
@@ -520,7 +524,7 @@ class Runner:
                          defer=True)
         self.norm_after(po, ly["mlp_norm"], M)
       if cfg.num_experts:
-        self._moe(ly["experts"], M)
+        pending = self._moe(ly["experts"], M)
       elif cfg.family == "gemma3":
         fused = self.fuses_next(ly["gu"], ly["down"], M, L.TNX_EPI_GELU_MUL)
         self.linear(ly["gu"], self.xn, self.act, M, epilogue=L.TNX_EPI_GELU_MUL, next_f=ly["down"])
@@ -538,7 +542,7 @@ class Runner:
       self.norm_after(pending, m.final_norm, M)
     return self.xn
 
-  def _moe(self, ex: ExpertBank, M: int):
+  def _moe(self, ex: ExpertBank, M: int) -> int:
     cfg = self.cfg
     k, E = cfg.num_experts_per_tok, cfg.num_experts
     ops.lora_down(self.xn, ex.router_t, self.scores, M=M)          # dense bf16 router
@@ -560,7 +564,10 @@ class Runner:
     d2.offsets, d2.sorted_route = self.offsets.data_ptr(), self.sorted_route.data_ptr()
     d2.epilogue, d2.y = L.TNX_EPI_STORE, self.y_route.data_ptr()
     ops.moe_gmm(d2)
+    if cfg.embed_dim % 8 == 0:   # the next norm adds the weighted combine to the residual stream
+      return _MOE_PENDING
     ops.moe_combine(self.y_route, self.topk_w, M, k, cfg.embed_dim, self.h, self.h)
+    return 1
 
   def head_desc(self, x, rows, part, temperature=1.0, targets=None, best_id=None, best_logp=None,
                 target_logp=None, lse=None, logits_out=None, forbidden=None, entropy=None,

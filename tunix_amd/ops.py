@@ -123,6 +123,14 @@ def rmsnorm_splitk(ws, split_k, w, y, eps, flavor, M, D, res_pre=None, h_out=Non
           "tnx_rmsnorm_splitk")
 
 
+def rmsnorm_moe_combine(y_route, topk_w, k, w, y, eps, flavor, M, D, res_pre=None, h_out=None, res_post=None):
+  """y = norm(h), h = bf16(bf16(sum_j topk_w[m, j] * y_route[m * k + j]) + res_pre): the weighted
+  combine of an MoE layer folded into the residual add + norm that consumes it."""
+  L.check(L.lib().tnx_rmsnorm_moe_combine(_stream(), _ptr(y_route), _ptr(topk_w), k, _ptr(res_pre), _ptr(h_out),
+                                          _ptr(w), _ptr(res_post), _ptr(y), M, D, float(eps), flavor),
+          "tnx_rmsnorm_moe_combine")
+
+
 def rmsnorm_pair(w, y, w2, y2, eps, flavor, M, D, x=None, ws=None, split_k=0, res_pre=None, h_out=None,
                  res_post=None):
   """y = [res_post +] norm(h) . w with h from x (or the split-k planes ws) [+ res_pre]; y2 = norm(y) . w2."""
