@@ -1046,12 +1046,17 @@ def test_moe_route_sort_gmm_combine(gpu, M, E, k, D, F):
     (256, 256, 4, 256, 288, 128, Q.INT4, False),  # 9 tile pairs per block, 2 per wave: runs span two blocks
     (256, 256, 4, 256, 576, 128, Q.NF4, True),
     (16, 48, 2, 384, 80, 128, Q.INT4, False),     # 5 column tiles: no pairs, the general kernel
+    (8, 512, 2, 512, 256, 128, Q.INT4, False),    # ~128 rows per expert: the 128 x 256 tiles of the many-row kernel
+    (8, 512, 2, 384, 512, 64, Q.NF4, True),
+    (8, 512, 2, 256, 768, 32, Q.INT4, False),
 ])
 def test_moe_gmm_skewed_routes(gpu, E, n_tok, k, K, N, group, qtype, mul):
   """The grouped GEMM alone, on routes built by hand: experts with no rows, with one row, with
-  exactly 16 and with more than 16 rows (several row blocks of one expert), gathered through a
-  shuffled route order; k-tile counts below the kernel's ring depth; both code books, two and
-  four scale slots, the plain and the SiLU-mul epilogue."""
+  exactly one row block and with more (several row blocks of one expert), gathered through a
+  shuffled route order; k-tile counts below the streaming kernel's ring depth; both code books,
+  two and four scale slots, the plain and the SiLU-mul epilogue; decode-sized batches (the
+  streaming kernel), a shape the general tile kernel takes, and many rows per expert (the
+  128 x 256 tiles of the many-row kernel)."""
   from tunix_amd import _lib as L
   from tunix_amd import ops
   rng = np.random.Generator(np.random.PCG64(2000 + E + N))
@@ -1059,6 +1064,8 @@ def test_moe_gmm_skewed_routes(gpu, E, n_tok, k, K, N, group, qtype, mul):
   if E == 16:
     cnt = np.zeros(E, dtype=np.int64)
     cnt[[0, 2, 3, 5, 6, 7]] = [40, 3, 17, 1, 16, n_routes - 77]
+  elif E == 8:   # empty experts, one row, exactly one 128-row block, one row more, several blocks
+    cnt = np.array([300, 0, 129, 128, 1, 200, n_routes - 758, 0], dtype=np.int64)
   else:
     ids = rng.integers(0, E - 3, size=n_routes)
     ids[:40] = 7                                    # one expert far above the average

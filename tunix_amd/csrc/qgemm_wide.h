@@ -38,7 +38,12 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-template <int SPT>
+// GROUPED: the grouped GEMM over routed tokens at many rows per expert.  A work-group takes one
+// 128-row block of one expert's routes (in expert-sorted order) and one column tile; block b ->
+// (expert, row block) is found from the expert offsets by a running sum; activation rows are
+// gathered through sorted_route (row = route / x_div), output rows are routes.  No adapter, no
+// lm_head statistics in this mode.
+template <int SPT, bool GROUPED = false>
 __global__ __launch_bounds__(256)
 void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   constexpr int RT = 4, CG = 2, PF = 3, AP = 8;   // 32-row tiles, 32-column groups per wave
@@ -61,25 +66,58 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   // moves every eight ids
   const int tiles_m = (int)((a.M + kWideRows - 1) / kWideRows), tiles_n = (int)((a.N + kWideCols - 1) / kWideCols);
   int mtile, ntile;
-  {
+  int expert = 0, m_end = 0;   // GROUPED: the block's expert and the end of its routes in sorted order
+  if constexpr (GROUPED) {
+    // column tiles of one row block sit next to each other; every wave finds the block's expert
+    // itself (same result in all of them: nothing is shared, no barrier)
+    const int b = (int)blockIdx.x / tiles_n;
+    ntile = (int)blockIdx.x % tiles_n;
+    int carry = 0, found_e = -1, found_rb = 0;
+    for (int base = 0; base < a.n_experts; base += 64) {
+      const int e = base + lane;
+      int nb = 0;
+      if (e < a.n_experts) nb = (a.offsets[e + 1] - a.offsets[e] + kWideRows - 1) / kWideRows;
+      int incl = nb;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int t = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += t;
+      }
+      const int first = carry + incl - nb;
+      const uint64_t hit = __ballot(nb > 0 && b >= first && b < first + nb);
+      if (hit) {
+        const int l = __ffsll((long long)hit) - 1;
+        found_e = base + l;
+        found_rb = b - __shfl(first, l, 64);
+      }
+      carry += __shfl(incl, 63, 64);
+    }
+    if (found_e < 0) return;   // past the last block (the grid covers an upper bound)
+    expert = __builtin_amdgcn_readfirstlane(found_e);
+    mtile = __builtin_amdgcn_readfirstlane(found_rb);
+    m_end = a.offsets[expert + 1];
+  } else {
     const int per_group = 8 * tiles_n;
     const int g = (int)blockIdx.x / per_group, r = (int)blockIdx.x % per_group;
     const int gm = min(8, tiles_m - g * 8);
     mtile = g * 8 + r % gm;
     ntile = r / gm;
   }
-  const int64_t m0 = (int64_t)mtile * kWideRows;
+  // first row of the tile (GROUPED: first position in the sorted route list)
+  const int64_t m0 = GROUPED ? (int64_t)a.offsets[expert] + (int64_t)mtile * kWideRows : (int64_t)mtile * kWideRows;
   const int64_t ntile0 = ((int64_t)ntile * 4 + wn) * 4;   // first packed 16-column tile of this wave
   const int64_t ntiles = a.N / 16;
   const int ktiles = (int)(a.K / KTILE);
-  const int rows_here = (int)min((int64_t)kWideRows, a.M - m0);
+  const int rows_here = (int)min((int64_t)kWideRows, (GROUPED ? (int64_t)m_end : a.M) - m0);
 
   // the activation resource starts at this work-group's first row: offsets stay small whatever
-  // M is, and rows past M lie beyond the resource and read zeros
-  const rsrc_t rx = make_rsrc(a.x + m0 * a.K, (uint64_t)rows_here * a.K * 2);
+  // M is, and rows past M lie beyond the resource and read zeros (GROUPED: the whole buffer,
+  // rows are gathered)
+  const rsrc_t rx = GROUPED ? make_rsrc(a.x, (uint64_t)(a.M / a.x_div) * a.K * 2)
+                            : make_rsrc(a.x + m0 * a.K, (uint64_t)rows_here * a.K * 2);
   const uint64_t ntk = (uint64_t)ntiles * ktiles;
-  const rsrc_t rc = make_rsrc(a.codes, ntk * 1024);
-  const rsrc_t rs = make_rsrc(a.scales, ntk * 16 * SPT * 2 + 16);
+  const rsrc_t rc = make_rsrc(a.codes + (GROUPED ? (int64_t)expert * a.codes_stride : 0), ntk * 1024);
+  const rsrc_t rs = make_rsrc(a.scales + (GROUPED ? (int64_t)expert * a.scales_stride : 0), ntk * 16 * SPT * 2 + 16);
   // Lane l: column l % 32 of a group = column (l % 16) of packed tile 2 cg + (l % 32) / 16.  A
   // packed tile holds, at chunk 16 q + c, the k-groups 8 q + 32 j (dword j) of its column c;
   // slab u of the MFMA wants k-group 2 u + l / 32 from this lane: chunk q = l / 32 gives the
@@ -88,6 +126,21 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   uint32_t coff[CG], soff[CG];
   const uint32_t xbase = ((uint32_t)(tid >> 4) * (uint32_t)a.K + (uint32_t)(tid & 15) * 8u) * 2u;
   const uint32_t xstride = 16u * (uint32_t)a.K * 2u;  // 16 rows further per pass
+  // GROUPED: the byte offset of each of this thread's eight rows (rows the block does not have:
+  // beyond the buffer, which reads zeros)
+  uint32_t xrow[GROUPED ? 8 : 1];
+  if constexpr (GROUPED) {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const int r = (tid >> 4) + 16 * c;
+      const int route = r < rows_here ? a.sorted_route[m0 + r] : -1;
+      xrow[c] = route >= 0 ? ((uint32_t)(route / a.x_div) * (uint32_t)a.K + (uint32_t)(tid & 15) * 8u) * 2u : 0xfffff000u;
+    }
+  }
+  auto xoff = [&](int c, uint32_t base, uint32_t stride) -> uint32_t {
+    if constexpr (GROUPED) return xrow[c];
+    return base + (uint32_t)c * stride;
+  };
 #pragma unroll
   for (int cg = 0; cg < CG; ++cg) {
     const uint32_t tile0 = (uint32_t)(ntile0 + 2 * cg + (l32 >> 4)) * (uint32_t)ktiles;
@@ -168,7 +221,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
     const uint32_t base = xbase ^ ((xbase ^ tbase) & m), stride = xstride ^ ((xstride ^ tstride) & m);
 #pragma unroll
     for (int c = 0; c < AP; ++c)
-      a_next[c] = __builtin_amdgcn_raw_buffer_load_b128(r, base + (uint32_t)c * stride, s, 0);
+      a_next[c] = __builtin_amdgcn_raw_buffer_load_b128(r, xoff(c, base, stride), s, 0);
   };
   auto load_scale = [&](auto Dc, int cg, int ktc) {
     constexpr int D = decltype(Dc)::value;
@@ -251,7 +304,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
       if ((i & 1) == 0) xf[NXT][i >> 1] = lds_ld128(xb + (uint32_t)((i >> 1) * 32 * A_LD * 2));
       if (ST) lds_st128(a_wr_nxt + (uint32_t)(i * 16 * A_LD * 2), a_next[i]);
       if (LD) {
-        a_next[i] = __builtin_amdgcn_raw_buffer_load_b128(xr, xo + (uint32_t)i * xst, xs, 0);
+        a_next[i] = __builtin_amdgcn_raw_buffer_load_b128(xr, xoff(i, xo, xst), xs, 0);
         if (i < 4) ring_c[D][i >> 1][i & 1] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff[i >> 1] + (uint32_t)(i & 1) * 512u, wkt * 1024, 0);
         else if (i < 6) load_scale(Dc, i - 4, wkt);
       }
@@ -481,7 +534,8 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
     for (int row = r0; row < kWideRows; row += rstep) {
       if (row >= rows_here || !col_ok) continue;
       u32x4 v = lds_ld128(stage + (uint32_t)((row * sld + ch * 8) * 2));
-      const int64_t o = (m0 + row) * ldy + col0 + ch * 8;
+      const int64_t orow = GROUPED ? (int64_t)a.sorted_route[m0 + row] : m0 + row;
+      const int64_t o = orow * ldy + col0 + ch * 8;
       if (a.epilogue == TNX_EPI_RESIDUAL) {
         const u32x4 res = *reinterpret_cast<const u32x4*>(a.residual + o);
 #pragma unroll

@@ -32,6 +32,7 @@ struct QLArgs {
   const int32_t* offsets;
   const int32_t* sorted_route;
   int x_div;
+  int n_experts;
   int64_t codes_stride, scales_stride;  // per-expert strides in elements
   // fused down-projection of the next linear's adapter (*_MUL epilogue of qgemm128)
   const uint16_t* next_a_t;
@@ -506,6 +507,22 @@ int launch_qgemm_wide(hipStream_t st, const QLArgs& a, const WideHead& h = WideH
   return TNX_OK;
 }
 
+// The grouped form: the grid covers an upper bound of the 128-row blocks, sum over the experts
+// of ceil(rows / 128) <= n_routes / 128 + E (work-groups past the last block exit at once).
+template <int SPT>
+int launch_qgemm_wide_grouped(hipStream_t st, const QLArgs& a) {
+  static std::once_flag once;
+  static int attr_rc = TNX_OK;
+  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm_wide_kernel<SPT, true>, kWideSmemBytes); });
+  if (attr_rc) return attr_rc;
+  const int64_t blocks = a.M / kWideRows + a.n_experts;
+  const unsigned wgs = (unsigned)(blocks * cdiv(a.N, kWideCols));
+  hipLaunchKernelGGL((qgemm_wide_kernel<SPT, true>), dim3(wgs), dim3(256), kWideSmemBytes, st, a,
+                     WideHead{nullptr, nullptr, nullptr, 0, 1.0f});
+  TNX_CHECK_LAUNCH("qgemm_wide_grouped");
+  return TNX_OK;
+}
+
 // Shapes the 128 x 256 kernel takes: enough rows to fill the device with its tiles, no k split,
 // a bf16 output whose rows can be written in 16-byte chunks, and an adapter (if any) of rank
 // <= 64 none of whose 256-column windows touches more than two segments.
@@ -771,6 +788,13 @@ extern "C" int tnx_moe_int4_gmm(void* stream, const tnx_moe_gmm_desc* d) {
   const int64_t max_rows = d->n_routes / d->k;
   const int64_t avg_rows = cdiv(d->n_routes, (int64_t)d->E);
   hipStream_t st = as_stream(stream);
+  a.n_experts = d->E;
+  // Many rows per expert (a prefill, a per-token log-probability pass): the 128 x 256 tiles of
+  // the many-row kernel, one expert's routes per row block.
+  const bool mul = d->epilogue == TNX_EPI_SILU_MUL;
+  if (avg_rows >= 96 && d->N % kWideCols == 0 && (mul ? d->N / 2 : d->N) % 8 == 0 && ((uintptr_t)d->y & 15) == 0 &&
+      (uint64_t)(d->n_routes / d->x_div) * (uint64_t)d->K * 2 < 0xfffff000ull && d->n_routes % d->x_div == 0)
+    return scales_per_tile(d->group) == 2 ? launch_qgemm_wide_grouped<2>(st, a) : launch_qgemm_wide_grouped<4>(st, a);
   if (max_rows <= 16 || avg_rows <= 8) {
     const int cus = device_cus();
     if (moe16_shape(a, d->E, cb, sb, cus)) return launch_moe16(st, a, d->E, cus);
