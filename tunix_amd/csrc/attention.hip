@@ -507,22 +507,39 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
 }
 
 // out[qv, d] = bf16( sum_c e^{m_c - M} O_c[d] / sum_c e^{m_c - M} l_c )
+// The (m, l) pairs of all chunks are fetched at once into LDS (one round trip instead of one
+// dependent load per chunk and pass); every thread then forms M, the weights and the sums in
+// chunk order, with its chunk outputs fetched eight at a time.  (Chunks without a key have
+// l = 0 and an O nobody wrote: selected away, never multiplied.)
 __global__ void attn_combine_kernel(const float* ws, int64_t n_qvec, int dh, int n_chunks,
                                     uint16_t* out) {
+  extern __shared__ float ml[];   // [n_chunks][2]
   const int64_t qv = blockIdx.x;
   const int d = threadIdx.x;
-  if (d >= dh) return;
   const float* p = ws + qv * n_chunks * (dh + 2);
+  for (int i = d; i < 2 * n_chunks; i += blockDim.x) ml[i] = p[(i >> 1) * (dh + 2) + (i & 1)];
+  __syncthreads();
+  if (d >= dh) return;
   float M = kNegBig;
   for (int c = 0; c < n_chunks; ++c)
-    if (p[c * (dh + 2) + 1] > 0.f) M = fmaxf(M, p[c * (dh + 2)]);
+    if (ml[2 * c + 1] > 0.f) M = fmaxf(M, ml[2 * c]);
   float L = 0.f, o = 0.f;
-  for (int c = 0; c < n_chunks; ++c) {
-    const float l = p[c * (dh + 2) + 1];
-    if (l <= 0.f) continue;
-    const float w = __expf(p[c * (dh + 2)] - M);
-    L += w * l;
-    o += w * p[c * (dh + 2) + 2 + d];
+  for (int c0 = 0; c0 < n_chunks; c0 += 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = p[min(c0 + u, n_chunks - 1) * (dh + 2) + 2 + d];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int c = c0 + u;
+      if (c < n_chunks) {
+        const float l = ml[2 * c + 1];
+        if (l > 0.f) {
+          const float w = __expf(ml[2 * c] - M);
+          L += w * l;
+          o += w * v[u];
+        }
+      }
+    }
   }
   out[qv * dh + d] = f2bf(L > 0.f ? o / L : 0.f);
 }
@@ -603,8 +620,8 @@ extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
   TNX_CHECK_LAUNCH("gqa_attn");
   if (a.n_chunks > 1) {
     const int64_t nq = d->B * d->T * d->Hq;
-    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)nq), dim3(d->dh), 0, st, a.ws, nq, d->dh,
-                       a.n_chunks, a.out);
+    hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)nq), dim3(d->dh), (size_t)a.n_chunks * 2 * sizeof(float), st,
+                       a.ws, nq, d->dh, a.n_chunks, a.out);
     TNX_CHECK_LAUNCH("gqa_attn_combine");
   }
   return TNX_OK;
