@@ -393,7 +393,13 @@ class Runner:
     ktiles = f.K // 128
     if blocks >= 200 or M > 128:
       return 1
-    return int(max(1, min(8, ktiles, 256 // blocks)))
+    split = int(max(1, min(8, ktiles, 256 // blocks)))
+    # A gate|up linear that runs unsplit applies its activation itself and can leave the next
+    # linear's adapter down-projection behind: two launches fewer (finishing pass, LoRA down),
+    # ≈ 9 us, against ≈ 1.1 us per k-tile the unsplit work-groups run longer.
+    if f.interleave2 and ktiles - math.ceil(ktiles / split) <= 7:
+      return 1
+    return split
 
   def linear(self, f: FusedLinear, x, y, M, epilogue=L.TNX_EPI_STORE, residual=None, defer=False,
              next_f: FusedLinear | None = None, t_ready: bool = False):
