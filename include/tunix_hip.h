@@ -56,7 +56,8 @@ extern "C" {
 #define TNX_EPI_F32 4       /* y(fp32) = acc, no rounding                                   */
 
 const char* tnx_last_error(void);
-/* Library/ABI version: (major << 16) | minor. */
+/* Library/ABI version: (major << 16) | minor.  The minor number counts additions that leave every
+ * existing entry point as it was (1: tnx_rmsnorm_moe_combine). */
 int tnx_version(void);
 
 /* ---------------------------------------------------------------------------------------

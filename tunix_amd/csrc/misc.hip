@@ -19,7 +19,7 @@ void tnx_set_error(const char* fmt, ...) {
 }
 
 extern "C" const char* tnx_last_error(void) { return g_err; }
-extern "C" int tnx_version(void) { return (1 << 16) | 0; }
+extern "C" int tnx_version(void) { return (1 << 16) | 1; }   // minor 1: tnx_rmsnorm_moe_combine added
 
 namespace {
 
