@@ -798,11 +798,14 @@ extern "C" int tnx_moe_int4_gmm(void* stream, const tnx_moe_gmm_desc* d) {
   if (avg_rows > 24 && d->N % kWideCols == 0 && (mul ? d->N / 2 : d->N) % 8 == 0 && ((uintptr_t)d->y & 15) == 0 &&
       (uint64_t)(d->n_routes / d->x_div) * (uint64_t)d->K * 2 < 0xfffff000ull && d->n_routes % d->x_div == 0)
     return scales_per_tile(d->group) == 2 ? launch_qgemm_wide_grouped<2>(st, a) : launch_qgemm_wide_grouped<4>(st, a);
-  if (max_rows <= 16 || avg_rows <= 8) {
+  // Up to about 12 rows per expert the streaming kernel (16-row blocks, an expert with more
+  // rows streams its weights once per block) beats the 32-row tiles: 87 + 48 against 96 + 56 us
+  // at 10 rows per expert, 90 + 49 against 96 + 58 us at 12, 112 + 54 against 98 + 60 us at 16.
+  if (max_rows <= 16 || avg_rows <= 12) {
     const int cus = device_cus();
     if (moe16_shape(a, d->E, cb, sb, cus)) return launch_moe16(st, a, d->E, cus);
-    return launch_moe<1, 2>(st, a, d->E, max_rows);
   }
+  if (max_rows <= 16 || avg_rows <= 8) return launch_moe<1, 2>(st, a, d->E, max_rows);
   if (max_rows <= 32 || avg_rows <= 24) return launch_moe<2, 2>(st, a, d->E, max_rows);
   return launch_moe<4, 2>(st, a, d->E, max_rows);
 }
