@@ -186,3 +186,24 @@ def test_threefry_seed_mirrors_jax_with_32_bit_integers():
   assert _threefry_seed(-1) == (0, 0xFFFFFFFF)
   assert _threefry_seed(-2 ** 31) == (0, 0x80000000)
   assert _threefry_seed(2 ** 32 + 5) == (0, 5)
+
+
+def test_split_k_choice_of_the_decode_linears():
+  """The k split the model picks per linear (host logic, no GPU): shapes that fill the device
+  run unsplit, few-block shapes split up to 8 ways, and a gate|up linear stays unsplit when the
+  split would save at most 7 k-tiles (its epilogue then replaces the finishing pass and the next
+  linear's LoRA down-projection); the override wins over everything."""
+  import types
+  from tunix_amd.model import Runner
+  m = Runner.__new__(Runner)
+  m.split_k_override = {}
+  lin = lambda name, K, N, il=False: types.SimpleNamespace(names=[f"layers.0.{name}"], K=K, N=N, interleave2=il)
+  assert m._split_k(lin("wq", 4096, 6144), 128) == 5            # Llama-3.1-8B q|k|v: 48 column blocks
+  assert m._split_k(lin("wo", 4096, 4096), 128) == 8
+  assert m._split_k(lin("w_down", 14336, 4096), 128) == 8
+  assert m._split_k(lin("w_gate", 4096, 28672, True), 128) == 1  # 224 blocks fill the device
+  assert m._split_k(lin("w_gate", 1152, 13824, True), 64) == 1   # Gemma3-1B: 108 blocks, a 2-way split saves 4 k-tiles
+  assert m._split_k(lin("w_gate", 4096, 2048, True), 64) == 8    # 16 blocks: the split saves 28 k-tiles
+  assert m._split_k(lin("wq", 4096, 6144), 8192) == 1            # many rows
+  m.split_k_override = {"w_gate": 3}
+  assert m._split_k(lin("w_gate", 1152, 13824, True), 64) == 3
