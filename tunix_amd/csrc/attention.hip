@@ -596,6 +596,8 @@ extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
     TNX_REQUIRE(d->q, "attn: null pointer");
   }
   if (a.n_chunks > 1) TNX_REQUIRE(d->ws, "attn: split key range needs a workspace");
+  // (the combine keeps the chunks' (max, sum) pairs in LDS: 8 bytes per chunk)
+  TNX_REQUIRE(a.n_chunks <= 4096, "attn: %d key chunks (S / kv_chunk), at most 4096", a.n_chunks);
   const int PT = 16 / a.Gp;
   const int64_t QT = cdiv(d->T, PT);
   TNX_REQUIRE(d->B * QT <= 65535 * 32, "attn: too many query tiles");
