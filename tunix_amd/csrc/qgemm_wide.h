@@ -29,7 +29,11 @@
 namespace {
 
 constexpr int kWideRows = 128, kWideCols = 256;
-constexpr size_t kWideSmemBytes = kBigLutBytes + 2 * (size_t)kWideRows * A_LD * 2;
+// LDS: two activation tiles of 128 rows x 128 k (256-byte rows, 16-byte chunks XOR-swizzled by
+// row) at 0 and 32 KB, the table behind them.
+constexpr uint32_t kWideTileBytes = kWideRows * KTILE * 2, kWideLutBase = 2 * kWideTileBytes;
+constexpr size_t kWideSmemBytes = kWideLutBase + kBigLutBytes;
+static_assert(kWideLutBase == 0x10000, "the table look-up forms its address with byte 2 = 1");
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
@@ -47,7 +51,6 @@ template <int SPT, bool GROUPED = false>
 __global__ __launch_bounds__(256)
 void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   constexpr int RT = 4, CG = 2, PF = 3, AP = 8;   // 32-row tiles, 32-column groups per wave
-  constexpr uint32_t ABYTES = kWideRows * A_LD * 2;
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wn = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -60,7 +63,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   asm volatile("" ::"s"(a.t_ld), "s"(a.t), "s"(a.lora_b), "s"(a.lora_scale), "s"(a.epilogue), "s"(a.y),
                "s"(a.residual));
   const float lvl0 = rbf(code_level_imm(a.qtype, tid & 15)), lvl1 = rbf(code_level_imm(a.qtype, (tid >> 4) & 15));
-  const uint32_t lane_off = (uint32_t)lane * 4u;
+  const uint32_t lane_off = (uint32_t)lane * 4u | kWideLutBase;   // byte 2 = 1: the table's base
 
   // work-group id -> (row block, column tile): groups of eight row blocks, the column tile
   // moves every eight ids
@@ -113,8 +116,16 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   // the activation resource starts at this work-group's first row: offsets stay small whatever
   // M is, and rows past M lie beyond the resource and read zeros (GROUPED: the whole buffer,
   // rows are gathered)
-  const rsrc_t rx = GROUPED ? make_rsrc(a.x, (uint64_t)(a.M / a.x_div) * a.K * 2)
-                            : make_rsrc(a.x + m0 * a.K, (uint64_t)rows_here * a.K * 2);
+  // (a raw descriptor in scalar registers: the loads that use it are written in assembly)
+  auto raw_rsrc = [](const void* p, uint64_t bytes) -> u32x4 {
+    const uint64_t q = (uint64_t)p;
+    const uint32_t n = (uint32_t)(bytes > 0xffffffffull ? 0xffffffffull : bytes);
+    return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)q),
+                 (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(q >> 32) & 0xffffu)),
+                 (uint32_t)__builtin_amdgcn_readfirstlane((int)n), 0x00020000u};
+  };
+  const u32x4 rx = GROUPED ? raw_rsrc(a.x, (uint64_t)(a.M / a.x_div) * a.K * 2)
+                           : raw_rsrc(a.x + m0 * a.K, (uint64_t)rows_here * a.K * 2);
   const uint64_t ntk = (uint64_t)ntiles * ktiles;
   const rsrc_t rc = make_rsrc(a.codes + (GROUPED ? (int64_t)expert * a.codes_stride : 0), ntk * 1024);
   const rsrc_t rs = make_rsrc(a.scales + (GROUPED ? (int64_t)expert * a.scales_stride : 0), ntk * 16 * SPT * 2 + 16);
@@ -124,7 +135,13 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   // even slabs (dword u / 2), chunk q = 2 + l / 32 the odd ones.  Column tiles past N start
   // beyond the buffer and read zeros.
   uint32_t coff[CG], soff[CG];
-  const uint32_t xbase = ((uint32_t)(tid >> 4) * (uint32_t)a.K + (uint32_t)(tid & 15) * 8u) * 2u;
+  // Activation tiles go from memory straight into LDS, 16 bytes per lane, a wave's 64 lanes
+  // into 1 KB = four consecutive 256-byte rows.  Thread t fills chunk t % 16 of rows t / 16 + 16 c
+  // (c = 0..7) and fetches for it the k-chunk (t % 16) ^ (row % 16): with the chunks of a row
+  // permuted like that, the 16 lanes that read one k-chunk of 16 consecutive rows for an MFMA
+  // fragment hit 16 different bank groups.
+  const uint32_t chs = (uint32_t)((tid & 15) ^ ((tid >> 4) & 15));
+  const uint32_t xbase = ((uint32_t)(tid >> 4) * (uint32_t)a.K + chs * 8u) * 2u;
   const uint32_t xstride = 16u * (uint32_t)a.K * 2u;  // 16 rows further per pass
   // GROUPED: the byte offset of each of this thread's eight rows (rows the block does not have:
   // beyond the buffer, which reads zeros)
@@ -134,7 +151,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
     for (int c = 0; c < 8; ++c) {
       const int r = (tid >> 4) + 16 * c;
       const int route = r < rows_here ? a.sorted_route[m0 + r] : -1;
-      xrow[c] = route >= 0 ? ((uint32_t)(route / a.x_div) * (uint32_t)a.K + (uint32_t)(tid & 15) * 8u) * 2u : 0xfffff000u;
+      xrow[c] = route >= 0 ? ((uint32_t)(route / a.x_div) * (uint32_t)a.K + chs * 8u) * 2u : 0xfffff000u;
     }
   }
   auto xoff = [&](int c, uint32_t base, uint32_t stride) -> uint32_t {
@@ -156,7 +173,6 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[rt][cg][i] = 0.f;
 
-  u32x4 a_next[AP];
   u32x4 ring_c[PF][CG][2];   // [.][.][0]: even slabs, [1]: odd slabs
   u32x2 ring_s[PF][CG];
   float sc[PF][CG][SPT];
@@ -206,22 +222,33 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
     for (int u = 0; u < 4; ++u) lbv[cg][u] = u32x4{0, 0, 0, 0};
   uint32_t tbase = 0;
   if (lora) {
-    const int ch = tid & 15;
+    const int ch = (int)chs;
     const int col = ((ch < 8) ? toff_a : toff_b) + min((ch & 7) * 8, a.lora_rank - 8);
     tbase = (uint32_t)((tid >> 4) * a.t_ld + col) * 2u;
   }
-  const rsrc_t rt_ = lora ? make_rsrc(a.t + m0 * a.t_ld, (uint64_t)rows_here * a.t_ld * 2) : rx;
+  const u32x4 rt_ = lora ? raw_rsrc(a.t + m0 * a.t_ld, (uint64_t)rows_here * a.t_ld * 2) : rx;
   const uint32_t tstride = (uint32_t)(16 * a.t_ld * 2);
 
-  auto load_a = [&](int kt) {
+  // One 16-byte-per-lane load into LDS at `lds` + 16 * lane (M0 carries the wave's base).  The
+  // compiler does not count these loads: its own waits for other loads can only turn out
+  // longer than needed (loads complete in order), and the waits for these are written by hand.
+  auto dma16 = [&](uint32_t lds, const u32x4& r, uint32_t voff, int soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds), "v"(voff), "s"(r), "s"(soff) : "memory", "m0");
+  };
+  const uint32_t dma_wave = (uint32_t)wn * 1024u;      // this wave's four rows within a 16-row pass
+  auto sel_rsrc = [&](bool ut) -> u32x4 {
+    const uint32_t m = 0u - (uint32_t)ut;
+    return u32x4{rx[0] ^ ((rx[0] ^ rt_[0]) & m), rx[1] ^ ((rx[1] ^ rt_[1]) & m), rx[2] ^ ((rx[2] ^ rt_[2]) & m), rx[3]};
+  };
+  auto load_a = [&](int kt, uint32_t buf) {
     const bool ut = lora && kt >= ktiles;
     const int s = ut ? 0 : min(kt, ktiles - 1) * (KTILE * 2);
-    const rsrc_t r = ut ? rt_ : rx;
+    const u32x4 r = sel_rsrc(ut);
     const uint32_t m = 0u - (uint32_t)ut;
     const uint32_t base = xbase ^ ((xbase ^ tbase) & m), stride = xstride ^ ((xstride ^ tstride) & m);
 #pragma unroll
-    for (int c = 0; c < AP; ++c)
-      a_next[c] = __builtin_amdgcn_raw_buffer_load_b128(r, xoff(c, base, stride), s, 0);
+    for (int c = 0; c < AP; ++c) dma16(buf + dma_wave + (uint32_t)c * 4096u, r, xoff(c, base, stride), s);
   };
   auto load_scale = [&](auto Dc, int cg, int ktc) {
     constexpr int D = decltype(Dc)::value;
@@ -252,35 +279,34 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
       }
     }
   };
-  uint32_t a_rd = kBigLutBytes + (uint32_t)(l32 * A_LD + lh * 8) * 2u;
-  uint32_t a_rd_nxt = a_rd + ABYTES;
-  uint32_t a_wr = kBigLutBytes + (uint32_t)((tid >> 4) * A_LD + (tid & 15) * 8) * 2u;
-  uint32_t a_wr_nxt = a_wr + ABYTES;
-  auto store_a = [&](uint32_t base) {
+  // Fragment addresses: slab u wants k-chunk 2 u + l / 32 of row l % 32 (+ 32 per row tile, an
+  // immediate).  xaddr[u] points into the tile slab u is read from next and flips to the other
+  // tile after each use; slab 0 is read one tile ahead (by slab 7 of the tile before).
+  uint32_t xaddr[8];
 #pragma unroll
-    for (int c = 0; c < AP; ++c) lds_st128(base + (uint32_t)(c * 16 * A_LD * 2), a_next[c]);
-  };
+  for (int u = 0; u < 8; ++u)
+    xaddr[u] = (uint32_t)l32 * 256u + (((uint32_t)(2 * u + lh) ^ (uint32_t)(l32 & 15)) * 16u) + (u == 0 ? kWideTileBytes : 0u);
+  uint32_t dma_buf = 0;     // the tile buffer that slab 7 of the current k-tile refills
 
   // One slab (16 k) = eight slots, one MFMA each (column group i / 4, row tile i % 4), written
   // in the order they should issue.  Slot i also carries, for code pair (group i / 4, byte i % 4):
   // the two f16 x scale products and the bf16 pack of that pair of the NEXT slab's weights, the
   // table look-up (address: one v_perm) of the same pair of the slab AFTER the next, which
   // overwrites the entry just consumed, and in even slots an activation fragment read for the
-  // next slab.  Slab 5 expands the next k-tile's scales, slab 6 stores the next activation tile
-  // (fetched by slab 7 of the tile before), the barrier sits between slabs 6 and 7 (the
-  // fragments slab 7 reads are the next tile's), and slab 7 issues the global loads:
-  // activations of k-tile kt + 2, weights of k-tile kt + PF into the ring stage this tile has
-  // finished with.
+  // next slab.  Slab 5 expands the next k-tile's scales; slab 6 requests the weights of k-tile
+  // kt + PF into the ring stage this tile has finished with; the barrier sits between slabs 6
+  // and 7 (the fragments slab 7 reads are the next tile's, requested by slab 7 of the tile
+  // before); slab 7 requests the activations of k-tile kt + 2 into the tile buffer this k-tile
+  // has been read from (every wave's fragment reads of it completed before the barrier).
   auto slab = [&](auto Uc, auto Dc, int kt, bool next_active) {
     constexpr int U = decltype(Uc)::value, D = decltype(Dc)::value, DN = (D + 1) % PF;
     constexpr int CUR = U & 1, NXT = CUR ^ 1;
     constexpr int UC = (U + 1) & 7, DC = U < 7 ? D : DN;   // slab whose weights are converted here
     constexpr int UL = (U + 2) & 7, DL = U < 6 ? D : DN;   // slab whose table entries are fetched here
-    constexpr bool ST = U == 6, LD = U == 7, EX = U == 5;
-    const uint32_t xb = (U < 7 ? a_rd : a_rd_nxt) + (uint32_t)(UC * 16 * 2);
+    constexpr bool LW = U == 6, LD = U == 7, EX = U == 5;
     const bool ut = lora && kt + 2 >= ktiles;      // LD: the activation tile to fetch is the adapter block
     const int xs = ut ? 0 : min(kt + 2, ktiles - 1) * (KTILE * 2);
-    const rsrc_t xr = ut ? rt_ : rx;
+    const u32x4 xr = LD ? sel_rsrc(ut) : rx;
     const uint32_t um = 0u - (uint32_t)ut;
     const uint32_t xo = xbase ^ ((xbase ^ tbase) & um), xst = xstride ^ ((xstride ^ tstride) & um);
     const int wkt = min(kt + PF, ktiles - 1);
@@ -299,12 +325,12 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
         cf0 = __builtin_fmaf((float)hh[0], sv, 0.0f);
         cf1 = __builtin_fmaf((float)hh[1], sv, 0.0f);
         const uint32_t w = ring_c[DL][cg][UL & 1][UL >> 1];
-        lp[cg][rt] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0400u + ((uint32_t)rt << 8)));
+        lp[cg][rt] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020400u + ((uint32_t)rt << 8)));
       }
-      if ((i & 1) == 0) xf[NXT][i >> 1] = lds_ld128(xb + (uint32_t)((i >> 1) * 32 * A_LD * 2));
-      if (ST) lds_st128(a_wr_nxt + (uint32_t)(i * 16 * A_LD * 2), a_next[i]);
-      if (LD) {
-        a_next[i] = __builtin_amdgcn_raw_buffer_load_b128(xr, xoff(i, xo, xst), xs, 0);
+      if ((i & 1) == 0) xf[NXT][i >> 1] = lds_ld128(xaddr[UC] + (uint32_t)((i >> 1) * 32 * 256));
+      if (i == 7) xaddr[UC] ^= kWideTileBytes;
+      if (LD) dma16(dma_buf + dma_wave + (uint32_t)i * 4096u, xr, xoff(i, xo, xst), xs);
+      if (LW) {
         if (i < 4) ring_c[D][i >> 1][i & 1] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff[i >> 1] + (uint32_t)(i & 1) * 512u, wkt * 1024, 0);
         else if (i < 6) load_scale(Dc, i - 4, wkt);
       }
@@ -326,27 +352,28 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
     slab(ic<4>{}, Dc, kt, next_active);
     slab(ic<5>{}, Dc, kt, next_active);
     slab(ic<6>{}, Dc, kt, next_active);
+    // the next tile's activations, requested by slab 7 of the tile before, have landed in LDS:
+    // the only younger loads are the six weight / scale loads slab 6 has just issued
+    __builtin_amdgcn_s_waitcnt(0x0f70 | 6);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     slab(ic<7>{}, Dc, kt, next_active);
-    const uint32_t r = a_rd; a_rd = a_rd_nxt; a_rd_nxt = r;
-    const uint32_t w = a_wr; a_wr = a_wr_nxt; a_wr_nxt = w;
+    dma_buf ^= kWideTileBytes;
   };
 
   // (order of the first loads: each is followed by at least as many later loads as it will be
   // in the steady state of the loop, so the counted waits of the loop body never have to fall
   // back to "everything outstanding" for the sake of the path that enters from here)
-  load_a(0);
+  load_a(0, 0u);
   load_w(ic<0>{}, 0);
   {  // table entry e = f16 pair (level[e & 15], level[e >> 4]), 64 copies rotated over the banks
-    uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
+    uint32_t* lut = reinterpret_cast<uint32_t*>(smem + kWideLutBase);
     const h16x2 h = {(_Float16)lvl0, (_Float16)lvl1};
     const uint32_t v = __builtin_bit_cast(uint32_t, h);
 #pragma unroll
     for (int c = 0; c < 64; ++c) lut[tid * 64 + ((c + lane) & 63)] = v;
   }
-  store_a(a_wr);
-  load_a(1);
+  load_a(1, kWideTileBytes);
   load_w(ic<1>{}, 1);
   load_w(ic<2>{}, 2);
   if (lora) {
@@ -360,15 +387,18 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
                                         (uint32_t)(u * 16 + lh * 8)) * 2u);
   }
   expand_scales(ic<0>{}, true);
+  // the first tile is in LDS: its eight loads are the oldest, and at least 26 follow them (three
+  // ring stages of six, the second tile's eight); vmcnt(20) also covers the first ring stage
+  __builtin_amdgcn_s_waitcnt(0x0f70 | (20 & 15) | ((20 >> 4) << 14));
   __syncthreads();
   // slab 0: table entries, conversion, fragments; then the table entries of slab 1
 #pragma unroll
   for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
     for (int b = 0; b < 4; ++b)
-      lp[cg][b] = lds_ld32(__builtin_amdgcn_perm(ring_c[0][cg][0][0], lane_off, 0x0c0c0400u + ((uint32_t)b << 8)));
+      lp[cg][b] = lds_ld32(__builtin_amdgcn_perm(ring_c[0][cg][0][0], lane_off, 0x0c020400u + ((uint32_t)b << 8)));
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) xf[0][rt] = lds_ld128(a_rd + (uint32_t)(rt * 32 * A_LD * 2));
+  for (int rt = 0; rt < RT; ++rt) xf[0][rt] = lds_ld128((xaddr[0] ^ kWideTileBytes) + (uint32_t)(rt * 32 * 256));
 #pragma unroll
   for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
@@ -383,7 +413,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
     for (int b = 0; b < 4; ++b)
-      lp[cg][b] = lds_ld32(__builtin_amdgcn_perm(ring_c[0][cg][1][0], lane_off, 0x0c0c0400u + ((uint32_t)b << 8)));
+      lp[cg][b] = lds_ld32(__builtin_amdgcn_perm(ring_c[0][cg][1][0], lane_off, 0x0c020400u + ((uint32_t)b << 8)));
   // whole turns of the ring without a branch inside (a conditional tile would make the waits
   // of the tile after it assume that its loads never happened), then the one or two tiles left
   int kt = 0;
@@ -398,7 +428,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   }
 
   if (lora) {
-    // The t block sits in the activation buffer the last k-tile left as "next" (now a_rd).  The
+    // The t block is k-tile number ktiles: it sits in tile buffer ktiles % 2.  The
     // two 16-column halves of a group may belong to different adapters (always so for a
     // gate | up pair): one pass per half then, the other half's lanes contributing zeros.
 #pragma unroll
@@ -410,7 +440,8 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) part[rt][i] = 0.f;
       for (int p = 0; p < (same ? 1 : 2); ++p) {
-        const uint32_t base = a_rd + (uint32_t)((toff[2 * cg + p] == toff_a ? 0 : 64) * 2);
+        const uint32_t half = toff[2 * cg + p] == toff_a ? 0u : 8u;   // first 16-byte chunk of the segment's 64 columns
+        const uint32_t base = (uint32_t)(ktiles & 1) * kWideTileBytes + (uint32_t)l32 * 256u;
         const bool mine = same || (l32 >> 4) == p;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -418,7 +449,8 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
             const u32x4 lb = mine ? lbv[cg][u] : u32x4{0, 0, 0, 0};
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt)
-              part[rt] = mfma32(lb, lds_ld128(base + (uint32_t)((rt * 32 * A_LD + u * 16) * 2)), part[rt]);
+              part[rt] = mfma32(lb, lds_ld128(base + (uint32_t)(rt * 32 * 256) +
+                                              (((half + (uint32_t)(2 * u + lh)) ^ (uint32_t)(l32 & 15)) * 16u)), part[rt]);
           }
         }
       }
@@ -428,6 +460,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
         for (int i = 0; i < 16; ++i) acc[rt][cg][i] += a.lora_scale * part[rt][i];
     }
   }
+  __builtin_amdgcn_s_waitcnt(0x0f70);   // no load into LDS is still on its way
   __syncthreads();  // every wave is done with the activation buffers: they become the output stage
 
   // The bf16 tile goes through LDS (row stride cols + 8 elements) and leaves as 16-byte chunks
@@ -436,7 +469,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   const bool mul = a.epilogue == TNX_EPI_SILU_MUL || a.epilogue == TNX_EPI_GELU_MUL;
   const int cols = mul ? kWideCols / 2 : kWideCols;      // output columns of the work-group
   const int sld = cols + 8;
-  const uint32_t stage = kBigLutBytes;
+  const uint32_t stage = 0;   // 128 rows x (256 + 8) columns: over both tiles and into the table, all dead now
   if (mul) {
     // a group is [16 gate columns | 16 up columns]: registers 4 b + e (b < 2) and 4 (b + 2) + e
 #pragma unroll
