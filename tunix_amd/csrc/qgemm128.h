@@ -29,9 +29,13 @@ typedef __attribute__((address_space(3))) uint32_t lds_u32;
 typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
 
 constexpr int kBigLutBytes = 256 * 256;
-// table, two activation buffers of max(32, rows) rows, adapter fragments (2 KiB per column tile)
-constexpr size_t big_abytes(int mt) { return (size_t)(mt < 2 ? 32 : 16 * mt) * A_LD * 2; }
-constexpr size_t big_smem_bytes(int nt, int mt) { return kBigLutBytes + 2 * big_abytes(mt) + 4 * (size_t)nt * 2048; }
+// LDS: two activation tiles of max(32, rows) rows x 128 k (256-byte rows whose 16-byte chunks
+// are XOR-swizzled by row) from address 0, the table at 64 KiB, adapter fragments (2 KiB per
+// column tile) behind it
+constexpr uint32_t kBigLutBase = 0x10000, kBigAdapterBase = kBigLutBase + kBigLutBytes;
+constexpr size_t big_abytes(int mt) { return (size_t)(mt < 2 ? 32 : 16 * mt) * KTILE * 2; }
+constexpr size_t big_smem_bytes(int nt, int mt) { return kBigAdapterBase + 4 * (size_t)nt * 2048; }
+static_assert(2 * big_abytes(8) <= kBigLutBase, "the activation tiles end where the table starts");
 
 // LDS accesses by absolute LDS byte address (the dynamic LDS block of these kernels starts at
 // address 0: they declare no static LDS).
@@ -93,7 +97,7 @@ void qgemm128_kernel(const QLArgs a) {
   // the two code-book levels of this thread's table entry, from literals: nothing at the start
   // of the kernel waits on memory except the loads of the first tiles
   const float lvl0 = rbf(code_level_imm(a.qtype, tid & 15)), lvl1 = rbf(code_level_imm(a.qtype, (tid >> 4) & 15));
-  const uint32_t lane_off = (uint32_t)lane * 4u;
+  const uint32_t lane_off = (uint32_t)lane * 4u | kBigLutBase;   // byte 2 = 1: the table's base
   const int64_t m0 = (int64_t)blockIdx.x * ROWS;
   const int64_t ntile0 = ((int64_t)blockIdx.y * 4 + wn) * NT;
   const int64_t ntiles = a.N / 16;
@@ -101,7 +105,15 @@ void qgemm128_kernel(const QLArgs a) {
   const int kt_begin = blockIdx.z * a.ktiles_per_split;
   const int kt_end = min(ktiles, kt_begin + a.ktiles_per_split);
 
-  const rsrc_t rx = make_rsrc(a.x, (uint64_t)a.M * a.K * 2);
+  // (raw descriptors in scalar registers: the loads that use them are written in assembly)
+  auto raw_rsrc = [](const void* p, uint64_t bytes) -> u32x4 {
+    const uint64_t q = (uint64_t)p;
+    const uint32_t n = (uint32_t)(bytes > 0xffffffffull ? 0xffffffffull : bytes);
+    return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)q),
+                 (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(q >> 32) & 0xffffu)),
+                 (uint32_t)__builtin_amdgcn_readfirstlane((int)n), 0x00020000u};
+  };
+  const u32x4 rx = raw_rsrc(a.x, (uint64_t)a.M * a.K * 2);
   const uint64_t ntk = (uint64_t)ntiles * ktiles;
   const rsrc_t rc = make_rsrc(a.codes, ntk * 1024);
   const rsrc_t rs = make_rsrc(a.scales, ntk * 16 * SPT * 2 + 16);
@@ -109,7 +121,21 @@ void qgemm128_kernel(const QLArgs a) {
   // scalar offset of the load.  Rows past M and column tiles past N start beyond the buffer
   // and read zeros.  A lane's 16 bytes of codes are four k-steps: this wave takes its half.
   uint32_t coff[NT], soff[NT];
-  const uint32_t xbase = ((uint32_t)(m0 + (tid >> 4)) * (uint32_t)a.K + (uint32_t)(tid & 15) * 8u) * 2u;
+  // Activation tiles go from memory straight into LDS, 16 bytes per lane: a wave's 64 lanes fill
+  // 1 KB = four consecutive 256-byte rows, the 512 threads 32 rows per pass.  Thread t fills
+  // chunk t % 16 of rows t / 16 + 32 c and fetches for it the k-chunk (t % 16) ^ (row % 16):
+  // the 16 lanes that read one k-chunk of 16 consecutive rows for an MFMA fragment then hit 16
+  // different bank groups.
+  const uint32_t chs = (uint32_t)((tid & 15) ^ ((tid >> 4) & 15));
+  const uint32_t xbase = ((uint32_t)(m0 + (tid >> 4)) * (uint32_t)a.K + chs * 8u) * 2u;
+  // One 16-byte-per-lane load into LDS at `lds` + 16 * lane (M0 carries the wave's base).  The
+  // compiler does not count these loads: its own waits for other loads can only turn out
+  // longer than needed (loads complete in order), and the waits for these are written by hand.
+  auto dma16 = [&](uint32_t lds, const u32x4& r, uint32_t voff, int soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds), "v"(voff), "s"(r), "s"(soff) : "memory", "m0");
+  };
+  const uint32_t dma_wave = (uint32_t)wv * 1024u;      // this wave's four rows within a 32-row pass
   const uint32_t xstride = 32u * (uint32_t)a.K * 2u;  // 32 rows further per chunk
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
@@ -125,7 +151,6 @@ void qgemm128_kernel(const QLArgs a) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) zero_acc(acc[mt][nt]);
 
-  u32x4 a_next[AP];
   u32x2 ring_c[PF][NT];
   uint32_t ring_s[PF][NT];
   float sc[PF][NT][SW];   // the scales of a ring stage as fp32
@@ -143,13 +168,11 @@ void qgemm128_kernel(const QLArgs a) {
     }
   };
   // What the first k-tile needs is requested here, ahead of the adapter bookkeeping below (a
-  // few hundred scalar and vector instructions that touch no memory).  The first activation
-  // tile has registers of its own (live only up to its store).
-  u32x4 a_first[AP];
+  // few hundred scalar and vector instructions that touch no memory).
   if (kt_begin < kt_end) {
 #pragma unroll
     for (int c = 0; c < AP; ++c)
-      a_first[c] = __builtin_amdgcn_raw_buffer_load_b128(rx, xbase + (uint32_t)c * xstride, kt_begin * (KTILE * 2), 0);
+      dma16(dma_wave + (uint32_t)c * 8192u, rx, xbase + (uint32_t)c * xstride, kt_begin * (KTILE * 2));
     load_w(ic<0>{}, kt_begin);
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -200,7 +223,7 @@ void qgemm128_kernel(const QLArgs a) {
   // B^T fragments of the adapter for this column group: fetched now, parked in the group's
   // 4 KiB of LDS behind the activation buffers until the epilogue (both waves of the group
   // write the same values; the barriers of the main loop order them before the reads)
-  const uint32_t lb_lds = kBigLutBytes + 2 * ABYTES + (uint32_t)wn * (uint32_t)(NT * 2048) + (uint32_t)lane * 16u;
+  const uint32_t lb_lds = kBigAdapterBase + (uint32_t)wn * (uint32_t)(NT * 2048) + (uint32_t)lane * 16u;
   uint32_t tbase = 0;
   u32x4 lbv[NT][2];  // live only until the main loop starts
 #pragma unroll
@@ -220,25 +243,28 @@ void qgemm128_kernel(const QLArgs a) {
                                         (uint32_t)(j * 32 + lq * 8)) * 2u);
   };
   if (lora_fast) {
-    const int ch = tid & 15;
+    const int ch = (int)chs;
     const int col = ((ch < 8) ? toff_a : toff_b) + min((ch & 7) * 8, a.lora_rank - 8);
     tbase = (uint32_t)((m0 + (tid >> 4)) * a.t_ld + col) * 2u;
   }
-  const rsrc_t rt = make_rsrc(lora_fast ? (const void*)a.t : (const void*)a.x,
-                              lora_fast ? (uint64_t)a.M * a.t_ld * 2 : (uint64_t)a.M * a.K * 2);
+  const u32x4 rt = raw_rsrc(lora_fast ? (const void*)a.t : (const void*)a.x,
+                            lora_fast ? (uint64_t)a.M * a.t_ld * 2 : (uint64_t)a.M * a.K * 2);
+  auto sel_rsrc = [&](bool ut) -> u32x4 {
+    const uint32_t m = 0u - (uint32_t)ut;
+    return u32x4{rx[0] ^ ((rx[0] ^ rt[0]) & m), rx[1] ^ ((rx[1] ^ rt[1]) & m), rx[2] ^ ((rx[2] ^ rt[2]) & m), rx[3]};
+  };
   const uint32_t tstride = (uint32_t)(32 * a.t_ld * 2);
 
   // k-tiles past the last one are clamped: their data is fetched but never multiplied
-  auto load_a = [&](int kt) {
+  auto load_a = [&](int kt, uint32_t buf) {
     const bool ut = lora_fast && kt >= kt_end;
     const int s = ut ? 0 : min(kt, ktiles - 1) * (KTILE * 2);
-    const rsrc_t r = ut ? rt : rx;
+    const u32x4 r = sel_rsrc(ut);
     // bit selects (not ?:, which the compiler turns into a private-memory table)
     const uint32_t m = 0u - (uint32_t)ut;
     const uint32_t base = xbase ^ ((xbase ^ tbase) & m), stride = xstride ^ ((xstride ^ tstride) & m);
 #pragma unroll
-    for (int c = 0; c < AP; ++c)
-      a_next[c] = __builtin_amdgcn_raw_buffer_load_b128(r, base + (uint32_t)c * stride, s, 0);
+    for (int c = 0; c < AP; ++c) dma16(buf + dma_wave + (uint32_t)c * 8192u, r, base + (uint32_t)c * stride, s);
   };
   // scales of ring stage D -> fp32; a k-tile past the end gets zero scales, which turns its
   // weights into zeros
@@ -262,11 +288,11 @@ void qgemm128_kernel(const QLArgs a) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       const uint32_t w = ring_c[D][nt][J];
-      // address bytes: [0] = lane * 4, [1] = code byte b of w, [2] = [3] = 0
-      dst[nt][0] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0400u));
-      dst[nt][1] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0500u));
-      dst[nt][2] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0600u));
-      dst[nt][3] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0700u));
+      // address bytes: [0] = lane * 4, [1] = code byte b of w, [2] = 1 (the table's base), [3] = 0
+      dst[nt][0] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020400u));
+      dst[nt][1] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020500u));
+      dst[nt][2] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020600u));
+      dst[nt][3] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020700u));
     }
   };
   // f16 level pair x fp32 scale -> bf16 pair
@@ -284,32 +310,25 @@ void qgemm128_kernel(const QLArgs a) {
       dst[nt] = r;
     }
   };
-  // LDS byte addresses of the two activation buffers as this lane reads (its k half) / writes them
-  uint32_t a_rd = kBigLutBytes + (uint32_t)(lm * A_LD + lq * 8 + kh * 64) * 2u;
-  uint32_t a_rd_nxt = a_rd + ABYTES;
-  uint32_t a_wr = kBigLutBytes + (uint32_t)((tid >> 4) * A_LD + (tid & 15) * 8) * 2u;
-  uint32_t a_wr_nxt = a_wr + ABYTES;
-  auto read_a = [&](u32x4 (&dst)[MT], uint32_t base, auto Jc) {
-    constexpr int J = decltype(Jc)::value;
-#pragma unroll
-    for (int m = 0; m < MT; ++m) dst[m] = lds_ld128(base + (uint32_t)((m * 16 * A_LD + J * 32) * 2));
-  };
-  // (with fewer than 32 rows the copy still moves 32: the extra rows are zeros or rows of
-  // nobody's tile, and land in LDS rows no fragment reads)
-  auto store_a = [&](uint32_t base) {
-#pragma unroll
-    for (int c = 0; c < AP; ++c) lds_st128(base + (uint32_t)(c * 32 * A_LD * 2), a_next[c]);
-  };
+  // LDS byte addresses of this lane's fragments: row l % 16 (+ 16 per row tile, an immediate),
+  // k-chunk 8 kh + 4 J + l / 16 of the wave's k-step J, swizzled by the row; the other step of
+  // the same tile is 64 bytes away under XOR.  a_cur1: step 1 of the current tile, a_nxt0: step 0
+  // of the next one (the two the loop reads); they trade places, and steps, after every k-tile.
+  // (With fewer than 32 rows a pass still moves 32: the extra rows are zeros or rows of nobody's
+  // tile, and land in LDS rows no fragment reads.)
+  uint32_t a_cur1 = (uint32_t)lm * 256u + (((uint32_t)(kh * 8 + 4 + lq) ^ (uint32_t)lm) * 16u);
+  uint32_t a_nxt0 = (a_cur1 ^ 64u) + ABYTES;
+  uint32_t dma_buf = 0;     // the tile buffer the second step of the current k-tile refills
   // One of this wave's two k-steps, written as NT * 8 units in the order they should issue: two
   // units per code pair of the step.  The MT * NT MFMAs are spread evenly over the units
   // (column tile-major: the first MT use the column tile whose conversion finished first).  An
   // even unit forms the two f16 x scale products of its pair of the NEXT step's weights, the odd
   // unit packs them to bf16.  The first half of the units also carries the LDS reads: one table
   // look-up each (pair u of the step AFTER the next, into the other half of lp) and the
-  // activation fragments of the next step; the second half the stores of the next activation
-  // tile (ST, first step: issued seven units before the barrier behind the step asks for them),
-  // followed at once by the loads of the activation tile after that one into the same registers
-  // (a whole k-tile before their store), or the weight loads (LD, second step).
+  // activation fragments of the next step; the second half the requests to memory: the weights of
+  // k-tile kt + PF into this tile's ring stage (ST, first step, ahead of the barrier), or the
+  // activations of k-tile kt + 2 into this tile's LDS buffer (LD, second step: behind the
+  // barrier, when no wave reads that buffer any more).
   // A scheduling barrier behind every unit keeps that order.
   auto kstep = [&](auto CURc, auto Dcc, auto Jcc, auto Dlc, auto Jlc, uint32_t rd_base, auto Jrc, auto STc,
                    auto LDc, auto EXc, int kt, bool ex_active) {
@@ -323,7 +342,7 @@ void qgemm128_kernel(const QLArgs a) {
     float f0 = 0.f, f1 = 0.f;
     const bool ut = lora_fast && kt >= kt_end;      // LD: the activation tile to fetch is the adapter block
     const int xs = ut ? 0 : min(kt, ktiles - 1) * (KTILE * 2);
-    const rsrc_t xr = ut ? rt : rx;
+    const u32x4 xr = sel_rsrc(ut);
     const uint32_t um = 0u - (uint32_t)ut;
     const uint32_t xo = xbase ^ ((xbase ^ tbase) & um), xst = xstride ^ ((xstride ^ tstride) & um);
     const int wkt = min(kt + (PF - 2), ktiles - 1);   // LD: weights of k-tile (this + PF)
@@ -344,18 +363,14 @@ void qgemm128_kernel(const QLArgs a) {
       }
       if (u < UNITS / 2) {   // all LDS reads in the first half: nothing of them is in flight at the barrier
         lp[NXT][u >> 2][u & 3] =
-            lds_ld32(__builtin_amdgcn_perm(ring_c[DL][u >> 2][JL], lane_off, 0x0c0c0400u + ((uint32_t)(u & 3) << 8)));
-        if (u < MT) af[NXT][u] = lds_ld128(rd_base + (uint32_t)((u * 16 * A_LD + JR * 32) * 2));
+            lds_ld32(__builtin_amdgcn_perm(ring_c[DL][u >> 2][JL], lane_off, 0x0c020400u + ((uint32_t)(u & 3) << 8)));
+        if (u < MT) af[NXT][u] = lds_ld128(rd_base + (uint32_t)(u * 16 * 256));
       } else {
         const int q = u - UNITS / 2;
-        if (ST && q == 0) {
-#pragma unroll
-          for (int c = 0; c < AP; ++c) lds_st128(a_wr_nxt + (uint32_t)(c * 32 * A_LD * 2), a_next[c]);
-        }
-        if (ST && q >= 1 && q <= AP)   // the registers just stored take the activation tile after the next
-          a_next[q - 1] = __builtin_amdgcn_raw_buffer_load_b128(xr, xo + (uint32_t)(q - 1) * xst, xs, 0);
-        if (LD) {
-          constexpr int DW = DL == 0 ? PF - 1 : DL - 1;   // the ring stage this k-tile has finished with
+        if (LD && q >= 1 && q <= AP)   // (after the barrier: every wave has read this tile's fragments)
+          dma16(dma_buf + dma_wave + (uint32_t)(q - 1) * 8192u, xr, xo + (uint32_t)(q - 1) * xst, xs);
+        if (ST) {
+          constexpr int DW = DC;   // the ring stage of this k-tile: all its codes have been looked up
           if (q >= 4 && q < 4 + NT) {
             ring_c[DW][q - 4] = __builtin_amdgcn_raw_buffer_load_b64(rc, coff[q - 4], wkt * 1024, 0);
           } else if (q >= 4 + NT && q < 4 + 2 * NT) {
@@ -381,30 +396,32 @@ void qgemm128_kernel(const QLArgs a) {
 
   // One k-tile of ring stage D = this wave's two k-steps.  On entry af[0] holds the activation
   // fragments of the first step, bfr[0] its weights and lp the table entries of the second.
-  // The one barrier of the k-tile sits between the steps (every wave has finished reading this
-  // tile and stored the next).  The first step fetches the activations of k-tile kt + 2, the
-  // second the weights of k-tile kt + PF into the ring stage this tile has finished with.
+  // The one barrier of the k-tile sits between the steps: every wave has finished reading this
+  // tile, and the next tile, requested by the second step of the tile before, has landed in LDS
+  // (the only younger loads are the 2 NT weight / scale loads the first step has just issued).
   auto tile = [&](auto Dc, int kt) {
     constexpr int d = decltype(Dc)::value, dn = (d + 1) % PF;
     const bool next_active = kt + 1 < kt_end;
     __builtin_amdgcn_sched_barrier(0);
-    kstep(ic<0>{}, Dc, ic<1>{}, ic<dn>{}, ic<0>{}, a_rd, ic<1>{}, ic<1>{}, ic<0>{}, ic<dn>{}, kt + 2, next_active);
+    kstep(ic<0>{}, Dc, ic<1>{}, ic<dn>{}, ic<0>{}, a_cur1, ic<1>{}, ic<1>{}, ic<0>{}, ic<dn>{}, kt + 2, next_active);
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * NT));
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
-    kstep(ic<1>{}, ic<dn>{}, ic<0>{}, ic<dn>{}, ic<1>{}, a_rd_nxt, ic<0>{}, ic<0>{}, ic<1>{}, ic<-1>{}, kt + 2, false);
-    const uint32_t r = a_rd; a_rd = a_rd_nxt; a_rd_nxt = r;
-    const uint32_t w = a_wr; a_wr = a_wr_nxt; a_wr_nxt = w;
+    kstep(ic<1>{}, ic<dn>{}, ic<0>{}, ic<dn>{}, ic<1>{}, a_nxt0, ic<0>{}, ic<0>{}, ic<1>{}, ic<-1>{}, kt + 2, false);
+    const uint32_t r = a_cur1;
+    a_cur1 = a_nxt0 ^ 64u;
+    a_nxt0 = r ^ 64u;
+    dma_buf ^= ABYTES;
   };
 
   if (kt_begin < kt_end) {
     // Order of the first loads: each is followed by at least as many later loads as it will be
     // in the steady state of the loop, so the counted waits of the loop body need not fall back
-    // to "everything outstanding" for the sake of the path that enters from here.  The first
-    // activation tile has registers of its own for that (live only up to its store).
+    // to "everything outstanding" for the sake of the path that enters from here.
     TNX_STAMP(7);
     {  // table entry e = f16 pair (level[e & 15], level[e >> 4]); copies rotated over banks,
        // half of them per thread; built while the first loads are in flight
-      uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
+      uint32_t* lut = reinterpret_cast<uint32_t*>(smem + kBigLutBase);
       const h16x2 h = {(_Float16)lvl0, (_Float16)lvl1};
       const uint32_t v = __builtin_bit_cast(uint32_t, h);
       const int e = tid & 255, c0 = (tid >> 8) * 32;
@@ -416,17 +433,19 @@ void qgemm128_kernel(const QLArgs a) {
     // memory queue, and the first tile is multiplied while the second one's data arrives.
     __builtin_amdgcn_sched_barrier(0);
     load_w(ic<1>{}, kt_begin + 1);
-    load_a(kt_begin + 1);
+    load_a(kt_begin + 1, ABYTES);
     load_w(ic<2>{}, kt_begin + 2);
     if (lora_fast) load_adapter_b();
     __builtin_amdgcn_sched_barrier(0);
     TNX_STAMP(1);
-#pragma unroll
-    for (int c = 0; c < AP; ++c) lds_st128(a_wr + (uint32_t)(c * 32 * A_LD * 2), a_first[c]);
     expand_scales(ic<0>{}, true);
+    // the first tile's AP loads are the oldest in flight; at least 3 x 2 NT weight / scale loads
+    // and the second tile's AP follow them
+    __builtin_amdgcn_s_waitcnt(0x0f70 | ((6 * NT + AP) & 15) | (((6 * NT + AP) >> 4) << 14));
     __syncthreads();  // table and first activation tile
     lut_issue(ic<0>{}, ic<0>{}, lp[1]);
-    read_a(af[0], a_rd, ic<0>{});
+#pragma unroll
+    for (int m = 0; m < MT; ++m) af[0][m] = lds_ld128((a_cur1 ^ 64u) + (uint32_t)(m * 16 * 256));
     convert(ic<0>{}, ic<0>{}, bfr[0], lp[1]);
     lut_issue(ic<0>{}, ic<1>{}, lp[0]);
     if (lora_fast) {
@@ -454,29 +473,34 @@ void qgemm128_kernel(const QLArgs a) {
 
   const bool has_rows = MT > 1 || kh == 0;
   const int64_t m0w = m0 + kh * (HM * 16);   // first row of the tile this wave finishes
-  const uint32_t row_lds = (uint32_t)(kh * (HM * 16) * A_LD * 2);
+  const uint32_t row_lds = (uint32_t)(kh * (HM * 16) * 256);
+  // every load into LDS has landed (the last k-tile requested one more tile): the epilogue
+  // reuses the buffers
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  const uint32_t n_tiles = (uint32_t)max(kt_end - kt_begin, 0);
+  const uint32_t t_buf = (n_tiles & 1u) * ABYTES;   // the adapter block is "k-tile" n_tiles of this split
 
   // The adapter's share of the rows this wave will finish, before the k halves meet: it needs
-  // nothing from the partner (the t block sits in the activation buffer the last k-tile left
-  // as "next", the B^T fragments in LDS since the prologue), so it runs while slower waves are
-  // still in their last k-tile.
+  // nothing from the partner (the t block sits in LDS as the k-tile after the last, the B^T
+  // fragments since the prologue), so it runs while slower waves are still in their last k-tile.
   f32x4 part[HM][NT];
 #pragma unroll
   for (int mt = 0; mt < HM; ++mt)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) zero_acc(part[mt][nt]);
   if (lora_fast && has_rows) {
-    const uint32_t tb = a_rd - (uint32_t)(kh * 64 * 2) + row_lds;
+    const uint32_t tb = t_buf + row_lds + (uint32_t)lm * 256u;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const uint32_t base = tb + (uint32_t)((toff[nt] == toff_a ? 0 : 64) * 2);
+      const uint32_t half = toff[nt] == toff_a ? 0u : 8u;   // first 16-byte chunk of the segment's 64 columns
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         if (j * 32 < a.lora_rank) {
           const u32x4 lbf = lds_ld128(lb_lds + (uint32_t)((nt * 2 + j) * 1024));
 #pragma unroll
           for (int mt = 0; mt < HM; ++mt)
-            part[mt][nt] = mfma16(lds_ld128(base + (uint32_t)((mt * 16 * A_LD + j * 32) * 2)), lbf, part[mt][nt]);
+            part[mt][nt] = mfma16(lds_ld128(tb + (uint32_t)(mt * 16 * 256) +
+                                            (((half + (uint32_t)(j * 4 + lq)) ^ (uint32_t)lm) * 16u)), lbf, part[mt][nt]);
         }
       }
     }
@@ -489,8 +513,8 @@ void qgemm128_kernel(const QLArgs a) {
   f32x4 out[HM][NT];
   {
     __syncthreads();  // every wave is done with the table
-    const uint32_t xw = (uint32_t)wv * 8192u + (uint32_t)lane * 16u;
-    const uint32_t xr = (uint32_t)(wv ^ 4) * 8192u + (uint32_t)lane * 16u;
+    const uint32_t xw = kBigLutBase + (uint32_t)wv * 8192u + (uint32_t)lane * 16u;
+    const uint32_t xr = kBigLutBase + (uint32_t)(wv ^ 4) * 8192u + (uint32_t)lane * 16u;
 #pragma unroll
     for (int m = 0; m < HM; ++m)
 #pragma unroll
@@ -531,7 +555,7 @@ void qgemm128_kernel(const QLArgs a) {
     // the tile is multiplied with the NEXT linear's adapter A (its LoRA down-projection, whose
     // K axis is this kernel's output axis), one fp32 fragment plane per work-group.
     constexpr int ACT_LD = 72;  // 64 act columns + 8 pad (bf16 elements)
-    const uint32_t act_lds = a_rd_nxt - (uint32_t)(lm * A_LD + lq * 8 + kh * 64) * 2u;
+    const uint32_t act_lds = t_buf ^ ABYTES;
     const int64_t ldy = a.N / 2;
     const int64_t wgcol0 = (int64_t)blockIdx.y * 64;      // first act column of the work-group
     const bool fuse_next = a.next_tpart != nullptr;
@@ -597,7 +621,7 @@ void qgemm128_kernel(const QLArgs a) {
     // (decode step 6.51 -> 6.42 ms; the same policy on the outputs of the norm and of attention,
     // which many work-groups re-read, measured neutral and is not used there).
     constexpr int T_LD = 36;   // floats per LDS row: 32 + 4, conflict-free for both passes
-    const uint32_t scr = kBigLutBytes + (uint32_t)wv * (16u * T_LD * 4u);
+    const uint32_t scr = (uint32_t)wv * (16u * T_LD * 4u);
     static_assert(MT < 4 || 8 * 16 * T_LD * 4 <= 2 * (int)ABYTES, "transposition scratch fits the activation buffers");
     const rsrc_t rp = make_rsrc(a.ws + (int64_t)blockIdx.z * a.M * a.N, (uint64_t)a.M * a.N * 4);
     const uint32_t col0 = (uint32_t)ntile0 * 16u;
