@@ -2,7 +2,8 @@
 //
 // A work-group of 4 waves owns 16*MT activation rows (MT = 8: a rollout batch of 128) and
 // 64*NT output columns; wave w owns NT column tiles of 16.  The activation tile [16*MT x 128k]
-// is staged in LDS once per k-tile (double buffered) and read as MFMA A fragments; weights go
+// is loaded straight into LDS once per k-tile (double buffered, 256-byte rows whose 16-byte
+// chunks are XOR-swizzled by row) and read as MFMA A fragments; weights go
 // HBM -> registers (one 128-bit buffer load per lane and k-tile for QW codes), are expanded to
 // bf16 through a bank-replicated LDS table and multiplied by their group scale in registers:
 // the MFMA B operand is bf16(bf16(level) * scale), i.e. the weight "dequantised to bf16", and
@@ -10,13 +11,13 @@
 //
 // Latency: a work-group runs alone on its CU (one wave per SIMD), so HBM latency is covered
 // by a register ring of PF weight k-tiles in flight per wave and the L2 latency of the
-// activations by one k-tile of register prefetch in front of the LDS double buffer.  All
-// loads are raw buffer loads: out-of-range rows / tiles read zeros without branches.
+// activations by requesting a tile one k-tile ahead of its use.  All loads are raw buffer
+// loads: out-of-range rows / tiles read zeros without branches.
 #pragma once
 #include "common.h"
 
 constexpr int KTILE = 128;
-constexpr int A_LD = KTILE + 8;  // bf16 elements per LDS row (272 B)
+constexpr int A_LD = KTILE;      // bf16 elements per LDS row (256 B, no padding: the chunks are swizzled)
 constexpr size_t tile_smem_bytes(int mt) {
   return 2 * (size_t)mt * 16 * A_LD * sizeof(uint16_t) + TNX_LUT_WORDS * sizeof(uint32_t);
 }
@@ -45,29 +46,45 @@ struct TileSrc {
 
 __device__ __forceinline__ void zero_acc(f32x4& v) { v = f32x4{0.f, 0.f, 0.f, 0.f}; }
 
-// Rows [m0, m0+16*MT) x k-tile kt of x -> registers; thread t owns the 16-byte chunks
-// t, t+256, ...  Rows beyond M read zeros (buffer bounds) or a clamped row (gather).
+// A buffer descriptor in scalar registers, for loads written in assembly.
+__device__ __forceinline__ u32x4 raw_rsrc(const void* p, uint64_t bytes) {
+  const uint64_t q = (uint64_t)p;
+  const uint32_t n = (uint32_t)(bytes > 0xffffffffull ? 0xffffffffull : bytes);
+  return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)q),
+               (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(q >> 32) & 0xffffu)),
+               (uint32_t)__builtin_amdgcn_readfirstlane((int)n), 0x00020000u};
+}
+// One 16-byte-per-lane load from a buffer straight into LDS, at byte address `lds` + 16 * lane
+// (M0 carries the wave-uniform base; lanes past the buffer write zeros).  The compiler does not
+// count these loads: its own waits for other loads can only turn out longer than needed (loads
+// complete in order), and the waits for these are written by hand (tnx_wait_vm).
+__device__ __forceinline__ void dma16(uint32_t lds, const u32x4& r, uint32_t voff, int soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :: "s"(lds), "v"(voff), "s"(r), "s"(soff) : "memory", "m0");
+}
+// s_waitcnt vmcnt(N) alone (the other counters at their maximum)
+#define tnx_wait_vm(N) __builtin_amdgcn_s_waitcnt(0x0f70 | ((N) & 15) | (((N) >> 4) << 14))
+
+// Rows [m0, m0+16*MT) x k-tile kt of x -> the LDS tile at byte address `lds`.  Thread t fills
+// chunk t % 16 of rows t / 16 + 16 c (a wave: 1 KB = four consecutive rows) and fetches for it
+// the k-chunk (t % 16) ^ (row % 16): the 16 lanes that read one k-chunk of 16 consecutive rows
+// as an MFMA fragment then hit 16 different bank groups.  Rows beyond M read zeros (buffer
+// bounds) or a clamped row (gather).
 template <int MT>
-__device__ __forceinline__ void load_a(const TileSrc& s, rsrc_t rx, int64_t m0, int kt, int tid,
-                                       u32x4 (&regs)[MT]) {
+__device__ __forceinline__ void load_a(const TileSrc& s, const u32x4& rx, int64_t m0, int kt, int tid,
+                                       uint32_t lds) {
+  const uint32_t wave_lds = lds + (uint32_t)__builtin_amdgcn_readfirstlane(tid >> 6) * 1024u;
+  const uint32_t ch = (uint32_t)((tid & 15) ^ ((tid >> 4) & 15));
 #pragma unroll
   for (int c = 0; c < MT; ++c) {
-    const int idx = tid + 256 * c;
-    const int row = idx >> 4, ch = idx & 15;
-    int64_t src = m0 + row;
+    int64_t src = m0 + (tid >> 4) + 16 * c;
     if (s.row_index) src = s.row_index[src < s.M ? src : s.M - 1] / s.row_div;
     // 32-bit offset: the host checks (rows + 128) * K * 2 < 4 GiB
-    regs[c] = buf_load128(rx, ((uint32_t)src * (uint32_t)s.K + (uint32_t)(kt * KTILE + ch * 8)) * 2u);
+    dma16(wave_lds + (uint32_t)c * 4096u, rx, ((uint32_t)src * (uint32_t)s.K + (uint32_t)kt * KTILE + ch * 8u) * 2u, 0);
   }
 }
-template <int MT>
-__device__ __forceinline__ void store_a(uint16_t* sA, int tid, const u32x4 (&regs)[MT]) {
-#pragma unroll
-  for (int c = 0; c < MT; ++c) {
-    const int idx = tid + 256 * c;
-    *reinterpret_cast<u32x4*>(sA + (idx >> 4) * A_LD + (idx & 15) * 8) = regs[c];
-  }
-}
+// LDS byte address of a __shared__ object
+__device__ __forceinline__ uint32_t lds_addr(const void* p) { return (uint32_t)(uintptr_t)p; }
 
 template <int MT, int NT, bool DENSE>
 __device__ __forceinline__ void tile_mainloop(const TileSrc& s, int64_t m0, int64_t ntile0,
@@ -76,8 +93,14 @@ __device__ __forceinline__ void tile_mainloop(const TileSrc& s, int64_t m0, int6
   const int tid = threadIdx.x, lane = tid & 63, lm = lane & 15, lq = lane >> 4;
   const int ktiles = (int)(s.K / KTILE);
   constexpr int kBufElems = MT * 16 * A_LD;
-  const rsrc_t rx = make_rsrc(s.x, (uint64_t)s.x_rows * s.K * 2);
-  u32x4 a_next[MT];
+  constexpr uint32_t kBufBytes = kBufElems * 2;
+  const u32x4 rx = raw_rsrc(s.x, (uint64_t)s.x_rows * s.K * 2);
+  const uint32_t lds_a = lds_addr(sA);
+  // this lane's fragment of row tile mt, k-step j: row l % 16, k-chunk 4 j + l / 16, swizzled
+  auto frag = [&](const uint16_t* buf, int mt, int j) -> u32x4 {
+    return *reinterpret_cast<const u32x4*>(reinterpret_cast<const unsigned char*>(buf) + mt * 4096 + lm * 256 +
+                                           (((j * 4 + lq) ^ lm) * 16));
+  };
 
   if constexpr (DENSE) {
     constexpr int PF = 2;  // weight k-tiles in flight
@@ -95,7 +118,7 @@ __device__ __forceinline__ void tile_mainloop(const TileSrc& s, int64_t m0, int6
               rw, ok ? (row * (uint32_t)s.K + (uint32_t)(kt * KTILE + j * 32 + lq * 8)) * 2u : 0xfffffff0u);
       }
     };
-    load_a<MT>(s, rx, m0, kt_begin, tid, a_next);
+    load_a<MT>(s, rx, m0, kt_begin, tid, lds_a);
 #pragma unroll
     for (int d = 0; d < PF; ++d) load_w(ring[d], kt_begin + d);
     for (int kt0 = kt_begin; kt0 < kt_end; kt0 += PF) {
@@ -104,29 +127,32 @@ __device__ __forceinline__ void tile_mainloop(const TileSrc& s, int64_t m0, int6
         const int kt = kt0 + d;
         const bool active = kt < kt_end;
         {
-          uint16_t* buf = sA + ((kt - kt_begin) & 1) * kBufElems;
-          if (active) store_a<MT>(buf, tid, a_next);
+          const uint32_t par = (uint32_t)((kt - kt_begin) & 1);
+          const uint16_t* buf = sA + par * kBufElems;
           u32x4 wf[NT][4];
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int j = 0; j < 4; ++j) wf[nt][j] = ring[d][nt][j];
-          __syncthreads();  // buffer (kt & 1) was last read two k-tiles ago
-          load_a<MT>(s, rx, m0, kt + 1, tid, a_next);
+          // this k-tile's activations have landed (the only younger loads: one ring stage of
+          // weights); every wave is past its reads of the other buffer, which the next tile takes
+          tnx_wait_vm(NT * 4);
+          __syncthreads();
+          load_a<MT>(s, rx, m0, kt + 1, tid, lds_a + (par ^ 1u) * kBufBytes);
           load_w(ring[d], kt + PF);
           if (active)
 #pragma unroll
           for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-              const u32x4 af =
-                  *reinterpret_cast<const u32x4*>(buf + (mt * 16 + lm) * A_LD + j * 32 + lq * 8);
+              const u32x4 af = frag(buf, mt, j);
 #pragma unroll
               for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = mfma16(af, wf[nt][j], acc[mt][nt]);
             }
         }
       }
     }
+    tnx_wait_vm(0);   // the tile requested last is not used, but must not land in LDS the caller reuses
   } else {
     constexpr int PF = 2;  // weight k-tiles in flight
     const int spt = scales_per_tile(s.group);  // scale slots per tile and column (2 or 4)
@@ -152,6 +178,7 @@ __device__ __forceinline__ void tile_mainloop(const TileSrc& s, int64_t m0, int6
       // layout (16 rows x 64 bytes per load, the four waves' requests meet in L1) -- no LDS
       // staging, no barrier in the loop, the waves drift apart and hide each other's waits.
       constexpr int PX = 3;
+      const rsrc_t rx1 = make_rsrc(s.x, (uint64_t)s.x_rows * s.K * 2);
       int64_t src = m0 + lm;
       if (s.row_index) src = s.row_index[src < s.M ? src : s.M - 1] / s.row_div;   // gather; rows past M: a clamped row, never stored
       const uint32_t xoff = ((uint32_t)src * (uint32_t)s.K + (uint32_t)(lq * 8)) * 2u;   // rows past M (no gather) lie beyond the resource: zeros
@@ -160,7 +187,7 @@ __device__ __forceinline__ void tile_mainloop(const TileSrc& s, int64_t m0, int6
       auto load_x = [&](u32x4 (&dst)[4], int kt) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          dst[j] = __builtin_amdgcn_raw_buffer_load_b128(rx, xoff, (kt * KTILE + j * 32) * 2, 0);
+          dst[j] = __builtin_amdgcn_raw_buffer_load_b128(rx1, xoff, (kt * KTILE + j * 32) * 2, 0);
       };
       const int kt_last = ktiles - 1;
 #pragma unroll
@@ -201,7 +228,7 @@ __device__ __forceinline__ void tile_mainloop(const TileSrc& s, int64_t m0, int6
     }
     // Loads are never predicated (k-tiles past the end read unused neighbouring or zero data)
     // and the trip count is padded to a multiple of PF, so every wait is counted exactly.
-    load_a<MT>(s, rx, m0, kt_begin, tid, a_next);
+    load_a<MT>(s, rx, m0, kt_begin, tid, lds_a);
 #pragma unroll
     for (int d = 0; d < PF; ++d) load_w(ring_c[d], ring_s[d], kt_begin + d);
     for (int kt0 = kt_begin; kt0 < kt_end; kt0 += PF) {
@@ -210,8 +237,8 @@ __device__ __forceinline__ void tile_mainloop(const TileSrc& s, int64_t m0, int6
         const int kt = kt0 + d;
         const bool active = kt < kt_end;
         {
-          uint16_t* buf = sA + ((kt - kt_begin) & 1) * kBufElems;
-          if (active) store_a<MT>(buf, tid, a_next);
+          const uint32_t par = (uint32_t)((kt - kt_begin) & 1);
+          const uint16_t* buf = sA + par * kBufElems;
           u32x4 cw[NT];
           float sc[NT][4];
 #pragma unroll
@@ -223,10 +250,12 @@ __device__ __forceinline__ void tile_mainloop(const TileSrc& s, int64_t m0, int6
 #pragma unroll
             for (int j = 0; j < 4; ++j) sc[nt][j] = spt == 2 ? f[j >> 1] : f[j];
           }
-          __syncthreads();  // buffer (kt & 1) was last read two k-tiles ago
-          // activations first, then the weights PF tiles ahead: the wait at the top of the
-          // next k-tile then only covers the activation loads
-          load_a<MT>(s, rx, m0, kt + 1, tid, a_next);
+          // this k-tile's activations have landed (the only younger loads: one ring stage of
+          // codes and scales); every wave is past its reads of the other buffer
+          tnx_wait_vm(NT * 2);
+          __syncthreads();
+          // activations first, then the weights PF tiles ahead
+          load_a<MT>(s, rx, m0, kt + 1, tid, lds_a + (par ^ 1u) * kBufBytes);
           load_w(ring_c[d], ring_s[d], kt + PF);
           if (active)
 #pragma unroll
@@ -236,8 +265,7 @@ __device__ __forceinline__ void tile_mainloop(const TileSrc& s, int64_t m0, int6
             for (int nt = 0; nt < NT; ++nt) bf[nt] = dequant8_scaled(cw[nt][j], lut_lane, sc[nt][j]);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-              const u32x4 af =
-                  *reinterpret_cast<const u32x4*>(buf + (mt * 16 + lm) * A_LD + j * 32 + lq * 8);
+              const u32x4 af = frag(buf, mt, j);
 #pragma unroll
               for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = mfma16(af, bf[nt], acc[mt][nt]);
             }
@@ -245,6 +273,7 @@ __device__ __forceinline__ void tile_mainloop(const TileSrc& s, int64_t m0, int6
         }
       }
     }
+    tnx_wait_vm(0);   // the tile requested last is not used, but must not land in LDS the caller reuses
   }
 }
 
