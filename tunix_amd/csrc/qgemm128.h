@@ -105,14 +105,6 @@ void qgemm128_kernel(const QLArgs a) {
   const int kt_begin = blockIdx.z * a.ktiles_per_split;
   const int kt_end = min(ktiles, kt_begin + a.ktiles_per_split);
 
-  // (raw descriptors in scalar registers: the loads that use them are written in assembly)
-  auto raw_rsrc = [](const void* p, uint64_t bytes) -> u32x4 {
-    const uint64_t q = (uint64_t)p;
-    const uint32_t n = (uint32_t)(bytes > 0xffffffffull ? 0xffffffffull : bytes);
-    return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)q),
-                 (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(q >> 32) & 0xffffu)),
-                 (uint32_t)__builtin_amdgcn_readfirstlane((int)n), 0x00020000u};
-  };
   const u32x4 rx = raw_rsrc(a.x, (uint64_t)a.M * a.K * 2);
   const uint64_t ntk = (uint64_t)ntiles * ktiles;
   const rsrc_t rc = make_rsrc(a.codes, ntk * 1024);
@@ -128,13 +120,8 @@ void qgemm128_kernel(const QLArgs a) {
   // different bank groups.
   const uint32_t chs = (uint32_t)((tid & 15) ^ ((tid >> 4) & 15));
   const uint32_t xbase = ((uint32_t)(m0 + (tid >> 4)) * (uint32_t)a.K + chs * 8u) * 2u;
-  // One 16-byte-per-lane load into LDS at `lds` + 16 * lane (M0 carries the wave's base).  The
-  // compiler does not count these loads: its own waits for other loads can only turn out
-  // longer than needed (loads complete in order), and the waits for these are written by hand.
-  auto dma16 = [&](uint32_t lds, const u32x4& r, uint32_t voff, int soff) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :: "s"(lds), "v"(voff), "s"(r), "s"(soff) : "memory", "m0");
-  };
+  // (dma16 of gemm_tile.h: the compiler does not count these loads, the waits for them are
+  // written by hand)
   const uint32_t dma_wave = (uint32_t)wv * 1024u;      // this wave's four rows within a 32-row pass
   const uint32_t xstride = 32u * (uint32_t)a.K * 2u;  // 32 rows further per chunk
 #pragma unroll
@@ -404,7 +391,7 @@ void qgemm128_kernel(const QLArgs a) {
     const bool next_active = kt + 1 < kt_end;
     __builtin_amdgcn_sched_barrier(0);
     kstep(ic<0>{}, Dc, ic<1>{}, ic<dn>{}, ic<0>{}, a_cur1, ic<1>{}, ic<1>{}, ic<0>{}, ic<dn>{}, kt + 2, next_active);
-    __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * NT));
+    tnx_wait_vm(2 * NT);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     kstep(ic<1>{}, ic<dn>{}, ic<0>{}, ic<dn>{}, ic<1>{}, a_nxt0, ic<0>{}, ic<0>{}, ic<1>{}, ic<-1>{}, kt + 2, false);
@@ -441,7 +428,7 @@ void qgemm128_kernel(const QLArgs a) {
     expand_scales(ic<0>{}, true);
     // the first tile's AP loads are the oldest in flight; at least 3 x 2 NT weight / scale loads
     // and the second tile's AP follow them
-    __builtin_amdgcn_s_waitcnt(0x0f70 | ((6 * NT + AP) & 15) | (((6 * NT + AP) >> 4) << 14));
+    tnx_wait_vm(6 * NT + AP);
     __syncthreads();  // table and first activation tile
     lut_issue(ic<0>{}, ic<0>{}, lp[1]);
 #pragma unroll
@@ -476,7 +463,7 @@ void qgemm128_kernel(const QLArgs a) {
   const uint32_t row_lds = (uint32_t)(kh * (HM * 16) * 256);
   // every load into LDS has landed (the last k-tile requested one more tile): the epilogue
   // reuses the buffers
-  __builtin_amdgcn_s_waitcnt(0x0f70);
+  tnx_wait_vm(0);
   const uint32_t n_tiles = (uint32_t)max(kt_end - kt_begin, 0);
   const uint32_t t_buf = (n_tiles & 1u) * ABYTES;   // the adapter block is "k-tile" n_tiles of this split
 

@@ -116,14 +116,6 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   // the activation resource starts at this work-group's first row: offsets stay small whatever
   // M is, and rows past M lie beyond the resource and read zeros (GROUPED: the whole buffer,
   // rows are gathered)
-  // (a raw descriptor in scalar registers: the loads that use it are written in assembly)
-  auto raw_rsrc = [](const void* p, uint64_t bytes) -> u32x4 {
-    const uint64_t q = (uint64_t)p;
-    const uint32_t n = (uint32_t)(bytes > 0xffffffffull ? 0xffffffffull : bytes);
-    return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)q),
-                 (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(q >> 32) & 0xffffu)),
-                 (uint32_t)__builtin_amdgcn_readfirstlane((int)n), 0x00020000u};
-  };
   const u32x4 rx = GROUPED ? raw_rsrc(a.x, (uint64_t)(a.M / a.x_div) * a.K * 2)
                            : raw_rsrc(a.x + m0 * a.K, (uint64_t)rows_here * a.K * 2);
   const uint64_t ntk = (uint64_t)ntiles * ktiles;
@@ -229,13 +221,8 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   const u32x4 rt_ = lora ? raw_rsrc(a.t + m0 * a.t_ld, (uint64_t)rows_here * a.t_ld * 2) : rx;
   const uint32_t tstride = (uint32_t)(16 * a.t_ld * 2);
 
-  // One 16-byte-per-lane load into LDS at `lds` + 16 * lane (M0 carries the wave's base).  The
-  // compiler does not count these loads: its own waits for other loads can only turn out
-  // longer than needed (loads complete in order), and the waits for these are written by hand.
-  auto dma16 = [&](uint32_t lds, const u32x4& r, uint32_t voff, int soff) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :: "s"(lds), "v"(voff), "s"(r), "s"(soff) : "memory", "m0");
-  };
+  // (dma16 of gemm_tile.h: the compiler does not count these loads, the waits for them are
+  // written by hand)
   const uint32_t dma_wave = (uint32_t)wn * 1024u;      // this wave's four rows within a 16-row pass
   auto sel_rsrc = [&](bool ut) -> u32x4 {
     const uint32_t m = 0u - (uint32_t)ut;
@@ -354,7 +341,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
     slab(ic<6>{}, Dc, kt, next_active);
     // the next tile's activations, requested by slab 7 of the tile before, have landed in LDS:
     // the only younger loads are the six weight / scale loads slab 6 has just issued
-    __builtin_amdgcn_s_waitcnt(0x0f70 | 6);
+    tnx_wait_vm(6);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     slab(ic<7>{}, Dc, kt, next_active);
@@ -389,7 +376,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   expand_scales(ic<0>{}, true);
   // the first tile is in LDS: its eight loads are the oldest, and at least 26 follow them (three
   // ring stages of six, the second tile's eight); vmcnt(20) also covers the first ring stage
-  __builtin_amdgcn_s_waitcnt(0x0f70 | (20 & 15) | ((20 >> 4) << 14));
+  tnx_wait_vm(20);
   __syncthreads();
   // slab 0: table entries, conversion, fragments; then the table entries of slab 1
 #pragma unroll
@@ -460,7 +447,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
         for (int i = 0; i < 16; ++i) acc[rt][cg][i] += a.lora_scale * part[rt][i];
     }
   }
-  __builtin_amdgcn_s_waitcnt(0x0f70);   // no load into LDS is still on its way
+  tnx_wait_vm(0);   // no load into LDS is still on its way
   __syncthreads();  // every wave is done with the activation buffers: they become the output stage
 
   // The bf16 tile goes through LDS (row stride cols + 8 elements) and leaves as 16-byte chunks
