@@ -156,6 +156,14 @@ def _pad_lora(a, b, rp):
     (64, 1152, 1024, 128, Q.INT4, 16, 3),
     (33, 768, 208, 256, Q.NF4, 0, 1),
     (130, 256, 48, 32, Q.INT4, 32, 1),
+    # the activation tiles' road into LDS at its corners: a single k-tile (the adapter block is the
+    # second tile), one whole turn of the weight ring, every row-tile count, uneven k splits
+    (128, 128, 256, 64, Q.NF4, 64, 1),
+    (16, 384, 256, 64, Q.INT4, 32, 1),
+    (32, 640, 384, 128, Q.NF4, 64, 2),
+    (100, 896, 512, 64, Q.INT4, 64, 3),
+    (17, 256, 128, 32, Q.NF4, 16, 1),
+    (64, 1024, 256, 64, Q.NF4, 32, 8),
 ])
 def test_qlinear_lora_matches_oracle(gpu, M, K, N, group, qtype, r, split):
   from tunix_amd import _lib as L
