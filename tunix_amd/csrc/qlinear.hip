@@ -256,6 +256,78 @@ __global__ __launch_bounds__(512) void lora_down_kernel(const uint16_t* x, int64
   }
 }
 
+// The same product with the operand rows taken through LDS.  A load that hands every lane of a
+// quarter-wave a different row (the MFMA operand layout: lane l holds row l % 16) is served one
+// lane at a time, ≈ 37 GB/s per compute unit however the data is cached; rows fetched as whole
+// kilobytes (a wave's 64 lanes on 1 KB of one row, straight into LDS) come at three times that.
+// The tm + tn rows of the tile are laid out one after the other (row stride `row_bytes`, K * 2
+// rounded up to 1 KB; 16-byte chunks XOR-swizzled by the row so that the fragment reads of 16
+// rows hit 16 bank groups), then every wave multiplies its eighth of the k-steps out of LDS.
+// Launched when the rows fit LDS and K is a multiple of 64; the wave sums reuse the tile's LDS.
+__global__ __launch_bounds__(512) void lora_down_lds_kernel(const uint16_t* x, int64_t M, int64_t K,
+                                                            const uint16_t* a_t, int R, uint16_t* t,
+                                                            int64_t t_ld, int tm, int tn, uint32_t row_bytes) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int lm = lane & 15, lq = lane >> 4;
+  const int64_t m0 = (int64_t)blockIdx.x * tm;
+  const int n0 = blockIdx.y * tn;
+  const uint32_t lds0 = lds_addr(smem);
+  {
+    // rows past M / R lie beyond the resource and arrive as zeros
+    const int64_t xrows = min((int64_t)tm, M - m0);
+    const int arows = min(tn, R - n0);
+    const u32x4 rx = raw_rsrc(x + m0 * K, (uint64_t)xrows * K * 2);
+    const u32x4 ra = raw_rsrc(a_t + (int64_t)n0 * K, (uint64_t)arows * K * 2);
+    const int per_row = (int)(row_bytes / 1024u), n_x = tm * per_row, n_all = (tm + tn) * per_row;
+    for (int q = wave; q < n_all; q += 8) {
+      const bool is_x = q < n_x;
+      const int qq = is_x ? q : q - n_x;
+      const int row = qq / per_row, blk = qq % per_row;
+      const int lrow = is_x ? row : tm + row;                     // row of the LDS tile
+      // lane j fills chunk 64 blk + j and fetches for it chunk 64 blk + (j ^ (row % 16))
+      const uint32_t voff = (uint32_t)row * (uint32_t)K * 2u + (uint32_t)blk * 1024u + (uint32_t)(lane ^ (lrow & 15)) * 16u;
+      // chunks past the row's K elements: beyond the resource for the last row, otherwise the next
+      // row's first bytes; no fragment read touches them
+      dma16(lds0 + (uint32_t)lrow * row_bytes + (uint32_t)blk * 1024u, is_x ? rx : ra, voff, 0);
+    }
+  }
+  tnx_wait_vm(0);
+  __syncthreads();
+  // operand rows of this lane: tile rows the output does not have are clamped (their products
+  // are never stored)
+  const unsigned char* ra_lds = smem + (uint32_t)min(lm, tm - 1) * row_bytes;
+  const unsigned char* rb_lds = smem + (uint32_t)(tm + min(lm, tn - 1)) * row_bytes;
+  auto ld = [](const unsigned char* p, uint32_t chunk) { return *reinterpret_cast<const u32x4*>(p + chunk * 16u); };
+  const uint32_t sa = (uint32_t)(min(lm, tm - 1) & 15), sb = (uint32_t)((tm + min(lm, tn - 1)) & 15);
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int ksteps = (int)(K / 64);
+#pragma unroll 4
+  for (int ks = wave; ks < ksteps; ks += 8) {
+    const uint32_t c0 = (uint32_t)(ks * 8 + lq * 2);            // this lane's two 16-byte chunks of the step
+    const u32x4 a0 = ld(ra_lds, c0 ^ sa), a1 = ld(ra_lds, (c0 + 1) ^ sa);
+    const u32x4 b0 = ld(rb_lds, c0 ^ sb), b1 = ld(rb_lds, (c0 + 1) ^ sb);
+    acc = mfma16(a0, b0, acc);
+    acc = mfma16(a1, b1, acc);
+  }
+  __syncthreads();   // every wave is done with the tile: its first 8 KB take the wave sums
+  float* red = reinterpret_cast<float*>(smem);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) red[(wave * 64 + lane) * 4 + i] = acc[i];
+  __syncthreads();
+  if (wave == 0) {
+    const bool b_on = lm < tn && n0 + lm < R;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < 8; ++w) sum += red[(w * 64 + lane) * 4 + i];
+      const int mi = lq * 4 + i;
+      if (mi < tm && m0 + mi < M && b_on) t[(m0 + mi) * t_ld + n0 + lm] = f2bf(sum);
+    }
+  }
+}
+
 // t[M, :R] = bf16(sum of fragment planes).  A plane holds, per (row tile, column tile, lane), the
 // four rows 4*(lane/16)+i of column lane%16 of a 16 x 16 tile, exactly as the MFMA that produced
 // it laid them out.  One work-group sums 8 consecutive lanes' values (128 bytes of every plane):
@@ -755,6 +827,19 @@ extern "C" int tnx_lora_down(void* stream, const uint16_t* x, int64_t M, int64_t
         }
   }
   dim3 grid((unsigned)cdiv(M, tm), (unsigned)cdiv(R, tn));
+  // the operand rows through LDS when they fit (rows of K * 2 bytes rounded up to whole KB)
+  const uint64_t row_bytes = (uint64_t)cdiv(K * 2, 1024) * 1024;
+  const uint64_t lds = std::max<uint64_t>((uint64_t)(tm + tn) * row_bytes, 8192);
+  if (K % 64 == 0 && lds <= 160 * 1024 && (uint64_t)(tm + 1) * (uint64_t)K * 2 < (1ull << 32)) {
+    static std::once_flag once;
+    static int attr_rc = TNX_OK;
+    std::call_once(once, [] { attr_rc = raise_lds_limit(&lora_down_lds_kernel, 160 * 1024); });
+    if (attr_rc) return attr_rc;
+    hipLaunchKernelGGL(lora_down_lds_kernel, grid, dim3(512), (size_t)lds, as_stream(stream), x, M, K, a_t, R, t, t_ld,
+                       tm, tn, (uint32_t)row_bytes);
+    TNX_CHECK_LAUNCH("lora_down_lds");
+    return TNX_OK;
+  }
   hipLaunchKernelGGL(lora_down_kernel, grid, dim3(512), 0, as_stream(stream), x, M, K, a_t, R, t, t_ld, tm, tn);
   TNX_CHECK_LAUNCH("lora_down");
   return TNX_OK;
