@@ -288,6 +288,19 @@ def test_lora_down_many_rows(gpu, M, K, R):
   assert (t[:, R:].float() == 7.0).all()
 
 
+@pytest.mark.parametrize("M,K,R", [(128, 4096, 64), (128, 4096, 192), (128, 14336, 64), (128, 6912, 128),
+                                   (8, 512, 32), (64, 1152, 16), (33, 2048, 128), (100, 96, 48), (5, 20480, 16)])
+def test_lora_down_decode_sizes(gpu, M, K, R):
+  """The down-projection at decode sizes: operand rows through LDS whole (K * rows fits), in pieces
+  (long rows), and the direct kernel (K not a multiple of 64); columns past R stay untouched."""
+  from tunix_amd import ops
+  x, a_t = rnd((M, K), 43), rnd((R, K), 44, 0.02)
+  t = torch.full((M, R + 32), 7.0, dtype=torch.bfloat16, device=gpu)
+  ops.lora_down(bf(x).to(gpu), bf(a_t).to(gpu), t)
+  assert_bf16_close(t[:, :R], Q.rb((bf(x).double() @ bf(a_t).t().double()).float()), what="lora_down decode")
+  assert (t[:, R:].float() == 7.0).all()
+
+
 def test_qlinear_invariants(gpu):
   """Zero codes give zero; B = 0 leaves the base result; scale linearity (exact powers of 2)."""
   from tunix_amd import ops

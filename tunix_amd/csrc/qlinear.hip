@@ -263,37 +263,23 @@ __global__ __launch_bounds__(512) void lora_down_kernel(const uint16_t* x, int64
 // The tm + tn rows of the tile are laid out one after the other (row stride `row_bytes`, K * 2
 // rounded up to 1 KB; 16-byte chunks XOR-swizzled by the row so that the fragment reads of 16
 // rows hit 16 bank groups), then every wave multiplies its eighth of the k-steps out of LDS.
-// Launched when the rows fit LDS and K is a multiple of 64; the wave sums reuse the tile's LDS.
+// Rows longer than LDS holds are taken in pieces of `kc` elements (a multiple of 512), one after
+// the other.  Launched when K is a multiple of 64; the wave sums reuse the tile's LDS.
 __global__ __launch_bounds__(512) void lora_down_lds_kernel(const uint16_t* x, int64_t M, int64_t K,
                                                             const uint16_t* a_t, int R, uint16_t* t,
-                                                            int64_t t_ld, int tm, int tn, uint32_t row_bytes) {
+                                                            int64_t t_ld, int tm, int tn, uint32_t row_bytes, int kc) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int lm = lane & 15, lq = lane >> 4;
   const int64_t m0 = (int64_t)blockIdx.x * tm;
   const int n0 = blockIdx.y * tn;
   const uint32_t lds0 = lds_addr(smem);
-  {
-    // rows past M / R lie beyond the resource and arrive as zeros
-    const int64_t xrows = min((int64_t)tm, M - m0);
-    const int arows = min(tn, R - n0);
-    const u32x4 rx = raw_rsrc(x + m0 * K, (uint64_t)xrows * K * 2);
-    const u32x4 ra = raw_rsrc(a_t + (int64_t)n0 * K, (uint64_t)arows * K * 2);
-    const int per_row = (int)(row_bytes / 1024u), n_x = tm * per_row, n_all = (tm + tn) * per_row;
-    for (int q = wave; q < n_all; q += 8) {
-      const bool is_x = q < n_x;
-      const int qq = is_x ? q : q - n_x;
-      const int row = qq / per_row, blk = qq % per_row;
-      const int lrow = is_x ? row : tm + row;                     // row of the LDS tile
-      // lane j fills chunk 64 blk + j and fetches for it chunk 64 blk + (j ^ (row % 16))
-      const uint32_t voff = (uint32_t)row * (uint32_t)K * 2u + (uint32_t)blk * 1024u + (uint32_t)(lane ^ (lrow & 15)) * 16u;
-      // chunks past the row's K elements: beyond the resource for the last row, otherwise the next
-      // row's first bytes; no fragment read touches them
-      dma16(lds0 + (uint32_t)lrow * row_bytes + (uint32_t)blk * 1024u, is_x ? rx : ra, voff, 0);
-    }
-  }
-  tnx_wait_vm(0);
-  __syncthreads();
+  // rows past M / R lie beyond the resource and arrive as zeros
+  const int64_t xrows = min((int64_t)tm, M - m0);
+  const int arows = min(tn, R - n0);
+  const u32x4 rx = raw_rsrc(x + m0 * K, (uint64_t)xrows * K * 2);
+  const u32x4 ra = raw_rsrc(a_t + (int64_t)n0 * K, (uint64_t)arows * K * 2);
+  const int per_row = (int)(row_bytes / 1024u), n_x = tm * per_row, n_all = (tm + tn) * per_row;
   // operand rows of this lane: tile rows the output does not have are clamped (their products
   // are never stored)
   const unsigned char* ra_lds = smem + (uint32_t)min(lm, tm - 1) * row_bytes;
@@ -301,14 +287,31 @@ __global__ __launch_bounds__(512) void lora_down_lds_kernel(const uint16_t* x, i
   auto ld = [](const unsigned char* p, uint32_t chunk) { return *reinterpret_cast<const u32x4*>(p + chunk * 16u); };
   const uint32_t sa = (uint32_t)(min(lm, tm - 1) & 15), sb = (uint32_t)((tm + min(lm, tn - 1)) & 15);
   f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int ksteps = (int)(K / 64);
+  for (int64_t k0 = 0; k0 < K; k0 += kc) {
+    if (k0 > 0) __syncthreads();   // every wave is done with the piece before
+    for (int q = wave; q < n_all; q += 8) {
+      const bool is_x = q < n_x;
+      const int qq = is_x ? q : q - n_x;
+      const int row = qq / per_row, blk = qq % per_row;
+      const int lrow = is_x ? row : tm + row;                     // row of the LDS tile
+      // lane j fills chunk 64 blk + j and fetches for it chunk 64 blk + (j ^ (row % 16))
+      const uint32_t voff = ((uint32_t)row * (uint32_t)K + (uint32_t)k0) * 2u + (uint32_t)blk * 1024u +
+                            (uint32_t)(lane ^ (lrow & 15)) * 16u;
+      // chunks past the row's K elements: beyond the resource for the last row, otherwise the next
+      // row's first bytes; no fragment read touches them
+      dma16(lds0 + (uint32_t)lrow * row_bytes + (uint32_t)blk * 1024u, is_x ? rx : ra, voff, 0);
+    }
+    tnx_wait_vm(0);
+    __syncthreads();
+    const int ksteps = (int)(min((int64_t)kc, K - k0) / 64);
 #pragma unroll 4
-  for (int ks = wave; ks < ksteps; ks += 8) {
-    const uint32_t c0 = (uint32_t)(ks * 8 + lq * 2);            // this lane's two 16-byte chunks of the step
-    const u32x4 a0 = ld(ra_lds, c0 ^ sa), a1 = ld(ra_lds, (c0 + 1) ^ sa);
-    const u32x4 b0 = ld(rb_lds, c0 ^ sb), b1 = ld(rb_lds, (c0 + 1) ^ sb);
-    acc = mfma16(a0, b0, acc);
-    acc = mfma16(a1, b1, acc);
+    for (int ks = wave; ks < ksteps; ks += 8) {
+      const uint32_t c0 = (uint32_t)(ks * 8 + lq * 2);            // this lane's two 16-byte chunks of the step
+      const u32x4 a0 = ld(ra_lds, c0 ^ sa), a1 = ld(ra_lds, (c0 + 1) ^ sa);
+      const u32x4 b0 = ld(rb_lds, c0 ^ sb), b1 = ld(rb_lds, (c0 + 1) ^ sb);
+      acc = mfma16(a0, b0, acc);
+      acc = mfma16(a1, b1, acc);
+    }
   }
   __syncthreads();   // every wave is done with the tile: its first 8 KB take the wave sums
   float* red = reinterpret_cast<float*>(smem);
@@ -827,16 +830,20 @@ extern "C" int tnx_lora_down(void* stream, const uint16_t* x, int64_t M, int64_t
         }
   }
   dim3 grid((unsigned)cdiv(M, tm), (unsigned)cdiv(R, tn));
-  // the operand rows through LDS when they fit (rows of K * 2 bytes rounded up to whole KB)
-  const uint64_t row_bytes = (uint64_t)cdiv(K * 2, 1024) * 1024;
+  // the operand rows through LDS, whole (rows of K * 2 bytes rounded up to whole KB) or, when LDS
+  // does not hold them, in pieces of kc elements (whole KB again)
+  int64_t kc = K;
+  if ((uint64_t)(tm + tn) * (uint64_t)cdiv(K * 2, 1024) * 1024 > 160 * 1024)
+    kc = (160 * 1024 / ((tm + tn) * 2)) / 512 * 512;
+  const uint64_t row_bytes = (uint64_t)cdiv(kc * 2, 1024) * 1024;
   const uint64_t lds = std::max<uint64_t>((uint64_t)(tm + tn) * row_bytes, 8192);
-  if (K % 64 == 0 && lds <= 160 * 1024 && (uint64_t)(tm + 1) * (uint64_t)K * 2 < (1ull << 32)) {
+  if (K % 64 == 0 && kc >= 512 && lds <= 160 * 1024 && (uint64_t)(tm + 1) * (uint64_t)K * 2 < (1ull << 32)) {
     static std::once_flag once;
     static int attr_rc = TNX_OK;
     std::call_once(once, [] { attr_rc = raise_lds_limit(&lora_down_lds_kernel, 160 * 1024); });
     if (attr_rc) return attr_rc;
     hipLaunchKernelGGL(lora_down_lds_kernel, grid, dim3(512), (size_t)lds, as_stream(stream), x, M, K, a_t, R, t, t_ld,
-                       tm, tn, (uint32_t)row_bytes);
+                       tm, tn, (uint32_t)row_bytes, (int)kc);
     TNX_CHECK_LAUNCH("lora_down_lds");
     return TNX_OK;
   }
