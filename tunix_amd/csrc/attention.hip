@@ -12,7 +12,7 @@
 #include "common.h"
 
 // Register stages of the key-block ring (head_dim <= 128).  Two: one block in flight while one is
-// computed.  A compute unit keeps about 16 KiB of reads in flight whatever its waves request, so a
+// computed.  A compute unit draws 21-28 GB/s from memory whatever its waves request, so a
 // third stage adds nothing to the stream, and its 72 registers push ring registers into AGPRs,
 // whose copies wait on loads in flight (measured: 46.5 / 64.8 us with two stages against
 // 47.9 / 67.3 us with three at contexts 528 / 768).

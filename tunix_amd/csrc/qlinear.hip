@@ -205,10 +205,12 @@ __global__ void splitk_finish_kernel(const QLArgs a) {
 }
 
 // t[M,R] = bf16(x . A): one tm x tn output tile (tm, tn <= 16) per work-group, K split over
-// 8 waves.  A compute unit draws only a few tens of GB/s from L2, so the op is bound by the
-// bytes one work-group must read, (tm + tn) rows of K elements: for decode-sized M the host
-// picks tiles smaller than the 16 x 16 MFMA shape (unused rows and columns are zero operands)
-// to spread the reads over every compute unit.
+// 8 waves.  The operands are loaded straight into the MFMA layout (every lane of a quarter-wave
+// its own row), which a compute unit serves one lane at a time, a few tens of GB/s: the op is
+// bound by the bytes one work-group must read, (tm + tn) rows of K elements, and for decode-sized
+// M the host picks tiles smaller than the 16 x 16 MFMA shape (unused rows and columns are zero
+// operands) to spread the reads over every compute unit.  (The kernel for K not a multiple of
+// 64; otherwise lora_down_lds_kernel below.)
 // The contraction may visit k in any order as long as both operands agree, so each lane takes
 // 16 consecutive elements per 64-wide step (two MFMAs): the four lanes of a row cover one whole
 // 128-byte line.
