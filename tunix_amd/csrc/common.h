@@ -123,13 +123,6 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
-// A 16-byte store that is written through to memory at once (the sc1 bit): for data that another
-// kernel, on other XCDs, reads next -- it neither waits in this XCD's L2 for the write-back at
-// the end of the launch nor skips the memory-side cache as a non-temporal store does.
-__device__ __forceinline__ void store_through(void* p, u32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
-}
-
 static inline hipStream_t as_stream(void* s) { return (hipStream_t)s; }
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
@@ -148,7 +141,6 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint64_t bytes) {
 // adopted for the packed weights of the GEMM, 1 us slower per launch, for the head's weight rows,
 // neutral, and for the norm's reads of the partial planes, slower.)
 constexpr int kStreamOnce = 2;   // the "nt" bit of the gfx940+ cache-policy operand
-constexpr int kWriteThrough = 16;  // its "sc1" bit on a store: written through to memory at once
 __device__ __forceinline__ u32x4 buf_load128(rsrc_t r, uint32_t byte_off) {
   return __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
 }

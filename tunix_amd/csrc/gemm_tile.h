@@ -58,8 +58,11 @@ __device__ __forceinline__ u32x4 raw_rsrc(const void* p, uint64_t bytes) {
 // (M0 carries the wave-uniform base; lanes past the buffer write zeros).  The compiler does not
 // count these loads: its own waits for other loads can only turn out longer than needed (loads
 // complete in order), and the waits for these are written by hand (tnx_wait_vm).
+// (The s_nop covers what the compiler's hazard handling cannot see inside the assembly: M0 written
+// just before its use, and a descriptor or offset register written by a vector instruction --
+// v_readfirstlane -- within the five slots before a memory instruction reads it.)
 __device__ __forceinline__ void dma16(uint32_t lds, const u32x4& r, uint32_t voff, int soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                :: "s"(lds), "v"(voff), "s"(r), "s"(soff) : "memory", "m0");
 }
 // s_waitcnt vmcnt(N) alone (the other counters at their maximum)

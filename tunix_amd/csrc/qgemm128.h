@@ -578,7 +578,7 @@ void qgemm128_kernel(const QLArgs a) {
       if (row >= ROWS) break;
       const u32x4 v = lds_ld128(act_lds + (uint32_t)((row * ACT_LD + ch * 8) * 2));
       if (m0 + row < a.M && wgcol0 + ch * 8 + 8 <= ldy)
-        store_through(y + (m0 + row) * ldy + wgcol0 + ch * 8, v);
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(y + (m0 + row) * ldy + wgcol0 + ch * 8));
     }
     if (fuse_next && wv < MT) {   // one row tile per wave; fewer rows leave plane slots unwritten
       float* plane = a.next_tpart + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * 8192;
@@ -593,7 +593,7 @@ void qgemm128_kernel(const QLArgs a) {
           f32x4 pacc = f32x4{0.f, 0.f, 0.f, 0.f};
           pacc = mfma16(af2[0], bn[n][0], pacc);
           pacc = mfma16(af2[1], bn[n][1], pacc);
-          store_through(plane + ((mt * 4 + n) * 64 + lane) * 4, __builtin_bit_cast(u32x4, pacc));
+          __builtin_nontemporal_store(pacc, reinterpret_cast<f32x4*>(plane + ((mt * 4 + n) * 64 + lane) * 4));
         }
       }
     }
@@ -604,13 +604,9 @@ void qgemm128_kernel(const QLArgs a) {
     // row tile goes through a wave-private corner of the activation buffers instead (idle since
     // the barriers of the exchange above) and leaves as two 16-byte stores per lane, 128-byte
     // runs (rows past M fall outside the plane's buffer and are dropped).  The planes are written
-    // once and read once, by another kernel on other XCDs: written through to memory at once
-    // (the sc1 bit).  With the default policy the launch ends with 15-16 MB of dirty lines to
-    // write back (decode step 6.51 ms); the non-temporal policy avoids that (6.42) but also keeps
-    // the planes out of the memory-side cache their reader would find them in; written through
-    // they cost 1 % of the step less again (6.17 -> 6.11 ms).  The activation tile and the
-    // adapter planes of the gate|up epilogue leave the same way (5.95 -> 5.89 ms); on the outputs
-    // of the norm and of attention the policy measured neutral and is not used.
+    // once and read once, by another kernel on other XCDs: stored with the non-temporal policy
+    // (decode step 6.51 -> 6.42 ms; the same policy on the outputs of the norm and of attention,
+    // which many work-groups re-read, measured neutral and is not used there).
     constexpr int T_LD = 36;   // floats per LDS row: 32 + 4, conflict-free for both passes
     const uint32_t scr = (uint32_t)wv * (16u * T_LD * 4u);
     static_assert(MT < 4 || 8 * 16 * T_LD * 4 <= 2 * (int)ABYTES, "transposition scratch fits the activation buffers");
@@ -634,7 +630,7 @@ void qgemm128_kernel(const QLArgs a) {
         const int r = (lane >> 3) + 8 * j, c4 = (lane & 7) * 4;
         const u32x4 v = lds_ld128(scr + (uint32_t)((r * T_LD + c4) * 4));
         const uint32_t off = ((uint32_t)(m0w + mt * 16 + r) * (uint32_t)a.N + col0 + (uint32_t)c4) * 4u;
-        __builtin_amdgcn_raw_buffer_store_b128(v, rp, off, 0, kWriteThrough);
+        __builtin_amdgcn_raw_buffer_store_b128(v, rp, off, 0, kStreamOnce);
       }
       asm volatile("" ::: "memory");
     }
