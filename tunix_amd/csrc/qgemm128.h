@@ -13,11 +13,13 @@
 //     bunch up and pull look-ups that have not returned yet into waits;
 //   * the code book is an LDS table of f16 level pairs indexed by a code byte, replicated 64
 //     times with a 256-byte entry stride, so that the LDS address of a look-up is one
-//     v_perm_b32: (byte << 8) | (lane << 2); every bf16-rounded level is exact in f16, and
-//     v_fma_mix_f32 multiplies the f16 half it selects with the fp32 scale in one instruction;
-//   * activations are double-buffered in LDS (one barrier per k-tile); packed codes and scales
-//     come through a three-deep register ring filled by buffer loads whose per-k-tile offset
-//     is a scalar, so the loop has no per-load address arithmetic.
+//     v_perm_b32: 0x10000 | (byte << 8) | (lane << 2); every bf16-rounded level is exact in
+//     f16, and v_fma_mix_f32 multiplies the f16 half it selects with the fp32 scale in one
+//     instruction;
+//   * activations are double-buffered in LDS (one barrier per k-tile) and go there straight
+//     from memory (16 bytes per lane, unpadded rows with XOR-swizzled chunks); packed codes and
+//     scales come through a three-deep register ring filled by buffer loads whose per-k-tile
+//     offset is a scalar, so the loop has no per-load address arithmetic.
 //
 // Included by qlinear.hip after QLArgs / store_tile.
 #pragma once
@@ -321,7 +323,8 @@ void qgemm128_kernel(const QLArgs a) {
                    auto LDc, auto EXc, int kt, bool ex_active) {
     constexpr int CUR = decltype(CURc)::value, NXT = CUR ^ 1;
     constexpr int DC = decltype(Dcc)::value, JC = decltype(Jcc)::value;
-    constexpr int DL = decltype(Dlc)::value, JL = decltype(Jlc)::value, JR = decltype(Jrc)::value;
+    constexpr int DL = decltype(Dlc)::value, JL = decltype(Jlc)::value;
+    (void)sizeof(Jrc);   // (the k-step of the fragments to read is part of rd_base)
     constexpr bool ST = decltype(STc)::value != 0, LD = decltype(LDc)::value != 0;
     constexpr int EX = decltype(EXc)::value;   // -1, or the ring stage whose scales to expand
     constexpr int UNITS = NT * 8, MPS = MT * NT;
