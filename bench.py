@@ -179,14 +179,16 @@ def many_rows_breakdown(model, rows, iters):
 # to a hash of the kernel's sources: the figure is reported only while the sources are the ones it
 # was measured on.
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "qgemm128_kernel_llama8b_decode_b128.json")
-KERNEL_SOURCES = ("qgemm128.h", "gemm_tile.h")
+# everything that decides what a GEMM launch reads and writes: the kernel and its tile loop, the
+# store-policy helpers, the dispatch, and the host's choice of the k split
+KERNEL_SOURCES = ("csrc/qgemm128.h", "csrc/gemm_tile.h", "csrc/common.h", "csrc/qlinear.hip", "model.py")
 
 
 def kernel_source_hash():
   import hashlib
   h = hashlib.sha256()
   for name in KERNEL_SOURCES:
-    with open(os.path.join(ROOT, "tunix_amd", "csrc", name), "rb") as f:
+    with open(os.path.join(ROOT, "tunix_amd", name), "rb") as f:
       h.update(f.read())
   return h.hexdigest()[:16]
 
@@ -606,11 +608,18 @@ def main():
       dst.copy_(src)
     # and a second yardstick for reads: 1 GiB fetched once with the 16-byte-per-lane buffer loads
     # the GEMM, attention and head kernels stream their operands with (stream_read_kernel)
-    from tunix_amd import ops as _ops
+    # (a probe of this benchmark, in its own shared object: not part of the product library)
+    import ctypes
+    probe = ctypes.CDLL(os.path.join(ROOT, "tunix_amd", "libtunix_probe.so"))
+    probe.tnx_probe_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int,
+                                            ctypes.c_void_p]
     big = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
     sink = torch.zeros(64, dtype=torch.int32, device=dev)
     for width in (16, 8, 16, 8):      # 8 bytes per lane: the GEMM's packed-code loads
-      _ops.stream_read(big, sink, width)
+      rc = probe.tnx_probe_stream_read(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
+                                       ctypes.c_void_p(big.data_ptr()), big.numel(), width,
+                                       ctypes.c_void_p(sink.data_ptr()))
+      assert rc == 0, "stream-read probe failed"
     torch.cuda.synchronize()
     del big
     many = many_rows_breakdown(model, 8192, max(2, args.kernel_iters // 5))

@@ -56,8 +56,21 @@ extern "C" {
 #define TNX_EPI_F32 4       /* y(fp32) = acc, no rounding                                   */
 
 const char* tnx_last_error(void);
-/* Library/ABI version: (major << 16) | minor.  The minor number counts additions that leave every
- * existing entry point as it was (1: tnx_rmsnorm_moe_combine). */
+/* Library / ABI version: (major << 16) | minor, the value tnx_version() returns.
+ * Rule: the MAJOR number changes whenever an existing entry point changes its argument list or
+ * meaning, or a descriptor struct changes its layout (a field added, removed, moved or retyped):
+ * a caller built against another major number must not call the library.  The MINOR number counts
+ * additions that leave every existing entry point and struct exactly as they were (new entry
+ * points, new enum values); a caller built against minor m runs on any minor >= m of the same
+ * major.  A caller checks tnx_version() >> 16 == TNX_ABI_VERSION_MAJOR and
+ * (tnx_version() & 0xffff) >= TNX_ABI_VERSION_MINOR before its first call.
+ * History: 1.0 first ABI; 1.1 added tnx_rmsnorm_moe_combine (and, against this rule, an argument
+ * of tnx_quantize_pack and a field of tnx_lmhead_desc); 2.0 states the rule, keeps those changes,
+ * adds tnx_attn_desc.segment_ids and the o_* fields of the fused adapter down-projection, and
+ * moves the measurement probe tnx_stream_read out of the library. */
+#define TNX_ABI_VERSION_MAJOR 2
+#define TNX_ABI_VERSION_MINOR 0
+#define TNX_ABI_VERSION ((TNX_ABI_VERSION_MAJOR << 16) | TNX_ABI_VERSION_MINOR)
 int tnx_version(void);
 
 /* ---------------------------------------------------------------------------------------
@@ -240,7 +253,8 @@ int tnx_rope_table(void* stream, const int32_t* positions, int64_t pos_ld, const
 
 /* ---------------------------------------------------------------------------------------
  * GQA attention over the KV cache for T query tokens per row (T = 1: decode).
- * Query token t of row b sits in cache slot c = *col_ptr + t and attends slot j iff
+ * Query token t of row b sits in cache slot c = *col_ptr + t (the caller keeps *col_ptr + T <=
+ * tok_ld, the ids one row of `tokens` holds) and attends slot j iff
  *   j <= c  and  tokens[b*tok_ld + j] != pad_id  and (window == 0 or j > c - window),
  * i.e. the mask of compute_attention_masks (tunix/generate/utils.py:34-58) /
  * make_causal_attn_mask (:61-83) and create_sliding_window_mask (gemma3/model.py:477-496),
@@ -282,6 +296,12 @@ typedef struct tnx_attn_desc {
   int qkv_split;
   const float* rope_sin;     /* fp32 [B, dh/2] from tnx_rope_table                           */
   const float* rope_cos;
+  /* Optional, packed batches (several sequences per row, compute_per_token_logps with
+   * segment_ids, tunix/rl/common.py:260-271, :408-418; qwen3/model.py:622-655): int32
+   * [B, tok_ld] segment id of every slot.  When given, slot j is attended iff j <= c (and the
+   * window test) and segment_ids[b, j] == segment_ids[b, c]; `tokens` and pad_id are not read
+   * (padding is its own segment, as the reference's packed callers arrange it). */
+  const int32_t* segment_ids;
 } tnx_attn_desc;
 size_t tnx_attn_ws_bytes(int64_t B, int64_t T, int64_t S, int Hq, int dh, int kv_chunk);
 int tnx_gqa_attn(void* stream, const tnx_attn_desc* h_desc);
@@ -353,14 +373,16 @@ int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* h_desc);
  * probability exceeds top_p are dropped, and one is drawn by Gumbel-max (jax.random.categorical)
  * with noise from threefry2x32 keyed by fold_in((key0,key1), *step_ptr) (sampler.py:516).
  * rng_variant selects jax's random_bits layout: 1 = partitionable (counter (0,n), x0^x1),
- * 0 = original (counter array split in halves).  k <= 0 or k >= V with top_p >= 1 draws from
- * the whole vocabulary.  logp_out = full-vocabulary log-softmax at the drawn id (:141-144).
- * k <= 1024.  With a workspace `ws` of tnx_sample_topk_ws_bytes(M, V, k) bytes (and
+ * 0 = original (counter array split in halves).  k <= 0 (no top-k) with top_p >= 1 draws from
+ * the whole vocabulary, noise indexed by vocabulary id (:118-121).  logp_out = full-vocabulary
+ * log-softmax at the drawn id (:141-144).
+ * 0 < k < V: k <= 1024.  With a workspace `ws` of tnx_sample_topk_ws_bytes(M, V, k) bytes (and
  * ceil(V / 8192) * k <= 4096, k <= 512) the row is processed in segments by many work-groups and a merging
  * launch; with ws = NULL one work-group per row does everything.  Both give the same result.
- * top_p < 1 without top_k (k <= 0) sorts every row completely, as the reference does with
- * jax.lax.top_k(k = V) (:126-127), and needs ws of tnx_sample_fullsort_ws_bytes(M, V) bytes
- * (four [M,V] arrays plus the sort's scratch; M * V < 2^31). */
+ * k <= 0 with top_p < 1, and k == V with any top_p, sort every row completely, as the reference
+ * does with jax.lax.top_k(k = V) (:126-127), draw over SORTED positions, and need ws of
+ * tnx_sample_fullsort_ws_bytes(M, V) bytes (M * V < 2^31).  k > V returns TNX_EINVAL
+ * (jax.lax.top_k raises). */
 size_t tnx_sample_topk_ws_bytes(int64_t M, int64_t V, int k);
 size_t tnx_sample_fullsort_ws_bytes(int64_t M, int64_t V);
 int tnx_sample_topk(void* stream, const float* logits, int64_t M, int64_t V, int k, float top_p,
@@ -474,13 +496,6 @@ int tnx_logp_drift(void* stream, const float* rollout_logp, const float* trainer
 int64_t tnx_logp_drift_static_max_rows(void);
 int tnx_logp_drift_static(void* stream, const float* rollout_logp, const float* trainer_logp,
                           const float* mask, int64_t B, int64_t T, float* out5);
-
-/* Measurement aid, no counterpart in the reference: reads `bytes` bytes at `src` exactly once with
- * the access pattern of this library's streaming kernels (buffer loads of bytes_per_lane = 16 or
- * 8 bytes per lane) and xors them into sink64[0..63] (64 device words).  A read of known size:
- * run it under a hardware fetch counter next to the kernels of interest to learn what the counter
- * reports per byte for this kind of load. */
-int tnx_stream_read(void* stream, const void* src, uint64_t bytes, int bytes_per_lane, uint32_t* sink64);
 
 /* Fill n 32-bit words with `value` (graph-capturable replacement for hipMemsetAsync). */
 int tnx_fill_u32(void* stream, uint32_t* p, int64_t n, uint32_t value);

@@ -38,9 +38,25 @@ def selective_log_softmax(logits: torch.Tensor, input_ids: torch.Tensor) -> torc
   return tgt - torch.logsumexp(lg, dim=-1)
 
 
-def process_ids(prompt_tokens: np.ndarray, completion_tokens: np.ndarray, pad_id: int):
-  """tunix/rl/common.py:234-291 (unpacked branch)."""
+def segment_attn_mask(segment_ids: np.ndarray) -> np.ndarray:
+  """[B, L, L] bool: query i attends key j iff j <= i and both carry the same segment id -- what the
+  splash-attention path of the packed mode computes from a causal mask kernel plus
+  SegmentIds(q, kv) (tunix/models/qwen3/model.py:622-655)."""
+  seg = np.asarray(segment_ids)
+  L = seg.shape[1]
+  causal = np.tril(np.ones((L, L), dtype=bool))
+  return (seg[:, :, None] == seg[:, None, :]) & causal[None]
+
+
+def process_ids(prompt_tokens: np.ndarray, completion_tokens: np.ndarray, pad_id: int,
+                segment_ids=None, segment_positions=None):
+  """tunix/rl/common.py:234-291.  Packed branch (:260-271): positions are the caller's
+  segment_positions (required), no padding mask; the model separates sequences by segment id."""
   ids = np.concatenate([prompt_tokens, completion_tokens], axis=1)
+  if segment_ids is not None:
+    if segment_positions is None:
+      raise ValueError("segment_positions must be explicitly provided for packed sequences. ")
+    return ids, np.asarray(segment_positions), segment_attn_mask(segment_ids)
   mask = np.concatenate([prompt_tokens != pad_id, completion_tokens != pad_id], axis=-1)
   positions = U.build_positions_from_mask(mask)
   attn_mask = U.make_causal_attn_mask(mask)
@@ -56,14 +72,27 @@ def compute_entropy_from_logits(logits: torch.Tensor) -> torch.Tensor:
 
 
 def compute_per_token_logps(ref_model, prompt_tokens, completion_tokens, pad_id,
-                            temperature: float = 1.0, chunk_size: int = 0, return_entropy: bool = False):
+                            temperature: float = 1.0, chunk_size: int = 0, return_entropy: bool = False,
+                            segment_ids=None, segment_positions=None):
   """tunix/rl/common.py:326-482: one full forward without cache, logits[:, -T-1:-1],
   optional temperature, gather - logsumexp.  chunk_size > 0 follows compute_chunked_logps
-  (:485-571): the head is applied per sequence chunk."""
+  (:485-571): the head is applied per sequence chunk.  Packed mode (segment_ids, :408-418): the
+  whole buffer is scored, logits_to_keep = L - 1, and the result is padded in front with one 0.0
+  so that logp[i] belongs to token[i] (:440-443, :468-472)."""
   ids, positions, attn_mask = process_ids(np.asarray(prompt_tokens), np.asarray(completion_tokens),
-                                          pad_id)
+                                          pad_id, segment_ids, segment_positions)
   B, Ltot = ids.shape
-  T = completion_tokens.shape[1]
+  T = completion_tokens.shape[1] if segment_ids is None else Ltot - 1
+  inner = _logps_of_last(ref_model, ids, positions, attn_mask, T, temperature, chunk_size, return_entropy)
+  if segment_ids is None:
+    return inner
+  pad = lambda x: torch.cat([torch.zeros(B, 1, dtype=x.dtype), x], dim=1)
+  return (pad(inner[0]), pad(inner[1])) if return_entropy else pad(inner)
+
+
+def _logps_of_last(ref_model, ids, positions, attn_mask, T, temperature, chunk_size, return_entropy):
+  """Shared tail of compute_per_token_logps: forward, keep logits[:, -T-1:-1], gather."""
+  B, Ltot = ids.shape
   cache = ref_model.init_cache(B, Ltot)
   tok = torch.from_numpy(ids.astype(np.int64))
   h = ref_model.hidden(tok, torch.from_numpy(positions.astype(np.int64)), cache,

@@ -62,7 +62,12 @@ def test_ctypes_table_matches_header():
 
 def test_version_and_argument_errors_without_gpu():
   lib = L.lib()
-  assert lib.tnx_version() >= 1
+  # the library, the header and the ctypes binding name one and the same ABI version
+  hdr = open(HEADER).read()
+  major = int(re.search(r"#define TNX_ABI_VERSION_MAJOR (\d+)", hdr).group(1))
+  minor = int(re.search(r"#define TNX_ABI_VERSION_MINOR (\d+)", hdr).group(1))
+  assert lib.tnx_version() == (major << 16) | minor
+  assert L.ABI_VERSION == (major, minor)
   cb, sb = ctypes.c_size_t(), ctypes.c_size_t()
   assert lib.tnx_qw_sizes(4096, 4096, 64, ctypes.byref(cb), ctypes.byref(sb)) == 0
   assert cb.value == 4096 * 4096 // 2
@@ -157,16 +162,19 @@ def test_missing_library_fails_loudly(monkeypatch):
 
 
 def test_sampling_plan_uses_one_predicate_for_path_and_workspace():
-  """top_k None / <= 0 / >= V all mean "no top-k" -- for the path AND for the workspace size, as
-  the library itself reads k: a top_k equal to the vocabulary with top_p < 1 must get the
-  full-row sort's workspace, not the (much smaller) segmented top-k one."""
+  """top_k None / <= 0 mean "no top-k"; top_k == V is a real top-k of the whole row in the
+  reference (jax.lax.top_k(k = V), draw over sorted positions: tunix/generate/sampler.py:118-134)
+  and takes the full sort whatever top_p; top_k > V raises as jax.lax.top_k does.  The same
+  predicate decides the workspace: a full sort must get the full-row sort's workspace, not the
+  (much smaller) segmented top-k one."""
   from tunix_amd.generate.sampler import sampling_plan
   V = 1000
   assert sampling_plan(None, 1.0, V) == (0, "head_draw")
   assert sampling_plan(0, 1.0, V) == (0, "head_draw")
-  assert sampling_plan(V, 1.0, V) == (0, "head_draw")
-  assert sampling_plan(V + 5, 0.9, V) == (0, "fullsort")
-  assert sampling_plan(V, 0.9, V) == (0, "fullsort")
+  assert sampling_plan(V, 1.0, V) == (V, "fullsort")
+  assert sampling_plan(V, 0.9, V) == (V, "fullsort")
+  with pytest.raises(ValueError, match="top_k"):
+    sampling_plan(V + 5, 0.9, V)
   assert sampling_plan(None, 0.9, V) == (0, "fullsort")
   assert sampling_plan(50, 0.9, V) == (50, "topk")
   assert sampling_plan(V - 1, 1.0, V) == (V - 1, "topk")

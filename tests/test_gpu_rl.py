@@ -88,6 +88,39 @@ def test_per_token_logps_chunking_and_batching_are_invariant(tiny, gpu):
   assert (one_by_one - full).abs().max().item() <= 1e-2
 
 
+def test_packed_per_token_logps(tiny, gpu):
+  """Packed batches (segment_ids / segment_positions: tunix/rl/common.py:260-271, :408-418): the
+  HIP path against the oracle's packed branch (itself pinned by packed == unpacked), against the
+  same sequences scored alone, and the shape / front padding of the result."""
+  from tunix_amd.rl import common
+  from packed_cases import packed_case
+  cfg, w, model = tiny
+  (A, Bq, Cq), ids, seg, pos = packed_case(cfg.vocab_size)
+  empty = np.zeros((2, 0), np.int32)
+  got = common.compute_per_token_logps(model, empty, ids, pad_id=0, segment_ids=seg, segment_positions=pos)
+  assert tuple(got.shape) == (2, 24) and (got[:, 0] == 0).all()
+  got = got.cpu().numpy()
+  ref = MR.RefModel(cfg, w)
+  want = R.compute_per_token_logps(ref, empty, ids, 0, segment_ids=seg, segment_positions=pos).numpy()
+  real = seg != 0
+  real[:, 0] = False
+  assert np.abs(got - want)[real].max() <= 2e-2
+  for row, off, q in ((0, 0, A), (0, 10, Bq), (1, 0, Cq)):
+    alone = common.compute_per_token_logps(model, q[None, :1], q[None, 1:], pad_id=0).cpu().numpy()[0]
+    # other key-block boundaries and GEMM row tiles than the packed pass: equal up to the bf16
+    # resolution of the logits
+    assert np.abs(got[row, off + 1: off + len(q)] - alone).max() <= 2e-2
+  # entropy comes padded the same way; a missing segment_positions raises as in the reference
+  lp, ent = common.compute_per_token_logps(model, empty, ids, pad_id=0, segment_ids=seg, segment_positions=pos,
+                                           return_entropy=True)
+  assert tuple(ent.shape) == (2, 24) and (ent[:, 0] == 0).all() and np.array_equal(lp.cpu().numpy(), got)
+  with pytest.raises(ValueError, match="segment_positions"):
+    common.compute_per_token_logps(model, empty, ids, pad_id=0, segment_ids=seg)
+  # without the segment ids the second sequence sees the first: its scores move
+  plain = common.compute_per_token_logps(model, ids[:, :1], ids[:, 1:], pad_id=0).cpu().numpy()
+  assert np.abs(plain[0, 10:] - got[0, 11:]).max() > 1e-3
+
+
 def test_per_token_logps_argument_errors(tiny, gpu):
   from tunix_amd.rl import common
   cfg, w, model = tiny

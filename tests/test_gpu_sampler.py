@@ -331,3 +331,74 @@ def test_full_state_replacement_requantises_in_place(tiny, gpu):
     sampler.update_params({"embed": w["embed"][:, :8]})
   with pytest.raises(ValueError, match="same structure"):
     sampler.update_params({"no_such_leaf": w["embed"]})
+
+
+def test_rejected_state_leaves_the_model_untouched(tiny, gpu):
+  """A state that is refused must not have changed anything: every name, fused-member set and
+  shape is checked before the first copy (the reference validates before it replaces,
+  tunix/generate/sampler.py:280-284, :322-325)."""
+  from tunix_amd import dummy_model
+  from tunix_amd.model import QLoRAModel
+  cfg, w, _ = tiny
+  model = QLoRAModel(cfg, w, gpu)
+  w2 = dummy_model.create_dummy_weights(cfg, seed=4242)
+  snap = {"embed": model.embed.clone(), "final_norm": model.final_norm.clone(),
+          "qkv0": model.layers[0]["qkv"].codes.clone(), "o0": model.layers[0]["o"].codes.clone(),
+          "a0": model.layers[0]["qkv"].a_t.clone(), "norm0": model.layers[0]["attn_norm"].clone()}
+
+  def untouched():
+    return (torch.equal(snap["embed"], model.embed) and torch.equal(snap["final_norm"], model.final_norm)
+            and torch.equal(snap["qkv0"], model.layers[0]["qkv"].codes)
+            and torch.equal(snap["o0"], model.layers[0]["o"].codes)
+            and torch.equal(snap["a0"], model.layers[0]["qkv"].a_t)
+            and torch.equal(snap["norm0"], model.layers[0]["attn_norm"]))
+
+  # valid leaves first in iteration order, the offending one last
+  with pytest.raises(ValueError, match="same structure"):   # wk / wv of the fused q|k|v missing
+    model.update_params({"embed": w2["embed"], "final_norm": w2["final_norm"], "l0.wo": w2["l0.wo"],
+                         "l0.attn_norm": w2["l0.attn_norm"], "l1.wq": w2["l1.wq"]})
+  assert untouched()
+  with pytest.raises(ValueError, match="same shape"):
+    model.update_params({"embed": w2["embed"], "l0.wo": w2["l0.wo"], "l1.wo": w2["l1.wo"][:, :64]})
+  assert untouched()
+  with pytest.raises(ValueError, match="same shape"):       # a LoRA leaf of another rank, after valid base leaves
+    model.update_params({"embed": w2["embed"], "l0.wq.lora_a": w2["l0.wq.lora_a"][:, :4],
+                         "l0.wq.lora_b": w2["l0.wq.lora_b"][:4]})
+  assert untouched()
+  lora2 = {k: v for k, v in w2.items() if ".lora_" in k}
+  bad = dict(lora2)
+  last = sorted(k for k in bad if k.endswith(".lora_b"))[-1]
+  bad[last] = bad[last][:, :8]
+  with pytest.raises(ValueError, match="same shape"):       # LoRA-only swap, one wrong shape at the end
+    model.update_lora(bad)
+  assert untouched()
+  model.update_params({"embed": w2["embed"]})                # and a valid partial state goes through
+  assert not torch.equal(snap["embed"], model.embed)
+
+
+def test_top_k_equal_to_the_vocabulary_sorts_the_row(tiny, gpu):
+  """top_k == V is a real top-k in the reference (jax.lax.top_k(k = V): the row is sorted and the
+  draw runs over sorted positions, tunix/generate/sampler.py:118-134), also with top_p = 1.0, so
+  its ids differ from those of top_k = None for the same seed; top_k > V raises."""
+  from oracle import threefry as TF
+  from tunix_amd.generate import CacheConfig, Sampler
+  from tunix_amd.generate.utils import IdTokenizer
+  cfg, w, model = tiny
+  B, P, T = 4, 16, 6
+  V = cfg.vocab_size
+  tok = IdTokenizer(V, pad_id=0, eos_id=1)
+  sampler = Sampler(model, tok, CacheConfig(P + T, cfg.num_layers, cfg.num_kv_heads, cfg.head_dim))
+  prompts = _prompts(B, P, V, 5, ragged=False)
+  out = sampler(prompts, T, max_prompt_length=P, temperature=0.8, top_p=1.0, top_k=V, seed=3,
+                return_logprobs=True, return_logits=True, eos_tokens=[-1])
+  tb = sampler._last_state.token_buffer.cpu().numpy()
+  key = TF.prng_key(3)
+  for c in range(P, P + T):
+    gpu_lg = torch.from_numpy(np.stack([out.logits[b][c - P] for b in range(B)]))
+    t_ref, lp_ref = SR.sample_top_p(gpu_lg, TF.fold_in(key, c - 1), 0.8, 1.0, V)
+    np.testing.assert_array_equal(t_ref.numpy(), tb[:, c])
+    np.testing.assert_allclose(np.array([out.logprobs[b][c - P] for b in range(B)]), lp_ref.numpy(), atol=2e-5)
+  plain = sampler(prompts, T, max_prompt_length=P, temperature=0.8, top_p=1.0, top_k=None, seed=3, eos_tokens=[-1])
+  assert not all(np.array_equal(x, y) for x, y in zip(out.tokens, plain.tokens))
+  with pytest.raises(ValueError, match="top_k"):
+    sampler(prompts, T, max_prompt_length=P, temperature=0.8, top_p=1.0, top_k=V + 1, seed=3)

@@ -272,3 +272,34 @@ def test_sampler_trainer_agreement_against_library_routines_and_closed_forms():
   np.testing.assert_allclose(anti["sampler_trainer/prob_diff_max"], 0.6, rtol=1e-5)
   empty = R.sampler_trainer_agreement(a, b, np.zeros_like(mask))
   assert all(v == 0 for v in empty.values())
+
+
+def test_packed_per_token_logps_equal_unpacked():
+  """The packed branch of compute_per_token_logps (tunix/rl/common.py:260-271, :408-418) must score
+  every sequence as if it stood alone: the gate the reference sets for packing (packed equals
+  unpacked, tests/rl/algo_core_test.py:51-143) applied to the forward pass.  A mask that leaks
+  across a segment boundary, positions that do not restart, or an output shifted by one all fail."""
+  from oracle import model_ref as MR
+  from tunix_amd import config, dummy_model
+  cfg = config.tiny_qwen3(vocab_size=512)
+  w = dummy_model.create_dummy_weights(cfg, seed=5)
+  ref = MR.RefModel(cfg, w, bf16=False)
+  from packed_cases import packed_case
+  (A, Bq, Cq), ids, seg, pos = packed_case(cfg.vocab_size)
+  empty = np.zeros((2, 0), np.int32)
+  packed = R.compute_per_token_logps(ref, empty, ids, 0, segment_ids=seg, segment_positions=pos).numpy()
+  assert packed.shape == (2, 24) and (packed[:, 0] == 0).all()
+  for row, off, q in ((0, 0, A), (0, 10, Bq), (1, 0, Cq)):
+    alone = R.compute_per_token_logps(ref, q[None, :1], q[None, 1:], 0).numpy()[0]
+    np.testing.assert_allclose(packed[row, off + 1: off + len(q)], alone, atol=1e-5)
+  # the mask itself, by brute force
+  m = R.segment_attn_mask(seg)
+  for b in range(2):
+    for i in range(24):
+      for j in range(24):
+        assert m[b, i, j] == (j <= i and seg[b, i] == seg[b, j])
+  # leaking across the boundary changes B's scores (the test has teeth)
+  leak = R.compute_per_token_logps(ref, empty, ids, 0, segment_ids=np.ones_like(seg), segment_positions=pos).numpy()
+  assert np.abs(leak[0, 11:] - packed[0, 11:]).max() > 1e-3
+  with pytest.raises(ValueError, match="segment_positions"):
+    R.compute_per_token_logps(ref, empty, ids, 0, segment_ids=seg)

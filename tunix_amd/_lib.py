@@ -11,6 +11,9 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtunix_hip.so")
 
+# the ABI this binding was written against (TNX_ABI_VERSION_MAJOR / _MINOR of include/tunix_hip.h)
+ABI_VERSION = (2, 0)
+
 TNX_Q_INT4, TNX_Q_NF4 = 0, 1
 TNX_NORM_LLAMA, TNX_NORM_QWEN3, TNX_NORM_GEMMA3 = 0, 1, 2
 TNX_ROPE_LLAMA, TNX_ROPE_QWEN3, TNX_ROPE_GEMMA3 = 0, 1, 2
@@ -58,6 +61,7 @@ class AttnDesc(C.Structure):
       ("tokens", _p), ("tok_ld", _i64), ("col_ptr", _p),
       ("kv_chunk", _i32), ("ws", _p), ("out", _p),
       ("qkv_ws", _p), ("qkv", _p), ("qkv_split", _i32), ("rope_sin", _p), ("rope_cos", _p),
+      ("segment_ids", _p),
   ]
 
 
@@ -125,7 +129,6 @@ SIGNATURES = {
     "tnx_logp_drift": (_i32, [_p, _p, _p, _p, _i64, _i64, _p, _p]),
     "tnx_logp_drift_static_max_rows": (_i64, []),
     "tnx_logp_drift_static": (_i32, [_p, _p, _p, _p, _i64, _i64, _p]),
-    "tnx_stream_read": (_i32, [_p, _p, C.c_uint64, _i32, _p]),
     "tnx_fill_u32": (_i32, [_p, _p, _i64, C.c_uint32]),
 }
 
@@ -146,6 +149,11 @@ def lib() -> C.CDLL:
           "g.build()'` (hipcc --offload-arch=gfx950); there is no CPU fallback"
       )
     handle = C.CDLL(LIB_PATH)
+    handle.tnx_version.restype = _i32
+    v = handle.tnx_version()
+    if (v >> 16) != ABI_VERSION[0] or (v & 0xffff) < ABI_VERSION[1]:
+      raise ImportError(f"{LIB_PATH} has ABI version {v >> 16}.{v & 0xffff}; this binding needs "
+                        f"{ABI_VERSION[0]}.x with x >= {ABI_VERSION[1]} (rebuild the library)")
     for name, (res, args) in SIGNATURES.items():
       fn = getattr(handle, name)
       fn.restype = res

@@ -31,8 +31,9 @@ struct AttnArgs {
   const uint16_t* q;
   const uint16_t* k;
   const uint16_t* v;
-  const int32_t* tokens;
+  const int32_t* tokens;       // token ids, or (seg_mode) the segment ids of a packed batch
   int64_t tok_ld;
+  int seg_mode;                // 0: a key counts when its token != pad_id; 1: when its segment id equals the query's
   const int32_t* col_ptr;
   int kv_chunk, n_chunks;
   float* ws;
@@ -104,6 +105,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
   const uint16_t* kbase = a.k + ((b * a.Hkv + hkv) * a.S) * DH;
   const uint16_t* vbase = a.v + ((b * a.Hkv + hkv) * a.S) * DH;
   const int32_t* tok = a.tokens + b * a.tok_ld;
+  // what a key's id is compared with: the pad id (the key counts when it differs), or, for packed
+  // batches, the segment id of this lane's query token (the key counts when it is equal)
+  // (loaded in both modes: a branch around a load would make the counted waits behind it inexact)
+  const int32_t id_q = tok[min((int64_t)c_n, a.tok_ld - 1)];
+  const int32_t id_ref = a.seg_mode ? id_q : a.pad_id;
+  const bool id_equal = a.seg_mode != 0;
   const int vcol = (8 * lm) % (DH < 128 ? DH : 128);     // DH=64: upper lanes duplicate
   // TOKVEC: 16-byte token loads; the host chooses them when rows are 16-byte aligned and hold
   // whole groups of four slots (keys beyond the range are masked by the range test anyway).  A
@@ -128,7 +135,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
   // the end) read zeros; they are masked by the range test anyway.
   const uint32_t slab_bytes = (uint32_t)a.S * DH * 2u;
   const rsrc_t rk = make_rsrc(kbase, slab_bytes), rv = make_rsrc(vbase, slab_bytes);
-  const rsrc_t rtok = make_rsrc(tok, (uint64_t)a.S * 4);
+  // (the row holds tok_ld ids: slots past them read zeros, and the range test masks them)
+  const rsrc_t rtok = make_rsrc(tok, (uint64_t)min(a.S, a.tok_ld) * 4);
   const uint32_t koff = (uint32_t)(lm * DH + lq * 8) * 2u;           // + tt * 16 keys, + j * 64 B
   const uint32_t voff = (uint32_t)(4 * lq * DH + vcol) * 2u;         // + s keys, + 16 keys, + h * 256 B
   auto load_block = [&](int kb, Stage& sg) {
@@ -167,7 +175,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       const int key = kb + (s < 4 ? 4 * lq + s : 16 + 4 * lq + (s - 4));
-      kvalid[s] = qvalid && key >= max(k_lo, lo_n) && key <= min(k_hi, key_hi) && sg.tk[s] != a.pad_id;
+      kvalid[s] = qvalid && key >= max(k_lo, lo_n) && key <= min(k_hi, key_hi) && ((sg.tk[s] == id_ref) == id_equal);
     }
     // ---- S^T = K . q^T ----
     f32x4 st[2];
@@ -566,9 +574,9 @@ extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
   TNX_REQUIRE(d->Hkv > 0 && d->Hq % d->Hkv == 0, "attn: Hq=%d not a multiple of Hkv=%d", d->Hq, d->Hkv);
   const int G = d->Hq / d->Hkv;
   TNX_REQUIRE(G <= 16, "attn: group size %d > 16 not supported", G);
-  TNX_REQUIRE(d->kcache && d->vcache && d->tokens && d->col_ptr && d->out, "attn: null pointer");
+  TNX_REQUIRE(d->kcache && d->vcache && (d->tokens || d->segment_ids) && d->col_ptr && d->out, "attn: null pointer");
   TNX_REQUIRE(d->kv_chunk >= 0 && d->kv_chunk % 32 == 0, "attn: kv_chunk must be a multiple of 32");
-  TNX_REQUIRE(d->tok_ld >= d->S || d->tok_ld > 0, "attn: bad tok_ld");
+  TNX_REQUIRE(d->tok_ld > 0, "attn: tok_ld=%lld must be positive", (long long)d->tok_ld);
   AttnArgs a;
   a.B = d->B; a.T = d->T; a.S = d->S; a.Hq = d->Hq; a.Hkv = d->Hkv; a.dh = d->dh;
   a.G = G; a.Gp = next_pow2(G);
@@ -581,7 +589,8 @@ extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
     a.scale_bf = 0.f;
   }
   a.window = d->window; a.pad_id = d->pad_id;
-  a.q = d->q; a.k = d->kcache; a.v = d->vcache; a.tokens = d->tokens; a.tok_ld = d->tok_ld;
+  a.q = d->q; a.k = d->kcache; a.v = d->vcache; a.tokens = d->segment_ids ? d->segment_ids : d->tokens; a.tok_ld = d->tok_ld;
+  a.seg_mode = d->segment_ids ? 1 : 0;
   a.col_ptr = d->col_ptr; a.kv_chunk = d->kv_chunk;
   a.n_chunks = d->kv_chunk > 0 ? (int)cdiv(d->S, d->kv_chunk) : 1;
   a.ws = d->ws; a.out = d->out;
@@ -603,7 +612,7 @@ extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
   TNX_REQUIRE(d->B * QT <= 65535 * 32, "attn: too many query tiles");
   dim3 grid((unsigned)a.n_chunks, (unsigned)d->Hkv, (unsigned)(d->B * QT));
   hipStream_t st = as_stream(stream);
-  const bool tv = (d->tok_ld % 4 == 0) && ((reinterpret_cast<uintptr_t>(d->tokens) & 15) == 0) && d->S % 4 == 0;
+  const bool tv = (d->tok_ld % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.tokens) & 15) == 0) && d->S % 4 == 0;
 #define TNX_ATTN_LAUNCH(DH, FUSE)                                                                \
   do {                                                                                           \
     if (tv) hipLaunchKernelGGL((attn_kernel<DH, FUSE, true>), grid, dim3(64), 0, st, a);         \

@@ -679,7 +679,7 @@ extern "C" size_t tnx_sample_fullsort_ws_bytes(int64_t M, int64_t V) {
 
 extern "C" size_t tnx_sample_topk_ws_bytes(int64_t M, int64_t V, int k) {
   if (M <= 0 || V <= 0) return 0;
-  if (k <= 0 || k >= V) k = 0;  // whole-vocabulary draw: (max, sum, noisy best, its id, its logit)
+  if (k <= 0 || k >= V) k = 0;  // whole-vocabulary draw: (max, sum, noisy best, its id, its logit); k == V takes the full sort
   return (size_t)(M * cdiv(V, kSegElems) * (k > 0 ? 2 + 2 * (int64_t)k : 5)) * sizeof(float);
 }
 
@@ -692,10 +692,15 @@ extern "C" int tnx_sample_topk(void* stream, const float* logits, int64_t M, int
   TNX_REQUIRE(M > 0 && V > 0 && V < (1ll << 31), "sample_topk: bad shape");
   TNX_REQUIRE(rng_variant == 0 || rng_variant == 1, "sample_topk: rng_variant must be 0 or 1");
   TNX_REQUIRE(temperature > 0.f, "sample_topk: temperature must be positive, got %f", temperature);
-  if (k <= 0 || k >= V) {
-    if (top_p < 1.0f) {
-      TNX_REQUIRE(ws, "sample_topk: top_p < 1 without top_k sorts the whole row and needs a workspace of "
-                      "tnx_sample_fullsort_ws_bytes(M, V) bytes");
+  // jax.lax.top_k refuses k beyond the last axis (sampler.py:126-127)
+  TNX_REQUIRE(k <= V, "sample_topk: top_k=%d exceeds the vocabulary (%lld)", k, (long long)V);
+  if (k <= 0 || k == V) {
+    // no top-k with top_p < 1, or a top-k of the whole vocabulary (whatever top_p): the reference
+    // sorts the row and draws over SORTED positions; only top_k absent with top_p >= 1 draws over
+    // vocabulary ids (sampler.py:118-127)
+    if (top_p < 1.0f || k == V) {
+      TNX_REQUIRE(ws, "sample_topk: top_p < 1 without top_k (or top_k == V) sorts the whole row and needs a "
+                      "workspace of tnx_sample_fullsort_ws_bytes(M, V) bytes");
       TNX_REQUIRE(M * V < (1ll << 31), "sample_topk: M * V too large for the full-row sort");
       FullSortWs w;
       TNX_REQUIRE(fullsort_layout(M, V, &w) == 0, "sample_topk: rocPRIM refused the sort configuration");

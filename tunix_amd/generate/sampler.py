@@ -41,13 +41,19 @@ def _threefry_seed(seed: int) -> tuple[int, int]:
 
 def sampling_plan(top_k: int | None, top_p: float, vocab_size: int) -> tuple[int, str]:
   """(k passed to tnx_sample_topk, which path it takes there) for a top_p-mode call
-  (sampler.py:105-148).  top_k None, <= 0 or >= vocab_size all mean "no top-k", exactly as the
-  library reads k (k <= 0 or k >= V): then top_p >= 1 is the categorical draw inside the head
-  ("head_draw") and top_p < 1 sorts whole rows ("fullsort", workspace of
-  tnx_sample_fullsort_ws_bytes); a real top-k uses the segmented selection ("topk", workspace of
+  (sampler.py:105-148).  top_k None or <= 0 means "no top-k" (:118): then top_p >= 1 is the
+  categorical draw inside the head ("head_draw", noise per vocabulary id) and top_p < 1 sorts whole
+  rows ("fullsort", workspace of tnx_sample_fullsort_ws_bytes).  top_k == vocab_size is a real
+  top-k in the reference -- jax.lax.top_k(k = V) sorts the row and the draw runs over sorted
+  positions, whatever top_p -- so it takes the full sort too; top_k > vocab_size raises as
+  jax.lax.top_k does.  Any other top_k uses the segmented selection ("topk", workspace of
   tnx_sample_topk_ws_bytes).  One predicate decides both the path and the workspace size."""
-  if top_k is None or top_k <= 0 or top_k >= vocab_size:
+  if top_k is None or top_k <= 0:
     return 0, ("head_draw" if top_p >= 1.0 else "fullsort")
+  if top_k > vocab_size:
+    raise ValueError(f"top_k={top_k} must be at most the vocabulary size {vocab_size}")
+  if top_k == vocab_size:
+    return int(top_k), "fullsort"
   return int(top_k), "topk"
 
 

@@ -8,9 +8,7 @@ kernel.  LoRA A/B stay separate buffers so that `update_lora` can swap them betw
 """
 from __future__ import annotations
 
-import json
 import math
-import os
 
 import numpy as np
 import torch
@@ -72,18 +70,39 @@ class FusedLinear:
         self._row_perm = (cc // 16) * 32 + h * 16 + (cc % 16)
       self.load_lora(weights)
 
-  def load_base(self, weights: dict):
-    """(Re-)quantises and packs the base kernels of every member from `weights` (all members of a
-    fused projection must be present, with the shapes the linear was built with)."""
-    ws = []
+  def check_base(self, weights: dict):
+    """Raises ValueError unless `weights` holds every member of this projection in the shape it was
+    built with; touches nothing."""
     for n, wd in zip(self.names, self.widths):
       if n not in weights:
         raise ValueError(f"New state must have the same structure as the old state: {n} is missing")
-      w = weights[n]
-      if tuple(w.shape) != (self.K, wd):
-        raise ValueError(f"New state must have the same shape as the old state: {n} {tuple(w.shape)} "
+      if tuple(weights[n].shape) != (self.K, wd):
+        raise ValueError(f"New state must have the same shape as the old state: {n} {tuple(weights[n].shape)} "
                          f"vs {(self.K, wd)}")
-      ws.append(w.to(device=self.device, dtype=torch.bfloat16))
+
+  def check_lora(self, weights: dict):
+    """Raises ValueError for an adapter leaf of this projection whose shape differs from the one
+    it was built with, or whose partner leaf is missing; touches nothing."""
+    if not self.has_lora:
+      return
+    for n, wd in zip(self.names, self.widths):
+      a, b = weights.get(n + ".lora_a"), weights.get(n + ".lora_b")
+      if a is None and b is None:
+        continue
+      if a is None or b is None:
+        raise ValueError(f"New state must have the same structure as the old state: {n} has one LoRA leaf only")
+      if tuple(a.shape) != (self.K, self.r) or tuple(b.shape) != (self.r, wd):
+        raise ValueError(
+            f"New state must have the same shape as the old state: {n} lora_a {tuple(a.shape)}"
+            f" lora_b {tuple(b.shape)} vs {(self.K, self.r)} / {(self.r, wd)}")
+
+  def load_base(self, weights: dict):
+    """(Re-)quantises and packs the base kernels of every member from `weights` (all members of a
+    fused projection must be present, with the shapes the linear was built with)."""
+    self.check_base(weights)
+    ws = []
+    for n, wd in zip(self.names, self.widths):
+      ws.append(weights[n].to(device=self.device, dtype=torch.bfloat16))
     w = torch.cat(ws, dim=1).contiguous() if len(ws) > 1 else ws[0].contiguous()
     codes, scales = ops.quantize_pack(w, self.group, self.qtype, self.interleave2, self.int4_bound)
     if self.codes is None:
@@ -96,16 +115,13 @@ class FusedLinear:
     """Copies lora_a [K,r] / lora_b [r,N_i] of every member into the kernel layout."""
     if not self.has_lora:
       return
+    self.check_lora(weights)
     b_full = torch.zeros(self.N, self.rp, dtype=torch.bfloat16, device=self.b_t.device)
     off = 0
     for i, (n, wd) in enumerate(zip(self.names, self.widths)):
       a = weights.get(n + ".lora_a")
       if a is not None:
         b = weights[n + ".lora_b"]
-        if tuple(a.shape) != (self.K, self.r) or tuple(b.shape) != (self.r, wd):
-          raise ValueError(
-              f"New state must have the same shape as the old state: {n} lora_a {tuple(a.shape)}"
-              f" lora_b {tuple(b.shape)} vs {(self.K, self.r)} / {(self.r, wd)}")
         self.a_t[i * self.rp: i * self.rp + self.r].copy_(a.to(self.a_t.device, torch.bfloat16).t())
         b_full[off: off + wd, : self.r].copy_(b.to(self.b_t.device, torch.bfloat16).t())
       off += wd
@@ -136,15 +152,21 @@ class ExpertBank:
     self.router_t = torch.empty(E, self.D, dtype=torch.bfloat16, device=device)
     self.load_base(weights)
 
-  def load_base(self, weights: dict):
-    """(Re-)quantises the experts and copies the router from `weights`, in place."""
-    cfg, prefix, device, E = self.cfg, self.prefix, self.device, self.E
+  def check_base(self, weights: dict):
+    """Raises ValueError unless `weights` holds the router and the three expert kernels in the
+    shapes the bank was built with; touches nothing."""
+    prefix, E = self.prefix, self.E
     for n, shape in ((prefix + "e_gate", (E, self.D, self.F)), (prefix + "e_up", (E, self.D, self.F)),
                      (prefix + "e_down", (E, self.F, self.D)), (prefix + "router", (self.D, E))):
       if n not in weights:
         raise ValueError(f"New state must have the same structure as the old state: {n} is missing")
       if tuple(weights[n].shape) != shape:
         raise ValueError(f"New state must have the same shape as the old state: {n} {tuple(weights[n].shape)} vs {shape}")
+
+  def load_base(self, weights: dict):
+    """(Re-)quantises the experts and copies the router from `weights`, in place."""
+    self.check_base(weights)
+    cfg, prefix, device, E = self.cfg, self.prefix, self.device, self.E
     g, u, d = weights[prefix + "e_gate"], weights[prefix + "e_up"], weights[prefix + "e_down"]
     cb, sb = ops.qw_sizes(self.D, 2 * self.F, cfg.group)
     cb2, sb2 = ops.qw_sizes(self.F, self.D, cfg.group)
@@ -210,13 +232,18 @@ class QLoRAModel:
       raise ValueError(
           "New state must have the same structure as the old state. "
           f"missing={sorted(expected - set(new_lora))} extra={sorted(set(new_lora) - expected)}")
-    for ly in self.layers:
-      for key in ("qkv", "o", "gu", "down"):
-        if key in ly:
-          ly[key].load_lora(new_lora)
-    if self.head is not None:
-      self.head.load_lora(new_lora)
+    linears = self._linears()
+    for f in linears:      # every shape is checked before the first copy: a rejected state changes nothing
+      f.check_lora(new_lora)
+    for f in linears:
+      f.load_lora(new_lora)
     torch.cuda.synchronize(self.device)
+
+  def _linears(self) -> list:
+    out = [ly[key] for ly in self.layers for key in ("qkv", "o", "gu", "down") if key in ly]
+    if self.head is not None:
+      out.append(self.head)
+    return out
 
   # full state replacement (tunix/generate/sampler.py:265-332; VanillaRollout.update_params,
   # tunix/rl/rollout/vanilla_rollout.py:92-121, merges a partial state into the old one first)
@@ -242,41 +269,60 @@ class QLoRAModel:
     if extra:
       raise ValueError(f"New state must have the same structure as the old state. extra={extra}")
 
-    def copy_into(dst: torch.Tensor, name: str, transpose: bool = False):
-      src = base[name].to(dev, bf)
-      src = src.t() if transpose else src
-      if tuple(src.shape) != tuple(dst.shape):
+    # First pass: every name, fused-member set and shape is checked and the work is only listed;
+    # a state that is rejected leaves the model exactly as it was (the reference validates the
+    # structure before it replaces anything, sampler.py:280-284, :322-325).
+    copies, reloads = [], []
+
+    def plan_copy(dst: torch.Tensor, name: str, transpose: bool = False):
+      shape = tuple(base[name].shape)[::-1] if transpose else tuple(base[name].shape)
+      if shape != tuple(dst.shape):
         raise ValueError(f"New state must have the same shape as the old state: {name} {tuple(base[name].shape)}")
-      dst.copy_(src)
+      copies.append((dst, name, transpose))
 
     if "embed" in base:
-      copy_into(self.embed, "embed")
+      plan_copy(self.embed, "embed")
     if "final_norm" in base:
-      copy_into(self.final_norm, "final_norm")
+      plan_copy(self.final_norm, "final_norm")
     if "lm_head" in base:
       if self.head is not None:
-        self.head.load_base(base)
+        self.head.check_base(base)
+        reloads.append(self.head)
       elif self.head_w is not None:
-        copy_into(self.head_w, "lm_head", transpose=True)
+        plan_copy(self.head_w, "lm_head", transpose=True)
     for i, ly in enumerate(self.layers):
       p = f"l{i}."
       for n in ("attn_norm", "mlp_norm", "q_norm", "k_norm", "post_attn_norm", "post_ffw_norm"):
         if p + n in base:
           if n not in ly:
             raise ValueError(f"New state must have the same structure as the old state. extra={[p + n]}")
-          copy_into(ly[n], p + n)
+          plan_copy(ly[n], p + n)
       for key in ("qkv", "o", "gu", "down"):
         if key in ly and any(n in base for n in ly[key].names):
-          ly[key].load_base(base)
+          ly[key].check_base(base)
+          reloads.append(ly[key])
       if "experts" in ly and any(p + n in base for n in ("router", "e_gate", "e_up", "e_down")):
-        ly["experts"].load_base(base)
+        ly["experts"].check_base(base)
+        reloads.append(ly["experts"])
+      elif "experts" not in ly and any(p + n in base for n in ("router", "e_gate", "e_up", "e_down")):
+        raise ValueError(f"New state must have the same structure as the old state. extra={[p + 'e_gate']}")
+    linears = self._linears()
     if lora:
-      for ly in self.layers:
-        for key in ("qkv", "o", "gu", "down"):
-          if key in ly:
-            ly[key].load_lora(lora)
-      if self.head is not None:
-        self.head.load_lora(lora)
+      known_lora = {n + sfx for n in self.cfg.lora_names() for sfx in (".lora_a", ".lora_b")}
+      extra = sorted(set(lora) - known_lora)
+      if extra:
+        raise ValueError(f"New state must have the same structure as the old state. extra={extra}")
+      for f in linears:
+        f.check_lora(lora)
+    # Second pass: nothing below raises for a reason the first pass could have seen.
+    for dst, name, transpose in copies:
+      src = base[name].to(dev, bf)
+      dst.copy_(src.t() if transpose else src)
+    for obj in reloads:
+      obj.load_base(base)
+    if lora:
+      for f in linears:
+        f.load_lora(lora)
     torch.cuda.synchronize(self.device)
 
   def weight_bytes(self) -> dict:
@@ -311,7 +357,7 @@ class Runner:
   """
 
   def __init__(self, model: QLoRAModel, B: int, T: int, S: int, pad_id: int, kv_chunk=None,
-               want_logits: bool = False):
+               want_logits: bool = False, split_k_override: dict | None = None):
     cfg = model.cfg
     self.model, self.cfg, self.B, self.T, self.S = model, cfg, B, T, S
     self.pad_id = int(pad_id)
@@ -341,8 +387,8 @@ class Runner:
       self.y_route = torch.empty(M * k, D, dtype=bf, device=dev)
     else:
       self.act = torch.empty(M, F, dtype=bf, device=dev)
-    # tuning knob: TUNIX_SPLIT_K='{"o": 4}' pins the k split of the linears with that name
-    self.split_k_override = json.loads(os.environ.get("TUNIX_SPLIT_K", "{}"))
+    # {"wo": 4} pins the k split of the linears of that name (a sweep's handle; empty in normal use)
+    self.split_k_override = dict(split_k_override or {})
     self.fuse_rope = True   # decode: RoPE + cache write inside the attention kernel where it can
     self.rope_sin = torch.empty(B, max(cfg.head_dim // 2, 1), dtype=torch.float32, device=dev)
     self.rope_cos = torch.empty_like(self.rope_sin)
@@ -459,9 +505,13 @@ class Runner:
     ops.rmsnorm_pair(w, self.h, w2, self.xn, cfg.norm_eps, _NORM[cfg.family], M, cfg.embed_dim,
                      res_post=self.h, **kw)
 
-  def forward_hidden(self, tokens, positions, col_ptr, kcache, vcache, B=None, T=None):
+  def forward_hidden(self, tokens, positions, col_ptr, kcache, vcache, B=None, T=None, segment_ids=None):
     """Runs all layers for tokens[b, col .. col+T) of each row; leaves the final-normed hidden
-    state in self.xn[:B*T].  kcache/vcache: lists of [B,Hkv,S,dh] tensors."""
+    state in self.xn[:B*T].  kcache/vcache: lists of [B,Hkv,S,dh] tensors.  segment_ids (int32,
+    the shape of `tokens`): a packed batch, attention stays inside a token's own segment."""
+    if segment_ids is not None and (tuple(segment_ids.shape) != tuple(tokens.shape)
+                                    or segment_ids.dtype != torch.int32 or not segment_ids.is_contiguous()):
+      raise ValueError("segment_ids must be a contiguous int32 tensor of the token buffer's shape")
     cfg, m = self.cfg, self.model
     B = self.B if B is None else B
     T = self.T if T is None else T
@@ -512,6 +562,8 @@ class Runner:
       ad.q, ad.kcache, ad.vcache = self.q.data_ptr(), kcache[i].data_ptr(), vcache[i].data_ptr()
       ad.tokens, ad.tok_ld, ad.col_ptr = tokens.data_ptr(), tokens.shape[1], col_ptr.data_ptr()
       ad.kv_chunk = self.kv_chunk if T == 1 else 0
+      if segment_ids is not None:
+        ad.segment_ids = segment_ids.data_ptr()
       ad.ws, ad.out = self.attn_ws.data_ptr(), self.attn.data_ptr()
       if fuse_rope:
         if qkv_split > 1:

@@ -259,12 +259,6 @@ def logp_drift_static(rollout_logp, trainer_logp, mask, out5):
                                         _ptr(out5)), "tnx_logp_drift_static")
 
 
-def stream_read(src: torch.Tensor, sink64: torch.Tensor, bytes_per_lane: int = 16):
-  """Reads every byte of `src` once with 16- or 8-byte buffer loads (a yardstick for fetch counters)."""
-  L.check(L.lib().tnx_stream_read(_stream(), _ptr(src), src.numel() * src.element_size(), bytes_per_lane,
-                                  _ptr(sink64)), "tnx_stream_read")
-
-
 def fill_u32(t: torch.Tensor, value: int = 0):
   assert t.element_size() == 4
   L.check(L.lib().tnx_fill_u32(_stream(), _ptr(t), t.numel(), value), "tnx_fill_u32")

@@ -46,8 +46,18 @@ def process_ids(prompt_tokens: torch.Tensor, completion_tokens: torch.Tensor, pa
 def compute_per_token_logps(model: QLoRAModel, prompt_tokens, completion_tokens, pad_id: int,
                             eos_id: int | None = None, *, temperature: float = 1.0,
                             chunk_size: int = 0, return_entropy: bool = False,
+                            segment_ids=None, segment_positions=None,
                             max_rows: int = 16384, logits_fp32: bool = False) -> torch.Tensor:
   """fp32 [B, completion_len]: log p(completion token | everything before it).
+
+  Packed batches (tunix/rl/common.py:260-271, :408-418, :440-443, :468-472): with `segment_ids`
+  [B, L] a row of completion_tokens holds several prompt + completion sequences one after the
+  other (prompt_tokens is then [B, 0]), `segment_positions` [B, L] gives every token its position
+  inside its own sequence (required, as in the reference), a token attends the earlier tokens of
+  its own segment only (the causal mask combined with equal segment ids, what the reference's
+  flash-attention path computes from SegmentIds: tunix/models/qwen3/model.py:622-655), no padding
+  mask is applied, every position but the first is scored and the result is [B, L] with 0.0 in
+  column 0, so that logp[i] belongs to token[i].
 
   prompt_tokens [B, P] (left padded) and completion_tokens [B, T] (right padded) are integer
   arrays or tensors.  `temperature` divides the logits as in the reference (:431-436: ignored
@@ -66,10 +76,24 @@ def compute_per_token_logps(model: QLoRAModel, prompt_tokens, completion_tokens,
     raise ValueError(f"prompt_tokens {tuple(pt.shape)} and completion_tokens {tuple(ct.shape)} "
                      "must be [B, P] and [B, T]")
   B, T = ct.shape
-  ids, positions = process_ids(pt, ct, pad_id)
+  seg = None
+  if segment_ids is not None:
+    if segment_positions is None:
+      raise ValueError("segment_positions must be explicitly provided for packed sequences. ")
+    ids = torch.cat([pt, ct], dim=1).to(torch.int32).contiguous()
+    as_i32 = lambda a: torch.as_tensor(np.asarray(a) if not isinstance(a, torch.Tensor) else a).to(dev, torch.int32).contiguous()
+    seg, positions = as_i32(segment_ids), as_i32(segment_positions)
+    if tuple(seg.shape) != tuple(ids.shape) or tuple(positions.shape) != tuple(ids.shape):
+      raise ValueError(f"segment_ids {tuple(seg.shape)} and segment_positions {tuple(positions.shape)} must "
+                       f"have the shape of the token buffer {tuple(ids.shape)}")
+    T = ids.shape[1] - 1          # every position but the first is scored (:440-443)
+    pad_front = True
+  else:
+    ids, positions = process_ids(pt, ct, pad_id)
+    pad_front = False
   Ltot = ids.shape[1]
-  if T == 0:
-    empty = torch.zeros(B, 0, dtype=torch.float32, device=dev)
+  if T <= 0:
+    empty = torch.zeros(B, Ltot if pad_front else 0, dtype=torch.float32, device=dev)
     return (empty, torch.zeros_like(empty)) if return_entropy else empty
   if Ltot < T + 1:
     raise ValueError("the first completion token needs at least one token before it")
@@ -92,7 +116,8 @@ def compute_per_token_logps(model: QLoRAModel, prompt_tokens, completion_tokens,
   for b0 in range(0, B, rows_b):
     nb = min(rows_b, B - b0)
     xn = runner.forward_hidden(ids[b0:b0 + nb], positions[b0:b0 + nb], runner.zero,
-                               [kc[:nb]] * cfg.num_layers, [vc[:nb]] * cfg.num_layers, B=nb, T=Ltot)
+                               [kc[:nb]] * cfg.num_layers, [vc[:nb]] * cfg.num_layers, B=nb, T=Ltot,
+                               segment_ids=None if seg is None else seg[b0:b0 + nb])
     # logits[:, -T-1:-1] predict the completion tokens (:462-467)
     xs = xsel[: nb * T]
     xs.view(nb, T, -1).copy_(xn[: nb * Ltot].view(nb, Ltot, -1)[:, Ltot - T - 1: Ltot - 1])
@@ -105,6 +130,9 @@ def compute_per_token_logps(model: QLoRAModel, prompt_tokens, completion_tokens,
         kw = dict(entropy=ent[b0:b0 + nb].view(-1)[r0:r0 + nr], part_entropy=part_ent)
       runner.run_head(xs[r0:r0 + nr], nr, temperature=temp, targets=tg[r0:r0 + nr],
                       target_logp=lp[r0:r0 + nr], logits_fp32=logits_fp32, **kw)
+  if pad_front:   # one 0.0 in front: logp[i] belongs to token[i] (:468-472)
+    front = lambda x: torch.cat([torch.zeros(B, 1, dtype=torch.float32, device=dev), x], dim=1)
+    return (front(out), front(ent)) if return_entropy else front(out)
   return (out, ent) if return_entropy else out
 
 
