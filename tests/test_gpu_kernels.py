@@ -1070,14 +1070,17 @@ def test_moe_route_sort_gmm_combine(gpu, M, E, k, D, F):
     (8, 512, 2, 512, 256, 128, Q.INT4, False),    # ~128 rows per expert: the 128 x 256 tiles of the many-row kernel
     (8, 512, 2, 384, 512, 64, Q.NF4, True),
     (8, 512, 2, 256, 768, 32, Q.INT4, False),
+    (8, 64, 2, 384, 96, 64, Q.NF4, False),        # 16 rows per expert on average: the 32-row tile kernel, whose
+    (8, 128, 2, 256, 96, 128, Q.INT4, False),     # activation rows are gathered straight into LDS; 32: its 64-row form
 ])
 def test_moe_gmm_skewed_routes(gpu, E, n_tok, k, K, N, group, qtype, mul):
   """The grouped GEMM alone, on routes built by hand: experts with no rows, with one row, with
   exactly one row block and with more (several row blocks of one expert), gathered through a
   shuffled route order; k-tile counts below the streaming kernel's ring depth; both code books,
   two and four scale slots, the plain and the SiLU-mul epilogue; decode-sized batches (the
-  streaming kernel), a shape the general tile kernel takes, and many rows per expert (the
-  128 x 256 tiles of the many-row kernel)."""
+  streaming kernel), a shape the general tile kernel takes, the 32- and 64-row tile kernels (whose
+  loads straight into LDS take their row offsets from the gathered route list), and many rows per
+  expert (the 128 x 256 tiles of the many-row kernel)."""
   from tunix_amd import _lib as L
   from tunix_amd import ops
   rng = np.random.Generator(np.random.PCG64(2000 + E + N))
@@ -1085,7 +1088,7 @@ def test_moe_gmm_skewed_routes(gpu, E, n_tok, k, K, N, group, qtype, mul):
   if E == 16:
     cnt = np.zeros(E, dtype=np.int64)
     cnt[[0, 2, 3, 5, 6, 7]] = [40, 3, 17, 1, 16, n_routes - 77]
-  elif E == 8:   # empty experts, one row, exactly one 128-row block, one row more, several blocks
+  elif E == 8 and n_routes >= 1024:   # empty experts, one row, exactly one 128-row block, one row more, several blocks
     cnt = np.array([300, 0, 129, 128, 1, 200, n_routes - 758, 0], dtype=np.int64)
   else:
     ids = rng.integers(0, E - 3, size=n_routes)
