@@ -66,8 +66,8 @@ const char* tnx_last_error(void);
  * (tnx_version() & 0xffff) >= TNX_ABI_VERSION_MINOR before its first call.
  * History: 1.0 first ABI; 1.1 added tnx_rmsnorm_moe_combine (and, against this rule, an argument
  * of tnx_quantize_pack and a field of tnx_lmhead_desc); 2.0 states the rule, keeps those changes,
- * adds tnx_attn_desc.segment_ids and the o_* fields of the fused adapter down-projection, and
- * moves the measurement probe tnx_stream_read out of the library. */
+ * adds tnx_attn_desc.segment_ids, reads top_k == V in tnx_sample_topk as a real top-k, and moves
+ * the measurement probe tnx_stream_read out of the library. */
 #define TNX_ABI_VERSION_MAJOR 2
 #define TNX_ABI_VERSION_MINOR 0
 #define TNX_ABI_VERSION ((TNX_ABI_VERSION_MAJOR << 16) | TNX_ABI_VERSION_MINOR)
@@ -381,7 +381,8 @@ int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* h_desc);
  * launch; with ws = NULL one work-group per row does everything.  Both give the same result.
  * k <= 0 with top_p < 1, and k == V with any top_p, sort every row completely, as the reference
  * does with jax.lax.top_k(k = V) (:126-127), draw over SORTED positions, and need ws of
- * tnx_sample_fullsort_ws_bytes(M, V) bytes (M * V < 2^31).  k > V returns TNX_EINVAL
+ * tnx_sample_fullsort_ws_bytes(M, V) bytes (two pairs of [M, V] key / id arrays for the library's
+ * own stable radix sort; M * V < 2^31).  k > V returns TNX_EINVAL
  * (jax.lax.top_k raises). */
 size_t tnx_sample_topk_ws_bytes(int64_t M, int64_t V, int k);
 size_t tnx_sample_fullsort_ws_bytes(int64_t M, int64_t V);

@@ -912,6 +912,41 @@ def test_sample_top_p_over_the_whole_vocabulary(gpu, V, top_p, variant):
     ops.sample_topk(logits.to(gpu), 0, top_p, temp, (int(key[0]), int(key[1])), variant, stp, None, ids, lp)
 
 
+@pytest.mark.parametrize("M,V", [(3, 100), (5, 4097), (4, 262144), (130, 2000)])
+def test_full_row_sort_is_stable_and_descending(gpu, M, V):
+  """The library's own radix sort behind the whole-row path (jax.lax.top_k(k = V): descending,
+  the lower index first among equal values): the sorted keys and ids it leaves in the workspace
+  against numpy's stable sort, bit for bit -- rows full of ties, negative values, zeros of both
+  signs, forbidden ids (-inf, sorted last), fewer elements than the sort has threads."""
+  from tunix_amd import ops
+  rng = np.random.default_rng(7 + V)
+  lg = rng.standard_normal((M, V)).astype(np.float32) * 4
+  lg[0] = np.round(lg[0])                               # a row of heavy ties
+  lg[1, ::3] = 0.0
+  lg[1, 1::7] = -0.0
+  lg[2, : V // 2] = lg[2, V // 2: 2 * (V // 2)]         # every value twice
+  temp = 0.7
+  forbidden = torch.tensor([1, V - 1, 17 % V], dtype=torch.int32, device=gpu)
+  ids = torch.empty(M, dtype=torch.int32, device=gpu)
+  lp = torch.empty(M, dtype=torch.float32, device=gpu)
+  stp = torch.tensor([3], dtype=torch.int32, device=gpu)
+  nb = ops.sample_fullsort_ws_bytes(M, V)
+  ws = torch.zeros(nb // 4, dtype=torch.float32, device=gpu)
+  ops.sample_topk(torch.from_numpy(lg).to(gpu), 0, 0.9, temp, (1, 2), 0, stp, ws, ids, lp, forbidden=forbidden)
+  torch.cuda.synchronize()
+  up = (M * V * 4 + 255) // 256 * 256 // 4
+  keys = ws[: M * V].view(M, V).cpu().numpy()
+  sids = ws[2 * up: 2 * up + M * V].view(torch.int32).view(M, V).cpu().numpy()
+  y = (torch.from_numpy(lg) / np.float32(temp)).numpy()
+  y[:, [1, V - 1, 17 % V]] = -np.inf
+  # descending with the lower index first among equals; -0.0 sorts below +0.0 (bit patterns)
+  for m in range(M):
+    order = np.lexsort((np.arange(V), np.signbit(y[m]) & (y[m] == 0), -y[m].astype(np.float64)))
+    assert np.array_equal(sids[m], order.astype(np.int32)), m
+    assert np.array_equal(keys[m].view(np.uint32), y[m][order].view(np.uint32)), m
+  assert 0 <= int(ids.min()) and int(ids.max()) < V
+
+
 def test_sample_commit_and_fill(gpu):
   from tunix_amd import ops
   B, Ld = 5, 12

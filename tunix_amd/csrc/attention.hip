@@ -25,6 +25,8 @@ namespace {
 struct AttnArgs {
   int64_t B, T, S;
   int Hq, Hkv, dh, G, Gp;
+  int gp_shift;                // Gp = 1 << gp_shift (the query group padded to a power of two)
+  unsigned QT;                 // query tiles per row: ceil(T / (16 / Gp))
   float scale_bf;  // bf16-rounded scale, 0 = none
   int window;
   int32_t pad_id;
@@ -60,14 +62,16 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
   constexpr int NS = DH > 128 ? 1 : TNX_ATTN_NS;        // register stages of the key-block pipeline
   const int lane = threadIdx.x, lm = lane & 15, lq = lane >> 4;
   const int chunk = blockIdx.x, hkv = blockIdx.y;
-  const int PT = 16 / a.Gp;                              // positions per query tile
-  const int QT = (int)((a.T + PT - 1) / PT);
-  const int64_t b = blockIdx.z / QT;
-  const int qt = blockIdx.z % QT;
+  // (shifts and one unsigned division: a general integer division costs some forty instructions,
+  // and the chain in front of this kernel's first loads had several of them)
+  const int PT = 16 >> a.gp_shift;                       // positions per query tile
+  const unsigned bz = blockIdx.z;
+  const int64_t b = FUSE != 0 ? bz : bz / a.QT;          // (the fused decode step has one query tile per row)
+  const int qt = FUSE != 0 ? 0 : (int)(bz - (unsigned)b * a.QT);
   const int col0 = *a.col_ptr;
 
   // query column of this lane (as B-fragment column and as softmax owner)
-  const int g = lm % a.Gp, tq = qt * PT + lm / a.Gp;
+  const int g = lm & (a.Gp - 1), tq = qt * PT + (lm >> a.gp_shift);
   const bool qvalid = g < a.G && tq < a.T;
   const int c_n = col0 + tq;                              // cache slot of the query token
   const int lo_n = a.window > 0 ? max(0, c_n - a.window + 1) : 0;
@@ -106,11 +110,16 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
   const uint16_t* vbase = a.v + ((b * a.Hkv + hkv) * a.S) * DH;
   const int32_t* tok = a.tokens + b * a.tok_ld;
   // what a key's id is compared with: the pad id (the key counts when it differs), or, for packed
-  // batches, the segment id of this lane's query token (the key counts when it is equal)
-  // (loaded in both modes: a branch around a load would make the counted waits behind it inexact)
-  const int32_t id_q = tok[min((int64_t)c_n, a.tok_ld - 1)];
-  const int32_t id_ref = a.seg_mode ? id_q : a.pad_id;
+  // batches, the segment id of this lane's query token (the key counts when it is equal).  The
+  // query's id is fetched behind the first key blocks and planes (a load in front of them would
+  // hold them back until the step counter it depends on has arrived), in both modes: a branch
+  // around a load would make the counted waits behind it inexact.
+  int32_t id_ref = a.pad_id;
   const bool id_equal = a.seg_mode != 0;
+  auto fetch_query_id = [&]() {
+    const int32_t id_q = tok[min((int64_t)c_n, a.tok_ld - 1)];
+    id_ref = a.seg_mode ? id_q : a.pad_id;
+  };
   const int vcol = (8 * lm) % (DH < 128 ? DH : 128);     // DH=64: upper lanes duplicate
   // TOKVEC: 16-byte token loads; the host chooses them when rows are 16-byte aligned and hold
   // whole groups of four slots (keys beyond the range are masked by the range test anyway).  A
@@ -252,7 +261,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
     // partial planes of this step's q / k / v go first: a wave's loads return in order, so
     // planes requested behind 32 KiB of keys and values would only be usable once those have
     // arrived, and the rotation would start late instead of running while the blocks stream in.
-    if constexpr (!fused) issue_ring();
+    if constexpr (!fused) {
+      issue_ring();
+      fetch_query_id();
+    }
     // the step's own key / value wait in LDS while the cached keys stream through the registers
     __shared__ u32x4 park[FUSE ? KS + NH : 1][64];
     if constexpr (fused) {
@@ -328,6 +340,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
           load_planes(0, p);
           __builtin_amdgcn_sched_barrier(0);
           issue_stage(0);
+          fetch_query_id();
           __builtin_amdgcn_sched_barrier(0);
           sum_planes(0, p);
           take_sincos();
@@ -337,6 +350,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
           __builtin_amdgcn_sched_barrier(0);
         } else {
           issue_ring();
+          fetch_query_id();
           take_sincos();
           for (int i4 = lane; i4 < n4; i4 += 64) {
               const int hsel = i4 / (DH / 4), d = (i4 % (DH / 4)) * 4;
@@ -477,7 +491,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
     for (int i = 0; i < 4; ++i) {
       const int n = 4 * lq + i;
       const float l = __shfl(l_run, n, 64);
-      const int gi = n % a.Gp, ti = qt * PT + n / a.Gp;
+      const int gi = n & (a.Gp - 1), ti = qt * PT + (n >> a.gp_shift);
       if (!(gi < a.G && ti < a.T) || !dvalid) continue;
       const float inv = l > 0.f ? 1.0f / l : 0.f;
       uint16_t* o = a.out + ((b * a.T + ti) * a.Hq + hkv * a.G + gi) * DH;
@@ -498,7 +512,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
     const int n = 4 * lq + i;
     const float l = __shfl(l_run, n, 64);
     const float m = __shfl(m_run, n, 64);
-    const int gi = n % a.Gp, ti = qt * PT + n / a.Gp;
+    const int gi = n & (a.Gp - 1), ti = qt * PT + (n >> a.gp_shift);
     if (!(gi < a.G && ti < a.T)) continue;
     const int64_t qv = (b * a.T + ti) * a.Hq + hkv * a.G + gi;
     float* p = a.ws + (qv * a.n_chunks + chunk) * (DH + 2);
@@ -580,6 +594,9 @@ extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
   AttnArgs a;
   a.B = d->B; a.T = d->T; a.S = d->S; a.Hq = d->Hq; a.Hkv = d->Hkv; a.dh = d->dh;
   a.G = G; a.Gp = next_pow2(G);
+  a.gp_shift = 0;
+  while ((1 << a.gp_shift) < a.Gp) ++a.gp_shift;
+  a.QT = (unsigned)cdiv(d->T, 16 / a.Gp);
   // bf16(scale), as a weak-typed python float multiplied into a bf16 array
   if (d->scale != 0.f) {
     uint32_t u; float f = d->scale; memcpy(&u, &f, 4);

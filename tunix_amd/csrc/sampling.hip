@@ -2,8 +2,6 @@
 // jax.random (fold_in -> random_bits -> uniform -> gumbel -> argmax), one work-group per row.
 #include <mutex>
 
-#include <rocprim/device/device_segmented_radix_sort.hpp>
-
 #include "common.h"
 #include "rng.h"
 
@@ -582,24 +580,102 @@ __global__ __launch_bounds__(NTH) void topk_merge_sample_kernel(
 }
 
 
-// ---- top-p over the whole vocabulary (top_k absent, top_p < 1) ------------------------------
-// sample_top_p then sorts the full row (jax.lax.top_k with k = V): a stable segmented radix sort
-// (rocPRIM) of (scaled logit, id) pairs per row, then one work-group per row that soft-maxes the
-// sorted row, keeps the entries whose exclusive cumulative probability is <= top_p and draws
-// by Gumbel-max with the noise of the SORTED position, as jax.random.categorical over the
-// sorted logits does.
-__global__ void fullsort_prepare_kernel(const float* logits, int64_t M, int64_t V, float temperature,
-                                        const int32_t* forbidden, int n_forbidden, float* keys,
-                                        int* ids, int* offsets) {
-  const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (n <= M) offsets[n] = (int)(n * V);
-  if (n >= M * V) return;
-  const int v = (int)(n % V);
-  float y = __fdiv_rn(logits[n], temperature);
-  for (int f = 0; f < n_forbidden; ++f)
-    if (forbidden[f] == v) y = kNegInf;
-  keys[n] = y;
-  ids[n] = v;
+// ---- top-p over the whole vocabulary (top_k absent with top_p < 1, or top_k == V) -------------
+// sample_top_p then sorts the full row (jax.lax.top_k with k = V: descending, the lower index first
+// among equal values): a stable least-significant-digit radix sort per row, written here (four
+// passes of eight bits over order-preserving keys), then one work-group per row that soft-maxes
+// the sorted row, keeps the entries whose exclusive cumulative probability is <= top_p and draws
+// by Gumbel-max with the noise of the SORTED position, as jax.random.categorical over the sorted
+// logits does.
+//
+// The sort: one work-group of kSortThreads threads per row.  Thread t owns the contiguous chunk
+// [t * per, (t + 1) * per) of the row, so "thread order, then position inside the chunk" is the
+// row's order and a counting sort that hands out positions in that order is stable.  Per pass:
+// every thread counts its chunk's digits into its own column of an LDS table [256 digits][threads]
+// (no atomics), the table is turned into exclusive offsets in (digit, thread) order -- each pair
+// of digit rows summed by one thread, the 256 digit totals scanned, the rows rewritten -- and
+// every thread walks its chunk again and moves each element to offset[digit][t]++.  Keys are the
+// bit patterns of the scaled logits mapped so that unsigned order is descending float order; the
+// first pass reads the logits themselves (dividing by the temperature and masking forbidden ids
+// on the way), the last one writes floats back.  Two (key, id) buffer pairs alternate; after the
+// fourth pass the sorted row is in the first pair.
+constexpr int kSortThreads = 128;
+constexpr int kSortLd = kSortThreads + 1;              // padded row of the table: bank-conflict-free scans
+constexpr size_t kSortLdsBytes = 256 * (size_t)kSortLd * sizeof(uint32_t);
+
+__device__ __forceinline__ uint32_t desc_key(float f) { return ~order_key(f); }   // ascending unsigned = descending float
+__device__ __forceinline__ float desc_key_inv(uint32_t k) {
+  const uint32_t o = ~k;
+  return __uint_as_float((o & 0x80000000u) ? (o & 0x7fffffffu) : ~o);
+}
+
+__global__ __launch_bounds__(kSortThreads) void fullsort_kernel(const float* logits, int64_t V, float temperature,
+                                                                const int32_t* forbidden, int n_forbidden,
+                                                                uint32_t* k0, int* i0, uint32_t* k1, int* i1) {
+  extern __shared__ uint32_t cnt[];                    // [256][kSortLd]
+  __shared__ uint32_t digit_base[256];
+  const int tid = threadIdx.x;
+  const int64_t row = blockIdx.x;
+  const int64_t per = (V + kSortThreads - 1) / kSortThreads;
+  const int64_t j0 = min(V, tid * per), j1 = min(V, j0 + per);
+  const float* lrow = logits + row * V;
+  uint32_t* ka = k0 + row * V;
+  int* ia = i0 + row * V;
+  uint32_t* kb = k1 + row * V;
+  int* ib = i1 + row * V;
+  // key of element j in pass 0: the scaled, masked logit (what tnx_sample_topk's other paths draw from)
+  auto first_key = [&](int64_t j) -> uint32_t {
+    float y = __fdiv_rn(lrow[j], temperature);
+    for (int f = 0; f < n_forbidden; ++f)
+      if (forbidden[f] == (int)j) y = kNegInf;
+    return desc_key(y);
+  };
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 8 * pass;
+    const uint32_t* src_k = (pass & 1) ? kb : ka;      // passes 1, 3 read the second pair
+    const int* src_i = (pass & 1) ? ib : ia;
+    uint32_t* dst_k = (pass & 1) ? ka : kb;
+    int* dst_i = (pass & 1) ? ia : ib;
+    for (int d = 0; d < 256; ++d) cnt[d * kSortLd + tid] = 0;
+    // (a thread touches only its own column until the barrier)
+    for (int64_t j = j0; j < j1; ++j) {
+      const uint32_t key = pass == 0 ? first_key(j) : src_k[j];
+      ++cnt[((key >> shift) & 255u) * kSortLd + tid];
+    }
+    __syncthreads();
+    // exclusive offsets in (digit, thread) order: the two digit rows of this thread summed, ...
+    uint32_t tot[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int d = 2 * tid + h;
+      uint32_t run = 0;
+      for (int t = 0; t < kSortThreads; ++t) {
+        const uint32_t c = cnt[d * kSortLd + t];
+        cnt[d * kSortLd + t] = run;
+        run += c;
+      }
+      tot[h] = run;
+      digit_base[d] = run;
+    }
+    __syncthreads();
+    // ... the digit totals scanned (256 values: every thread walks the ones below its own two), ...
+    uint32_t base = 0;
+    for (int d = 0; d < 2 * tid; ++d) base += digit_base[d];
+    __syncthreads();
+    digit_base[2 * tid] = base;
+    digit_base[2 * tid + 1] = base + tot[0];
+    __syncthreads();
+    // ... and every element moved to its digit's base + its (thread, position) rank
+    for (int64_t j = j0; j < j1; ++j) {
+      const uint32_t key = pass == 0 ? first_key(j) : src_k[j];
+      const int id = pass == 0 ? (int)j : src_i[j];
+      const uint32_t d = (key >> shift) & 255u;
+      const uint32_t pos = digit_base[d] + cnt[d * kSortLd + tid]++;
+      dst_k[pos] = pass == 3 ? __float_as_uint(desc_key_inv(key)) : key;
+      dst_i[pos] = id;
+    }
+    __syncthreads();   // the pass's writes are visible to the work-group's next pass; the table is free
+  }
 }
 
 __global__ __launch_bounds__(NTH) void fullsort_sample_kernel(const float* skeys, const int* sids, int64_t V,
@@ -647,33 +723,25 @@ __global__ __launch_bounds__(NTH) void fullsort_sample_kernel(const float* skeys
 }
 
 struct FullSortWs {
-  size_t keys_in, keys_out, ids_in, ids_out, offsets, temp, temp_bytes, total;
+  size_t keys_a, keys_b, ids_a, ids_b, total;
 };
-int fullsort_layout(int64_t M, int64_t V, FullSortWs* w) {
+void fullsort_layout(int64_t M, int64_t V, FullSortWs* w) {
   const size_t n = (size_t)(M * V);
   auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
-  size_t temp_bytes = 0;
-  const hipError_t e = rocprim::segmented_radix_sort_pairs_desc(
-      nullptr, temp_bytes, (const float*)nullptr, (float*)nullptr, (const int*)nullptr, (int*)nullptr,
-      (unsigned)n, (unsigned)M, (const int*)nullptr, (const int*)nullptr, 0, 32, (hipStream_t)0);
-  if (e != hipSuccess) return -1;
   size_t o = 0;
-  w->keys_in = o; o += up(n * 4);
-  w->keys_out = o; o += up(n * 4);
-  w->ids_in = o; o += up(n * 4);
-  w->ids_out = o; o += up(n * 4);
-  w->offsets = o; o += up((size_t)(M + 1) * 4);
-  w->temp = o; o += up(temp_bytes);
-  w->temp_bytes = temp_bytes;
+  w->keys_a = o; o += up(n * 4);
+  w->keys_b = o; o += up(n * 4);
+  w->ids_a = o; o += up(n * 4);
+  w->ids_b = o; o += up(n * 4);
   w->total = o;
-  return 0;
 }
 
 }  // namespace
 
 extern "C" size_t tnx_sample_fullsort_ws_bytes(int64_t M, int64_t V) {
   FullSortWs w;
-  if (M <= 0 || V <= 0 || M * V >= (1ll << 31) || fullsort_layout(M, V, &w) != 0) return 0;
+  if (M <= 0 || V <= 0 || M * V >= (1ll << 31)) return 0;
+  fullsort_layout(M, V, &w);
   return w.total;
 }
 
@@ -703,23 +771,25 @@ extern "C" int tnx_sample_topk(void* stream, const float* logits, int64_t M, int
                       "workspace of tnx_sample_fullsort_ws_bytes(M, V) bytes");
       TNX_REQUIRE(M * V < (1ll << 31), "sample_topk: M * V too large for the full-row sort");
       FullSortWs w;
-      TNX_REQUIRE(fullsort_layout(M, V, &w) == 0, "sample_topk: rocPRIM refused the sort configuration");
+      fullsort_layout(M, V, &w);
       unsigned char* base = reinterpret_cast<unsigned char*>(ws);
-      float* kin = reinterpret_cast<float*>(base + w.keys_in);
-      float* kout = reinterpret_cast<float*>(base + w.keys_out);
-      int* iin = reinterpret_cast<int*>(base + w.ids_in);
-      int* iout = reinterpret_cast<int*>(base + w.ids_out);
-      int* off = reinterpret_cast<int*>(base + w.offsets);
-      const int64_t n = M * V;
-      hipLaunchKernelGGL(fullsort_prepare_kernel, dim3((unsigned)cdiv(n + 1, 256)), dim3(256), 0, as_stream(stream),
-                         logits, M, V, temperature, forbidden, forbidden ? n_forbidden : 0, kin, iin, off);
-      TNX_CHECK_LAUNCH("sample_topk (sort keys)");
-      size_t tb = w.temp_bytes;
-      const hipError_t e = rocprim::segmented_radix_sort_pairs_desc(
-          base + w.temp, tb, (const float*)kin, kout, (const int*)iin, iout, (unsigned)n, (unsigned)M,
-          (const int*)off, (const int*)(off + 1), 0, 32, as_stream(stream));
-      TNX_REQUIRE(e == hipSuccess, "sample_topk: segmented sort failed: %s", hipGetErrorString(e));
-      hipLaunchKernelGGL(fullsort_sample_kernel, dim3((unsigned)M), dim3(NTH), 0, as_stream(stream), kout, iout, V,
+      uint32_t* ka = reinterpret_cast<uint32_t*>(base + w.keys_a);
+      uint32_t* kb = reinterpret_cast<uint32_t*>(base + w.keys_b);
+      int* ia = reinterpret_cast<int*>(base + w.ids_a);
+      int* ib = reinterpret_cast<int*>(base + w.ids_b);
+      static std::once_flag sort_once;
+      static hipError_t sort_rc = hipSuccess;
+      std::call_once(sort_once, [] {
+        sort_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(fullsort_kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSortLdsBytes);
+      });
+      TNX_REQUIRE(sort_rc == hipSuccess, "sample_topk: cannot raise the dynamic LDS limit of the sort");
+      hipLaunchKernelGGL(fullsort_kernel, dim3((unsigned)M), dim3(kSortThreads), kSortLdsBytes, as_stream(stream), logits,
+                         V, temperature, forbidden, forbidden ? n_forbidden : 0, ka, ia, kb, ib);
+      TNX_CHECK_LAUNCH("sample_topk (sort)");
+      // (four passes: the sorted floats and their ids are back in the first pair)
+      hipLaunchKernelGGL(fullsort_sample_kernel, dim3((unsigned)M), dim3(NTH), 0, as_stream(stream),
+                         reinterpret_cast<const float*>(ka), ia, V,
                          top_p, key0, key1, rng_variant, step_ptr, M, ids_out, logp_out);
       TNX_CHECK_LAUNCH("sample_topk (sorted draw)");
       return TNX_OK;
