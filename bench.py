@@ -15,7 +15,9 @@ Extra objects on the line:
   roofline      the kernel with the largest share of a step (the quantised GEMM), timed in
                 isolation with events on its launch stream; roofline_hbm prices the same
                 launches against the HBM roof
-  kernels       the same measurement for every kernel family of the step
+  kernels_isolated  the same measurement for every kernel family of the step, each alone in its own
+                replayed graph (the linears with their LoRA down-projection and a finishing pass):
+                not a breakdown of ms_per_step -- the step's kernel trace is under profiles/
   fused_logps   the standalone per-token log-probability workload at training scale
   cpu_baseline  the CPU oracle (a port of the reference's JAX path) timed on this host on a
                 bounded sample and scaled linearly
@@ -763,9 +765,12 @@ def main():
       "hbm_roofline_frac_step": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
       "step_bytes": int(step_bytes), "prefill_s": round(prefill_s, 3),
       "roofline": roofline, "roofline_hbm": roofline_linears, "roofline_many_rows": many,
-      "kernels": {k: {"us": round(v["ms"] * 1e3, 2), "GBps": round(v["gbs"], 1),
-                      "TFLOPs": round(v["tflops"], 1), "ms_per_step": round(v["step_ms"], 4)}
-                  for k, v in kern.items()},
+      # each family alone in its own replayed graph at the mean context -- the linears with their
+      # LoRA down-projection and a finishing pass that the decode chain folds into its consumers --
+      # so these do NOT add up to ms_per_step; the step's own kernel trace is in profiles/
+      "kernels_isolated": {k: {"us": round(v["ms"] * 1e3, 2), "launches_per_step": v["per_step"],
+                               "GBps": round(v["gbs"], 1), "TFLOPs": round(v["tflops"], 1)}
+                           for k, v in kern.items()},
   }
   if first_steps is not None:
     result["first_steps"] = first_steps
