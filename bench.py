@@ -187,12 +187,7 @@ KERNEL_SOURCES = ("csrc/qgemm128.h", "csrc/gemm_tile.h", "csrc/common.h", "csrc/
 
 
 def kernel_source_hash():
-  import hashlib
-  h = hashlib.sha256()
-  for name in KERNEL_SOURCES:
-    with open(os.path.join(ROOT, "tunix_amd", name), "rb") as f:
-      h.update(f.read())
-  return h.hexdigest()[:16]
+  return source_hash(KERNEL_SOURCES)
 
 
 def measured_traffic():
@@ -264,6 +259,71 @@ def write_traffic_profile(fetch_csv, write_csv):
       "write_bytes_per_launch": int(sum(w_shapes) / 4 * 1024),
   }
   with open(TRAFFIC_PROFILE, "w") as f:
+    json.dump(rec, f, indent=1)
+    f.write("\n")
+  print(json.dumps(rec, indent=1))
+
+
+# The same for the many-row kernel on the standalone log-probability pass (one launch = 16384 rows
+# x 128256 columns): counter runs of `bench.py --fused-logps`.
+FUSED_TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "qgemm_wide_kernel_fused_logps_131072rows.json")
+FUSED_KERNEL_SOURCES = ("csrc/qgemm_wide.h", "csrc/gemm_tile.h", "csrc/common.h", "csrc/qlinear.hip",
+                        "csrc/lmhead.hip")
+
+
+def source_hash(names):
+  import hashlib
+  h = hashlib.sha256()
+  for name in names:
+    with open(os.path.join(ROOT, "tunix_amd", name), "rb") as f:
+      h.update(f.read())
+  return h.hexdigest()[:16]
+
+
+def fused_measured_traffic():
+  try:
+    with open(FUSED_TRAFFIC_PROFILE) as f:
+      prof = json.load(f)
+  except (OSError, ValueError):
+    return None
+  if prof.get("kernel_source_sha256_16") != source_hash(FUSED_KERNEL_SOURCES):
+    return None
+  return int(prof["read_bytes_per_launch"] + prof["write_bytes_per_launch"])
+
+
+def write_fused_traffic_profile(fetch_csv, write_csv):
+  """Rebuilds the tracked traffic record of the log-probability pass from two `rocprofv3 --pmc`
+  runs of `bench.py --fused-logps` (FETCH_SIZE in one, WRITE_SIZE in the other; KiB per dispatch of
+  qgemm_wide_kernel).  FETCH_SIZE is scaled with the factor the decode GEMM's record holds for
+  buffer loads (its 1 GiB yardstick reads)."""
+  import csv
+
+  def mean(path, counter):
+    v = [float(r["Counter_Value"]) for r in csv.DictReader(open(path))
+         if r["Counter_Name"] == counter and "qgemm_wide_kernel" in r["Kernel_Name"]]
+    if not v:
+      raise SystemExit(f"no qgemm_wide_kernel dispatches with {counter} in {path}")
+    return sum(v) / len(v), len(v)
+
+  with open(TRAFFIC_PROFILE) as f:
+    factor = float(json.load(f)["fetch_counter_factor"])
+  fk, nf = mean(fetch_csv, "FETCH_SIZE")
+  wk, nw = mean(write_csv, "WRITE_SIZE")
+  rows, D, V, r = 16384, 4096, 128256, 64
+  rec = {
+      "kernel": "qgemm_wide_kernel<4> (head-statistics epilogue)",
+      "workload": "one launch of the standalone log-probability pass: 16384 rows x 4096 -> 128256, int4 g128 + LoRA r64",
+      "kernel_source_sha256_16": source_hash(FUSED_KERNEL_SOURCES),
+      "kernel_sources": list(FUSED_KERNEL_SOURCES),
+      "fetch_counter_factor": factor, "write_counter_factor": 1.0,
+      "dispatches": {"fetch_run": nf, "write_run": nw},
+      "counter_kib_per_launch": {"FETCH_SIZE": round(fk, 1), "WRITE_SIZE": round(wk, 1)},
+      "read_bytes_per_launch": int(fk * 1024 * factor), "write_bytes_per_launch": int(wk * 1024),
+      # what one launch must move: hidden rows + packed head + adapter once, statistics out
+      "algorithmic_bytes_per_launch": int(rows * D * 2 + D * V // 2 + (D // 128) * V * 2 + V * r * 2 + rows * r * 2
+                                          + rows * (V // 128) * 16),
+  }
+  with open(FUSED_TRAFFIC_PROFILE, "w") as f:
     json.dump(rec, f, indent=1)
     f.write("\n")
   print(json.dumps(rec, indent=1))
@@ -452,7 +512,9 @@ def fused_logps_workload(rows, chunk, iters):
                  "rows_per_launch": chunk},
       "roofline": {"kernel": "qgemm_wide_kernel (statistics epilogue)", "bound": "mfma",
                    "achieved": round(flops / (ms * 1e-3) / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                   "frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}}
+                   "frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                   # HBM bytes of one 16384-row launch, from the tracked counter record
+                   "traffic": fused_measured_traffic() if chunk == 16384 else None}}
 
 
 def config_workload(name, steps):
@@ -543,6 +605,9 @@ def main():
                        "rollout's context range")
   ap.add_argument("--summarize-trace", metavar="CSV", default=None,
                   help="no GPU work: tabulate one decode step of a rocprofv3 kernel-trace csv of this script")
+  ap.add_argument("--write-fused-traffic-profile", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"), default=None,
+                  help="rebuild profiles/qgemm_wide_kernel_fused_logps_131072rows.json from the counter csv files "
+                       "of two `rocprofv3 --pmc FETCH_SIZE | WRITE_SIZE -- python3 bench.py --fused-logps` runs")
   ap.add_argument("--write-traffic-profile", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"), default=None,
                   help="no GPU work: rebuild profiles/qgemm128_kernel_llama8b_decode_b128.json from the counter csvs "
                        "of two `rocprofv3 --pmc FETCH_SIZE | WRITE_SIZE -- python3 bench.py --kernels-only` runs")
@@ -559,6 +624,9 @@ def main():
     return
   if args.summarize_counters:
     summarize_counters(args.summarize_counters)
+    return
+  if args.write_fused_traffic_profile:
+    write_fused_traffic_profile(*args.write_fused_traffic_profile)
     return
   if args.write_traffic_profile:
     write_traffic_profile(*args.write_traffic_profile)

@@ -281,7 +281,7 @@ __global__ __launch_bounds__(512) void lora_down_lds_kernel(const uint16_t* x, i
   const int arows = min(tn, R - n0);
   const u32x4 rx = raw_rsrc(x + m0 * K, (uint64_t)xrows * K * 2);
   const u32x4 ra = raw_rsrc(a_t + (int64_t)n0 * K, (uint64_t)arows * K * 2);
-  const int per_row = (int)(row_bytes / 1024u), n_x = tm * per_row, n_all = (tm + tn) * per_row;
+  const int per_row = (int)(row_bytes / 1024u);
   // operand rows of this lane: tile rows the output does not have are clamped (their products
   // are never stored)
   const unsigned char* ra_lds = smem + (uint32_t)min(lm, tm - 1) * row_bytes;
@@ -291,17 +291,22 @@ __global__ __launch_bounds__(512) void lora_down_lds_kernel(const uint16_t* x, i
   f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int64_t k0 = 0; k0 < K; k0 += kc) {
     if (k0 > 0) __syncthreads();   // every wave is done with the piece before
-    for (int q = wave; q < n_all; q += 8) {
-      const bool is_x = q < n_x;
-      const int qq = is_x ? q : q - n_x;
-      const int row = qq / per_row, blk = qq % per_row;
-      const int lrow = is_x ? row : tm + row;                     // row of the LDS tile
+    // this wave's kilobytes: q = wave, wave + 8, ... of the (row, kilobyte) pairs, walked without a
+    // division (per_row is a run-time value: an integer division per request, some forty scalar
+    // instructions, stretched the issue of the 20 requests over longer than they take to arrive)
+    int lrow = 0, blk = wave;                                   // row of the LDS tile, kilobyte of the row
+    while (blk >= per_row) { blk -= per_row; ++lrow; }
+    while (lrow < tm + tn) {
+      const bool is_x = lrow < tm;
+      const int row = is_x ? lrow : lrow - tm;
       // lane j fills chunk 64 blk + j and fetches for it chunk 64 blk + (j ^ (row % 16))
       const uint32_t voff = ((uint32_t)row * (uint32_t)K + (uint32_t)k0) * 2u + (uint32_t)blk * 1024u +
                             (uint32_t)(lane ^ (lrow & 15)) * 16u;
       // chunks past the row's K elements: beyond the resource for the last row, otherwise the next
       // row's first bytes; no fragment read touches them
       dma16(lds0 + (uint32_t)lrow * row_bytes + (uint32_t)blk * 1024u, is_x ? rx : ra, voff, 0);
+      blk += 8;
+      while (blk >= per_row) { blk -= per_row; ++lrow; }
     }
     tnx_wait_vm(0);
     __syncthreads();
@@ -346,9 +351,19 @@ __global__ __launch_bounds__(256) void lora_reduce_kernel(const float* tpart, in
   const int64_t mb = blockIdx.y;
   if (n * 16 >= R) return;                     // same for the whole work-group
   const float* p = tpart + mb * ncb * 8192 + (int64_t)q * 4;
+  // A thread's planes (every 32nd) are requested eight at a time before the first is added: one
+  // memory round trip per eight instead of one per plane (a loop of load-then-add waits for each
+  // plane in turn, and the planes come from memory).  Planes past the last are clamped loads
+  // whose values are not added; the order of the additions is the planes' order.
   f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-  for (int64_t cb = sl; cb < ncb; cb += 32) s += *reinterpret_cast<const f32x4*>(p + cb * 8192);
+  for (int64_t cb0 = sl; cb0 < ncb; cb0 += 256) {
+    f32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const f32x4*>(p + min(cb0 + 32 * u, ncb - 1) * 8192);
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (cb0 + 32 * u < ncb) s += v[u];
+  }
   red[sl][g] = s;
   __syncthreads();
   if (sl != 0) return;
