@@ -154,6 +154,30 @@ def test_product_does_not_import_the_oracle():
         assert not re.search(r"^\s*(from|import)\s+oracle\b", text, re.M), os.path.join(dirpath, f)
 
 
+def test_ffi_handlers_cover_the_documented_targets_and_call_declared_entry_points():
+  """csrc/tunix_ffi.cc (the jax.ffi handlers, built only where jaxlib's headers exist) defines the
+  twelve targets INTEGRATION.md lists and calls nothing the header does not declare."""
+  src = open(os.path.join(ROOT, "tunix_amd", "csrc", "tunix_ffi.cc")).read()
+  targets = set(re.findall(r"XLA_FFI_DEFINE_HANDLER_SYMBOL\((tnx_\w+_ffi)", src))
+  doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+  documented = set(re.findall(r"`(tnx_\w+_ffi)`", doc))
+  assert targets == documented and len(targets) == 12, (targets ^ documented)
+  called = set(re.findall(r"\b(tnx_[a-z0-9_]+)\s*\(", src)) - {t for t in targets}
+  assert called <= set(_declared()), called - set(_declared())
+
+
+def test_binding_refuses_another_abi_version(monkeypatch):
+  """A library of another major version (or an older minor one) must not be called."""
+  monkeypatch.setattr(L, "_lib", None)
+  monkeypatch.setattr(L, "ABI_VERSION", (L.ABI_VERSION[0] + 1, 0))
+  with pytest.raises(ImportError, match="ABI version"):
+    L.lib()
+  monkeypatch.setattr(L, "_lib", None)
+  monkeypatch.setattr(L, "ABI_VERSION", (L.ABI_VERSION[0] - 1, L.ABI_VERSION[1] + 1))   # back to the real major, a newer minor
+  with pytest.raises(ImportError, match="ABI version"):
+    L.lib()
+
+
 def test_missing_library_fails_loudly(monkeypatch):
   monkeypatch.setattr(L, "_lib", None)
   monkeypatch.setattr(L, "LIB_PATH", "/nonexistent/libtunix_hip.so")

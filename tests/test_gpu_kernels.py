@@ -201,6 +201,11 @@ def test_qlinear_lora_matches_oracle(gpu, M, K, N, group, qtype, r, split):
     (520, 128, 13440, 32, Q.NF4, 0, None, "residual"),           # ragged last column tile, group 32, one k-tile
     (1024, 512, 8448, 64, Q.INT4, 32, None, "silu"),             # gate|up pair with its two adapters
     (515, 640, 16896, 64, Q.NF4, 0, None, "gelu"),
+    # integer codes are converted without the table: group 32 (four scales per k-tile) over one
+    # and over five k-tiles, ragged rows with an adapter
+    (520, 128, 13440, 32, Q.INT4, 0, None, "residual"),
+    (515, 640, 16896, 32, Q.INT4, 0, None, "gelu"),
+    (1100, 256, 7424, 64, Q.INT4, 64, None, "store"),
 ])
 def test_qlinear_many_rows_matches_oracle(gpu, M, K, N, group, qtype, r, seg_widths, epi):
   """Row counts that go to the 128 x 256-tile kernel (prefill, per-token logps): every epilogue,
@@ -272,8 +277,10 @@ def test_qlinear_many_rows_matches_oracle(gpu, M, K, N, group, qtype, r, seg_wid
   ops.qlinear(ops.make_qlinear_desc(M=M, K=K, N=N, group=group, qtype=qtype, x=gx, codes=c, scales=s, y=y,
                                     epilogue=e, **kw))
   torch.cuda.synchronize()
+  # act(gate) * up: gate and up may each be one ulp off; linear + residual: a linear output one ulp
+  # off can move the rounded sum by one more step of the sum's own (finer) spacing
   assert_bf16_close(y, ref, atol=1e-5 if mul else 1e-6, min_equal=0.9 if mul else 0.97, what=f"wide {epi}", mag=mag,
-                    ulps=3 if mul else 1)   # act(gate) * up: gate and up may each be one ulp off
+                    ulps=3 if mul else 2 if epi == "residual" else 1)
 
 
 @pytest.mark.parametrize("M,K,R", [(12300, 256, 192), (6200, 384, 128), (700, 128, 32)])

@@ -47,7 +47,17 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
 // (expert, row block) is found from the expert offsets by a running sum; activation rows are
 // gathered through sorted_route (row = route / x_div), output rows are routes.  No adapter, no
 // lm_head statistics in this mode.
-template <int SPT, bool GROUPED = false>
+//
+// INT4: the integer code book needs no table.  A code byte is (k even | k odd << 4) and a dword
+// holds the lane's four pairs of one slab; masked into the mantissa of an f16 whose exponent makes
+// one mantissa step worth exactly one level -- 0x6400 (1024, step 1) for a nibble at bit 0, 0x5400
+// (64, step 1/16) for a nibble at bit 4 -- the nibbles of bytes 0 and 2 become an f16 pair
+// (1024 + n | 1024 + n) or (64 + n | 64 + n) with one v_and_or_b32, those of bytes 1 and 3 after
+// one shift by 8, and one packed f16 add of -1032 or -72 leaves the exact levels n - 8.  Entry j
+// of a slab is then: 0 = even k of bytes 0 | 2, 1 = odd k of bytes 0 | 2, 2 / 3 = the same of
+// bytes 1 | 3; the pair of byte b is half b / 2 of entries 2 (b % 2) and 2 (b % 2) + 1.  That is
+// one VALU instruction more per MFMA than the table path and one LDS instruction fewer.
+template <int SPT, bool GROUPED = false, bool INT4 = false>
 __global__ __launch_bounds__(256)
 void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   constexpr int RT = 4, CG = 2, PF = 3, AP = 8;   // 32-row tiles, 32-column groups per wave
@@ -100,10 +110,10 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
     mtile = __builtin_amdgcn_readfirstlane(found_rb);
     m_end = a.offsets[expert + 1];
   } else {
-    const int per_group = 8 * tiles_n;
+    const int per_group = 32 * tiles_n;
     const int g = (int)blockIdx.x / per_group, r = (int)blockIdx.x % per_group;
-    const int gm = min(8, tiles_m - g * 8);
-    mtile = g * 8 + r % gm;
+    const int gm = min(32, tiles_m - g * 32);
+    mtile = g * 32 + r % gm;
     ntile = r / gm;
   }
   // first row of the tile (GROUPED: first position in the sorted route list)
@@ -170,7 +180,10 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   float sc[PF][CG][SPT];
   u32x4 xf[2][RT];           // activation fragments of the current / next slab
   u32x4 wf[2][CG];           // weight fragments of the current / next slab
-  uint32_t lp[CG][4];        // table entries (f16 level pairs) of the slab after the next
+  // f16 level pairs of the slab after the next (table path: entry b = the pair of byte b, looked
+  // up into the place of the entry just consumed; INT4: entries as described above, the slab's
+  // parity picks the set, since a set is read until its slab has been converted)
+  uint32_t lp[INT4 ? 2 : 1][CG][4];
   float cf0 = 0.f, cf1 = 0.f;  // products of the pair whose pack is still to come
 
   // LoRA: the k-tile after the last one is the 128-row block of t = bf16(x . A), columns
@@ -269,6 +282,33 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   // Fragment addresses: slab u wants k-chunk 2 u + l / 32 of row l % 32 (+ 32 per row tile, an
   // immediate).  xaddr[u] points into the tile slab u is read from next and flips to the other
   // tile after each use; slab 0 is read one tile ahead (by slab 7 of the tile before).
+  // (masks in scalar registers, the exponents in vector registers: one v_and_or_b32 each, which
+  // takes no literal and only one scalar operand)
+  uint32_t mask_lo = 0x000f000fu, mask_hi = 0x00f000f0u, magic_lo = 0x64006400u, magic_hi = 0x54005400u;
+  if constexpr (INT4) asm volatile("" : "+s"(mask_lo), "+s"(mask_hi), "+v"(magic_lo), "+v"(magic_hi));
+  // entry j of the dword w of one slab (see INT4 above) / the table's entry for byte j of w
+  auto level_entry = [&](uint32_t w, int j) -> uint32_t {
+    if constexpr (INT4) {
+      const uint32_t src = j < 2 ? w : w >> 8;
+      const uint32_t m = (j & 1) ? ((src & mask_hi) | magic_hi) : ((src & mask_lo) | magic_lo);
+      const h16x2 bias = (j & 1) ? h16x2{(_Float16)-72.0f, (_Float16)-72.0f} : h16x2{(_Float16)-1032.0f, (_Float16)-1032.0f};
+      return __builtin_bit_cast(uint32_t, __builtin_bit_cast(h16x2, m) + bias);
+    } else {
+      return lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020400u + ((uint32_t)j << 8)));
+    }
+  };
+  // the two levels of byte b of a slab's dword times the scale sv, from that slab's entries
+  auto pair_products = [&](const uint32_t (&e)[4], int b, float sv, float& p0, float& p1) {
+    if constexpr (INT4) {
+      const h16x2 he = __builtin_bit_cast(h16x2, e[2 * (b & 1)]), ho = __builtin_bit_cast(h16x2, e[2 * (b & 1) + 1]);
+      p0 = __builtin_fmaf((float)he[b >> 1], sv, 0.0f);
+      p1 = __builtin_fmaf((float)ho[b >> 1], sv, 0.0f);
+    } else {
+      const h16x2 hh = __builtin_bit_cast(h16x2, e[b]);
+      p0 = __builtin_fmaf((float)hh[0], sv, 0.0f);
+      p1 = __builtin_fmaf((float)hh[1], sv, 0.0f);
+    }
+  };
   uint32_t xaddr[8];
 #pragma unroll
   for (int u = 0; u < 8; ++u)
@@ -307,12 +347,9 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
         // belongs to the fragment the MFMAs of slots 4-7 of THIS slab multiply
         if (i == 0) wf[CUR][CG - 1][3] = cvt_pk_bf16(cf0, cf1);
         else wf[NXT][(i - 1) >> 2][(i - 1) & 3] = cvt_pk_bf16(cf0, cf1);
-        const h16x2 hh = __builtin_bit_cast(h16x2, lp[cg][rt]);
         const float sv = sc[DC][cg][SPT == 2 ? (UC >> 2) : (UC >> 1)];
-        cf0 = __builtin_fmaf((float)hh[0], sv, 0.0f);
-        cf1 = __builtin_fmaf((float)hh[1], sv, 0.0f);
-        const uint32_t w = ring_c[DL][cg][UL & 1][UL >> 1];
-        lp[cg][rt] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020400u + ((uint32_t)rt << 8)));
+        pair_products(lp[INT4 ? (UC & 1) : 0][cg], rt, sv, cf0, cf1);
+        lp[INT4 ? (UL & 1) : 0][cg][rt] = level_entry(ring_c[DL][cg][UL & 1][UL >> 1], rt);
       }
       if ((i & 1) == 0) xf[NXT][i >> 1] = lds_ld128(xaddr[UC] + (uint32_t)((i >> 1) * 32 * 256));
       if (i == 7) xaddr[UC] ^= kWideTileBytes;
@@ -353,7 +390,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   // back to "everything outstanding" for the sake of the path that enters from here)
   load_a(0, 0u);
   load_w(ic<0>{}, 0);
-  {  // table entry e = f16 pair (level[e & 15], level[e >> 4]), 64 copies rotated over the banks
+  if constexpr (!INT4) {  // table entry e = f16 pair (level[e & 15], level[e >> 4]), 64 copies rotated over the banks
     uint32_t* lut = reinterpret_cast<uint32_t*>(smem + kWideLutBase);
     const h16x2 h = {(_Float16)lvl0, (_Float16)lvl1};
     const uint32_t v = __builtin_bit_cast(uint32_t, h);
@@ -382,25 +419,20 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
 #pragma unroll
   for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
-    for (int b = 0; b < 4; ++b)
-      lp[cg][b] = lds_ld32(__builtin_amdgcn_perm(ring_c[0][cg][0][0], lane_off, 0x0c020400u + ((uint32_t)b << 8)));
+    for (int b = 0; b < 4; ++b) lp[0][cg][b] = level_entry(ring_c[0][cg][0][0], b);
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) xf[0][rt] = lds_ld128((xaddr[0] ^ kWideTileBytes) + (uint32_t)(rt * 32 * 256));
 #pragma unroll
   for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-      const h16x2 hh = __builtin_bit_cast(h16x2, lp[cg][b]);
-      const float sv = sc[0][cg][0];
-      cf0 = __builtin_fmaf((float)hh[0], sv, 0.0f);
-      cf1 = __builtin_fmaf((float)hh[1], sv, 0.0f);
+      pair_products(lp[0][cg], b, sc[0][cg][0], cf0, cf1);
       if (cg < CG - 1 || b < 3) wf[0][cg][b] = cvt_pk_bf16(cf0, cf1);   // the last pair: slot 0 of the loop
     }
 #pragma unroll
   for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
-    for (int b = 0; b < 4; ++b)
-      lp[cg][b] = lds_ld32(__builtin_amdgcn_perm(ring_c[0][cg][1][0], lane_off, 0x0c020400u + ((uint32_t)b << 8)));
+    for (int b = 0; b < 4; ++b) lp[INT4 ? 1 : 0][cg][b] = level_entry(ring_c[0][cg][1][0], b);
   // whole turns of the ring without a branch inside (a conditional tile would make the waits
   // of the tile after it assume that its loads never happened), then the one or two tiles left
   int kt = 0;
@@ -541,8 +573,52 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
         }
       }
     };
-    if (h.temperature == 1.0f) reduce(std::true_type{});
-    else reduce(std::false_type{});
+    // A block that lies wholly inside the vocabulary, no entropy term asked for (every block of a
+    // log-probability pass over a head whose width is a multiple of 128): the same arithmetic in
+    // the same order without the per-element column tests, and the target's logit is read from its
+    // place in the staged row instead of being compared for 128 times.
+    auto reduce_full = [&](auto unit_c) {
+      constexpr bool unit = decltype(unit_c)::value;
+      const int c0i = (int)c0;
+      if (tg >= c0i && tg < c0i + 128) {
+        const uint32_t w = lds_ld32(base + (uint32_t)((tg - c0i) >> 1) * 4u);
+        const float raw = ((tg - c0i) & 1) ? bfhi(w) : bflo(w);
+        tgt = unit ? raw : __fdiv_rn(raw, h.temperature);
+      }
+#pragma unroll 4
+      for (int ch = 0; ch < 16; ++ch) {
+        const u32x4 v = lds_ld128(base + (uint32_t)(ch * 16));
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          const float raw = (q & 1) ? bfhi(v[q >> 1]) : bflo(v[q >> 1]);
+          const float l = unit ? raw : __fdiv_rn(raw, h.temperature);
+          if (l > mx) {
+            mx = l;
+            idx = c0i + ch * 8 + q;
+          }
+        }
+      }
+      if (mx != ninf) {
+#pragma unroll 4
+        for (int ch = 0; ch < 16; ++ch) {
+          const u32x4 v = lds_ld128(base + (uint32_t)(ch * 16));
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            const float raw = (q & 1) ? bfhi(v[q >> 1]) : bflo(v[q >> 1]);
+            const float l = unit ? raw : __fdiv_rn(raw, h.temperature);
+            se += __expf(l - mx);
+          }
+        }
+      }
+    };
+    const bool plain = c0 + 128 <= a.N && h.part_ent == nullptr;
+    if (h.temperature == 1.0f) {
+      if (plain) reduce_full(std::true_type{});
+      else reduce(std::true_type{});
+    } else {
+      if (plain) reduce_full(std::false_type{});
+      else reduce(std::false_type{});
+    }
     float* p = h.part + (grow * h.nvb + pb) * 4;
     p[0] = mx;
     p[1] = __int_as_float(idx);

@@ -587,32 +587,43 @@ int launch_qgemm128(hipStream_t st, const QLArgs& a) {
   return TNX_OK;
 }
 
-template <int SPT>
-int launch_qgemm_wide(hipStream_t st, const QLArgs& a, const WideHead& h = WideHead{nullptr, nullptr, nullptr, 0, 1.0f}) {
+template <int SPT, bool INT4>
+int launch_qgemm_wide_as(hipStream_t st, const QLArgs& a, const WideHead& h) {
   static std::once_flag once;
   static int attr_rc = TNX_OK;
-  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm_wide_kernel<SPT>, kWideSmemBytes); });
+  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm_wide_kernel<SPT, false, INT4>, kWideSmemBytes); });
   if (attr_rc) return attr_rc;
   const unsigned wgs = (unsigned)(cdiv(a.M, kWideRows) * cdiv(a.N, kWideCols));
-  hipLaunchKernelGGL((qgemm_wide_kernel<SPT>), dim3(wgs), dim3(256), kWideSmemBytes, st, a, h);
+  hipLaunchKernelGGL((qgemm_wide_kernel<SPT, false, INT4>), dim3(wgs), dim3(256), kWideSmemBytes, st, a, h);
   TNX_CHECK_LAUNCH("qgemm_wide");
   return TNX_OK;
 }
 
+// integer codes take the instantiation that converts them without the table
+template <int SPT>
+int launch_qgemm_wide(hipStream_t st, const QLArgs& a, const WideHead& h = WideHead{nullptr, nullptr, nullptr, 0, 1.0f}) {
+  return a.qtype == TNX_Q_INT4 ? launch_qgemm_wide_as<SPT, true>(st, a, h) : launch_qgemm_wide_as<SPT, false>(st, a, h);
+}
+
 // The grouped form: the grid covers an upper bound of the 128-row blocks, sum over the experts
 // of ceil(rows / 128) <= n_routes / 128 + E (work-groups past the last block exit at once).
-template <int SPT>
-int launch_qgemm_wide_grouped(hipStream_t st, const QLArgs& a) {
+template <int SPT, bool INT4>
+int launch_qgemm_wide_grouped_as(hipStream_t st, const QLArgs& a) {
   static std::once_flag once;
   static int attr_rc = TNX_OK;
-  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm_wide_kernel<SPT, true>, kWideSmemBytes); });
+  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm_wide_kernel<SPT, true, INT4>, kWideSmemBytes); });
   if (attr_rc) return attr_rc;
   const int64_t blocks = a.M / kWideRows + a.n_experts;
   const unsigned wgs = (unsigned)(blocks * cdiv(a.N, kWideCols));
-  hipLaunchKernelGGL((qgemm_wide_kernel<SPT, true>), dim3(wgs), dim3(256), kWideSmemBytes, st, a,
+  hipLaunchKernelGGL((qgemm_wide_kernel<SPT, true, INT4>), dim3(wgs), dim3(256), kWideSmemBytes, st, a,
                      WideHead{nullptr, nullptr, nullptr, 0, 1.0f});
   TNX_CHECK_LAUNCH("qgemm_wide_grouped");
   return TNX_OK;
+}
+
+template <int SPT>
+int launch_qgemm_wide_grouped(hipStream_t st, const QLArgs& a) {
+  return a.qtype == TNX_Q_INT4 ? launch_qgemm_wide_grouped_as<SPT, true>(st, a) : launch_qgemm_wide_grouped_as<SPT, false>(st, a);
 }
 
 // Shapes the 128 x 256 kernel takes: enough rows to fill the device with its tiles, no k split,
