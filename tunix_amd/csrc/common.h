@@ -95,6 +95,51 @@ __device__ __forceinline__ void build_lut(uint32_t* lut, int qtype, int tid, int
       lut[byte * TNX_LUT_COPIES + ((c + tid) & (TNX_LUT_COPIES - 1))] = v;
   }
 }
+// The integer code book without a table.  A code byte is (k even | k odd << 4) and a dword holds
+// a lane's four code bytes of one k-step.  Masked into the mantissa of an f16 whose exponent makes
+// one mantissa step worth exactly one level -- 0x6400 (1024, step 1) for a nibble at bit 0, 0x5400
+// (64, step 1/16) for a nibble at bit 4 -- the nibbles of bytes 0 and 2 become an f16 pair
+// (1024 + n | 1024 + n) or (64 + n | 64 + n) with one v_and_or_b32, those of bytes 1 and 3 after
+// one shift by 8, and one packed f16 add of -1032 or -72 leaves the exact levels n - 8.  Entry j
+// of a dword is then: 0 = the even k of bytes 0 | 2, 1 = the odd k of bytes 0 | 2, 2 / 3 = the
+// same of bytes 1 | 3; the pair of byte b is half b / 2 of entries 2 (b % 2) and 2 (b % 2) + 1.
+// One VALU instruction more per pair than the table path, and no LDS instruction.
+struct Int4Magic {
+  uint32_t mask_lo = 0x000f000fu, mask_hi = 0x00f000f0u, magic_lo = 0x64006400u, magic_hi = 0x54005400u;
+  uint32_t bias_lo = 0xe408e408u, bias_hi = 0xd480d480u;   // f16 pairs (-1032 | -1032), (-72 | -72)
+  // Kept in registers as opaque values, so that the compiler forms v_and_or_b32 (which takes no
+  // literal and only one scalar operand): the exponents in vector registers; masks and biases in
+  // scalar registers, or in vector registers too for a kernel that has no scalar registers left
+  // (out of them, the compiler parks loop-carried scalars in vector registers and then hands
+  // one to an assembly operand that must be scalar).
+  template <bool VEC>
+  __device__ __forceinline__ void pin() {
+    asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));
+    if constexpr (VEC) asm volatile("" : "+v"(mask_lo), "+v"(mask_hi), "+v"(bias_lo), "+v"(bias_hi));
+    else asm volatile("" : "+s"(mask_lo), "+s"(mask_hi), "+s"(bias_lo), "+s"(bias_hi));
+  }
+};
+__device__ __forceinline__ uint32_t int4_entry(const Int4Magic& m, uint32_t w, int j) {
+  typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+  const uint32_t src = j < 2 ? w : w >> 8;
+  const uint32_t v = (j & 1) ? ((src & m.mask_hi) | m.magic_hi) : ((src & m.mask_lo) | m.magic_lo);
+  const f16x2_t sum = __builtin_bit_cast(f16x2_t, v) + __builtin_bit_cast(f16x2_t, (j & 1) ? m.bias_hi : m.bias_lo);
+  return __builtin_bit_cast(uint32_t, sum);
+}
+// the two levels of code byte b, as f16: from a dword's four entries above (INT4) or from the
+// table's four entries, one per byte
+template <bool INT4>
+__device__ __forceinline__ void level_pair(const uint32_t (&e)[4], int b, _Float16& l0, _Float16& l1) {
+  typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+  if constexpr (INT4) {
+    l0 = __builtin_bit_cast(f16x2_t, e[2 * (b & 1)])[b >> 1];
+    l1 = __builtin_bit_cast(f16x2_t, e[2 * (b & 1) + 1])[b >> 1];
+  } else {
+    const f16x2_t h = __builtin_bit_cast(f16x2_t, e[b]);
+    l0 = h[0];
+    l1 = h[1];
+  }
+}
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {

@@ -71,7 +71,8 @@ __device__ unsigned long long tnx_stamps[8];
 // MT = row tiles of 16 (8 for 65+ rows; 1, 2, 4 for decode batches of up to 16, 32, 64 rows: the
 // weight stream and its dequantisation are the same, the MFMA, fragment and activation work
 // shrink with the rows).
-template <int NT, int SPT, int MT>
+// INT4: integer codes, converted without the table (Int4Magic in common.h).
+template <int NT, int SPT, int MT, bool INT4 = false>
 __global__ __launch_bounds__(512)
 void qgemm128_kernel(const QLArgs a) {
   constexpr int HM = (MT + 1) / 2, PF = 3;   // HM: row tiles a wave finishes after the k halves meet
@@ -100,6 +101,20 @@ void qgemm128_kernel(const QLArgs a) {
   // of the kernel waits on memory except the loads of the first tiles
   const float lvl0 = rbf(code_level_imm(a.qtype, tid & 15)), lvl1 = rbf(code_level_imm(a.qtype, (tid >> 4) & 15));
   const uint32_t lane_off = (uint32_t)lane * 4u | kBigLutBase;   // byte 2 = 1: the table's base
+  Int4Magic magic;
+  if constexpr (INT4) magic.pin<true>();
+  // entry j of a k-step's code dword: Int4Magic's, or the table's entry for byte j
+  auto level_entry = [&](uint32_t w, int j) -> uint32_t {
+    if constexpr (INT4) {
+      // (tied to its place in the unit order like the look-up it replaces: an instruction without
+      // side effects is otherwise free to move across the scheduling barriers)
+      uint32_t e = int4_entry(magic, w, j);
+      asm volatile("" : "+v"(e));
+      return e;
+    } else {
+      return lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020400u + ((uint32_t)j << 8)));
+    }
+  };
   const int64_t m0 = (int64_t)blockIdx.x * ROWS;
   const int64_t ntile0 = ((int64_t)blockIdx.y * 4 + wn) * NT;
   const int64_t ntiles = a.N / 16;
@@ -277,11 +292,9 @@ void qgemm128_kernel(const QLArgs a) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       const uint32_t w = ring_c[D][nt][J];
-      // address bytes: [0] = lane * 4, [1] = code byte b of w, [2] = 1 (the table's base), [3] = 0
-      dst[nt][0] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020400u));
-      dst[nt][1] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020500u));
-      dst[nt][2] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020600u));
-      dst[nt][3] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020700u));
+      // table address bytes: [0] = lane * 4, [1] = code byte b of w, [2] = 1 (the table's base), [3] = 0
+#pragma unroll
+      for (int j = 0; j < 4; ++j) dst[nt][j] = level_entry(w, j);
     }
   };
   // f16 level pair x fp32 scale -> bf16 pair
@@ -293,8 +306,9 @@ void qgemm128_kernel(const QLArgs a) {
       u32x4 r;
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
-        const h16x2 h = __builtin_bit_cast(h16x2, src[nt][b]);
-        r[b] = cvt_pk_bf16(__builtin_fmaf((float)h[0], s, 0.0f), __builtin_fmaf((float)h[1], s, 0.0f));
+        _Float16 l0, l1;
+        level_pair<INT4>(src[nt], b, l0, l1);
+        r[b] = cvt_pk_bf16(__builtin_fmaf((float)l0, s, 0.0f), __builtin_fmaf((float)l1, s, 0.0f));
       }
       dst[nt] = r;
     }
@@ -331,7 +345,10 @@ void qgemm128_kernel(const QLArgs a) {
     static_assert(UNITS % MPS == 0 && 4 + 2 * NT <= UNITS / 2 && AP <= 4, "unit layout");
     float f0 = 0.f, f1 = 0.f;
     const bool ut = lora_fast && kt >= kt_end;      // LD: the activation tile to fetch is the adapter block
-    const int xs = ut ? 0 : min(kt, ktiles - 1) * (KTILE * 2);
+    // (INT4: left alone, the compiler keeps this wave-uniform offset in a vector register in that
+    // instantiation and hands it to the load's scalar operand as it is)
+    const int xs_ = ut ? 0 : min(kt, ktiles - 1) * (KTILE * 2);
+    const int xs = INT4 ? __builtin_amdgcn_readfirstlane(xs_) : xs_;
     const u32x4 xr = sel_rsrc(ut);
     const uint32_t um = 0u - (uint32_t)ut;
     const uint32_t xo = xbase ^ ((xbase ^ tbase) & um), xst = xstride ^ ((xstride ^ tstride) & um);
@@ -344,16 +361,16 @@ void qgemm128_kernel(const QLArgs a) {
         acc[m][nt] = mfma16(af[CUR][m], bfr[CUR][nt], acc[m][nt]);
       }
       if ((u & 1) == 0) {
-        const h16x2 h = __builtin_bit_cast(h16x2, lp[CUR][pnt][pb]);
+        _Float16 l0, l1;
+        level_pair<INT4>(lp[CUR][pnt], pb, l0, l1);
         const float sv = sc[DC][pnt][SPT == 2 ? 0 : JC];
-        f0 = __builtin_fmaf((float)h[0], sv, 0.0f);
-        f1 = __builtin_fmaf((float)h[1], sv, 0.0f);
+        f0 = __builtin_fmaf((float)l0, sv, 0.0f);
+        f1 = __builtin_fmaf((float)l1, sv, 0.0f);
       } else {
         bfr[NXT][pnt][pb] = cvt_pk_bf16(f0, f1);
       }
       if (u < UNITS / 2) {   // all LDS reads in the first half: nothing of them is in flight at the barrier
-        lp[NXT][u >> 2][u & 3] =
-            lds_ld32(__builtin_amdgcn_perm(ring_c[DL][u >> 2][JL], lane_off, 0x0c020400u + ((uint32_t)(u & 3) << 8)));
+        lp[NXT][u >> 2][u & 3] = level_entry(ring_c[DL][u >> 2][JL], u & 3);
         if (u < MT) af[NXT][u] = lds_ld128(rd_base + (uint32_t)(u * 16 * 256));
       } else {
         const int q = u - UNITS / 2;
@@ -409,7 +426,8 @@ void qgemm128_kernel(const QLArgs a) {
     // in the steady state of the loop, so the counted waits of the loop body need not fall back
     // to "everything outstanding" for the sake of the path that enters from here.
     TNX_STAMP(7);
-    {  // table entry e = f16 pair (level[e & 15], level[e >> 4]); copies rotated over banks,
+    if constexpr (!INT4) {
+       // table entry e = f16 pair (level[e & 15], level[e >> 4]); copies rotated over banks,
        // half of them per thread; built while the first loads are in flight
       uint32_t* lut = reinterpret_cast<uint32_t*>(smem + kBigLutBase);
       const h16x2 h = {(_Float16)lvl0, (_Float16)lvl1};

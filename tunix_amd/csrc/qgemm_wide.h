@@ -47,16 +47,7 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
 // (expert, row block) is found from the expert offsets by a running sum; activation rows are
 // gathered through sorted_route (row = route / x_div), output rows are routes.  No adapter, no
 // lm_head statistics in this mode.
-//
-// INT4: the integer code book needs no table.  A code byte is (k even | k odd << 4) and a dword
-// holds the lane's four pairs of one slab; masked into the mantissa of an f16 whose exponent makes
-// one mantissa step worth exactly one level -- 0x6400 (1024, step 1) for a nibble at bit 0, 0x5400
-// (64, step 1/16) for a nibble at bit 4 -- the nibbles of bytes 0 and 2 become an f16 pair
-// (1024 + n | 1024 + n) or (64 + n | 64 + n) with one v_and_or_b32, those of bytes 1 and 3 after
-// one shift by 8, and one packed f16 add of -1032 or -72 leaves the exact levels n - 8.  Entry j
-// of a slab is then: 0 = even k of bytes 0 | 2, 1 = odd k of bytes 0 | 2, 2 / 3 = the same of
-// bytes 1 | 3; the pair of byte b is half b / 2 of entries 2 (b % 2) and 2 (b % 2) + 1.  That is
-// one VALU instruction more per MFMA than the table path and one LDS instruction fewer.
+// INT4: integer codes, converted without the table (Int4Magic in common.h).
 template <int SPT, bool GROUPED = false, bool INT4 = false>
 __global__ __launch_bounds__(256)
 void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
@@ -282,32 +273,19 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   // Fragment addresses: slab u wants k-chunk 2 u + l / 32 of row l % 32 (+ 32 per row tile, an
   // immediate).  xaddr[u] points into the tile slab u is read from next and flips to the other
   // tile after each use; slab 0 is read one tile ahead (by slab 7 of the tile before).
-  // (masks in scalar registers, the exponents in vector registers: one v_and_or_b32 each, which
-  // takes no literal and only one scalar operand)
-  uint32_t mask_lo = 0x000f000fu, mask_hi = 0x00f000f0u, magic_lo = 0x64006400u, magic_hi = 0x54005400u;
-  if constexpr (INT4) asm volatile("" : "+s"(mask_lo), "+s"(mask_hi), "+v"(magic_lo), "+v"(magic_hi));
-  // entry j of the dword w of one slab (see INT4 above) / the table's entry for byte j of w
+  Int4Magic magic;
+  if constexpr (INT4) magic.pin<false>();
+  // entry j of the dword w of one slab: Int4Magic's, or the table's entry for byte j of w
   auto level_entry = [&](uint32_t w, int j) -> uint32_t {
-    if constexpr (INT4) {
-      const uint32_t src = j < 2 ? w : w >> 8;
-      const uint32_t m = (j & 1) ? ((src & mask_hi) | magic_hi) : ((src & mask_lo) | magic_lo);
-      const h16x2 bias = (j & 1) ? h16x2{(_Float16)-72.0f, (_Float16)-72.0f} : h16x2{(_Float16)-1032.0f, (_Float16)-1032.0f};
-      return __builtin_bit_cast(uint32_t, __builtin_bit_cast(h16x2, m) + bias);
-    } else {
-      return lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020400u + ((uint32_t)j << 8)));
-    }
+    if constexpr (INT4) return int4_entry(magic, w, j);
+    else return lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020400u + ((uint32_t)j << 8)));
   };
   // the two levels of byte b of a slab's dword times the scale sv, from that slab's entries
   auto pair_products = [&](const uint32_t (&e)[4], int b, float sv, float& p0, float& p1) {
-    if constexpr (INT4) {
-      const h16x2 he = __builtin_bit_cast(h16x2, e[2 * (b & 1)]), ho = __builtin_bit_cast(h16x2, e[2 * (b & 1) + 1]);
-      p0 = __builtin_fmaf((float)he[b >> 1], sv, 0.0f);
-      p1 = __builtin_fmaf((float)ho[b >> 1], sv, 0.0f);
-    } else {
-      const h16x2 hh = __builtin_bit_cast(h16x2, e[b]);
-      p0 = __builtin_fmaf((float)hh[0], sv, 0.0f);
-      p1 = __builtin_fmaf((float)hh[1], sv, 0.0f);
-    }
+    _Float16 l0, l1;
+    level_pair<INT4>(e, b, l0, l1);
+    p0 = __builtin_fmaf((float)l0, sv, 0.0f);
+    p1 = __builtin_fmaf((float)l1, sv, 0.0f);
   };
   uint32_t xaddr[8];
 #pragma unroll

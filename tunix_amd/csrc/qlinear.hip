@@ -574,17 +574,23 @@ int prepare_qgemm128(Kern kern, size_t bytes) {
   return raise_lds_limit(kern, bytes);
 }
 
-template <int NT, int SPT, int MT>
-int launch_qgemm128(hipStream_t st, const QLArgs& a) {
+template <int NT, int SPT, int MT, bool INT4>
+int launch_qgemm128_as(hipStream_t st, const QLArgs& a) {
   static std::once_flag once;
   static int attr_rc = TNX_OK;
   constexpr size_t kSmem = big_smem_bytes(NT, MT);
-  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm128_kernel<NT, SPT, MT>, kSmem); });
+  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm128_kernel<NT, SPT, MT, INT4>, kSmem); });
   if (attr_rc) return attr_rc;
   dim3 grid((unsigned)cdiv(a.M, 16 * MT), (unsigned)cdiv(a.N, 64 * NT), (unsigned)a.split_k);
-  hipLaunchKernelGGL((qgemm128_kernel<NT, SPT, MT>), grid, dim3(512), kSmem, st, a);
+  hipLaunchKernelGGL((qgemm128_kernel<NT, SPT, MT, INT4>), grid, dim3(512), kSmem, st, a);
   TNX_CHECK_LAUNCH("qgemm128");
   return TNX_OK;
+}
+
+// integer codes take the instantiation that converts them without the table
+template <int NT, int SPT, int MT>
+int launch_qgemm128(hipStream_t st, const QLArgs& a) {
+  return a.qtype == TNX_Q_INT4 ? launch_qgemm128_as<NT, SPT, MT, true>(st, a) : launch_qgemm128_as<NT, SPT, MT, false>(st, a);
 }
 
 template <int SPT, bool INT4>
@@ -599,7 +605,6 @@ int launch_qgemm_wide_as(hipStream_t st, const QLArgs& a, const WideHead& h) {
   return TNX_OK;
 }
 
-// integer codes take the instantiation that converts them without the table
 template <int SPT>
 int launch_qgemm_wide(hipStream_t st, const QLArgs& a, const WideHead& h = WideHead{nullptr, nullptr, nullptr, 0, 1.0f}) {
   return a.qtype == TNX_Q_INT4 ? launch_qgemm_wide_as<SPT, true>(st, a, h) : launch_qgemm_wide_as<SPT, false>(st, a, h);
