@@ -119,10 +119,17 @@ struct Int4Magic {
     else asm volatile("" : "+s"(mask_lo), "+s"(mask_hi), "+s"(bias_lo), "+s"(bias_hi));
   }
 };
+// entry j with the offsets still on: 1024 + n (even j) or 64 + n (odd j) in both halves.  A kernel
+// with registers to spare multiplies these with the scale s and adds -1032 s or -72 s in the same
+// fused multiply-add (exact: the sum (n - 8) s has at most 12 significant bits) and saves the
+// packed add.
+__device__ __forceinline__ uint32_t int4_entry_offset(const Int4Magic& m, uint32_t w, int j) {
+  const uint32_t src = j < 2 ? w : w >> 8;
+  return (j & 1) ? ((src & m.mask_hi) | m.magic_hi) : ((src & m.mask_lo) | m.magic_lo);
+}
 __device__ __forceinline__ uint32_t int4_entry(const Int4Magic& m, uint32_t w, int j) {
   typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
-  const uint32_t src = j < 2 ? w : w >> 8;
-  const uint32_t v = (j & 1) ? ((src & m.mask_hi) | m.magic_hi) : ((src & m.mask_lo) | m.magic_lo);
+  const uint32_t v = int4_entry_offset(m, w, j);
   const f16x2_t sum = __builtin_bit_cast(f16x2_t, v) + __builtin_bit_cast(f16x2_t, (j & 1) ? m.bias_hi : m.bias_lo);
   return __builtin_bit_cast(uint32_t, sum);
 }

@@ -169,6 +169,16 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   u32x4 ring_c[PF][CG][2];   // [.][.][0]: even slabs, [1]: odd slabs
   u32x2 ring_s[PF][CG];
   float sc[PF][CG][SPT];
+  // INT4: the entries keep their offsets (1024 + n | 64 + n), and the products subtract them
+  // again as -1032 s | -72 s in the multiply-add
+  float sb[INT4 ? PF : 1][CG][SPT][2];
+  auto set_scale = [&](int d, int cg, int j, float v) {
+    sc[d][cg][j] = v;
+    if constexpr (INT4) {
+      sb[d][cg][j][0] = v * -1032.0f;
+      sb[d][cg][j][1] = v * -72.0f;
+    }
+  };
   u32x4 xf[2][RT];           // activation fragments of the current / next slab
   u32x4 wf[2][CG];           // weight fragments of the current / next slab
   // f16 level pairs of the slab after the next (table path: entry b = the pair of byte b, looked
@@ -266,7 +276,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
 #pragma unroll
       for (int j = 0; j < SPT; ++j) {
         const uint32_t w = ring_s[D][cg][j >> 1];
-        sc[D][cg][j] = active ? ((j & 1) ? bfhi(w) : bflo(w)) : 0.f;
+        set_scale(D, cg, j, active ? ((j & 1) ? bfhi(w) : bflo(w)) : 0.f);
       }
     }
   };
@@ -275,17 +285,18 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   // tile after each use; slab 0 is read one tile ahead (by slab 7 of the tile before).
   Int4Magic magic;
   if constexpr (INT4) magic.pin<false>();
-  // entry j of the dword w of one slab: Int4Magic's, or the table's entry for byte j of w
+  // entry j of the dword w of one slab: Int4Magic's (offsets on), or the table's entry for byte j of w
   auto level_entry = [&](uint32_t w, int j) -> uint32_t {
-    if constexpr (INT4) return int4_entry(magic, w, j);
+    if constexpr (INT4) return int4_entry_offset(magic, w, j);
     else return lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c020400u + ((uint32_t)j << 8)));
   };
-  // the two levels of byte b of a slab's dword times the scale sv, from that slab's entries
-  auto pair_products = [&](const uint32_t (&e)[4], int b, float sv, float& p0, float& p1) {
+  // the two levels of byte b of a slab's dword times scale j of ring stage d, from that slab's entries
+  auto pair_products = [&](const uint32_t (&e)[4], int b, int d, int cg, int j, float& p0, float& p1) {
     _Float16 l0, l1;
     level_pair<INT4>(e, b, l0, l1);
-    p0 = __builtin_fmaf((float)l0, sv, 0.0f);
-    p1 = __builtin_fmaf((float)l1, sv, 0.0f);
+    const float sv = sc[d][cg][j];
+    p0 = __builtin_fmaf((float)l0, sv, INT4 ? sb[INT4 ? d : 0][cg][j][0] : 0.0f);
+    p1 = __builtin_fmaf((float)l1, sv, INT4 ? sb[INT4 ? d : 0][cg][j][1] : 0.0f);
   };
   uint32_t xaddr[8];
 #pragma unroll
@@ -325,8 +336,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
         // belongs to the fragment the MFMAs of slots 4-7 of THIS slab multiply
         if (i == 0) wf[CUR][CG - 1][3] = cvt_pk_bf16(cf0, cf1);
         else wf[NXT][(i - 1) >> 2][(i - 1) & 3] = cvt_pk_bf16(cf0, cf1);
-        const float sv = sc[DC][cg][SPT == 2 ? (UC >> 2) : (UC >> 1)];
-        pair_products(lp[INT4 ? (UC & 1) : 0][cg], rt, sv, cf0, cf1);
+        pair_products(lp[INT4 ? (UC & 1) : 0][cg], rt, DC, cg, SPT == 2 ? (UC >> 2) : (UC >> 1), cf0, cf1);
         lp[INT4 ? (UL & 1) : 0][cg][rt] = level_entry(ring_c[DL][cg][UL & 1][UL >> 1], rt);
       }
       if ((i & 1) == 0) xf[NXT][i >> 1] = lds_ld128(xaddr[UC] + (uint32_t)((i >> 1) * 32 * 256));
@@ -338,7 +348,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
       }
       if (EX && i < CG * SPT) {
         const uint32_t w = ring_s[DN][i / SPT][(i % SPT) >> 1];
-        sc[DN][i / SPT][i % SPT] = next_active ? (((i % SPT) & 1) ? bfhi(w) : bflo(w)) : 0.f;
+        set_scale(DN, i / SPT, i % SPT, next_active ? (((i % SPT) & 1) ? bfhi(w) : bflo(w)) : 0.f);
       }
       __builtin_amdgcn_sched_barrier(0);   // slots issue in the order written
     }
@@ -404,7 +414,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-      pair_products(lp[0][cg], b, sc[0][cg][0], cf0, cf1);
+      pair_products(lp[0][cg], b, 0, cg, 0, cf0, cf1);
       if (cg < CG - 1 || b < 3) wf[0][cg][b] = cvt_pk_bf16(cf0, cf1);   // the last pair: slot 0 of the loop
     }
 #pragma unroll
