@@ -206,6 +206,9 @@ def test_qlinear_lora_matches_oracle(gpu, M, K, N, group, qtype, r, split):
     (520, 128, 13440, 32, Q.INT4, 0, None, "residual"),
     (515, 640, 16896, 32, Q.INT4, 0, None, "gelu"),
     (1100, 256, 7424, 64, Q.INT4, 64, None, "store"),
+    # 40 row blocks: one full group of 32 of the work-group id -> tile map and a ragged one of 8
+    (5000, 128, 2048, 64, Q.INT4, 0, None, "store"),
+    (4200, 128, 2304, 64, Q.NF4, 16, None, "store"),
 ])
 def test_qlinear_many_rows_matches_oracle(gpu, M, K, N, group, qtype, r, seg_widths, epi):
   """Row counts that go to the 128 x 256-tile kernel (prefill, per-token logps): every epilogue,
