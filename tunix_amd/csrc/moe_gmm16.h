@@ -58,7 +58,9 @@ __device__ __forceinline__ void moe_static_for(F&& f) {
 }
 
 // MUL: the SiLU(gate) * up epilogue over interleaved gate / up tiles; SPT: scale slots per k-tile
-template <bool MUL, int SPT>
+// INT4: integer codes, converted without the table (Int4Magic in common.h; the level offsets are
+// subtracted in the scale multiply-add)
+template <bool MUL, int SPT, bool INT4>
 __global__ __launch_bounds__(kMoeWaves * 64) void moe_gmm16_kernel(const QLArgs a, const int E) {
   constexpr int R = kMoeRing;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -76,7 +78,7 @@ __global__ __launch_bounds__(kMoeWaves * 64) void moe_gmm16_kernel(const QLArgs 
   for (int i = tid; i <= E; i += kMoeWaves * 64) offs[i] = a.offsets[i];
   for (int i = tid; i < n_routes; i += kMoeWaves * 64) routes[i] = a.sorted_route[i];
   static_assert(kMoeWaves == 8, "the table is written by 512 threads");
-  {  // table entry e = f16 pair (level[e & 15], level[e >> 4]), 64 copies rotated over the banks
+  if constexpr (!INT4) {  // table entry e = f16 pair (level[e & 15], level[e >> 4]), 64 copies rotated over the banks
     const float lvl0 = rbf(code_level_imm(a.qtype, tid & 15)), lvl1 = rbf(code_level_imm(a.qtype, (tid >> 4) & 15));
     uint32_t* lut = reinterpret_cast<uint32_t*>(smem);
     const h16x2 h = {(_Float16)lvl0, (_Float16)lvl1};
@@ -139,6 +141,8 @@ __global__ __launch_bounds__(kMoeWaves * 64) void moe_gmm16_kernel(const QLArgs 
   const rsrc_t rc = make_rsrc(a.codes, (uint64_t)E * a.codes_stride * 4);
   const rsrc_t rs = make_rsrc(a.scales, (uint64_t)E * a.scales_stride * 2);
   const uint32_t lane_off = (uint32_t)lane * 4u;
+  Int4Magic magic;
+  if constexpr (INT4) magic.pin<false>();
   const uint32_t cvoff = (uint32_t)lane * 16u;
   const uint32_t svoff = (uint32_t)lm * (uint32_t)(SPT * 2);
   const uint32_t ctile = (uint32_t)ktiles * 1024u, stile = (uint32_t)ktiles * (uint32_t)(16 * SPT * 2);
@@ -206,15 +210,24 @@ __global__ __launch_bounds__(kMoeWaves * 64) void moe_gmm16_kernel(const QLArgs 
     auto look = [&](int g) {
       const uint32_t w = ring_c[D][g & 1][g >> 1];
 #pragma unroll
-      for (int k = 0; k < 4; ++k)
-        lp[g % 3][k] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0400u + ((uint32_t)k << 8)));
+      for (int k = 0; k < 4; ++k) {
+        if constexpr (INT4) {
+          uint32_t e = int4_entry_offset(magic, w, k);
+          asm volatile("" : "+v"(e));   // (stays where the look-up it replaces would be issued)
+          lp[g % 3][k] = e;
+        } else {
+          lp[g % 3][k] = lds_ld32(__builtin_amdgcn_perm(w, lane_off, 0x0c0c0400u + ((uint32_t)k << 8)));
+        }
+      }
     };
     auto conv = [&](int g) {
       const float s = scale_of(g);
+      const float b0 = INT4 ? s * -1032.0f : 0.0f, b1 = INT4 ? s * -72.0f : 0.0f;
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
-        const h16x2 h = __builtin_bit_cast(h16x2, lp[g % 3][k]);
-        bw[g & 1][k] = cvt_pk_bf16(__builtin_fmaf((float)h[0], s, 0.0f), __builtin_fmaf((float)h[1], s, 0.0f));
+        _Float16 l0, l1;
+        level_pair<INT4>(lp[g % 3], k, l0, l1);
+        bw[g & 1][k] = cvt_pk_bf16(__builtin_fmaf((float)l0, s, b0), __builtin_fmaf((float)l1, s, b1));
       }
     };
     look(0);

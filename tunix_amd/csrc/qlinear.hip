@@ -685,22 +685,27 @@ bool moe16_shape(const QLArgs& a, int E, size_t codes_bytes, size_t scales_bytes
   return moe16_smem_bytes(E, a.M) <= 160 * 1024;
 }
 
-template <bool MUL, int SPT>
+template <bool MUL, int SPT, bool INT4>
 int launch_moe16_t(hipStream_t st, const QLArgs& a, int E, int cus) {
   static std::once_flag once;
   static int attr_rc = TNX_OK;
-  std::call_once(once, [] { attr_rc = prepare_qgemm128(&moe_gmm16_kernel<MUL, SPT>, 160 * 1024); });
+  std::call_once(once, [] { attr_rc = prepare_qgemm128(&moe_gmm16_kernel<MUL, SPT, INT4>, 160 * 1024); });
   if (attr_rc) return attr_rc;
-  hipLaunchKernelGGL((moe_gmm16_kernel<MUL, SPT>), dim3((unsigned)cus), dim3(kMoeWaves * 64), moe16_smem_bytes(E, a.M), st, a, E);
+  hipLaunchKernelGGL((moe_gmm16_kernel<MUL, SPT, INT4>), dim3((unsigned)cus), dim3(kMoeWaves * 64), moe16_smem_bytes(E, a.M), st, a, E);
   TNX_CHECK_LAUNCH("moe_gmm16");
   return TNX_OK;
+}
+
+template <bool MUL, int SPT>
+int launch_moe16_q(hipStream_t st, const QLArgs& a, int E, int cus) {
+  return a.qtype == TNX_Q_INT4 ? launch_moe16_t<MUL, SPT, true>(st, a, E, cus) : launch_moe16_t<MUL, SPT, false>(st, a, E, cus);
 }
 
 int launch_moe16(hipStream_t st, const QLArgs& a, int E, int cus) {
   const bool mul = a.epilogue == TNX_EPI_SILU_MUL;
   if (scales_per_tile(a.group) == 2)
-    return mul ? launch_moe16_t<true, 2>(st, a, E, cus) : launch_moe16_t<false, 2>(st, a, E, cus);
-  return mul ? launch_moe16_t<true, 4>(st, a, E, cus) : launch_moe16_t<false, 4>(st, a, E, cus);
+    return mul ? launch_moe16_q<true, 2>(st, a, E, cus) : launch_moe16_q<false, 2>(st, a, E, cus);
+  return mul ? launch_moe16_q<true, 4>(st, a, E, cus) : launch_moe16_q<false, 4>(st, a, E, cus);
 }
 
 int device_cus() {
