@@ -794,22 +794,29 @@ def main():
   # rollout sampling: one categorical draw over the whole vocabulary per row and step), through
   # the public Sampler call; two rollouts of different length, so that prefill, graph capture
   # and host work cancel.  Reported beside the headline (greedy) number, never instead of it.
-  sampling = None
+  sampling = recipe = None
   if args.sampling_steps > 0:
     prompts = [ids[b] for b in range(B)]
-    times = []
-    for n in (4, 4 + args.sampling_steps):
-      torch.cuda.synchronize()
-      t0 = time.perf_counter()
-      sampler(prompts, n, max_prompt_length=P, temperature=1.0, top_p=1.0, top_k=None, seed=7,
-              return_logprobs=True, eos_tokens=[-1])
-      torch.cuda.synchronize()
-      times.append(time.perf_counter() - t0)
-    s_ms = (times[1] - times[0]) / args.sampling_steps * 1e3
-    sampling = {"mode": "temperature 1.0, top_p 1.0, no top-k (categorical over the vocabulary)",
-                "steps": args.sampling_steps, "ms_per_step": round(s_ms, 4),
-                "tokens_per_s": round(B / (s_ms * 1e-3), 1), "context_range": [P + 4, P + 4 + args.sampling_steps]}
-    log(f"sampling variant: {s_ms:.3f} ms/step over {args.sampling_steps} steps from context {P + 4}")
+
+    def variant(label, **kw):
+      times = []
+      for n in (4, 4 + args.sampling_steps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        sampler(prompts, n, max_prompt_length=P, seed=7, return_logprobs=True, eos_tokens=[-1], **kw)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+      s_ms = (times[1] - times[0]) / args.sampling_steps * 1e3
+      log(f"sampling variant ({label}): {s_ms:.3f} ms/step over {args.sampling_steps} steps from context {P + 4}")
+      return {"mode": label, "steps": args.sampling_steps, "ms_per_step": round(s_ms, 4),
+              "tokens_per_s": round(B / (s_ms * 1e-3), 1), "context_range": [P + 4, P + 4 + args.sampling_steps]}
+
+    sampling = variant("temperature 1.0, top_p 1.0, no top-k (categorical over the vocabulary)",
+                       temperature=1.0, top_p=1.0, top_k=None)
+    # the sampling settings of the reference's own Llama-3.1-8B GRPO recipe
+    # (examples/rl/grpo/gsm8k/configs/llama3.1_8b.yaml: temperature 0.9, top_p 1.0, top_k 50)
+    recipe = variant("temperature 0.9, top_p 1.0, top-k 50 (the reference's Llama-3.1-8B GRPO recipe)",
+                     temperature=0.9, top_p=1.0, top_k=50)
 
   kern = kernel_breakdown(model, runner, st, int(round(mean_ctx)), args.kernel_iters)
   for name, v in kern.items():
@@ -844,6 +851,7 @@ def main():
     result["first_steps"] = first_steps
   if sampling is not None:
     result["sampling_variant"] = sampling
+    result["sampling_recipe"] = recipe
   if not args.no_fused_logps:
     del sampler, st, runner, graph
     torch.cuda.empty_cache()
