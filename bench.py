@@ -163,7 +163,7 @@ def many_rows_breakdown(model, rows, iters):
         M=rows, K=f.K, N=f.N, group=f.group, qtype=f.qtype, x=x, codes=f.codes, scales=f.scales, y=y,
         epilogue=epi, lora_rank=f.rp, lora_nseg=(-1 if f.interleave2 else len(f.names)),
         lora_seg_end=f.seg_end, lora_seg_toff=f.seg_toff, t=t, t_ld=t.shape[1] if t is not None else 0,
-        lora_b=f.b_t if f.has_lora else None, lora_scale=f.lora_scale)
+        lora_b=f.b_t if f.has_lora else None, lora_scale=f.lora_scale, w_expanded=f.expanded)
     ms = time_loop(lambda: ops.qlinear(d), iters, per_graph=2, warm=1)
     flops = 2.0 * rows * f.K * f.N
     out[key] = {"us": round(ms * 1e3, 1), "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1)}

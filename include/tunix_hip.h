@@ -67,8 +67,9 @@ const char* tnx_last_error(void);
  * History: 1.0 first ABI; 1.1 added tnx_rmsnorm_moe_combine (and, against this rule, an argument
  * of tnx_quantize_pack and a field of tnx_lmhead_desc); 2.0 states the rule, keeps those changes,
  * adds tnx_attn_desc.segment_ids, reads top_k == V in tnx_sample_topk as a real top-k, and moves
- * the measurement probe tnx_stream_read out of the library. */
-#define TNX_ABI_VERSION_MAJOR 2
+ * the measurement probe tnx_stream_read out of the library; 3.0 adds tnx_qw_expand /
+ * tnx_qw_expanded_bytes and the w_expanded field of tnx_qlinear_desc and tnx_lmhead_desc. */
+#define TNX_ABI_VERSION_MAJOR 3
 #define TNX_ABI_VERSION_MINOR 0
 #define TNX_ABI_VERSION ((TNX_ABI_VERSION_MAJOR << 16) | TNX_ABI_VERSION_MINOR)
 int tnx_version(void);
@@ -111,6 +112,18 @@ int tnx_quantize_pack(void* stream, const void* w, int w_is_f32, int64_t K, int6
 int tnx_qw_dequant(void* stream, const uint32_t* codes, const uint16_t* scales, int64_t K,
                    int64_t N, int group, int qtype, int interleave2, float* w_out);
 
+/* Optional second copy of a frozen weight for calls with many rows (512 and more: prefill,
+ * compute_per_token_logps): the same values w^ = bf16(bf16(level) * scale), 2 bytes per weight,
+ * laid out as the matrix-instruction fragments of the many-row kernel, which then loads them as
+ * they are instead of converting codes in its loop (results are bit-identical; the kernel is
+ * bound by its instruction mix there, not by the 4x larger weight stream).  288 GB of HBM hold
+ * it beside the packed weights: 14 GB for the 7 G linear weights of Llama-3.1-8B.  Pass the copy
+ * as tnx_qlinear_desc.w_expanded / tnx_lmhead_desc.w_expanded; calls with few rows ignore it.
+ * No counterpart in the reference (XLA materialises a dequantised bf16 W on every call). */
+size_t tnx_qw_expanded_bytes(int64_t K, int64_t N);
+int tnx_qw_expand(void* stream, const uint32_t* codes, const uint16_t* scales, int64_t K, int64_t N,
+                  int group, int qtype, uint16_t* w_expanded /* 16-byte aligned */);
+
 /* ---------------------------------------------------------------------------------------
  * Quantized linear fused with the LoRA delta:  y = epi( x . dequant(W) + lora_scale * t . B )
  * replaces Einsum.__call__ / nnx.Linear as rewritten by qwix (llama3/model.py:216-218,
@@ -150,6 +163,7 @@ typedef struct tnx_qlinear_desc {
   const uint16_t* next_a_t; /* bf16 [next_rank, N/2]: A_next transposed                     */
   int next_rank;            /* multiple of 16, <= 64                                        */
   float* next_tpart;        /* fp32 [ceil(M/128) * ceil(N/128)][8192]                       */
+  const uint16_t* w_expanded; /* optional: tnx_qw_expand of (codes, scales); NULL: none       */
 } tnx_qlinear_desc;
 
 int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* h_desc);
@@ -362,6 +376,7 @@ typedef struct tnx_lmhead_desc {
    * every sum and the log-softmax run in fp32.  Log-probabilities then agree with an fp64
    * evaluation of the same bf16 operands to 1e-4 instead of to bf16 resolution. */
   int logits_fp32;
+  const uint16_t* w_expanded; /* optional, quantised head: tnx_qw_expand of (codes, scales)  */
 } tnx_lmhead_desc;
 int64_t tnx_lmhead_nblocks(int64_t V);
 int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* h_desc);

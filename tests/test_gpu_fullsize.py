@@ -362,3 +362,32 @@ def test_fused_logps_at_the_bench_launch_size(gpu):
   # logits of a random target are N(0, sigma^2) with sigma^2 = D * 0.02^2, so the mean
   # log-probability is -(log V + sigma^2 / 2) up to the quantisation of the weights
   assert abs(float(tlp.mean()) + np.log(V) + D * 0.02 ** 2 / 2) < 0.1
+
+
+def test_expanded_weight_copy_gives_the_same_whole_sequence_pass(gpu):
+  """One layer of the 8B shape, 32 x 96 tokens (3072 rows: every linear on the many-row GEMM): the model that keeps
+  the converted second copy of its NF4 weights and the one that converts codes in the loop give
+  bit-identical per-token log-probabilities, and a base-weight update refreshes the copy."""
+  from tunix_amd import config, dummy_model
+  from tunix_amd.model import QLoRAModel
+  from tunix_amd.rl.common import compute_per_token_logps
+  cfg = config.llama31_8b(num_layers=1, vocab_size=4096)
+  w = dummy_model.create_dummy_weights(cfg, seed=20261, device=gpu)
+  packed = QLoRAModel(cfg, w, gpu, expand_many_rows=False)
+  expanded = QLoRAModel(cfg, w, gpu, expand_many_rows=True)
+  assert all(f.expanded is None for f in packed._linears())
+  assert all(f.expanded is not None for f in expanded._linears())
+  g = np.random.Generator(np.random.PCG64(20261))
+  prompt = torch.from_numpy(g.integers(2, cfg.vocab_size, size=(32, 32)).astype(np.int32)).to(gpu)
+  completion = torch.from_numpy(g.integers(2, cfg.vocab_size, size=(32, 64)).astype(np.int32)).to(gpu)
+  a = compute_per_token_logps(packed, prompt, completion, pad_id=0, eos_id=1)
+  b = compute_per_token_logps(expanded, prompt, completion, pad_id=0, eos_id=1)
+  assert torch.isfinite(a).all() and torch.equal(a, b)
+  # new base weights for one projection: both models re-quantise, the copy follows
+  w2 = dict(w)
+  w2["l0.wo"] = (w["l0.wo"].float() * 1.5).to(w["l0.wo"].dtype)
+  packed.update_params(w2)
+  expanded.update_params(w2)
+  a2 = compute_per_token_logps(packed, prompt, completion, pad_id=0, eos_id=1)
+  b2 = compute_per_token_logps(expanded, prompt, completion, pad_id=0, eos_id=1)
+  assert torch.equal(a2, b2) and not torch.equal(a, a2)

@@ -279,7 +279,13 @@ def test_qlinear_many_rows_matches_oracle(gpu, M, K, N, group, qtype, r, seg_wid
     kw["residual"] = bf(res).to(gpu)
   ops.qlinear(ops.make_qlinear_desc(M=M, K=K, N=N, group=group, qtype=qtype, x=gx, codes=c, scales=s, y=y,
                                     epilogue=e, **kw))
+  # the same call fed with the converted second copy of the weight (the fragments the kernel
+  # would have formed from the codes): bit for bit the same output
+  y2 = torch.full_like(y, float("nan"))
+  ops.qlinear(ops.make_qlinear_desc(M=M, K=K, N=N, group=group, qtype=qtype, x=gx, codes=c, scales=s, y=y2,
+                                    epilogue=e, w_expanded=ops.qw_expand(c, s, K, N, group, qtype), **kw))
   torch.cuda.synchronize()
+  assert torch.equal(y.view(torch.int16), y2.view(torch.int16)), "expanded weights: output differs"
   # act(gate) * up: gate and up may each be one ulp off; linear + residual: a linear output one ulp
   # off can move the rounded sum by one more step of the sum's own (finer) spacing
   assert_bf16_close(y, ref, atol=1e-5 if mul else 1e-6, min_equal=0.9 if mul else 0.97, what=f"wide {epi}", mag=mag,

@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtunix_hip.so")
 
 # the ABI this binding was written against (TNX_ABI_VERSION_MAJOR / _MINOR of include/tunix_hip.h)
-ABI_VERSION = (2, 0)
+ABI_VERSION = (3, 0)
 
 TNX_Q_INT4, TNX_Q_NF4 = 0, 1
 TNX_NORM_LLAMA, TNX_NORM_QWEN3, TNX_NORM_GEMMA3 = 0, 1, 2
@@ -36,6 +36,7 @@ class QLinearDesc(C.Structure):
       ("epilogue", _i32), ("residual", _p), ("y", _p),
       ("split_k", _i32), ("ws", _p),
       ("next_a_t", _p), ("next_rank", _i32), ("next_tpart", _p),
+      ("w_expanded", _p),
   ]
 
 
@@ -77,6 +78,7 @@ class LmHeadDesc(C.Structure):
       ("part_entropy", _p), ("entropy", _p),
       ("part_draw", _p), ("draw_key0", C.c_uint32), ("draw_key1", C.c_uint32), ("draw_rng_variant", _i32),
       ("draw_step_ptr", _p), ("draw_id", _p), ("draw_logp", _p), ("logits_fp32", _i32),
+      ("w_expanded", _p),
   ]
 
 
@@ -96,6 +98,8 @@ SIGNATURES = {
     "tnx_qw_sizes": (_i32, [_i64, _i64, _i32, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "tnx_quantize_pack": (_i32, [_p, _p, _i32, _i64, _i64, _i32, _i32, _i32, _f32, _p, _p]),
     "tnx_qw_dequant": (_i32, [_p, _p, _p, _i64, _i64, _i32, _i32, _i32, _p]),
+    "tnx_qw_expanded_bytes": (C.c_size_t, [_i64, _i64]),
+    "tnx_qw_expand": (_i32, [_p, _p, _p, _i64, _i64, _i32, _i32, _p]),
     "tnx_qlinear_lora": (_i32, [_p, C.POINTER(QLinearDesc)]),
     "tnx_splitk_finish": (_i32, [_p, C.POINTER(QLinearDesc)]),
     "tnx_lora_reduce": (_i32, [_p, _p, _i64, _i64, _i32, _p, _i64]),

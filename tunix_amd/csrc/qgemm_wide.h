@@ -47,10 +47,21 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
 // (expert, row block) is found from the expert offsets by a running sum; activation rows are
 // gathered through sorted_route (row = route / x_div), output rows are routes.  No adapter, no
 // lm_head statistics in this mode.
-// INT4: integer codes, converted without the table (Int4Magic in common.h).
-template <int SPT, bool GROUPED = false, bool INT4 = false>
+// MODE: where the bf16 weight fragments come from.  kWideTable: codes through the LDS table;
+// kWideInt4: integer codes converted without the table (Int4Magic in common.h); kWidePre: a copy
+// of the weights that was converted once, bf16(bf16(level) * scale), and laid out as the
+// fragments themselves (tnx_qw_expand: [column tile][k-tile][wave][column group][slab][lane] x
+// 16 bytes), so that a lane's fragment of a slab is one 16-byte load and the loop has neither
+// conversion instructions nor look-ups.  The frozen base weights of a model fit HBM a second time
+// in that form; rows in the hundreds of thousands per weight byte make its four times larger
+// stream irrelevant.  Same MFMA sequence on the same operand bits: results are bit-identical.
+constexpr int kWideTable = 0, kWideInt4 = 1, kWidePre = 2;
+constexpr int kWidePreStages = 12;   // slabs of weight fragments in flight (1.5 k-tiles)
+template <int SPT, bool GROUPED = false, int MODE = kWideTable>
 __global__ __launch_bounds__(256)
 void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
+  constexpr bool INT4 = MODE == kWideInt4, PRE = MODE == kWidePre;
+  static_assert(!(PRE && GROUPED), "the grouped form reads packed codes");
   constexpr int RT = 4, CG = 2, PF = 3, AP = 8;   // 32-row tiles, 32-column groups per wave
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -66,8 +77,9 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   const float lvl0 = rbf(code_level_imm(a.qtype, tid & 15)), lvl1 = rbf(code_level_imm(a.qtype, (tid >> 4) & 15));
   const uint32_t lane_off = (uint32_t)lane * 4u | kWideLutBase;   // byte 2 = 1: the table's base
 
-  // work-group id -> (row block, column tile): groups of eight row blocks, the column tile
-  // moves every eight ids
+  // work-group id -> (row block, column tile): groups of 32 row blocks, the column tile moves
+  // every 32 ids (ids go round-robin to the eight XCDs: the four row blocks an XCD holds at a
+  // time share the column tile's weights in its L2)
   const int tiles_m = (int)((a.M + kWideRows - 1) / kWideRows), tiles_n = (int)((a.N + kWideCols - 1) / kWideCols);
   int mtile, ntile;
   int expert = 0, m_end = 0;   // GROUPED: the block's expert and the end of its routes in sorted order
@@ -101,10 +113,11 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
     mtile = __builtin_amdgcn_readfirstlane(found_rb);
     m_end = a.offsets[expert + 1];
   } else {
-    const int per_group = 32 * tiles_n;
+    constexpr int GR = 32;
+    const int per_group = GR * tiles_n;
     const int g = (int)blockIdx.x / per_group, r = (int)blockIdx.x % per_group;
-    const int gm = min(32, tiles_m - g * 32);
-    mtile = g * 32 + r % gm;
+    const int gm = min(GR, tiles_m - g * GR);
+    mtile = g * GR + r % gm;
     ntile = r / gm;
   }
   // first row of the tile (GROUPED: first position in the sorted route list)
@@ -181,6 +194,19 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   };
   u32x4 xf[2][RT];           // activation fragments of the current / next slab
   u32x4 wf[2][CG];           // weight fragments of the current / next slab
+  // PRE: the fragments of the next kWidePreStages slabs, loaded as they are; stage = slab % stages
+  u32x4 wr[PRE ? kWidePreStages : 1][CG];
+  const rsrc_t re = make_rsrc(PRE ? (const void*)a.w_pre : (const void*)a.x,
+                              PRE ? (uint64_t)tiles_n * (uint64_t)ktiles * 65536u : 0u);
+  uint32_t evoff[CG];
+#pragma unroll
+  for (int cg = 0; cg < CG; ++cg) evoff[cg] = (uint32_t)(((wn * CG + cg) * 8 * 64 + lane) * 16);
+  // slab `sl` (counted from this work-group's first k-tile) of column group cg -> its stage
+  auto load_pre = [&](int sl, int u, int cg) {
+    const int kt_ = min(sl >> 3, ktiles - 1);
+    wr[PRE ? sl % kWidePreStages : 0][cg] =
+        __builtin_amdgcn_raw_buffer_load_b128(re, evoff[cg] + (uint32_t)u * 1024u, (ntile * ktiles + kt_) * 65536, 0);
+  };
   // f16 level pairs of the slab after the next (table path: entry b = the pair of byte b, looked
   // up into the place of the entry just consumed; INT4: entries as described above, the slab's
   // parity picks the set, since a set is read until its slab has been converted)
@@ -329,6 +355,18 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int cg = i >> 2, rt = i & 3;
+      if constexpr (PRE) {
+        // the fragment as loaded; once a column group's four MFMAs have read it, its stage takes
+        // the same group's fragment of the slab kWidePreStages further on
+        constexpr int SL = D * 8 + U;
+        acc[rt][cg] = mfma32(wr[SL % kWidePreStages][cg], xf[CUR][rt], acc[rt][cg]);
+        if (rt == 3) {
+          const int sl = kt * 8 + U + kWidePreStages;   // (kt counts from this work-group's first k-tile: no k split here)
+          const int kt_ = min(sl >> 3, ktiles - 1);
+          wr[SL % kWidePreStages][cg] = __builtin_amdgcn_raw_buffer_load_b128(
+              re, evoff[cg] + (uint32_t)((U + kWidePreStages) & 7) * 1024u, (ntile * ktiles + kt_) * 65536, 0);
+        }
+      } else {
       acc[rt][cg] = mfma32(wf[CUR][cg], xf[CUR][rt], acc[rt][cg]);
       {
         // the pack of the pair before this one (a slot behind its products: packed in the same
@@ -339,14 +377,15 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
         pair_products(lp[INT4 ? (UC & 1) : 0][cg], rt, DC, cg, SPT == 2 ? (UC >> 2) : (UC >> 1), cf0, cf1);
         lp[INT4 ? (UL & 1) : 0][cg][rt] = level_entry(ring_c[DL][cg][UL & 1][UL >> 1], rt);
       }
+      }
       if ((i & 1) == 0) xf[NXT][i >> 1] = lds_ld128(xaddr[UC] + (uint32_t)((i >> 1) * 32 * 256));
       if (i == 7) xaddr[UC] ^= kWideTileBytes;
       if (LD) dma16(dma_buf + dma_wave + (uint32_t)i * 4096u, xr, xoff(i, xo, xst), xs);
-      if (LW) {
+      if (LW && !PRE) {
         if (i < 4) ring_c[D][i >> 1][i & 1] = __builtin_amdgcn_raw_buffer_load_b128(rc, coff[i >> 1] + (uint32_t)(i & 1) * 512u, wkt * 1024, 0);
         else if (i < 6) load_scale(Dc, i - 4, wkt);
       }
-      if (EX && i < CG * SPT) {
+      if (EX && !PRE && i < CG * SPT) {
         const uint32_t w = ring_s[DN][i / SPT][(i % SPT) >> 1];
         set_scale(DN, i / SPT, i % SPT, next_active ? (((i % SPT) & 1) ? bfhi(w) : bflo(w)) : 0.f);
       }
@@ -365,8 +404,9 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
     slab(ic<5>{}, Dc, kt, next_active);
     slab(ic<6>{}, Dc, kt, next_active);
     // the next tile's activations, requested by slab 7 of the tile before, have landed in LDS:
-    // the only younger loads are the six weight / scale loads slab 6 has just issued
-    tnx_wait_vm(6);
+    // the only younger loads are the six weight / scale loads slab 6 has just issued (PRE: the
+    // second fragment load of that slab 7 and the two of each slab since, fifteen)
+    tnx_wait_vm(PRE ? 14 : 6);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     slab(ic<7>{}, Dc, kt, next_active);
@@ -377,8 +417,15 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   // in the steady state of the loop, so the counted waits of the loop body never have to fall
   // back to "everything outstanding" for the sake of the path that enters from here)
   load_a(0, 0u);
-  load_w(ic<0>{}, 0);
-  if constexpr (!INT4) {  // table entry e = f16 pair (level[e & 15], level[e >> 4]), 64 copies rotated over the banks
+  if constexpr (PRE) {
+#pragma unroll
+    for (int sl = 0; sl < kWidePreStages; ++sl)
+#pragma unroll
+      for (int cg = 0; cg < CG; ++cg) load_pre(sl, sl & 7, cg);
+  } else {
+    load_w(ic<0>{}, 0);
+  }
+  if constexpr (MODE == kWideTable) {  // table entry e = f16 pair (level[e & 15], level[e >> 4]), 64 copies rotated over the banks
     uint32_t* lut = reinterpret_cast<uint32_t*>(smem + kWideLutBase);
     const h16x2 h = {(_Float16)lvl0, (_Float16)lvl1};
     const uint32_t v = __builtin_bit_cast(uint32_t, h);
@@ -386,8 +433,10 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
     for (int c = 0; c < 64; ++c) lut[tid * 64 + ((c + lane) & 63)] = v;
   }
   load_a(1, kWideTileBytes);
-  load_w(ic<1>{}, 1);
-  load_w(ic<2>{}, 2);
+  if constexpr (!PRE) {
+    load_w(ic<1>{}, 1);
+    load_w(ic<2>{}, 2);
+  }
   if (lora) {
     const rsrc_t rb = make_rsrc(a.lora_b, (uint64_t)a.N * a.lora_rank * 2);
 #pragma unroll
@@ -398,29 +447,34 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
           lbv[cg][u] = buf_load128(rb, (((uint32_t)(ntile0 + 2 * cg) * 16u + (uint32_t)l32) * (uint32_t)a.lora_rank +
                                         (uint32_t)(u * 16 + lh * 8)) * 2u);
   }
-  expand_scales(ic<0>{}, true);
+  if constexpr (!PRE) expand_scales(ic<0>{}, true);
   // the first tile is in LDS: its eight loads are the oldest, and at least 26 follow them (three
   // ring stages of six, the second tile's eight); vmcnt(20) also covers the first ring stage
-  tnx_wait_vm(20);
+  // (PRE: 24 fragment loads and the second tile's eight follow them)
+  tnx_wait_vm(PRE ? 32 : 20);
   __syncthreads();
   // slab 0: table entries, conversion, fragments; then the table entries of slab 1
+  if constexpr (!PRE) {
 #pragma unroll
-  for (int cg = 0; cg < CG; ++cg)
+    for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
-    for (int b = 0; b < 4; ++b) lp[0][cg][b] = level_entry(ring_c[0][cg][0][0], b);
+      for (int b = 0; b < 4; ++b) lp[0][cg][b] = level_entry(ring_c[0][cg][0][0], b);
+  }
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) xf[0][rt] = lds_ld128((xaddr[0] ^ kWideTileBytes) + (uint32_t)(rt * 32 * 256));
+  if constexpr (!PRE) {
 #pragma unroll
-  for (int cg = 0; cg < CG; ++cg)
+    for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      pair_products(lp[0][cg], b, 0, cg, 0, cf0, cf1);
-      if (cg < CG - 1 || b < 3) wf[0][cg][b] = cvt_pk_bf16(cf0, cf1);   // the last pair: slot 0 of the loop
-    }
+      for (int b = 0; b < 4; ++b) {
+        pair_products(lp[0][cg], b, 0, cg, 0, cf0, cf1);
+        if (cg < CG - 1 || b < 3) wf[0][cg][b] = cvt_pk_bf16(cf0, cf1);   // the last pair: slot 0 of the loop
+      }
 #pragma unroll
-  for (int cg = 0; cg < CG; ++cg)
+    for (int cg = 0; cg < CG; ++cg)
 #pragma unroll
-    for (int b = 0; b < 4; ++b) lp[INT4 ? 1 : 0][cg][b] = level_entry(ring_c[0][cg][1][0], b);
+      for (int b = 0; b < 4; ++b) lp[INT4 ? 1 : 0][cg][b] = level_entry(ring_c[0][cg][1][0], b);
+  }
   // whole turns of the ring without a branch inside (a conditional tile would make the waits
   // of the tile after it assume that its loads never happened), then the one or two tiles left
   int kt = 0;

@@ -38,6 +38,8 @@ struct QLArgs {
   const uint16_t* next_a_t;
   int next_rank;
   float* next_tpart;
+  // optional: the weights converted once into the many-row kernel's fragments (tnx_qw_expand)
+  const uint16_t* w_pre;
 };
 // Second argument of the 128 x 256 kernel: with `part` set it reduces its tile to lm_head
 // statistics instead of storing it.
@@ -455,6 +457,37 @@ __global__ void qw_dequant_kernel(const uint32_t* codes, const uint16_t* scales,
   out[k * N + c] = rbf(rbf(code_level(qtype, (word >> (4 * i)) & 15)) * s);
 }
 
+// The converted copy for the many-row kernel: block (column tile of 256, k-tile) = 64 KB =
+// [wave 4][column group 2][slab 8][lane 64] x 16 bytes, a lane's eight bf16 being the weights
+// bf16(bf16(level) * scale) of packed column 64 wave + 32 group + lane % 32 of the tile at
+// k = 128 kt + 16 slab + 8 (lane / 32) .. + 7: the A fragment of one 32x32x16 MFMA.  Columns past N
+// are zeros.  One thread per 16 bytes.
+__global__ __launch_bounds__(256) void qw_expand_kernel(const uint32_t* codes, const uint16_t* scales, int64_t K,
+                                                         int64_t N, int group, int qtype, u32x4* out) {
+  const int ntile = blockIdx.x, kt = blockIdx.y, ktiles = (int)(K / KTILE);
+  const int wn = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  const int spt = scales_per_tile(group);
+  for (int cg = 0; cg < 2; ++cg) {
+    const int64_t nt16 = (int64_t)ntile * 16 + wn * 4 + 2 * cg + (l32 >> 4);
+    const int c16 = l32 & 15;
+    const bool live = nt16 < N / 16;
+    const int64_t tile = (live ? nt16 : 0) * ktiles + kt;
+    for (int u = 0; u < 8; ++u) {
+      const int g8 = 2 * u + lh;                       // the 8-deep k group: k = 8 g8 = 8 q + 32 j
+      const uint32_t w = codes[(tile * 64 + (g8 & 3) * 16 + c16) * 4 + (g8 >> 2)];
+      const float sv = bf2f(scales[(tile * 16 + c16) * spt + (16 * u) / (KTILE / spt)]);
+      u32x4 r;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const uint32_t byte = (w >> (8 * b)) & 255u;
+        r[b] = pack2bf(rbf(code_level(qtype, byte & 15)) * sv, rbf(code_level(qtype, byte >> 4)) * sv);
+      }
+      if (!live) r = u32x4{0, 0, 0, 0};
+      out[((((int64_t)ntile * ktiles + kt) * 4 + wn) * 2 + cg) * 512 + u * 64 + lane] = r;
+    }
+  }
+}
+
 QLArgs to_args(const tnx_qlinear_desc* d) {
   QLArgs a;
   a.M = d->M; a.K = d->K; a.N = d->N; a.group = d->group; a.qtype = d->qtype;
@@ -468,6 +501,7 @@ QLArgs to_args(const tnx_qlinear_desc* d) {
   a.ktiles_per_split = (ktiles + a.split_k - 1) / a.split_k;
   a.offsets = nullptr; a.sorted_route = nullptr; a.x_div = 1; a.codes_stride = 0; a.scales_stride = 0;
   a.next_a_t = d->next_a_t; a.next_rank = d->next_rank; a.next_tpart = d->next_tpart;
+  a.w_pre = d->w_expanded;
   return a;
 }
 
@@ -593,21 +627,26 @@ int launch_qgemm128(hipStream_t st, const QLArgs& a) {
   return a.qtype == TNX_Q_INT4 ? launch_qgemm128_as<NT, SPT, MT, true>(st, a) : launch_qgemm128_as<NT, SPT, MT, false>(st, a);
 }
 
-template <int SPT, bool INT4>
+template <int SPT, int MODE>
 int launch_qgemm_wide_as(hipStream_t st, const QLArgs& a, const WideHead& h) {
   static std::once_flag once;
   static int attr_rc = TNX_OK;
-  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm_wide_kernel<SPT, false, INT4>, kWideSmemBytes); });
+  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm_wide_kernel<SPT, false, MODE>, kWideSmemBytes); });
   if (attr_rc) return attr_rc;
   const unsigned wgs = (unsigned)(cdiv(a.M, kWideRows) * cdiv(a.N, kWideCols));
-  hipLaunchKernelGGL((qgemm_wide_kernel<SPT, false, INT4>), dim3(wgs), dim3(256), kWideSmemBytes, st, a, h);
+  hipLaunchKernelGGL((qgemm_wide_kernel<SPT, false, MODE>), dim3(wgs), dim3(256), kWideSmemBytes, st, a, h);
   TNX_CHECK_LAUNCH("qgemm_wide");
   return TNX_OK;
 }
 
 template <int SPT>
 int launch_qgemm_wide(hipStream_t st, const QLArgs& a, const WideHead& h = WideHead{nullptr, nullptr, nullptr, 0, 1.0f}) {
-  return a.qtype == TNX_Q_INT4 ? launch_qgemm_wide_as<SPT, true>(st, a, h) : launch_qgemm_wide_as<SPT, false>(st, a, h);
+  // the converted copy when the caller keeps one (its block offsets are 32-bit); else integer
+  // codes take the instantiation that converts them without the table
+  if (a.w_pre && cdiv(a.N, kWideCols) * (a.K / KTILE) * 65536 < (int64_t)1 << 31)
+    return launch_qgemm_wide_as<2, kWidePre>(st, a, h);
+  return a.qtype == TNX_Q_INT4 ? launch_qgemm_wide_as<SPT, kWideInt4>(st, a, h)
+                               : launch_qgemm_wide_as<SPT, kWideTable>(st, a, h);
 }
 
 // The grouped form: the grid covers an upper bound of the 128-row blocks, sum over the experts
@@ -616,11 +655,11 @@ template <int SPT, bool INT4>
 int launch_qgemm_wide_grouped_as(hipStream_t st, const QLArgs& a) {
   static std::once_flag once;
   static int attr_rc = TNX_OK;
-  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm_wide_kernel<SPT, true, INT4>, kWideSmemBytes); });
+  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm_wide_kernel<SPT, true, INT4 ? kWideInt4 : kWideTable>, kWideSmemBytes); });
   if (attr_rc) return attr_rc;
   const int64_t blocks = a.M / kWideRows + a.n_experts;
   const unsigned wgs = (unsigned)(blocks * cdiv(a.N, kWideCols));
-  hipLaunchKernelGGL((qgemm_wide_kernel<SPT, true, INT4>), dim3(wgs), dim3(256), kWideSmemBytes, st, a,
+  hipLaunchKernelGGL((qgemm_wide_kernel<SPT, true, INT4 ? kWideInt4 : kWideTable>), dim3(wgs), dim3(256), kWideSmemBytes, st, a,
                      WideHead{nullptr, nullptr, nullptr, 0, 1.0f});
   TNX_CHECK_LAUNCH("qgemm_wide_grouped");
   return TNX_OK;
@@ -763,6 +802,26 @@ extern "C" int tnx_qw_dequant(void* stream, const uint32_t* codes, const uint16_
   return TNX_OK;
 }
 
+extern "C" size_t tnx_qw_expanded_bytes(int64_t K, int64_t N) {
+  if (K <= 0 || N <= 0 || K % KTILE != 0) return 0;
+  return (size_t)(cdiv(N, kWideCols) * (K / KTILE)) * 65536u;
+}
+
+extern "C" int tnx_qw_expand(void* stream, const uint32_t* codes, const uint16_t* scales, int64_t K, int64_t N,
+                             int group, int qtype, uint16_t* w_expanded) {
+  int rc = tnx_qw_sizes(K, N, group, nullptr, nullptr);
+  if (rc) return rc;
+  TNX_REQUIRE(codes && scales && w_expanded, "qw_expand: null pointer");
+  TNX_REQUIRE(qtype == TNX_Q_INT4 || qtype == TNX_Q_NF4, "qw_expand: bad qtype %d", qtype);
+  TNX_REQUIRE(((uintptr_t)w_expanded & 15) == 0, "qw_expand: the output must be 16-byte aligned");
+  TNX_REQUIRE(K / KTILE <= 65535, "qw_expand: K=%lld too large", (long long)K);
+  dim3 grid((unsigned)cdiv(N, kWideCols), (unsigned)(K / KTILE));
+  hipLaunchKernelGGL(qw_expand_kernel, grid, dim3(256), 0, as_stream(stream), codes, scales, K, N, group, qtype,
+                     reinterpret_cast<u32x4*>(w_expanded));
+  TNX_CHECK_LAUNCH("qw_expand");
+  return TNX_OK;
+}
+
 extern "C" int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* d) {
   int rc = check_desc(d);
   if (rc) return rc;
@@ -799,6 +858,7 @@ int tnx_internal_wide_head(hipStream_t st, const tnx_lmhead_desc* d, float tempe
   a.t_ld = d->t_ld; a.t = d->t; a.lora_b = d->lora_b; a.lora_scale = d->lora_scale;
   a.epilogue = TNX_EPI_STORE; a.y = d->part;   // the shape test looks at a stored tile
   a.split_k = 1; a.ktiles_per_split = (int)(d->D / KTILE); a.x_div = 1;
+  a.w_pre = d->w_expanded;
   if (!wide_shape(a)) return 1;
   a.y = nullptr;
   const WideHead h{d->part, part_ent, d->targets, nvb, temperature};

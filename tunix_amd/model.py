@@ -47,6 +47,7 @@ class FusedLinear:
     self.group, self.qtype, self.int4_bound = cfg.group, cfg.qtype, cfg.int4_bound
     self.device = device
     self.codes = self.scales = None
+    self.expanded = None   # optional second copy for calls with many rows (`expand`)
     self.load_base(weights)
     r = cfg.lora_rank
     self.has_lora = any((n + ".lora_a") in weights for n in names)
@@ -110,6 +111,24 @@ class FusedLinear:
     else:   # in place: captured graphs and descriptors keep their pointers
       self.codes.copy_(codes)
       self.scales.copy_(scales)
+      if self.expanded is not None:
+        self.expanded.copy_(ops.qw_expand(self.codes, self.scales, self.K, self.N, self.group, self.qtype))
+
+  def expanded_bytes(self) -> int:
+    return int(L.lib().tnx_qw_expanded_bytes(self.K, self.N))
+
+  def expand(self):
+    """Keeps a second copy of the frozen weight, converted to bf16 in the many-row kernel's
+    fragment order (2 bytes per weight): prefill and per-token-logps passes then load it instead
+    of converting codes in their loop.  Decode steps never read it."""
+    if self.expanded is None and self.wants_expansion():
+      self.expanded = ops.qw_expand(self.codes, self.scales, self.K, self.N, self.group, self.qtype)
+
+  def wants_expansion(self) -> bool:
+    """A table code book (NF4) gains 9-17 % on the many-row kernel from the copy; integer codes
+    are converted there without a table at the copy's speed, so they get none.  (The kernel
+    addresses the copy with 32-bit offsets.)"""
+    return self.qtype != L.TNX_Q_INT4 and self.expanded_bytes() < (1 << 31)
 
   def load_lora(self, weights: dict):
     """Copies lora_a [K,r] / lora_b [r,N_i] of every member into the kernel layout."""
@@ -185,7 +204,10 @@ class ExpertBank:
 class QLoRAModel:
   """Packed weights of one model on one GPU."""
 
-  def __init__(self, cfg: ModelConfig, weights: dict, device="cuda"):
+  def __init__(self, cfg: ModelConfig, weights: dict, device="cuda", expand_many_rows: bool | None = None):
+    """expand_many_rows: keep the converted second copy of every dense quantised linear
+    (`FusedLinear.expand`) for the calls with many rows.  None (default): when the copies take
+    less than a quarter of the device memory that is free once the model is built."""
     L.lib()  # fail loudly when the HIP library is missing
     self.cfg = cfg
     self.device = torch.device(device)
@@ -221,6 +243,13 @@ class QLoRAModel:
       ly["rope_scale"] = sf
       self.layers.append(ly)
     torch.cuda.synchronize(dev)
+    if expand_many_rows is None:
+      need = sum(f.expanded_bytes() for f in self._linears() if f.wants_expansion())
+      expand_many_rows = need <= torch.cuda.mem_get_info(dev)[0] // 4
+    if expand_many_rows:
+      for f in self._linears():
+        f.expand()
+      torch.cuda.synchronize(dev)
 
   # weight sync: LoRA-only replacement (tunix/generate/sampler.py:333-352)
   def update_lora(self, new_lora: dict):
@@ -467,7 +496,7 @@ class Runner:
         lora_nseg=(-1 if f.interleave2 else len(f.names)), lora_seg_end=f.seg_end,
         lora_seg_toff=f.seg_toff, t=self.t if f.has_lora else None, t_ld=self.t.shape[1],
         lora_b=f.b_t if f.has_lora else None, lora_scale=f.lora_scale, split_k=split,
-        ws=self.splitk_ws if split > 1 else None, **kw)
+        ws=self.splitk_ws if split > 1 else None, w_expanded=f.expanded, **kw)
     if kw:
       ops.qlinear(d)
       ops.lora_reduce(self.next_tpart, M, math.ceil(f.N / 128), next_f.rp, self.t)
@@ -637,6 +666,8 @@ class Runner:
     if m.head is not None:
       f = m.head
       d.codes, d.scales, d.group, d.qtype = f.codes.data_ptr(), f.scales.data_ptr(), f.group, f.qtype
+      if f.expanded is not None:
+        d.w_expanded = f.expanded.data_ptr()
       if f.has_lora:
         d.lora_rank, d.t, d.t_ld = f.rp, self.t.data_ptr(), self.t.shape[1]
         d.lora_b, d.lora_scale = f.b_t.data_ptr(), f.lora_scale

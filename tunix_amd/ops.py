@@ -63,7 +63,7 @@ def qw_dequant(codes, scales, K, N, group, qtype, interleave2=False) -> torch.Te
 def make_qlinear_desc(*, M, K, N, group, qtype, x, codes, scales, y, epilogue=L.TNX_EPI_STORE,
                       residual=None, lora_rank=0, lora_nseg=1, lora_seg_end=(), lora_seg_toff=(),
                       t=None, t_ld=0, lora_b=None, lora_scale=0.0, split_k=1, ws=None,
-                      next_a_t=None, next_rank=0, next_tpart=None):
+                      next_a_t=None, next_rank=0, next_tpart=None, w_expanded=None):
   d = L.QLinearDesc()
   d.M, d.K, d.N, d.group, d.qtype = M, K, N, group, qtype
   d.x, d.codes, d.scales, d.y = _ptr(x), _ptr(codes), _ptr(scales), _ptr(y)
@@ -76,7 +76,19 @@ def make_qlinear_desc(*, M, K, N, group, qtype, x, codes, scales, y, epilogue=L.
   d.t, d.t_ld, d.lora_b, d.lora_scale = _ptr(t), t_ld, _ptr(lora_b), lora_scale
   d.split_k, d.ws = split_k, _ptr(ws)
   d.next_a_t, d.next_rank, d.next_tpart = _ptr(next_a_t), next_rank, _ptr(next_tpart)
+  d.w_expanded = _ptr(w_expanded)
   return d
+
+
+def qw_expand(codes, scales, K, N, group, qtype):
+  """The second, converted copy of a packed weight for calls with many rows (tnx_qw_expand):
+  bf16, 2 bytes per weight, in the many-row kernel's fragment order."""
+  import torch
+  n = int(L.lib().tnx_qw_expanded_bytes(K, N)) // 2
+  out = torch.empty(n, dtype=torch.bfloat16, device=codes.device)
+  L.check(L.lib().tnx_qw_expand(_stream(), _ptr(codes), _ptr(scales), K, N, group, qtype, _ptr(out)),
+          "tnx_qw_expand")
+  return out
 
 
 def qlinear(desc: L.QLinearDesc, finish: bool = True):
