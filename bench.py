@@ -311,7 +311,7 @@ def write_fused_traffic_profile(fetch_csv, write_csv):
   wk, nw = mean(write_csv, "WRITE_SIZE")
   rows, D, V, r = 16384, 4096, 128256, 64
   rec = {
-      "kernel": "qgemm_wide_kernel<4> (head-statistics epilogue)",
+      "kernel": "qgemm_wide_kernel (head-statistics epilogue)",
       "workload": "one launch of the standalone log-probability pass: 16384 rows x 4096 -> 128256, int4 g128 + LoRA r64",
       "kernel_source_sha256_16": source_hash(FUSED_KERNEL_SOURCES),
       "kernel_sources": list(FUSED_KERNEL_SOURCES),
