@@ -68,7 +68,8 @@ const char* tnx_last_error(void);
  * of tnx_quantize_pack and a field of tnx_lmhead_desc); 2.0 states the rule, keeps those changes,
  * adds tnx_attn_desc.segment_ids, reads top_k == V in tnx_sample_topk as a real top-k, and moves
  * the measurement probe tnx_stream_read out of the library; 3.0 adds tnx_qw_expand /
- * tnx_qw_expanded_bytes and the w_expanded field of tnx_qlinear_desc and tnx_lmhead_desc. */
+ * tnx_qw_expanded_bytes, tnx_dense_expand and the w_expanded field of tnx_qlinear_desc and
+ * tnx_lmhead_desc. */
 #define TNX_ABI_VERSION_MAJOR 3
 #define TNX_ABI_VERSION_MINOR 0
 #define TNX_ABI_VERSION ((TNX_ABI_VERSION_MAJOR << 16) | TNX_ABI_VERSION_MINOR)
@@ -123,6 +124,10 @@ int tnx_qw_dequant(void* stream, const uint32_t* codes, const uint16_t* scales, 
 size_t tnx_qw_expanded_bytes(int64_t K, int64_t N);
 int tnx_qw_expand(void* stream, const uint32_t* codes, const uint16_t* scales, int64_t K, int64_t N,
                   int group, int qtype, uint16_t* w_expanded /* 16-byte aligned */);
+/* The same layout from a dense bf16 matrix w[N][K] (an unquantised or tied lm_head, [V][D]): a
+ * log-probability pass over 512 rows or more then runs the head on the many-row kernel
+ * (tnx_lmhead_desc.w_expanded next to w_bf16) instead of the 128 x 128 one. */
+int tnx_dense_expand(void* stream, const uint16_t* w_bf16, int64_t K, int64_t N, uint16_t* w_expanded);
 
 /* ---------------------------------------------------------------------------------------
  * Quantized linear fused with the LoRA delta:  y = epi( x . dequant(W) + lora_scale * t . B )
@@ -376,7 +381,8 @@ typedef struct tnx_lmhead_desc {
    * every sum and the log-softmax run in fp32.  Log-probabilities then agree with an fp64
    * evaluation of the same bf16 operands to 1e-4 instead of to bf16 resolution. */
   int logits_fp32;
-  const uint16_t* w_expanded; /* optional, quantised head: tnx_qw_expand of (codes, scales)  */
+  const uint16_t* w_expanded; /* optional: tnx_qw_expand of (codes, scales), or
+                                 tnx_dense_expand of w_bf16                                   */
 } tnx_lmhead_desc;
 int64_t tnx_lmhead_nblocks(int64_t V);
 int tnx_lmhead_logp(void* stream, const tnx_lmhead_desc* h_desc);

@@ -375,8 +375,11 @@ def test_expanded_weight_copy_gives_the_same_whole_sequence_pass(gpu):
   w = dummy_model.create_dummy_weights(cfg, seed=20261, device=gpu)
   packed = QLoRAModel(cfg, w, gpu, expand_many_rows=False)
   expanded = QLoRAModel(cfg, w, gpu, expand_many_rows=True)
-  assert all(f.expanded is None for f in packed._linears())
-  assert all(f.expanded is not None for f in expanded._linears())
+  assert all(f.expanded is None for f in packed._linears()) and packed.head_expanded is None
+  assert all(f.expanded is not None for f in expanded._linears()) and expanded.head_expanded is not None
+  # (the dense head's copy sends the head itself to another kernel, with another summation order:
+  # checked on its own below; the linears' copies change no bit)
+  head_copy, expanded.head_expanded = expanded.head_expanded, None
   g = np.random.Generator(np.random.PCG64(20261))
   prompt = torch.from_numpy(g.integers(2, cfg.vocab_size, size=(32, 32)).astype(np.int32)).to(gpu)
   completion = torch.from_numpy(g.integers(2, cfg.vocab_size, size=(32, 64)).astype(np.int32)).to(gpu)
@@ -391,3 +394,18 @@ def test_expanded_weight_copy_gives_the_same_whole_sequence_pass(gpu):
   a2 = compute_per_token_logps(packed, prompt, completion, pad_id=0, eos_id=1)
   b2 = compute_per_token_logps(expanded, prompt, completion, pad_id=0, eos_id=1)
   assert torch.equal(a2, b2) and not torch.equal(a, a2)
+  # the dense head through its copy (the many-row kernel's statistics epilogue instead of the
+  # 128 x 128 head kernel): same logits up to the rounding of a bf16 logit whose fp32 sum came
+  # out in another order
+  expanded.head_expanded = head_copy
+  c2 = compute_per_token_logps(expanded, prompt, completion, pad_id=0, eos_id=1)
+  assert torch.isfinite(c2).all() and not torch.equal(c2, b2)
+  assert (c2 - b2).abs().max().item() < 2e-2 and (c2 - b2).abs().mean().item() < 2e-3
+  # ... and an update of the head refreshes the copy
+  w3 = dict(w2)
+  w3["lm_head"] = (w["lm_head"].float() * 0.5).to(w["lm_head"].dtype)
+  expanded.update_params(w3)
+  packed.update_params(w3)
+  c3 = compute_per_token_logps(expanded, prompt, completion, pad_id=0, eos_id=1)
+  a3 = compute_per_token_logps(packed, prompt, completion, pad_id=0, eos_id=1)
+  assert (c3 - a3).abs().max().item() < 2e-2 and (c3 - c2).abs().max().item() > 0.05

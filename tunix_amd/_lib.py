@@ -100,6 +100,7 @@ SIGNATURES = {
     "tnx_qw_dequant": (_i32, [_p, _p, _p, _i64, _i64, _i32, _i32, _i32, _p]),
     "tnx_qw_expanded_bytes": (C.c_size_t, [_i64, _i64]),
     "tnx_qw_expand": (_i32, [_p, _p, _p, _i64, _i64, _i32, _i32, _p]),
+    "tnx_dense_expand": (_i32, [_p, _p, _i64, _i64, _p]),
     "tnx_qlinear_lora": (_i32, [_p, C.POINTER(QLinearDesc)]),
     "tnx_splitk_finish": (_i32, [_p, C.POINTER(QLinearDesc)]),
     "tnx_lora_reduce": (_i32, [_p, _p, _i64, _i64, _i32, _p, _i64]),

@@ -488,6 +488,20 @@ __global__ __launch_bounds__(256) void qw_expand_kernel(const uint32_t* codes, c
   }
 }
 
+// The same layout from a dense bf16 matrix w[N][K] (an unquantised or tied lm_head): a permutation.
+__global__ __launch_bounds__(256) void dense_expand_kernel(const uint16_t* w, int64_t K, int64_t N, u32x4* out) {
+  const int ntile = blockIdx.x, kt = blockIdx.y, ktiles = (int)(K / KTILE);
+  const int wn = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  for (int cg = 0; cg < 2; ++cg) {
+    const int64_t col = (int64_t)ntile * 256 + wn * 64 + cg * 32 + l32;
+    for (int u = 0; u < 8; ++u) {
+      u32x4 r = u32x4{0, 0, 0, 0};
+      if (col < N) r = *reinterpret_cast<const u32x4*>(w + col * K + (int64_t)kt * KTILE + u * 16 + lh * 8);
+      out[((((int64_t)ntile * ktiles + kt) * 4 + wn) * 2 + cg) * 512 + u * 64 + lane] = r;
+    }
+  }
+}
+
 QLArgs to_args(const tnx_qlinear_desc* d) {
   QLArgs a;
   a.M = d->M; a.K = d->K; a.N = d->N; a.group = d->group; a.qtype = d->qtype;
@@ -645,6 +659,7 @@ int launch_qgemm_wide(hipStream_t st, const QLArgs& a, const WideHead& h = WideH
   // codes take the instantiation that converts them without the table
   if (a.w_pre && cdiv(a.N, kWideCols) * (a.K / KTILE) * 65536 < (int64_t)1 << 31)
     return launch_qgemm_wide_as<2, kWidePre>(st, a, h);
+  TNX_REQUIRE(a.codes && a.scales, "quantised GEMM: no packed weights and no usable expanded copy");
   return a.qtype == TNX_Q_INT4 ? launch_qgemm_wide_as<SPT, kWideInt4>(st, a, h)
                                : launch_qgemm_wide_as<SPT, kWideTable>(st, a, h);
 }
@@ -822,6 +837,17 @@ extern "C" int tnx_qw_expand(void* stream, const uint32_t* codes, const uint16_t
   return TNX_OK;
 }
 
+extern "C" int tnx_dense_expand(void* stream, const uint16_t* w_bf16, int64_t K, int64_t N, uint16_t* w_expanded) {
+  TNX_REQUIRE(w_bf16 && w_expanded, "dense_expand: null pointer");
+  TNX_REQUIRE(K > 0 && N > 0 && K % KTILE == 0 && K / KTILE <= 65535, "dense_expand: K=%lld must be a positive multiple of 128", (long long)K);
+  TNX_REQUIRE(((uintptr_t)w_expanded & 15) == 0 && ((uintptr_t)w_bf16 & 15) == 0, "dense_expand: pointers must be 16-byte aligned");
+  dim3 grid((unsigned)cdiv(N, kWideCols), (unsigned)(K / KTILE));
+  hipLaunchKernelGGL(dense_expand_kernel, grid, dim3(256), 0, as_stream(stream), w_bf16, K, N,
+                     reinterpret_cast<u32x4*>(w_expanded));
+  TNX_CHECK_LAUNCH("dense_expand");
+  return TNX_OK;
+}
+
 extern "C" int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* d) {
   int rc = check_desc(d);
   if (rc) return rc;
@@ -845,20 +871,28 @@ extern "C" int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* d) {
 // the shape is not one the kernel takes (the caller then uses its own kernel), 0 when launched.
 int tnx_internal_wide_head(hipStream_t st, const tnx_lmhead_desc* d, float temperature, int64_t nvb,
                            float* part_ent) {
-  if (d->w_bf16 || d->logits_out || d->forbidden || d->draw_id || d->logits_fp32) return 1;   // (its tile is staged in bf16)
-  if (d->group < 32 || d->group % 32 != 0 || (d->group <= KTILE ? KTILE % d->group != 0 : d->group % KTILE != 0) ||
-      d->D % d->group != 0)
-    return 1;
-  if ((uint64_t)d->D * (uint64_t)d->V / 2 >= (1ull << 32)) return 1;
+  if (d->logits_out || d->forbidden || d->draw_id || d->logits_fp32) return 1;   // (its tile is staged in bf16)
+  // a dense head comes here only through its expanded copy (tnx_dense_expand)
+  const bool dense = d->w_bf16 != nullptr;
+  const bool pre_ok = d->w_expanded && d->D % KTILE == 0 &&
+                      cdiv(d->V, kWideCols) * (d->D / KTILE) * 65536 < (int64_t)1 << 31;
+  if (dense) {
+    if (!pre_ok || d->V % 16 != 0 || d->lora_rank > 0) return 1;
+  } else {
+    if (d->group < 32 || d->group % 32 != 0 || (d->group <= KTILE ? KTILE % d->group != 0 : d->group % KTILE != 0) ||
+        d->D % d->group != 0)
+      return 1;
+    if ((uint64_t)d->D * (uint64_t)d->V / 2 >= (1ull << 32)) return 1;
+  }
   QLArgs a;
   memset(&a, 0, sizeof(a));
-  a.M = d->M; a.K = d->D; a.N = d->V; a.group = d->group; a.qtype = d->qtype;
+  a.M = d->M; a.K = d->D; a.N = d->V; a.group = dense ? KTILE : d->group; a.qtype = d->qtype;
   a.x = d->x; a.codes = d->codes; a.scales = d->scales;
   a.lora_rank = d->lora_rank; a.lora_nseg = 1; a.lora_seg_end[0] = d->V;
   a.t_ld = d->t_ld; a.t = d->t; a.lora_b = d->lora_b; a.lora_scale = d->lora_scale;
   a.epilogue = TNX_EPI_STORE; a.y = d->part;   // the shape test looks at a stored tile
   a.split_k = 1; a.ktiles_per_split = (int)(d->D / KTILE); a.x_div = 1;
-  a.w_pre = d->w_expanded;
+  a.w_pre = pre_ok ? d->w_expanded : nullptr;
   if (!wide_shape(a)) return 1;
   a.y = nullptr;
   const WideHead h{d->part, part_ent, d->targets, nvb, temperature};

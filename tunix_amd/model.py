@@ -243,12 +243,22 @@ class QLoRAModel:
       ly["rope_scale"] = sf
       self.layers.append(ly)
     torch.cuda.synchronize(dev)
+    # a dense (unquantised or tied) head in the many-row kernel's fragment order, same purpose
+    self.head_expanded = None
+    dense_head = self.head_w if self.head_w is not None else (self.embed if self.head is None else None)
+    head_need = 0
+    if dense_head is not None and cfg.embed_dim % 128 == 0 and cfg.vocab_size % 16 == 0:
+      head_need = int(L.lib().tnx_qw_expanded_bytes(cfg.embed_dim, cfg.vocab_size))
+      if head_need >= (1 << 31):
+        head_need = 0
     if expand_many_rows is None:
-      need = sum(f.expanded_bytes() for f in self._linears() if f.wants_expansion())
+      need = head_need + sum(f.expanded_bytes() for f in self._linears() if f.wants_expansion())
       expand_many_rows = need <= torch.cuda.mem_get_info(dev)[0] // 4
     if expand_many_rows:
       for f in self._linears():
         f.expand()
+      if head_need:
+        self.head_expanded = ops.dense_expand(dense_head)
       torch.cuda.synchronize(dev)
 
   # weight sync: LoRA-only replacement (tunix/generate/sampler.py:333-352)
@@ -349,6 +359,9 @@ class QLoRAModel:
       dst.copy_(src.t() if transpose else src)
     for obj in reloads:
       obj.load_base(base)
+    if self.head_expanded is not None and any(n in ("embed", "lm_head") for _, n, _ in copies):
+      src = self.head_w if self.head_w is not None else self.embed
+      self.head_expanded.copy_(ops.dense_expand(src))
     if lora:
       for f in linears:
         f.load_lora(lora)
@@ -673,6 +686,8 @@ class Runner:
         d.lora_b, d.lora_scale = f.b_t.data_ptr(), f.lora_scale
     else:
       d.w_bf16 = (m.head_w if m.head_w is not None else m.embed).data_ptr()
+      if m.head_expanded is not None:
+        d.w_expanded = m.head_expanded.data_ptr()
     d.temperature = float(temperature)
     d.logits_fp32 = 1 if logits_fp32 else 0
     if forbidden is not None:

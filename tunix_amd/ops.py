@@ -91,6 +91,15 @@ def qw_expand(codes, scales, K, N, group, qtype):
   return out
 
 
+def dense_expand(w):
+  """The same copy for a dense bf16 matrix w [N, K] (an unquantised or tied lm_head [V, D])."""
+  import torch
+  N, K = w.shape
+  out = torch.empty(int(L.lib().tnx_qw_expanded_bytes(K, N)) // 2, dtype=torch.bfloat16, device=w.device)
+  L.check(L.lib().tnx_dense_expand(_stream(), _ptr(w), K, N, _ptr(out)), "tnx_dense_expand")
+  return out
+
+
 def qlinear(desc: L.QLinearDesc, finish: bool = True):
   """finish=False leaves the split-k partial planes in desc.ws for a consumer that sums them
   itself (rmsnorm_splitk)."""
