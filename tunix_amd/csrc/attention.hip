@@ -27,6 +27,7 @@ struct AttnArgs {
   int Hq, Hkv, dh, G, Gp;
   int gp_shift;                // Gp = 1 << gp_shift (the query group padded to a power of two)
   unsigned QT;                 // query tiles per row: ceil(T / (16 / Gp))
+  unsigned QTG;                // (attn_tiles_kernel) groups of QW query tiles per row
   float scale_bf;  // bf16-rounded scale, 0 = none
   int window;
   int32_t pad_id;
@@ -528,6 +529,233 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DH > 128 ? 2
   }
 }
 
+// Many query positions per row (prefill, whole-sequence log-probability passes): the wave above
+// loads 16 KB of keys and values per 32-key block for sixteen MFMAs, i.e. it runs at what a
+// compute unit can draw from L2, not at its matrix rate.  This form gives one wave QW
+// consecutive query tiles: every loaded block, and the in-lane transposition of its value rows,
+// serves QW x 16 query columns.  Each tile sees the same 32-key blocks in the same order with
+// the same arithmetic as it would in a wave of its own (a block wholly before a tile's window
+// or after its causal limit leaves its running maximum, sum and output untouched: p = 0,
+// alpha = exp(0)), so results are bit-identical to the kernel above.  No fused rotation, no key
+// split (those are decode modes).
+template <int DH, bool TOKVEC, int QW>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void attn_tiles_kernel(const AttnArgs a) {
+  constexpr int KS = DH / 32;
+  constexpr int NH = DH > 128 ? DH / 128 : 1;
+  constexpr int NS = 2;
+  const int lane = threadIdx.x, lm = lane & 15, lq = lane >> 4;
+  const int hkv = blockIdx.y;
+  const int PT = 16 >> a.gp_shift;
+  const unsigned bz = blockIdx.z;
+  const int64_t b = bz / a.QTG;
+  // (the longest tiles of a row are handed out first: a tile's work grows with its position)
+  const int qt0 = ((int)a.QTG - 1 - (int)(bz - (unsigned)b * a.QTG)) * QW;
+  const int col0 = *a.col_ptr;
+  const int g = lm & (a.Gp - 1);
+
+  int c_n[QW], lo_n[QW];
+  bool qvalid[QW];
+  u32x4 qf[QW][KS];
+#pragma unroll
+  for (int w = 0; w < QW; ++w) {
+    const int tq = (qt0 + w) * PT + (lm >> a.gp_shift);
+    qvalid[w] = g < a.G && tq < a.T;
+    c_n[w] = col0 + tq;
+    lo_n[w] = a.window > 0 ? max(0, c_n[w] - a.window + 1) : 0;
+    const int64_t qvec = (b * a.T + (qvalid[w] ? tq : 0)) * a.Hq + hkv * a.G + (qvalid[w] ? g : 0);
+#pragma unroll
+    for (int j = 0; j < KS; ++j) {
+      qf[w][j] = u32x4{0, 0, 0, 0};
+      if (qvalid[w]) qf[w][j] = *reinterpret_cast<const u32x4*>(a.q + qvec * DH + j * 32 + lq * 8);
+    }
+  }
+  // key range of the QW tiles together
+  const int t_last = min((int)a.T - 1, (qt0 + QW) * PT - 1);
+  const int k_hi = col0 + t_last;
+  const int k_lo = a.window > 0 ? max(0, col0 + qt0 * PT - a.window + 1) : 0;
+
+  f32x4 O[QW][NH][8];
+  float m_run[QW], l_run[QW];
+#pragma unroll
+  for (int w = 0; w < QW; ++w) {
+    m_run[w] = kNegBig;
+    l_run[w] = 0.f;
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) O[w][h][jj] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const uint16_t* kbase = a.k + ((b * a.Hkv + hkv) * a.S) * DH;
+  const uint16_t* vbase = a.v + ((b * a.Hkv + hkv) * a.S) * DH;
+  const int32_t* tok = a.tokens + b * a.tok_ld;
+  int32_t id_ref[QW];
+  const bool id_equal = a.seg_mode != 0;
+  const int vcol = (8 * lm) % (DH < 128 ? DH : 128);
+  struct Stage {
+    u32x4 kf[2][KS];
+    u32x4 vf[NH][8];
+    int tk[8];
+  };
+  const uint32_t slab_bytes = (uint32_t)a.S * DH * 2u;
+  const rsrc_t rk = make_rsrc(kbase, slab_bytes), rv = make_rsrc(vbase, slab_bytes);
+  const rsrc_t rtok = make_rsrc(tok, (uint64_t)min(a.S, a.tok_ld) * 4);
+  const uint32_t koff = (uint32_t)(lm * DH + lq * 8) * 2u;
+  const uint32_t voff = (uint32_t)(4 * lq * DH + vcol) * 2u;
+  // (the blocks are re-read by the waves of the later tiles of this row: default cache policy)
+  auto load_block = [&](int kb, Stage& sg) {
+    const uint32_t kb_bytes = (uint32_t)kb * (DH * 2u);
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      const uint32_t o = koff + kb_bytes + (uint32_t)(tt * 16 * DH * 2);
+#pragma unroll
+      for (int j = 0; j < KS; ++j) sg.kf[tt][j] = __builtin_amdgcn_raw_buffer_load_b128(rk, o + (uint32_t)(j * 64), 0, 0);
+    }
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const uint32_t o = voff + kb_bytes + (uint32_t)(((s < 4 ? s : 12 + s)) * DH * 2);
+#pragma unroll
+      for (int h = 0; h < NH; ++h) sg.vf[h][s] = __builtin_amdgcn_raw_buffer_load_b128(rv, o + (uint32_t)(h * 256), 0, 0);
+    }
+    if constexpr (TOKVEC) {
+      const u32x4 t0 = __builtin_amdgcn_raw_buffer_load_b128(rtok, (uint32_t)(kb + 4 * lq) * 4u, 0, 0);
+      const u32x4 t1 = __builtin_amdgcn_raw_buffer_load_b128(rtok, (uint32_t)(kb + 16 + 4 * lq) * 4u, 0, 0);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        sg.tk[s] = (int)t0[s];
+        sg.tk[4 + s] = (int)t1[s];
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < 8; ++s)
+        sg.tk[s] = (int)__builtin_amdgcn_raw_buffer_load_b32(
+            rtok, (uint32_t)(kb + (s < 4 ? 4 * lq + s : 16 + 4 * lq + (s - 4))) * 4u, 0, 0);
+    }
+  };
+  auto compute_block = [&](int kb, const Stage& sg) {
+    u32x4 pa[QW];
+#pragma unroll
+    for (int w = 0; w < QW; ++w) {
+      bool kvalid[8];
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        const int key = kb + (s < 4 ? 4 * lq + s : 16 + 4 * lq + (s - 4));
+        kvalid[s] = qvalid[w] && key >= max(k_lo, lo_n[w]) && key <= min(k_hi, c_n[w]) &&
+                    ((sg.tk[s] == id_ref[w]) == id_equal);
+      }
+      f32x4 st[2];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        st[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < KS; ++j) st[tt] = mfma16(sg.kf[tt][j], qf[w][j], st[tt]);
+      }
+      float sv[8];
+      float bmax = kNegBig;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        float x = rbf(st[s >> 2][s & 3]);
+        if (a.scale_bf != 0.f) x = rbf(x * a.scale_bf);
+        sv[s] = x;
+        if (kvalid[s]) bmax = fmaxf(bmax, x);
+      }
+      bmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
+      bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+      const float m_new = fmaxf(m_run[w], bmax);
+      const float alpha = __expf(m_run[w] - m_new);
+      m_run[w] = m_new;
+      float p[8], psum = 0.f;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        p[s] = kvalid[s] ? __expf(sv[s] - m_new) : 0.f;
+        psum += p[s];
+      }
+      l_run[w] = l_run[w] * alpha + psum;
+      pa[w][0] = pack2bf(p[0], p[1]);
+      pa[w][1] = pack2bf(p[2], p[3]);
+      pa[w][2] = pack2bf(p[4], p[5]);
+      pa[w][3] = pack2bf(p[6], p[7]);
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+        float ar[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ar[i] = __shfl(alpha, 4 * lq + i, 64);
+#pragma unroll
+        for (int h = 0; h < NH; ++h)
+#pragma unroll
+          for (int jj = 0; jj < 8; ++jj)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) O[w][h][jj][i] *= ar[i];
+      }
+    }
+    // O += P . V: a value fragment is transposed once and multiplied with every tile's P
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) {
+        const uint32_t sel = (jj & 1) ? 0x07060302u : 0x05040100u;
+        u32x4 bfrag;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          bfrag[r] = __builtin_amdgcn_perm(sg.vf[h][2 * r + 1][jj >> 1], sg.vf[h][2 * r][jj >> 1], sel);
+#pragma unroll
+        for (int w = 0; w < QW; ++w) O[w][h][jj] = mfma16(pa[w], bfrag, O[w][h][jj]);
+      }
+  };
+  {
+    Stage sg[NS];
+    const int kb0 = k_lo & ~31;
+    const int kb_last = k_hi & ~31;
+    const bool any = kb0 <= k_hi;
+#pragma unroll
+    for (int u = 0; u < NS - 1; ++u) load_block(min(kb0 + 32 * u, kb_last), sg[u]);
+#pragma unroll
+    for (int w = 0; w < QW; ++w) {
+      const int32_t id_q = tok[min((int64_t)c_n[w], a.tok_ld - 1)];
+      id_ref[w] = a.seg_mode ? id_q : a.pad_id;
+    }
+    if (any) {
+      const int nblk = ((kb_last - kb0) >> 5) + 1;
+      int i = 0;
+      for (; i + NS <= nblk; i += NS) {
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+          const int kbu = kb0 + 32 * (i + u);
+          load_block(min(kbu + 32 * (NS - 1), kb_last), sg[(u + NS - 1) % NS]);
+          __builtin_amdgcn_sched_barrier(0);
+          compute_block(kbu, sg[u]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < NS - 1; ++u)
+        if (i + u < nblk) compute_block(kb0 + 32 * (i + u), sg[u]);
+    }
+  }
+  const bool dvalid = 8 * lm < (DH < 128 ? DH : 128);
+#pragma unroll
+  for (int w = 0; w < QW; ++w) {
+    float lr = l_run[w];
+    lr += __shfl_xor(lr, 16, 64);
+    lr += __shfl_xor(lr, 32, 64);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = 4 * lq + i;
+      const float l = __shfl(lr, n, 64);
+      const int gi = n & (a.Gp - 1), ti = (qt0 + w) * PT + (n >> a.gp_shift);
+      if (!(gi < a.G && ti < a.T) || !dvalid) continue;
+      const float inv = l > 0.f ? 1.0f / l : 0.f;
+      uint16_t* o = a.out + ((b * a.T + ti) * a.Hq + hkv * a.G + gi) * DH;
+#pragma unroll
+      for (int h = 0; h < NH; ++h) {
+        u32x4 wv;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          wv[r] = pack2bf(O[w][h][2 * r][i] * inv, O[w][h][2 * r + 1][i] * inv);
+        *reinterpret_cast<u32x4*>(o + h * 128 + 8 * lm) = wv;
+      }
+    }
+  }
+}
+
 // out[qv, d] = bf16( sum_c e^{m_c - M} O_c[d] / sum_c e^{m_c - M} l_c )
 // The (m, l) pairs of all chunks are fetched at once into LDS (one round trip instead of one
 // dependent load per chunk and pass); every thread then forms M, the weights and the sums in
@@ -597,6 +825,7 @@ extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
   a.gp_shift = 0;
   while ((1 << a.gp_shift) < a.Gp) ++a.gp_shift;
   a.QT = (unsigned)cdiv(d->T, 16 / a.Gp);
+  a.QTG = 1;
   // bf16(scale), as a weak-typed python float multiplied into a bf16 array
   if (d->scale != 0.f) {
     uint32_t u; float f = d->scale; memcpy(&u, &f, 4);
@@ -635,6 +864,21 @@ extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
     if (tv) hipLaunchKernelGGL((attn_kernel<DH, FUSE, true>), grid, dim3(64), 0, st, a);         \
     else hipLaunchKernelGGL((attn_kernel<DH, FUSE, false>), grid, dim3(64), 0, st, a);           \
   } while (0)
+  // many query positions, no key split, no fused rotation: four query tiles per wave
+  constexpr int kTilesPerWave = 2;
+  if (!a.rope_sin && a.n_chunks == 1 && d->dh <= 128 && QT >= 2 * kTilesPerWave) {
+    a.QTG = (unsigned)cdiv(QT, kTilesPerWave);
+    dim3 tgrid(1u, (unsigned)d->Hkv, (unsigned)(d->B * a.QTG));
+    if (d->dh == 64) {
+      if (tv) hipLaunchKernelGGL((attn_tiles_kernel<64, true, kTilesPerWave>), tgrid, dim3(64), 0, st, a);
+      else hipLaunchKernelGGL((attn_tiles_kernel<64, false, kTilesPerWave>), tgrid, dim3(64), 0, st, a);
+    } else {
+      if (tv) hipLaunchKernelGGL((attn_tiles_kernel<128, true, kTilesPerWave>), tgrid, dim3(64), 0, st, a);
+      else hipLaunchKernelGGL((attn_tiles_kernel<128, false, kTilesPerWave>), tgrid, dim3(64), 0, st, a);
+    }
+    TNX_CHECK_LAUNCH("gqa_attn (tiles)");
+    return TNX_OK;
+  }
   switch (d->dh) {
     case 64: TNX_ATTN_LAUNCH(64, 0); break;
     case 128:
