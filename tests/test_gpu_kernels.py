@@ -1373,6 +1373,46 @@ def test_attention_with_fused_rope_equals_rope_then_attention(gpu, kv_chunk, win
   assert (d <= ulp).all(), (d.max().item(), (d / ulp).max().item())
 
 
+@pytest.mark.parametrize("family,dh,Hq,Hkv", [("llama3", 128, 8, 2), ("gemma3", 256, 4, 1), ("qwen3", 64, 6, 3)])
+def test_rope_row_kernel_equals_the_per_head_kernel(gpu, family, dh, Hq, Hkv):
+  """Rotation + cache write without q / k norm at many rows (512 in one call: the row kernel, 16-byte
+  accesses, one sine / cosine per (row, i) for all heads) against the same rows in calls of 128
+  (the per-head kernel): q and both caches bit for bit."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  from tunix_amd.model import _ROPE, rope_timescale
+  B, T, S, col = 4, 128, 160, 9
+  ld = (Hq + 2 * Hkv) * dh
+  g = torch.Generator().manual_seed(96)
+  qkv = torch.randn(B, T, ld, generator=g).to(torch.bfloat16).to(gpu)
+  pos = torch.randint(0, 2000, (B, S), generator=g, dtype=torch.int32).to(gpu)
+  ts = torch.from_numpy(rope_timescale(dh, 1e6)).to(gpu)
+  colp = torch.tensor([col], dtype=torch.int32, device=gpu)
+
+  def run(rows_per_call):
+    q = torch.zeros(B, T, Hq * dh, dtype=torch.bfloat16, device=gpu)
+    kc = torch.zeros(B, Hkv, S, dh, dtype=torch.bfloat16, device=gpu)
+    vc = torch.zeros_like(kc)
+    for b0 in range(0, B, rows_per_call):
+      nb = min(rows_per_call, B - b0)
+      rd = L.RopeDesc()
+      rd.B, rd.T, rd.S, rd.Hq, rd.Hkv, rd.dh = nb, T, S, Hq, Hkv, dh
+      rd.rope_flavor, rd.rope_scale, rd.timescale, rd.qk_norm = _ROPE[family], 8.0 if family == "gemma3" else 1.0, ts.data_ptr(), -1
+      rd.q_prescale = dh ** -0.5 if family == "gemma3" else 0.0
+      rd.qkv, rd.positions, rd.pos_ld, rd.col_ptr = qkv[b0:].data_ptr(), pos[b0:].data_ptr(), S, colp.data_ptr()
+      rd.q_out, rd.kcache, rd.vcache = q[b0:].data_ptr(), kc[b0:].data_ptr(), vc[b0:].data_ptr()
+      ops.rope_kvwrite(rd)
+    torch.cuda.synchronize()
+    return q, kc, vc
+
+  one = run(B)        # 512 rows in one call
+  four = run(1)       # 128 rows per call
+  for name, x, y in zip(("q", "k cache", "v cache"), one, four):
+    diff = (x.float() - y.float()).abs()
+    assert torch.equal(x, y), (name, int((diff > 0).sum()), diff.max().item(), torch.nonzero(diff > 0)[:4].tolist())
+  assert one[0].float().abs().max() > 0.1 and one[1][:, :, col: col + T].float().abs().max() > 0.5
+
+
 @pytest.mark.parametrize("family", ["llama3", "qwen3"])
 def test_rope_from_splitk_planes_equals_finish_then_rope(gpu, family):
   """The rope / cache-write kernel fed with the partial planes of a split-k qkv linear against

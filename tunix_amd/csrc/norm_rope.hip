@@ -433,6 +433,73 @@ __global__ void rope_kernel(const RopeArgs a) {
   }
 }
 
+// Many rows, no q / k norm (a Llama prefill or whole-sequence pass): one work-group per token row,
+// 16-byte accesses, and the sine / cosine of a (row, i) computed once for all heads instead of
+// once per head.  Thread (ch, h0) owns the eight pairs i = 8 ch .. + 7 of heads h0, h0 + hstep, ...;
+// the arithmetic per element is rope_kernel's, so the outputs are bit-identical.
+__global__ __launch_bounds__(256) void rope_rows_kernel(const RopeArgs a) {
+  const int64_t row = blockIdx.x;
+  const int64_t b = row / a.T, t = row % a.T;
+  const int half = a.dh / 2, CH = half / 8, heads = a.Hq + 2 * a.Hkv;
+  const int ch = threadIdx.x % CH, h0 = threadIdx.x / CH, hstep = 256 / CH;
+  const int col = *a.col_ptr;
+  const int ld = heads * a.dh;
+  const int slot = (int)((col + t) % a.S);
+  const int i0 = ch * 8;
+  const float pos = (float)a.positions[b * a.pos_ld + col + t];
+  float sn[8], cs[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float ang = __fdiv_rn(pos, a.timescale[i0 + e]);
+    if (a.rope_flavor == TNX_ROPE_GEMMA3) ang = __fdiv_rn(ang, a.rope_scale);
+    sn[e] = sinf(ang);
+    cs[e] = cosf(ang);
+    if (a.rope_flavor == TNX_ROPE_QWEN3) {
+      sn[e] = rbf(sn[e]);
+      cs[e] = rbf(cs[e]);
+    }
+  }
+  for (int head = h0; head < heads; head += hstep) {
+    const uint16_t* src = a.qkv + row * ld + (int64_t)head * a.dh + i0;
+    const u32x4 v1 = *reinterpret_cast<const u32x4*>(src), v2 = *reinterpret_cast<const u32x4*>(src + half);
+    uint16_t* dst;
+    if (head >= a.Hq + a.Hkv) {   // V: plain copy into the cache slot
+      dst = a.vcache + (((b * a.Hkv + (head - a.Hq - a.Hkv)) * a.S) + slot) * a.dh + i0;
+      *reinterpret_cast<u32x4*>(dst) = v1;
+      *reinterpret_cast<u32x4*>(dst + half) = v2;
+      continue;
+    }
+    const bool is_q = head < a.Hq;
+    u32x4 o1v, o2v;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float o1[2], o2[2];
+#pragma unroll
+      for (int hsel = 0; hsel < 2; ++hsel) {
+        const int e = 2 * r + hsel;
+        const float x1 = hsel ? bfhi(v1[r]) : bflo(v1[r]), x2 = hsel ? bfhi(v2[r]) : bflo(v2[r]);
+        if (a.rope_flavor == TNX_ROPE_QWEN3) {
+          o1[hsel] = rbf(rbf(x1 * cs[e]) - rbf(x2 * sn[e]));
+          o2[hsel] = rbf(rbf(x2 * cs[e]) + rbf(x1 * sn[e]));
+        } else {
+          o1[hsel] = rbf(__fsub_rn(__fmul_rn(x1, cs[e]), __fmul_rn(x2, sn[e])));
+          o2[hsel] = rbf(__fadd_rn(__fmul_rn(x2, cs[e]), __fmul_rn(x1, sn[e])));
+        }
+        if (is_q && a.q_prescale_bf != 0.f) {
+          o1[hsel] = rbf(o1[hsel] * a.q_prescale_bf);
+          o2[hsel] = rbf(o2[hsel] * a.q_prescale_bf);
+        }
+      }
+      o1v[r] = pack2bf(o1[0], o1[1]);
+      o2v[r] = pack2bf(o2[0], o2[1]);
+    }
+    if (is_q) dst = a.q_out + (row * a.Hq + head) * a.dh + i0;
+    else dst = a.kcache + (((b * a.Hkv + (head - a.Hq)) * a.S) + slot) * a.dh + i0;
+    *reinterpret_cast<u32x4*>(dst) = o1v;
+    *reinterpret_cast<u32x4*>(dst + half) = o2v;
+  }
+}
+
 // sin / cos of angle = position / timescale[i] for the token in column *col_ptr of every row: the
 // values rope_kernel computes for the Llama rotation, once per decode step instead of per layer.
 __global__ void rope_table_kernel(const int32_t* positions, int64_t pos_ld, const int32_t* col_ptr,
@@ -561,6 +628,15 @@ extern "C" int tnx_qknorm_rope_kvwrite(void* stream, const tnx_rope_desc* d) {
   a.qkv = d->qkv; a.positions = d->positions; a.pos_ld = d->pos_ld; a.col_ptr = d->col_ptr;
   a.timescale = d->timescale; a.q_out = d->q_out; a.kcache = d->kcache; a.vcache = d->vcache;
   a.ws = d->qkv_ws; a.split_k = d->split_k;
+  // many rows of a model without q / k norm, from the finished linear output: the row kernel
+  const int chunks = d->dh / 16;
+  const bool aligned = (((uintptr_t)d->qkv | (uintptr_t)d->q_out | (uintptr_t)d->kcache | (uintptr_t)d->vcache) & 15) == 0;
+  if (d->qk_norm < 0 && !d->qkv_ws && d->B * d->T >= 256 && d->dh % 16 == 0 && chunks <= 256 && 256 % chunks == 0 &&
+      aligned) {
+    hipLaunchKernelGGL(rope_rows_kernel, dim3((unsigned)(d->B * d->T)), dim3(256), 0, as_stream(stream), a);
+    TNX_CHECK_LAUNCH("qknorm_rope_kvwrite (rows)");
+    return TNX_OK;
+  }
   dim3 grid((unsigned)(d->B * d->T), (unsigned)(d->Hq + 2 * d->Hkv));
   hipLaunchKernelGGL(rope_kernel, grid, dim3(d->dh / 2 < 64 ? 64 : d->dh / 2), 0, as_stream(stream), a);
   TNX_CHECK_LAUNCH("qknorm_rope_kvwrite");
