@@ -565,6 +565,23 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
         }
   }
   __syncthreads();
+  if (h.part != nullptr && h.logits_out != nullptr) {
+    // the raw logits (no temperature) as fp32: a wave writes one row of the tile at a time, a
+    // lane four columns (1 KB per row, whole lines)
+    const int64_t c0 = (int64_t)ntile * kWideCols + lane * 4;
+    for (int row = wn; row < rows_here; row += 4) {
+      const u32x2 v = *reinterpret_cast<const __attribute__((address_space(3))) u32x2*>(
+          static_cast<uintptr_t>(stage + (uint32_t)((row * sld + lane * 4) * 2)));
+      float* o = h.logits_out + (m0 + row) * a.N + c0;
+      if (c0 + 4 <= a.N) {
+        *reinterpret_cast<f32x4*>(o) = f32x4{bflo(v[0]), bfhi(v[0]), bflo(v[1]), bfhi(v[1])};
+      } else {
+        const float x[4] = {bflo(v[0]), bfhi(v[0]), bflo(v[1]), bfhi(v[1])};
+        for (int e = 0; e < 4; ++e)
+          if (c0 + e < a.N) o[e] = x[e];
+      }
+    }
+  }
   if (h.part != nullptr) {
     // lm_head: thread (row, half) reduces the row's 128 staged logits of column block
     // 2 * ntile + half to (max, first arg-max, sum of exp(l - max), logit of the row's target)

@@ -49,6 +49,7 @@ struct WideHead {
   const int32_t* targets;    // optional [M]
   int64_t nvb;               // 128-column blocks of the vocabulary
   float temperature;
+  float* logits_out;         // optional fp32 [M, N]: the raw logits (the staged bf16 values), or null
 };
 
 __device__ __forceinline__ float silu_bf16(float g) {
@@ -654,7 +655,7 @@ int launch_qgemm_wide_as(hipStream_t st, const QLArgs& a, const WideHead& h) {
 }
 
 template <int SPT>
-int launch_qgemm_wide(hipStream_t st, const QLArgs& a, const WideHead& h = WideHead{nullptr, nullptr, nullptr, 0, 1.0f}) {
+int launch_qgemm_wide(hipStream_t st, const QLArgs& a, const WideHead& h = WideHead{nullptr, nullptr, nullptr, 0, 1.0f, nullptr}) {
   // the converted copy when the caller keeps one (its block offsets are 32-bit); else integer
   // codes take the instantiation that converts them without the table
   if (a.w_pre && cdiv(a.N, kWideCols) * (a.K / KTILE) * 65536 < (int64_t)1 << 31)
@@ -675,7 +676,7 @@ int launch_qgemm_wide_grouped_as(hipStream_t st, const QLArgs& a) {
   const int64_t blocks = a.M / kWideRows + a.n_experts;
   const unsigned wgs = (unsigned)(blocks * cdiv(a.N, kWideCols));
   hipLaunchKernelGGL((qgemm_wide_kernel<SPT, true, INT4 ? kWideInt4 : kWideTable>), dim3(wgs), dim3(256), kWideSmemBytes, st, a,
-                     WideHead{nullptr, nullptr, nullptr, 0, 1.0f});
+                     WideHead{nullptr, nullptr, nullptr, 0, 1.0f, nullptr});
   TNX_CHECK_LAUNCH("qgemm_wide_grouped");
   return TNX_OK;
 }
@@ -688,8 +689,8 @@ int launch_qgemm_wide_grouped(hipStream_t st, const QLArgs& a) {
 // Shapes the 128 x 256 kernel takes: enough rows to fill the device with its tiles, no k split,
 // a bf16 output whose rows can be written in 16-byte chunks, and an adapter (if any) of rank
 // <= 64 none of whose 256-column windows touches more than two segments.
-bool wide_shape(const QLArgs& a) {
-  if (a.split_k > 1 || a.next_tpart || a.M < 512) return false;
+bool wide_shape(const QLArgs& a, int64_t min_rows = 512) {
+  if (a.split_k > 1 || a.next_tpart || a.M < min_rows) return false;
   if (cdiv(a.M, kWideRows) * cdiv(a.N, kWideCols) < 256) return false;
   const bool mul = a.epilogue == TNX_EPI_SILU_MUL || a.epilogue == TNX_EPI_GELU_MUL;
   if (!mul && a.epilogue != TNX_EPI_STORE && a.epilogue != TNX_EPI_RESIDUAL) return false;
@@ -871,7 +872,7 @@ extern "C" int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* d) {
 // the shape is not one the kernel takes (the caller then uses its own kernel), 0 when launched.
 int tnx_internal_wide_head(hipStream_t st, const tnx_lmhead_desc* d, float temperature, int64_t nvb,
                            float* part_ent) {
-  if (d->logits_out || d->forbidden || d->draw_id || d->logits_fp32) return 1;   // (its tile is staged in bf16)
+  if (d->forbidden || d->draw_id || d->logits_fp32) return 1;   // (its tile is staged in bf16)
   // a dense head comes here only through its expanded copy (tnx_dense_expand)
   const bool dense = d->w_bf16 != nullptr;
   const bool pre_ok = d->w_expanded && d->D % KTILE == 0 &&
@@ -893,9 +894,12 @@ int tnx_internal_wide_head(hipStream_t st, const tnx_lmhead_desc* d, float tempe
   a.epilogue = TNX_EPI_STORE; a.y = d->part;   // the shape test looks at a stored tile
   a.split_k = 1; a.ktiles_per_split = (int)(d->D / KTILE); a.x_div = 1;
   a.w_pre = pre_ok ? d->w_expanded : nullptr;
-  if (!wide_shape(a)) return 1;
+  // A dense head's copy is streamed at any row count: at a decode batch the launch is bound by
+  // the weight stream, and this kernel re-reads the activations once per 256 columns where the
+  // 128 x 128 head kernel re-reads them once per 128, as many bytes again as the weights.
+  if (!wide_shape(a, dense ? 1 : 512)) return 1;
   a.y = nullptr;
-  const WideHead h{d->part, part_ent, d->targets, nvb, temperature};
+  const WideHead h{d->part, part_ent, d->targets, nvb, temperature, d->logits_out};
   return scales_per_tile(a.group) == 2 ? launch_qgemm_wide<2>(st, a, h) : launch_qgemm_wide<4>(st, a, h);
 }
 
