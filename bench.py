@@ -312,16 +312,16 @@ def write_fused_traffic_profile(fetch_csv, write_csv):
   rows, D, V, r = 16384, 4096, 128256, 64
   rec = {
       "kernel": "qgemm_wide_kernel (head-statistics epilogue)",
-      "workload": "one launch of the standalone log-probability pass: 16384 rows x 4096 -> 128256, int4 g128 + LoRA r64",
+      "workload": "one launch of the standalone log-probability pass: 16384 rows x 4096 -> 128256, int4 g128 + LoRA r64, "
+                  "the head read from its expanded bf16 copy",
       "kernel_source_sha256_16": source_hash(FUSED_KERNEL_SOURCES),
       "kernel_sources": list(FUSED_KERNEL_SOURCES),
       "fetch_counter_factor": factor, "write_counter_factor": 1.0,
       "dispatches": {"fetch_run": nf, "write_run": nw},
       "counter_kib_per_launch": {"FETCH_SIZE": round(fk, 1), "WRITE_SIZE": round(wk, 1)},
       "read_bytes_per_launch": int(fk * 1024 * factor), "write_bytes_per_launch": int(wk * 1024),
-      # what one launch must move: hidden rows + packed head + adapter once, statistics out
-      "algorithmic_bytes_per_launch": int(rows * D * 2 + D * V // 2 + (D // 128) * V * 2 + V * r * 2 + rows * r * 2
-                                          + rows * (V // 128) * 16),
+      # what one launch must move: hidden rows + the head's bf16 copy + adapter once, statistics out
+      "algorithmic_bytes_per_launch": int(rows * D * 2 + D * V * 2 + V * r * 2 + rows * r * 2 + rows * (V // 128) * 16),
   }
   with open(FUSED_TRAFFIC_PROFILE, "w") as f:
     json.dump(rec, f, indent=1)
@@ -452,11 +452,13 @@ def summarize_counters(path):
     print(line)
 
 
-def fused_logps_workload(rows, chunk, iters):
+def fused_logps_workload(rows, chunk, iters, expanded=True):
   """The standalone per-token log-probability case at training scale: hidden states
   [rows, 4096] bf16 N(0,1) x an int4 (group 128) + LoRA r64 lm_head of 128256 columns ->
   log-softmax -> gather at random targets -> GRPO clipped ratio; logits never reach HBM.
-  Timed with HIP events around `iters` passes after one warm-up pass."""
+  expanded: the kernel reads the frozen head from its converted copy (tnx_qw_expand, what
+  QLoRAModel keeps for its many-row calls; same bits as converting the codes in the loop, which
+  expanded=False measures).  Timed with HIP events around `iters` passes after one warm-up pass."""
   import torch
   from tunix_amd import _lib as L
   from tunix_amd import ops
@@ -470,6 +472,7 @@ def fused_logps_workload(rows, chunk, iters):
   targets = torch.randint(0, V, (rows,), generator=g, device=dev, dtype=torch.int32)
   codes, scales = ops.quantize_pack(w, group, 0)
   del w
+  w_exp = ops.qw_expand(codes, scales, D, V, group, 0) if expanded else None
   t = torch.zeros(rows, r, dtype=torch.bfloat16, device=dev)
   nvb = ops.lmhead_nblocks(V)
   part = torch.empty(chunk * nvb * 4, dtype=torch.float32, device=dev)
@@ -486,6 +489,8 @@ def fused_logps_workload(rows, chunk, iters):
       d.x, d.codes, d.scales, d.group, d.qtype = x[r0:].data_ptr(), codes.data_ptr(), scales.data_ptr(), group, 0
       d.lora_rank, d.t, d.t_ld, d.lora_b, d.lora_scale = r, t[r0:].data_ptr(), r, b_t.data_ptr(), 1.0
       d.temperature = 1.0
+      if w_exp is not None:
+        d.w_expanded = w_exp.data_ptr()
       d.targets, d.part, d.target_logp = targets[r0:].data_ptr(), part.data_ptr(), logp[r0:].data_ptr()
       ops.lmhead(d)
     ops.grpo_ratio(logp, ref, adv, min(4096, rows), 0.2, 0.2, ratio=ratio, loss=loss)
@@ -502,19 +507,20 @@ def fused_logps_workload(rows, chunk, iters):
   ms = e0.elapsed_time(e1) / iters
   flops = 2.0 * rows * D * V + 2.0 * rows * r * (D + V)
   assert bool(torch.isfinite(logp).all()) and bool(torch.isfinite(loss).all())
-  del x, codes, scales, b_t, part
+  del x, codes, scales, b_t, part, w_exp
   torch.cuda.empty_cache()
   return {
       "metric": "fused per-token logps rows/sec @1 MI355X (int4 g128 + LoRA r64 head, 4096 x 128256)",
       "value": round(rows / (ms * 1e-3), 1), "unit": "rows/s", "n_gpus": 1, "steps": iters, "warmup": 1,
       "ms_per_step": round(ms, 3), "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
       "config": {"workload": "standalone fused lm_head -> log-softmax -> gather -> GRPO ratio", "rows": rows,
-                 "rows_per_launch": chunk},
+                 "rows_per_launch": chunk,
+                 "head_operand": "expanded bf16 copy of the int4 head" if expanded else "int4 codes converted in the loop"},
       "roofline": {"kernel": "qgemm_wide_kernel (statistics epilogue)", "bound": "mfma",
                    "achieved": round(flops / (ms * 1e-3) / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                    "frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                    # HBM bytes of one 16384-row launch, from the tracked counter record
-                   "traffic": fused_measured_traffic() if chunk == 16384 else None}}
+                   "traffic": fused_measured_traffic() if chunk == 16384 and expanded else None}}
 
 
 def config_workload(name, steps):
@@ -595,6 +601,9 @@ def main():
                   help="instead of the decode benchmark: the standalone fused per-token log-probability "
                        "workload (32 x 4096 rows, quantised 128256-column head), its own JSON line")
   ap.add_argument("--fused-logps-rows", type=int, default=131072)
+  ap.add_argument("--fused-logps-codes", action="store_true",
+                  help="the log-probability workload converts the head's int4 codes in its loop "
+                       "instead of reading the head's expanded copy")
   ap.add_argument("--no-fused-logps", action="store_true",
                   help="leave the standalone log-probability workload out of the default run's line")
   ap.add_argument("--config", choices=["c1", "c2", "c3", "c4"], default="c3",
@@ -617,7 +626,8 @@ def main():
   if args.fused_logps:
     if args.gpus != 1:
       sys.exit("bench.py measures one GPU; --gpus must be 1")
-    print(json.dumps(fused_logps_workload(args.fused_logps_rows, 16384, max(1, args.kernel_iters // 10))), flush=True)
+    print(json.dumps(fused_logps_workload(args.fused_logps_rows, 16384, max(1, args.kernel_iters // 10),
+                                          expanded=not args.fused_logps_codes)), flush=True)
     return
   if args.summarize_trace:
     summarize_step_trace(args.summarize_trace)
@@ -855,7 +865,7 @@ def main():
   if not args.no_fused_logps:
     del sampler, st, runner, graph
     torch.cuda.empty_cache()
-    fl = fused_logps_workload(args.fused_logps_rows, 16384, 2)
+    fl = fused_logps_workload(args.fused_logps_rows, 16384, 2, expanded=not args.fused_logps_codes)
     result["fused_logps"] = {k: fl[k] for k in ("metric", "value", "unit", "ms_per_step", "config", "roofline")}
     log(f"fused logps: {fl['ms_per_step']} ms per pass over {args.fused_logps_rows} rows, {fl['roofline']['achieved']} TFLOP/s")
   if not args.no_cpu_baseline:

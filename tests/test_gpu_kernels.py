@@ -206,9 +206,9 @@ def test_qlinear_lora_matches_oracle(gpu, M, K, N, group, qtype, r, split):
     (520, 128, 13440, 32, Q.INT4, 0, None, "residual"),
     (515, 640, 16896, 32, Q.INT4, 0, None, "gelu"),
     (1100, 256, 7424, 64, Q.INT4, 64, None, "store"),
-    # 40 row blocks: one full group of 32 of the work-group id -> tile map and a ragged one of 8
-    (5000, 128, 2048, 64, Q.INT4, 0, None, "store"),
-    (4200, 128, 2304, 64, Q.NF4, 16, None, "store"),
+    # 71 / 66 row blocks: one full group of 64 of the work-group id -> tile map and a ragged one
+    (9000, 128, 2048, 64, Q.INT4, 0, None, "store"),
+    (8400, 128, 2304, 64, Q.NF4, 16, None, "store"),
 ])
 def test_qlinear_many_rows_matches_oracle(gpu, M, K, N, group, qtype, r, seg_widths, epi):
   """Row counts that go to the 128 x 256-tile kernel (prefill, per-token logps): every epilogue,
@@ -691,6 +691,16 @@ def test_lmhead_many_rows_quantized_head(gpu, M, D, V, group, qtype, r, entropy)
   np.testing.assert_allclose(blp.cpu().numpy(), (got.max(-1).values - ref_lse).numpy(), atol=2e-5)
   if entropy:
     np.testing.assert_allclose(ent.cpu().numpy(), rl_ref.compute_entropy_from_logits(got).numpy(), rtol=0, atol=5e-5)
+  # the same head read from its converted copy (two work-groups per compute unit): same bits
+  first = [v.clone() for v in (best, blp, tlp, lse, ent if entropy else lse)]
+  for v in (blp, tlp, lse, ent, part, pent):
+    v.fill_(float("nan"))
+  w_exp = ops.qw_expand(c, s, D, V, group, qtype)
+  d.w_expanded = w_exp.data_ptr()
+  ops.lmhead(d)
+  torch.cuda.synchronize()
+  for u, v in zip(first, (best, blp, tlp, lse, ent if entropy else lse)):
+    assert torch.equal(u, v), "expanded head: statistics differ"
   logits = Q.rb(Q.qlinear_lora(x, codes, scale, group, qtype, a, b, lora_scale=1.0) if r else
                 Q.qlinear_lora(x, codes, scale, group, qtype, None, None, lora_scale=0.0))
   ref_t = rl_ref.selective_log_softmax(logits / np.float32(temperature), targets)

@@ -1,6 +1,6 @@
 // The quantised GEMM for many rows (prefill, per-token logps): output tile 128 rows x 256
-// columns per work-group of four waves, one per SIMD with the whole register file (the 128
-// accumulator registers of a wave's 128 x 64 block next to the operand pipeline).  Same weight
+// columns per work-group of four waves, one per SIMD (the 128 accumulator registers of a wave's
+// 128 x 64 block next to the operand pipeline).  Same weight
 // format, table look-up and conversion as qgemm128_kernel; what differs follows from what a
 // wave that has its SIMD to itself can issue:
 //
@@ -18,10 +18,12 @@
 //   * a slab is written as eight slots in issue order, one MFMA each with its share of the
 //     work for the following slabs; a scheduling barrier behind every slot keeps that order.
 //
-// Work-groups are numbered so that the eight XCDs (consecutive work-group ids go to
-// consecutive XCDs) each walk one 128-row block across the column tiles: a block's activations
-// stay in that XCD's L2 while the weights of a column tile, wanted by all eight at about the
-// same time, come out of the memory-side cache.
+// Work-groups are numbered in groups of 64 row blocks per column tile (consecutive work-group
+// ids go to consecutive XCDs): the eight row blocks an XCD works on at a time want the same
+// column tile's weights, which its L2 then holds for all of them.
+//
+// From the expanded copy of the weights (kWidePre) a wave needs half the register file, and
+// two work-groups share a compute unit, two waves a SIMD.
 //
 // Included by qlinear.hip after qgemm128.h.
 #pragma once
@@ -56,9 +58,18 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
 // in that form; rows in the hundreds of thousands per weight byte make its four times larger
 // stream irrelevant.  Same MFMA sequence on the same operand bits: results are bit-identical.
 constexpr int kWideTable = 0, kWideInt4 = 1, kWidePre = 2;
-constexpr int kWidePreStages = 12;   // slabs of weight fragments in flight (1.5 k-tiles)
+// kWidePre keeps so little besides its accumulators in registers that two of its waves fit one
+// SIMD (128 accumulator registers + 128 others each) and two of its work-groups one compute unit
+// (68 KB of LDS each: the two activation tiles, later the output stage): each covers the other's
+// barriers, first loads and epilogue.
+constexpr int kWidePreStages = 6;   // slabs of weight fragments in flight per wave
+constexpr size_t kWidePreSmemBytes = 68 * 1024;
+static_assert(kWidePreSmemBytes >= 2 * kWideTileBytes && kWidePreSmemBytes >= kWideRows * (kWideCols + 8) * 2,
+              "the activation tiles and the output stage fit");
+static_assert(24 % kWidePreStages == 0, "a stage keeps its slot over the three unrolled k-tiles");
 template <int SPT, bool GROUPED = false, int MODE = kWideTable>
 __global__ __launch_bounds__(256)
+__attribute__((amdgpu_waves_per_eu(MODE == kWidePre ? 2 : 1, MODE == kWidePre ? 2 : 1)))
 void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   constexpr bool INT4 = MODE == kWideInt4, PRE = MODE == kWidePre;
   static_assert(!(PRE && GROUPED), "the grouped form reads packed codes");
@@ -77,8 +88,8 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   const float lvl0 = rbf(code_level_imm(a.qtype, tid & 15)), lvl1 = rbf(code_level_imm(a.qtype, (tid >> 4) & 15));
   const uint32_t lane_off = (uint32_t)lane * 4u | kWideLutBase;   // byte 2 = 1: the table's base
 
-  // work-group id -> (row block, column tile): groups of 32 row blocks, the column tile moves
-  // every 32 ids (ids go round-robin to the eight XCDs: the four row blocks an XCD holds at a
+  // work-group id -> (row block, column tile): groups of 64 row blocks, the column tile moves
+  // every 64 ids (ids go round-robin to the eight XCDs: the eight row blocks an XCD holds at a
   // time share the column tile's weights in its L2)
   const int tiles_m = (int)((a.M + kWideRows - 1) / kWideRows), tiles_n = (int)((a.N + kWideCols - 1) / kWideCols);
   int mtile, ntile;
@@ -113,7 +124,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
     mtile = __builtin_amdgcn_readfirstlane(found_rb);
     m_end = a.offsets[expert + 1];
   } else {
-    constexpr int GR = 32;
+    constexpr int GR = 64;
     const int per_group = GR * tiles_n;
     const int g = (int)blockIdx.x / per_group, r = (int)blockIdx.x % per_group;
     const int gm = min(GR, tiles_m - g * GR);
@@ -437,7 +448,9 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
     load_w(ic<1>{}, 1);
     load_w(ic<2>{}, 2);
   }
-  if (lora) {
+  // the adapter's B^T fragments: up front, or (two work-groups per unit: no registers to park
+  // them in) behind the loop, where the other work-group covers their round trip
+  auto load_adapter_b = [&]() {
     const rsrc_t rb = make_rsrc(a.lora_b, (uint64_t)a.N * a.lora_rank * 2);
 #pragma unroll
     for (int cg = 0; cg < CG; ++cg)
@@ -446,12 +459,14 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
         if (u * 16 < a.lora_rank)
           lbv[cg][u] = buf_load128(rb, (((uint32_t)(ntile0 + 2 * cg) * 16u + (uint32_t)l32) * (uint32_t)a.lora_rank +
                                         (uint32_t)(u * 16 + lh * 8)) * 2u);
-  }
+  };
+  constexpr bool LATE_B = PRE;
+  if (lora && !LATE_B) load_adapter_b();
   if constexpr (!PRE) expand_scales(ic<0>{}, true);
   // the first tile is in LDS: its eight loads are the oldest, and at least 26 follow them (three
   // ring stages of six, the second tile's eight); vmcnt(20) also covers the first ring stage
   // (PRE: 24 fragment loads and the second tile's eight follow them)
-  tnx_wait_vm(PRE ? 32 : 20);
+  tnx_wait_vm(PRE ? 2 * kWidePreStages + 8 : 20);
   __syncthreads();
   // slab 0: table entries, conversion, fragments; then the table entries of slab 1
   if constexpr (!PRE) {
@@ -489,6 +504,7 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
   }
 
   if (lora) {
+    if constexpr (LATE_B) load_adapter_b();
     // The t block is k-tile number ktiles: it sits in tile buffer ktiles % 2.  The
     // two 16-column halves of a group may belong to different adapters (always so for a
     // gate | up pair): one pass per half then, the other half's lanes contributing zeros.

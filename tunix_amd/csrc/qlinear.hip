@@ -646,10 +646,11 @@ template <int SPT, int MODE>
 int launch_qgemm_wide_as(hipStream_t st, const QLArgs& a, const WideHead& h) {
   static std::once_flag once;
   static int attr_rc = TNX_OK;
-  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm_wide_kernel<SPT, false, MODE>, kWideSmemBytes); });
+  constexpr size_t kSmem = MODE == kWidePre ? kWidePreSmemBytes : kWideSmemBytes;
+  std::call_once(once, [] { attr_rc = prepare_qgemm128(&qgemm_wide_kernel<SPT, false, MODE>, kSmem); });
   if (attr_rc) return attr_rc;
   const unsigned wgs = (unsigned)(cdiv(a.M, kWideRows) * cdiv(a.N, kWideCols));
-  hipLaunchKernelGGL((qgemm_wide_kernel<SPT, false, MODE>), dim3(wgs), dim3(256), kWideSmemBytes, st, a, h);
+  hipLaunchKernelGGL((qgemm_wide_kernel<SPT, false, MODE>), dim3(wgs), dim3(256), kSmem, st, a, h);
   TNX_CHECK_LAUNCH("qgemm_wide");
   return TNX_OK;
 }

@@ -125,10 +125,10 @@ class FusedLinear:
       self.expanded = ops.qw_expand(self.codes, self.scales, self.K, self.N, self.group, self.qtype)
 
   def wants_expansion(self) -> bool:
-    """A table code book (NF4) gains 9-17 % on the many-row kernel from the copy; integer codes
-    are converted there without a table at the copy's speed, so they get none.  (The kernel
+    """From the copy the many-row kernel runs two work-groups per compute unit: 8-10 % over
+    integer codes converted in the loop, 20-25 % over a table code book (NF4).  (The kernel
     addresses the copy with 32-bit offsets.)"""
-    return self.qtype != L.TNX_Q_INT4 and self.expanded_bytes() < (1 << 31)
+    return self.expanded_bytes() < (1 << 31)
 
   def load_lora(self, weights: dict):
     """Copies lora_a [K,r] / lora_b [r,N_i] of every member into the kernel layout."""
