@@ -69,9 +69,9 @@ const char* tnx_last_error(void);
  * adds tnx_attn_desc.segment_ids, reads top_k == V in tnx_sample_topk as a real top-k, and moves
  * the measurement probe tnx_stream_read out of the library; 3.0 adds tnx_qw_expand /
  * tnx_qw_expanded_bytes, tnx_dense_expand and the w_expanded field of tnx_qlinear_desc and
- * tnx_lmhead_desc. */
+ * tnx_lmhead_desc; 3.1 adds tnx_sample_topk_head / tnx_sample_topk_head_ok. */
 #define TNX_ABI_VERSION_MAJOR 3
-#define TNX_ABI_VERSION_MINOR 0
+#define TNX_ABI_VERSION_MINOR 1
 #define TNX_ABI_VERSION ((TNX_ABI_VERSION_MAJOR << 16) | TNX_ABI_VERSION_MINOR)
 int tnx_version(void);
 
@@ -411,6 +411,21 @@ int tnx_sample_topk(void* stream, const float* logits, int64_t M, int64_t V, int
                     float temperature, uint32_t key0, uint32_t key1, int rng_variant,
                     const int32_t* forbidden, int n_forbidden, const int32_t* step_ptr, float* ws,
                     int32_t* ids_out, float* logp_out);
+
+/* The same draw for 0 < k < V straight after a tnx_lmhead_logp call over the same rows, in one
+ * launch that reads k x 128 logits per row instead of the row: the k best logits of a row lie in
+ * the k blocks of 128 columns with the largest block maxima, which the head has left in its
+ * workspace.  `logits` is that call's logits_out, `part` its workspace, `lse` its lse output
+ * (needed when logp_out is given); the call must have used the same `temperature` and the same
+ * `forbidden` list.  Ids are those of tnx_sample_topk on the same logits; logp_out is taken
+ * against the head's log-sum-exp (the two sum the row's exponentials in different orders).
+ * Shapes: tnx_sample_topk_head_ok(V, k) != 0, i.e. k <= 64 and V <= 524288; otherwise TNX_EINVAL
+ * and the caller uses tnx_sample_topk.  No workspace. */
+int tnx_sample_topk_head_ok(int64_t V, int k);
+int tnx_sample_topk_head(void* stream, const float* logits, const float* part, const float* lse,
+                         int64_t M, int64_t V, int k, float top_p, float temperature, uint32_t key0,
+                         uint32_t key1, int rng_variant, const int32_t* forbidden, int n_forbidden,
+                         const int32_t* step_ptr, int32_t* ids_out, float* logp_out);
 
 /* Sampler bookkeeping of one step (tunix/generate/sampler.py:529-535, :692-703):
  *   col = *step_ptr; tokens[b, col+1] = ids[b]; logprobs[b, col+1] = logp[b] (if given);

@@ -168,12 +168,13 @@ def test_ffi_handlers_cover_the_documented_targets_and_call_declared_entry_point
 
 def test_binding_refuses_another_abi_version(monkeypatch):
   """A library of another major version (or an older minor one) must not be called."""
+  major, minor = L.ABI_VERSION
   monkeypatch.setattr(L, "_lib", None)
-  monkeypatch.setattr(L, "ABI_VERSION", (L.ABI_VERSION[0] + 1, 0))
+  monkeypatch.setattr(L, "ABI_VERSION", (major + 1, 0))
   with pytest.raises(ImportError, match="ABI version"):
     L.lib()
   monkeypatch.setattr(L, "_lib", None)
-  monkeypatch.setattr(L, "ABI_VERSION", (L.ABI_VERSION[0] - 1, L.ABI_VERSION[1] + 1))   # back to the real major, a newer minor
+  monkeypatch.setattr(L, "ABI_VERSION", (major, minor + 1))   # the real major, a newer minor
   with pytest.raises(ImportError, match="ABI version"):
     L.lib()
 

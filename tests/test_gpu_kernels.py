@@ -890,6 +890,128 @@ def test_sample_topk_matches_oracle(gpu, k, top_p, variant, segmented, V):
   np.testing.assert_allclose(lp.cpu().numpy(), lp_ref2.numpy(), atol=2e-5)
 
 
+def _block_stats(logits, temp, forbidden=None):
+  """What a head call at temperature `temp` leaves for tnx_sample_topk_head: per 128-column block
+  the largest scaled (and masked) logit in slot 0 of its four statistics, and the row's lse."""
+  M, V = logits.shape
+  q = logits / np.float32(temp)
+  if forbidden:
+    q[:, forbidden] = -np.inf
+  nvb = (V + 127) // 128
+  pad = torch.full((M, nvb * 128), -np.inf)
+  pad[:, :V] = q
+  part = torch.zeros(M, nvb, 4)
+  part[:, :, 0] = pad.view(M, nvb, 128).max(-1).values
+  return part, torch.logsumexp(q.double(), -1).float()
+
+
+@pytest.mark.parametrize("V", [3000, 40001, 262144])
+@pytest.mark.parametrize("k,top_p,variant", [(50, 1.0, 0), (64, 0.7, 0), (8, 0.9, 1), (1, 1.0, 0)])
+def test_sample_topk_head_matches_oracle(gpu, k, top_p, variant, V):
+  """The one-launch top-k draw that starts from the head's block maxima, against the oracle's
+  sample_top_p and against tnx_sample_topk on the same logits: ids exactly, log-probabilities to
+  2e-5; ties inside the top-k, across blocks and at the far end of the row; forbidden ids."""
+  from tunix_amd import ops
+  M = 16
+  assert ops.sample_topk_head_ok(V, k)
+  g = torch.Generator().manual_seed(60)
+  logits = (torch.randn(M, V, generator=g) * 2).float()
+  logits[:, 17] = logits[:, 29]
+  top = torch.topk(logits, 3, dim=1).values
+  logits[:, V - 7] = top[:, 1]
+  logits[:, V // 2] = top[:, 2]
+  key = TF.prng_key(1234)
+  step, temp = 77, 0.7
+  stp = torch.tensor([step], dtype=torch.int32, device=gpu)
+  gl = logits.to(gpu)
+  for forbidden in (None, [int(torch.argmax(logits[0])), 5]):
+    masked = logits.clone()
+    if forbidden:
+      masked[:, forbidden] = -np.inf
+    tok_ref, lp_ref = SR.sample_top_p(masked, TF.fold_in(key, step), temp, top_p, k, partitionable=bool(variant))
+    part, lse = _block_stats(logits.clone(), temp, forbidden)
+    fb = torch.tensor(forbidden, dtype=torch.int32, device=gpu) if forbidden else None
+    ids = torch.full((M,), -1, dtype=torch.int32, device=gpu)
+    lp = torch.empty(M, dtype=torch.float32, device=gpu)
+    ops.sample_topk_head(gl, part.to(gpu), lse.to(gpu), k, top_p, temp, (int(key[0]), int(key[1])), variant, stp,
+                         ids, lp, forbidden=fb)
+    ids2, lp2 = torch.empty_like(ids), torch.empty_like(lp)
+    ws = torch.empty(max(ops.sample_topk_ws_bytes(M, V, k) // 4, 1), dtype=torch.float32, device=gpu)
+    ops.sample_topk(gl, k, top_p, temp, (int(key[0]), int(key[1])), variant, stp, ws, ids2, lp2, forbidden=fb)
+    torch.cuda.synchronize()
+    assert ids.cpu().long().tolist() == tok_ref.tolist()
+    assert torch.equal(ids, ids2)
+    np.testing.assert_allclose(lp.cpu().numpy(), lp_ref.numpy(), atol=2e-5)
+    np.testing.assert_allclose(lp.cpu().numpy(), lp2.cpu().numpy(), atol=2e-5)
+
+
+@pytest.mark.parametrize("V,k", [(50000, 50), (300000, 64), (300000, 3), (130, 64)])
+def test_sample_topk_head_with_massive_ties(gpu, V, k):
+  """Only a handful of distinct values: every block has the same maximum (more than 2048 equal
+  block maxima at V = 300000: the exact radix select of the block stage) and thousands of
+  elements tie at the k-th value (the same path of the element stage); the k lowest indices among
+  them are taken.  V = 130: two blocks, the second with two columns."""
+  from tunix_amd import ops
+  M, top_p, temp, step = 6, 0.95, 1.0, 3
+  g = torch.Generator().manual_seed(61)
+  logits = torch.round(torch.randn(M, V, generator=g)).float()
+  logits[0] = 1.0
+  logits[1, : V // 2] = 5.0
+  key = TF.prng_key(99)
+  tok_ref, lp_ref = SR.sample_top_p(logits, TF.fold_in(key, step), temp, top_p, k)
+  part, lse = _block_stats(logits.clone(), temp)
+  ids = torch.full((M,), -1, dtype=torch.int32, device=gpu)
+  lp = torch.empty(M, dtype=torch.float32, device=gpu)
+  stp = torch.tensor([step], dtype=torch.int32, device=gpu)
+  ops.sample_topk_head(logits.to(gpu), part.to(gpu), lse.to(gpu), k, top_p, temp, (int(key[0]), int(key[1])), 0, stp,
+                       ids, lp)
+  torch.cuda.synchronize()
+  assert ids.cpu().long().tolist() == tok_ref.tolist()
+  # (log-softmax in fp64: an fp32 sum over 300000 exponentials of this size is itself 2e-4 off)
+  lp64 = torch.log_softmax(logits.double() / temp, -1).gather(1, tok_ref[:, None])[:, 0]
+  np.testing.assert_allclose(lp.cpu().numpy(), lp64.float().numpy(), atol=2e-5)
+
+
+def test_sample_topk_head_after_a_head_call(gpu):
+  """The pairing the sampler uses: a dense head at the sampling temperature writes logits, block
+  statistics and lse; the draw from them equals tnx_sample_topk's on the logits and the oracle's."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  M, D, V, k, top_p, temp, step = 70, 256, 8208, 50, 0.9, 0.8, 5
+  x, w = rnd((M, D), 154), rnd((D, V), 155, 0.3)
+  gx, gw = bf(x).to(gpu), bf(w).t().contiguous().to(gpu)
+  key = TF.prng_key(31)
+  nvb = ops.lmhead_nblocks(V)
+  stp = torch.tensor([step], dtype=torch.int32, device=gpu)
+  for expanded in (False, True):
+    d = L.LmHeadDesc()
+    d.M, d.D, d.V, d.x, d.w_bf16, d.temperature = M, D, V, gx.data_ptr(), gw.data_ptr(), temp
+    w_exp = ops.dense_expand(gw) if expanded else None
+    if expanded:
+      d.w_expanded = w_exp.data_ptr()
+    part = torch.empty(M * nvb * 4, dtype=torch.float32, device=gpu)
+    lg_out = torch.empty(M, V, dtype=torch.float32, device=gpu)
+    lse = torch.empty(M, dtype=torch.float32, device=gpu)
+    d.part, d.logits_out, d.lse = part.data_ptr(), lg_out.data_ptr(), lse.data_ptr()
+    ops.lmhead(d)
+    ids = torch.full((M,), -1, dtype=torch.int32, device=gpu)
+    lp = torch.empty(M, dtype=torch.float32, device=gpu)
+    ops.sample_topk_head(lg_out, part, lse, k, top_p, temp, (int(key[0]), int(key[1])), 0, stp, ids, lp)
+    ids2, lp2 = torch.empty_like(ids), torch.empty_like(lp)
+    ws = torch.empty(ops.sample_topk_ws_bytes(M, V, k) // 4, dtype=torch.float32, device=gpu)
+    ops.sample_topk(lg_out, k, top_p, temp, (int(key[0]), int(key[1])), 0, stp, ws, ids2, lp2)
+    torch.cuda.synchronize()
+    tok_ref, lp_ref = SR.sample_top_p(lg_out.cpu(), TF.fold_in(key, step), temp, top_p, k)
+    assert ids.cpu().long().tolist() == tok_ref.tolist()
+    assert torch.equal(ids, ids2)
+    np.testing.assert_allclose(lp.cpu().numpy(), lp_ref.numpy(), atol=2e-5)
+    # the block maxima are bit for bit the maxima of the scaled logits the draw recomputes
+    q = (lg_out / np.float32(temp)).cpu()
+    pad = torch.full((M, nvb * 128), -np.inf)
+    pad[:, :V] = q
+    assert torch.equal(part.view(M, nvb, 4)[:, :, 0].cpu(), pad.view(M, nvb, 128).max(-1).values)
+
+
 @pytest.mark.parametrize("segmented", [False, True])
 def test_sample_topk_with_massive_ties(gpu, segmented):
   """Logits with only a handful of distinct values: thousands of elements tie at the k-th value,

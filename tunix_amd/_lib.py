@@ -12,7 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtunix_hip.so")
 
 # the ABI this binding was written against (TNX_ABI_VERSION_MAJOR / _MINOR of include/tunix_hip.h)
-ABI_VERSION = (3, 0)
+ABI_VERSION = (3, 1)
 
 TNX_Q_INT4, TNX_Q_NF4 = 0, 1
 TNX_NORM_LLAMA, TNX_NORM_QWEN3, TNX_NORM_GEMMA3 = 0, 1, 2
@@ -120,6 +120,9 @@ SIGNATURES = {
     "tnx_sample_fullsort_ws_bytes": (C.c_size_t, [_i64, _i64]),
     "tnx_sample_topk": (_i32, [_p, _p, _i64, _i64, _i32, _f32, _f32, C.c_uint32, C.c_uint32, _i32,
                                _p, _i32, _p, _p, _p, _p]),
+    "tnx_sample_topk_head_ok": (_i32, [_i64, _i32]),
+    "tnx_sample_topk_head": (_i32, [_p, _p, _p, _p, _i64, _i64, _i32, _f32, _f32, C.c_uint32, C.c_uint32, _i32,
+                                    _p, _i32, _p, _p, _p]),
     "tnx_sample_commit": (_i32, [_p, _p, _p, _i64, _p, _i64, _p, _p, _p, _i32, _p]),
     "tnx_moe_route_topk": (_i32, [_p, _p, _i64, _i32, _i32, _p, _p]),
     "tnx_moe_sort_routes": (_i32, [_p, _p, _i64, _i32, _i32, _p, _p, _p]),

@@ -580,6 +580,252 @@ __global__ __launch_bounds__(NTH) void topk_merge_sample_kernel(
 }
 
 
+// ---- top-k from the head's own block statistics, one launch -----------------------------------
+// The head leaves, per row and 128-column block, the block's largest scaled logit.  Under the
+// order of the selection (larger value, then lower index) the k best elements of a row lie in
+// the k best blocks ordered by (block maximum, then lower block): a block outside them has k
+// blocks whose best element comes before every one of its own.  So one work-group per row picks
+// those blocks from the statistics, fetches only their logits (k x 128 instead of the row), and
+// selects, ranks and draws as the two launches above do: same candidates, same draw.  The
+// log-probability is taken against the head's own log-sum-exp of the row.
+constexpr int kBlkCols = 128;        // columns per statistics block (tnx_lmhead_nblocks)
+constexpr int kBlkThreads = 512;
+constexpr int kBlkMaxBlocks = 4096;  // block maxima of a row held in LDS
+constexpr int kBlkMaxK = kSegElems / kBlkCols;
+
+struct SelectScratch {
+  float lst_v[kListMax];
+  int lst_i[kListMax];
+  uint32_t hist[256];
+  float red_f[kBlkThreads / 64];
+  uint32_t wave_cnt[kBlkThreads / 64];
+  uint32_t sel, rem, cnt, base;
+};
+
+// The k best of v[0..n) (LDS) under (larger value, then lower id), id of position i = gi(i),
+// positions in id order; result ranked best first in cv / ci [0..k) (LDS), padded with
+// (-inf, 0x7fffffff) when n < k.  Every thread of the work-group calls it; it ends on a barrier.
+template <class IdxFn>
+__device__ void select_best(const float* v, int n, int k, IdxFn gi, float* cv, int* ci, SelectScratch& s) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int kWaves = kBlkThreads / 64;
+  auto rank_list = [&](const float* lv, const int* li, int c) {   // c <= kListMax candidates -> ranks
+    for (int t = tid; t < c; t += kBlkThreads) {
+      const float mv = lv[t];
+      const int mi = li[t];
+      int r = 0;
+      for (int q = 0; q < c; ++q) {
+        const float x = lv[q];
+        r += (x > mv || (x == mv && li[q] < mi)) ? 1 : 0;
+      }
+      if (r < k) {
+        cv[r] = mv;
+        ci[r] = mi;
+      }
+    }
+  };
+  __syncthreads();
+  for (int i = tid; i < k; i += kBlkThreads) {
+    cv[i] = kNegInf;
+    ci[i] = 0x7fffffff;
+  }
+  if (tid == 0) s.cnt = 0;
+  // pivot: every wave offers the j-th largest of its threads' maxima, j = ceil(k / waves); at
+  // least k elements lie at or above the smallest offer, every tie at the k-th value included
+  float lm = kNegInf;
+  for (int i = tid; i < n; i += kBlkThreads) lm = fmaxf(lm, v[i]);
+#pragma unroll
+  for (int size = 2; size <= 64; size <<= 1)
+#pragma unroll
+    for (int st = size >> 1; st > 0; st >>= 1) {
+      const float y = __shfl_xor(lm, st, 64);
+      const bool up = (lane & size) == 0, low = (lane & st) == 0;
+      lm = (up == low) ? fmaxf(lm, y) : fminf(lm, y);
+    }
+  const int j = (k + kWaves - 1) / kWaves;
+  const float offer = __shfl(lm, j - 1, 64);
+  if (lane == 0) s.red_f[wave] = offer;
+  __syncthreads();
+  float pivot = s.red_f[0];
+  for (int w = 1; w < kWaves; ++w) pivot = fminf(pivot, s.red_f[w]);
+  for (int i = tid; i < n; i += kBlkThreads) {
+    const float x = v[i];
+    if (x >= pivot) {
+      const uint32_t p = atomicAdd(&s.cnt, 1u);
+      if (p < kListMax) {
+        s.lst_v[p] = x;
+        s.lst_i[p] = gi(i);
+      }
+    }
+  }
+  __syncthreads();
+  const int c = (int)s.cnt;
+  if (c <= kListMax) {
+    rank_list(s.lst_v, s.lst_i, c);
+    __syncthreads();
+    return;
+  }
+  // more than kListMax elements at or above the pivot (many equal values): exact radix select of
+  // the k-th key, the elements above it in any order, those equal to it by lowest position
+  uint32_t prefix = 0, mask = 0;
+  if (tid == 0) s.rem = (uint32_t)k;
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    if (tid < 256) s.hist[tid] = 0;
+    __syncthreads();
+    for (int i = tid; i < n; i += kBlkThreads) {
+      const uint32_t kk = order_key(v[i]);
+      if ((kk & mask) == prefix) atomicAdd(&s.hist[(kk >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    if (tid == 0) {
+      uint32_t cum = 0, rem = s.rem;
+      int b = 255;
+      for (; b > 0; --b) {
+        if (cum + s.hist[b] >= rem) break;
+        cum += s.hist[b];
+      }
+      s.sel = (uint32_t)b;
+      s.rem = rem - cum;
+    }
+    __syncthreads();
+    prefix |= s.sel << shift;
+    mask |= 0xffu << shift;
+  }
+  const uint32_t thr = prefix, r_eq = s.rem;
+  if (tid == 0) {
+    s.cnt = 0;
+    s.base = 0;
+  }
+  __syncthreads();
+  for (int i = tid; i < n; i += kBlkThreads) {
+    const float x = v[i];
+    if (order_key(x) > thr) {
+      const uint32_t p = atomicAdd(&s.cnt, 1u);
+      s.lst_v[p] = x;
+      s.lst_i[p] = gi(i);
+    }
+  }
+  __syncthreads();
+  const uint32_t n_gt = s.cnt;   // < k
+  for (int i0 = 0; i0 < n; i0 += kBlkThreads) {
+    if (s.base >= r_eq) break;
+    const int i = i0 + tid;
+    const bool eq = i < n && order_key(v[i]) == thr;
+    const uint64_t bal = __ballot(eq);
+    const uint32_t before = (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) s.wave_cnt[wave] = (uint32_t)__popcll(bal);
+    __syncthreads();
+    uint32_t woff = 0, tot = 0;
+    for (int w = 0; w < kWaves; ++w) {
+      if (w < wave) woff += s.wave_cnt[w];
+      tot += s.wave_cnt[w];
+    }
+    const uint32_t pos = s.base + woff + before;
+    if (eq && pos < r_eq) {
+      s.lst_v[n_gt + pos] = v[i];
+      s.lst_i[n_gt + pos] = gi(i);
+    }
+    __syncthreads();
+    if (tid == 0) s.base += tot;
+    __syncthreads();
+  }
+  __syncthreads();
+  rank_list(s.lst_v, s.lst_i, k);
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(kBlkThreads) void topk_blocks_sample_kernel(
+    const float* logits, const float* part, const float* lse, int64_t V, int nvb, int k, float top_p,
+    float temperature, const int32_t* forbidden, int n_forbidden, uint32_t key0, uint32_t key1, int variant,
+    const int32_t* step_ptr, int64_t M, int32_t* ids_out, float* logp_out) {
+  __shared__ __align__(16) float buf[kSegElems];   // the block maxima, then the gathered logits
+  __shared__ SelectScratch sc;
+  __shared__ float cv[kBlkMaxK];
+  __shared__ int ci[kBlkMaxK];
+  __shared__ int blk[kBlkMaxK];
+  __shared__ float prob[kBlkMaxK], excl[kBlkMaxK];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t row = blockIdx.x;
+  // 1. the k best blocks by (maximum, then lower block)
+  for (int b = tid; b < nvb; b += kBlkThreads) buf[b] = part[(row * nvb + b) * 4];
+  const int kb = min(k, nvb);
+  select_best(buf, nvb, kb, [](int i) { return i; }, cv, ci, sc);
+  // 2. in block order, so that positions in LDS are in id order
+  if (tid < kb) {
+    const int me = ci[tid];
+    int r = 0;
+    for (int q = 0; q < kb; ++q) r += ci[q] < me ? 1 : 0;
+    blk[r] = me;
+  }
+  __syncthreads();
+  // 3. their logits, scaled and masked as the sampling launches do
+  const float* lr = logits + row * V;
+  const int n2 = kb * kBlkCols;
+  const bool vec = (reinterpret_cast<uintptr_t>(lr) & 15) == 0 && V % 4 == 0;
+  for (int e = tid * 4; e < n2; e += kBlkThreads * 4) {
+    const int64_t col = (int64_t)blk[e >> 7] * kBlkCols + (e & 127);
+    float x[4];
+    if (vec && col + 4 <= V) {
+      const f32x4 q = *reinterpret_cast<const f32x4*>(lr + col);
+      x[0] = q[0]; x[1] = q[1]; x[2] = q[2]; x[3] = q[3];
+    } else {
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) x[jj] = col + jj < V ? lr[col + jj] : 0.f;
+    }
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      float y = col + jj < V ? __fdiv_rn(x[jj], temperature) : kNegInf;
+      for (int f = 0; f < n_forbidden; ++f)
+        if (forbidden[f] == (int32_t)(col + jj)) y = kNegInf;
+      buf[e + jj] = y;
+    }
+  }
+  // 4. the k best of those (select_best starts on a barrier)
+  select_best(buf, n2, k, [&](int i) { return blk[i >> 7] * kBlkCols + (i & 127); }, cv, ci, sc);
+  // 5. softmax over the k sorted logits, top-p cut, gumbel arg-max (as topk_merge_sample_kernel)
+  uint32_t ks0 = 0u, ks1 = (uint32_t)(*step_ptr);
+  threefry2x32(key0, key1, ks0, ks1);
+  const float mx = cv[0];
+  if (wave == 0) {
+    const float e = lane < k ? expf(cv[lane] - mx) : 0.f;
+    const float tot = wave_sum(e);
+    prob[lane] = e / tot;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float c = 0.f;
+    for (int jj = 0; jj < k; ++jj) {
+      c += prob[jj];
+      excl[jj] = c - prob[jj];
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    ArgMax g;
+    g.v = kNegInf;
+    g.i = 0x7fffffff;
+    if (lane < k) {
+      const float lgt = excl[lane] > top_p ? kNegInf : cv[lane];
+      g.v = lgt + gumbel_from_bits(random_bits(ks0, ks1, (uint64_t)(row * k + lane), (uint64_t)(M * k), variant));
+      g.i = lane;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      ArgMax y;
+      y.v = __shfl_xor(g.v, o, 64);
+      y.i = __shfl_xor(g.i, o, 64);
+      g = better(g, y);
+    }
+    if (lane == 0) {
+      const int w = g.i < k ? g.i : 0;   // (no finite candidate at all: the best-ranked one)
+      ids_out[row] = ci[w];
+      if (logp_out) logp_out[row] = cv[w] - lse[row];
+    }
+  }
+}
+
+
 // ---- top-p over the whole vocabulary (top_k absent with top_p < 1, or top_k == V) -------------
 // sample_top_p then sorts the full row (jax.lax.top_k with k = V: descending, the lower index first
 // among equal values): a stable least-significant-digit radix sort per row, written here (four
@@ -821,5 +1067,28 @@ extern "C" int tnx_sample_topk(void* stream, const float* logits, int64_t M, int
                      V, k, top_p, key0, key1, rng_variant, step_ptr, M, temperature, forbidden,
                      forbidden ? n_forbidden : 0, ids_out, logp_out);
   TNX_CHECK_LAUNCH("sample_topk");
+  return TNX_OK;
+}
+
+extern "C" int tnx_sample_topk_head_ok(int64_t V, int k) {
+  return k > 0 && k < V && k <= kBlkMaxK && cdiv(V, kBlkCols) <= kBlkMaxBlocks ? 1 : 0;
+}
+
+extern "C" int tnx_sample_topk_head(void* stream, const float* logits, const float* part, const float* lse,
+                                    int64_t M, int64_t V, int k, float top_p, float temperature, uint32_t key0,
+                                    uint32_t key1, int rng_variant, const int32_t* forbidden, int n_forbidden,
+                                    const int32_t* step_ptr, int32_t* ids_out, float* logp_out) {
+  TNX_REQUIRE(logits && part && step_ptr && ids_out, "sample_topk_head: null pointer");
+  TNX_REQUIRE(!logp_out || lse, "sample_topk_head: log-probabilities need the head's log-sum-exp");
+  TNX_REQUIRE(M > 0 && V > 0 && V < (1ll << 31), "sample_topk_head: bad shape");
+  TNX_REQUIRE(rng_variant == 0 || rng_variant == 1, "sample_topk_head: rng_variant must be 0 or 1");
+  TNX_REQUIRE(temperature > 0.f, "sample_topk_head: temperature must be positive, got %f", temperature);
+  TNX_REQUIRE(tnx_sample_topk_head_ok(V, k),
+              "sample_topk_head: needs 0 < top_k <= %d, top_k < V and V <= %d (top_k=%d, V=%lld): use tnx_sample_topk",
+              kBlkMaxK, kBlkMaxBlocks * kBlkCols, k, (long long)V);
+  hipLaunchKernelGGL(topk_blocks_sample_kernel, dim3((unsigned)M), dim3(kBlkThreads), 0, as_stream(stream), logits,
+                     part, lse, V, (int)cdiv(V, kBlkCols), k, top_p, temperature, forbidden, forbidden ? n_forbidden : 0,
+                     key0, key1, rng_variant, step_ptr, M, ids_out, logp_out);
+  TNX_CHECK_LAUNCH("sample_topk_head");
   return TNX_OK;
 }

@@ -47,7 +47,9 @@ def sampling_plan(top_k: int | None, top_p: float, vocab_size: int) -> tuple[int
   top-k in the reference -- jax.lax.top_k(k = V) sorts the row and the draw runs over sorted
   positions, whatever top_p -- so it takes the full sort too; top_k > vocab_size raises as
   jax.lax.top_k does.  Any other top_k uses the segmented selection ("topk", workspace of
-  tnx_sample_topk_ws_bytes).  One predicate decides both the path and the workspace size."""
+  tnx_sample_topk_ws_bytes) or, for the shapes tnx_sample_topk_head_ok accepts (top_k <= 64), the
+  one-launch draw from the head's block statistics, which selects the same candidates.  One
+  predicate decides both the path and the workspace size."""
   if top_k is None or top_k <= 0:
     return 0, ("head_draw" if top_p >= 1.0 else "fullsort")
   if top_k > vocab_size:
@@ -145,6 +147,15 @@ class Sampler:
                       logits_out=runner.logits,
                       draw=dict(part=mode["part_draw"], key=mode["key"], variant=self.rng_variant,
                                 step=st.step, ids=mode["ids"], logp=mode["logp"]))
+      ids, lp = mode["ids"], (mode["logp"] if want_lp else None)
+    elif mode.get("head_lse") is not None:
+      # top-k of at most 64: the head runs at the sampling temperature and leaves per-block
+      # maxima and the row's log-sum-exp; the draw then reads only the k best blocks' logits
+      runner.run_head(x, runner.B, temperature=mode["temperature"], forbidden=mode["forbidden"],
+                      lse=mode["head_lse"], logits_out=runner.logits)
+      ops.sample_topk_head(runner.logits, runner.part, mode["head_lse"], mode["top_k"], mode["top_p"],
+                           mode["temperature"], mode["key"], self.rng_variant, st.step, mode["ids"],
+                           mode["logp"], forbidden=mode["forbidden"])
       ids, lp = mode["ids"], (mode["logp"] if want_lp else None)
     else:
       runner.run_head(x, runner.B, best_id=runner.best_id, logits_out=runner.logits)
@@ -255,6 +266,8 @@ class Sampler:
                   ws=torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device=dev),
                   ids=torch.empty(B, dtype=torch.int32, device=dev),
                   logp=torch.empty(B, dtype=torch.float32, device=dev))
+      if path == "topk" and ops.sample_topk_head_ok(cfg.vocab_size, k):
+        mode["head_lse"] = torch.empty(B, dtype=torch.float32, device=dev)
       if k == 0 and top_p >= 1.0:
         mode["part_draw"] = torch.empty(B * ops.lmhead_nblocks(cfg.vocab_size) * 3, dtype=torch.float32,
                                         device=dev)

@@ -204,6 +204,24 @@ def sample_topk(logits, k, top_p, temperature, key, rng_variant, step_ptr, ws, i
           "tnx_sample_topk")
 
 
+def sample_topk_head_ok(V, k) -> bool:
+  """Whether tnx_sample_topk_head takes this vocabulary size and top_k."""
+  return bool(L.lib().tnx_sample_topk_head_ok(int(V), int(k)))
+
+
+def sample_topk_head(logits, part, lse, k, top_p, temperature, key, rng_variant, step_ptr, ids_out, logp_out,
+                     forbidden=None):
+  """The top-k / top-p draw from the statistics a head call left behind (tnx_sample_topk_head):
+  logits, part and lse are that call's logits_out, workspace and lse output, and the call used
+  the same temperature and forbidden list."""
+  M, V = logits.shape
+  L.check(L.lib().tnx_sample_topk_head(_stream(), _ptr(logits), _ptr(part), _ptr(lse), M, V, int(k), float(top_p),
+                                       float(temperature), key[0], key[1], rng_variant,
+                                       _ptr(forbidden), 0 if forbidden is None else forbidden.numel(),
+                                       _ptr(step_ptr), _ptr(ids_out), _ptr(logp_out)),
+          "tnx_sample_topk_head")
+
+
 def sample_commit(ids, logp, tokens, logprobs, done, eos, step_ptr):
   B = ids.shape[0]
   L.check(L.lib().tnx_sample_commit(_stream(), _ptr(ids), _ptr(logp), B, _ptr(tokens),
