@@ -427,10 +427,11 @@ def summarize_step_trace(path):
     print(f"| {name:34s} | {n:5d} | {busy / 1e3:8.1f} | {busy / n / 1e3:7.2f} | {span / n / 1e3:22.2f} |")
 
 
-def summarize_counters(path):
-  """Prints, per kernel, the mean of every counter in a `rocprofv3 --pmc ...` counter-collection
-  csv of this script (one row per dispatch and counter), and, where the counters are there, the
-  L1 -> L2 read latency per request and the address-translation miss rate."""
+def summarize_counters(path, by_grid=False):
+  """Prints, per kernel (by_grid: per kernel and grid size, which keeps a kernel's decode-sized
+  launches apart from its many-row ones), the mean of every counter in a `rocprofv3 --pmc ...`
+  counter-collection csv of this script (one row per dispatch and counter), and, where the
+  counters are there, the L1 -> L2 read latency per request and the address-translation miss rate."""
   import collections
   import csv
   import re
@@ -438,7 +439,10 @@ def summarize_counters(path):
   for row in csv.DictReader(open(path)):
     name = row["Kernel_Name"].replace("(anonymous namespace)::", "")
     m = re.search(r"([A-Za-z_0-9]+(<[^(]*>)?)\(", name)
-    agg[(m.group(1) if m else name)[:48]][row["Counter_Name"]].append(float(row["Counter_Value"]))
+    key = (m.group(1) if m else name)[:48]
+    if by_grid:
+      key = f"{key[:34]} grid {row.get('Grid_Size', '?')}"
+    agg[key][row["Counter_Name"]].append(float(row["Counter_Value"]))
   for name, counters in sorted(agg.items()):
     mean = {c: sum(v) / len(v) for c, v in counters.items()}
     n = max(len(v) for v in counters.values())
@@ -622,6 +626,7 @@ def main():
                        "of two `rocprofv3 --pmc FETCH_SIZE | WRITE_SIZE -- python3 bench.py --kernels-only` runs")
   ap.add_argument("--summarize-counters", metavar="CSV", default=None,
                   help="no GPU work: per-kernel means of a rocprofv3 --pmc counter-collection csv of this script")
+  ap.add_argument("--by-grid", action="store_true", help="with --summarize-counters: one line per kernel and grid size")
   args = ap.parse_args()
   if args.fused_logps:
     if args.gpus != 1:
@@ -633,7 +638,7 @@ def main():
     summarize_step_trace(args.summarize_trace)
     return
   if args.summarize_counters:
-    summarize_counters(args.summarize_counters)
+    summarize_counters(args.summarize_counters, args.by_grid)
     return
   if args.write_fused_traffic_profile:
     write_fused_traffic_profile(*args.write_fused_traffic_profile)
