@@ -571,6 +571,64 @@ def test_gqa_attention_matches_oracle(gpu, B, T, S, Hq, Hkv, dh, col, chunk, win
   assert diff.mean().item() <= 2e-3
 
 
+@pytest.mark.parametrize("B,T,S,Hq,Hkv,col,window,seg", [
+    (2, 256, 256, 8, 2, 0, 0, False),       # 64 query tiles per row: eight work-groups of eight tiles
+    (3, 200, 320, 32, 8, 40, 0, False),     # a ragged last group, queries that start at column 40
+    (2, 192, 192, 8, 1, 0, 48, False),      # sliding window: blocks before a tile's window are skipped
+    (2, 160, 160, 4, 4, 0, 0, True),        # one query head per kv head, a packed batch (segment ids)
+    (1, 100, 128, 16, 2, 0, 0, False),      # eight query heads per kv head: two positions per tile
+])
+def test_gqa_attention_through_lds_equals_the_per_wave_form(gpu, B, T, S, Hq, Hkv, col, window, seg):
+  """Many query positions at head_dim 128: the work-group kernel that stages keys and values through
+  LDS against the kernel in which every wave loads its own (taken when the id row is not 16-byte
+  aligned): bit for bit, pads inside the rows included; and the aligned result against the oracle."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  dh, pad = 128, 0
+  g = torch.Generator().manual_seed(70 + T)
+  if seg:
+    ids = torch.sort(torch.randint(1, 4, (B, S), generator=g, dtype=torch.int32), dim=1).values
+  else:
+    ids = torch.randint(1, 100, (B, S), generator=g, dtype=torch.int32)
+    ids[0, :5] = pad
+    ids[B - 1, 9] = pad
+  q = bf(rnd((B, T, Hq, dh), 71)).reshape(B * T, Hq * dh).to(gpu)
+  kc, vc = bf(rnd((B, Hkv, S, dh), 72)).to(gpu), bf(rnd((B, Hkv, S, dh), 73)).to(gpu)
+  colp = torch.tensor([col], dtype=torch.int32, device=gpu)
+  aligned = ids.to(gpu).contiguous()
+  shifted_buf = torch.zeros(B * (S + 4) + 4, dtype=torch.int32, device=gpu)
+  shifted = shifted_buf[1: 1 + B * (S + 4)].view(B, S + 4)       # rows start 4 bytes off a 16-byte boundary
+  shifted[:, :S] = aligned
+  outs = []
+  for tk, ld in ((aligned, S), (shifted, S + 4)):
+    d = L.AttnDesc()
+    d.B, d.T, d.S, d.Hq, d.Hkv, d.dh = B, T, S, Hq, Hkv, dh
+    d.scale, d.window, d.pad_id = dh ** -0.5, window, pad
+    out = torch.full((B * T, Hq * dh), 7.0, dtype=torch.bfloat16, device=gpu)
+    d.q, d.kcache, d.vcache = q.data_ptr(), kc.data_ptr(), vc.data_ptr()
+    if seg:
+      d.segment_ids = tk.data_ptr()
+    else:
+      d.tokens = tk.data_ptr()
+    d.tok_ld, d.col_ptr, d.kv_chunk, d.out = ld, colp.data_ptr(), 0, out.data_ptr()
+    ops.gqa_attn(d)
+    outs.append(out)
+  torch.cuda.synchronize()
+  assert shifted.data_ptr() % 16 != 0 and aligned.data_ptr() % 16 == 0
+  assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+  if not seg and col == 0:
+    ref = _attn_ref(q.float().cpu().view(B, T, Hq, dh), kc.float().cpu(), vc.float().cpu(), ids, pad, col, T,
+                    dh ** -0.5, window)
+    got = outs[0].view(B, T, Hq, dh).float().cpu()
+    valid = torch.ones(B, T, dtype=torch.bool)
+    for b in range(B):
+      for t in range(T):
+        if not ((ids[b, :col + t + 1] != pad).any()) or ids[b, col + t] == pad:
+          valid[b, t] = False
+    diff = (got - ref).abs()[valid]
+    assert diff.max().item() <= 2.0 ** -6 * max(1.0, ref.abs().max().item()), diff.max().item()
+
+
 @pytest.mark.parametrize("M,D,V,dense", [(8, 512, 32000, True), (128, 512, 4096, True),
                                          (130, 256, 1040, True),   # two row blocks, partial last column block
                                          (50, 256, 1040, False), (130, 256, 4096, False)])

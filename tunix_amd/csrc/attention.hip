@@ -9,7 +9,10 @@
 // inside each lane with v_perm_b32 to form B fragments; nothing goes through LDS.
 #include <string.h>
 
+#include <mutex>
+
 #include "common.h"
+#include "gemm_tile.h"   // dma16, raw_rsrc, tnx_wait_vm
 
 // Register stages of the key-block ring (head_dim <= 128).  Two: one block in flight while one is
 // computed.  A compute unit draws 21-28 GB/s from memory whatever its waves request, so a
@@ -756,6 +759,223 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
   }
 }
 
+// The same for head_dim 128 with keys and values staged through LDS: a work-group of four waves
+// takes 4 x QW consecutive query tiles of one (row, kv head), and every 32-key block is requested
+// once per work-group straight into LDS (16 bytes per lane, key rows with their 16-byte chunks
+// XOR-swizzled by row so that the fragment reads of 16 rows hit 16 bank groups; value rows as they
+// are; the block's 32 token / segment ids next to them), two blocks in flight.  A wave reads its
+// fragments from there instead of drawing them through its own loads in the MFMA operand layout,
+// which the memory path serves a few lanes at a time, and two such work-groups per compute unit
+// (227 registers per lane, 68 KB of LDS) put the softmax arithmetic of one wave under the MFMAs of
+// another.  Two query tiles per wave: with three the kernel spills.  Every wave computes exactly
+// the blocks attn_tiles_kernel would give it, in the same order with the same arithmetic: outputs
+// are bit-identical.
+typedef uint32_t __attribute__((address_space(3))) lds_word_t;
+typedef u32x4 __attribute__((address_space(3))) lds_vec_t;
+__device__ __forceinline__ u32x4 attn_lds128(uint32_t addr) {
+  return *reinterpret_cast<const lds_vec_t*>(static_cast<uintptr_t>(addr));
+}
+constexpr uint32_t kWgStageBytes = 8192 + 8192 + 1024;   // 32 keys x 256 B, 32 values x 256 B, ids
+// blocks in LDS: one computed, three in flight (three / six measured 3 % / 50 % slower: with six a
+// compute unit holds one work-group instead of two)
+constexpr int kWgStages = 4;
+template <int QW>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_wg_kernel(const AttnArgs a) {
+  constexpr int DH = 128, KS = 4;
+  extern __shared__ __align__(16) unsigned char smem_a[];
+  const uint32_t lds0 = lds_addr(smem_a);
+  const int tid = threadIdx.x, lane = tid & 63, lm = lane & 15, lq = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int hkv = blockIdx.y;
+  const int PT = 16 >> a.gp_shift;
+  const unsigned bz = blockIdx.z;
+  const int64_t b = bz / a.QTG;
+  // (the longest groups of a row are handed out first: a tile's work grows with its position)
+  const int qt_wg = ((int)a.QTG - 1 - (int)(bz - (unsigned)b * a.QTG)) * (4 * QW);
+  const int qt0 = qt_wg + wave * QW;
+  const int col0 = *a.col_ptr;
+  const int g = lm & (a.Gp - 1);
+
+  int c_n[QW], lo_n[QW];
+  bool qvalid[QW];
+  u32x4 qf[QW][KS];
+#pragma unroll
+  for (int w = 0; w < QW; ++w) {
+    const int tq = (qt0 + w) * PT + (lm >> a.gp_shift);
+    qvalid[w] = g < a.G && tq < a.T;
+    c_n[w] = col0 + tq;
+    lo_n[w] = a.window > 0 ? max(0, c_n[w] - a.window + 1) : 0;
+    const int64_t qvec = (b * a.T + (qvalid[w] ? tq : 0)) * a.Hq + hkv * a.G + (qvalid[w] ? g : 0);
+#pragma unroll
+    for (int j = 0; j < KS; ++j) {
+      qf[w][j] = u32x4{0, 0, 0, 0};
+      if (qvalid[w]) qf[w][j] = *reinterpret_cast<const u32x4*>(a.q + qvec * DH + j * 32 + lq * 8);
+    }
+  }
+  // key range of this wave's QW tiles (as in attn_tiles_kernel) and of the work-group's 4 QW
+  const bool wave_live = qt0 * PT < a.T;
+  const int k_hi = col0 + min((int)a.T - 1, (qt0 + QW) * PT - 1);
+  const int k_lo = a.window > 0 ? max(0, col0 + qt0 * PT - a.window + 1) : 0;
+  const int k_hi_wg = col0 + min((int)a.T - 1, (qt_wg + 4 * QW) * PT - 1);
+  const int k_lo_wg = a.window > 0 ? max(0, col0 + qt_wg * PT - a.window + 1) : 0;
+  const int kb0_wg = k_lo_wg & ~31;
+  const int nblk_wg = (((k_hi_wg & ~31) - kb0_wg) >> 5) + 1;
+  const int kb0 = k_lo & ~31, kb_last = k_hi & ~31;
+  const bool any = wave_live && kb0 <= k_hi;
+
+  f32x4 O[QW][8];
+  float m_run[QW], l_run[QW];
+#pragma unroll
+  for (int w = 0; w < QW; ++w) {
+    m_run[w] = kNegBig;
+    l_run[w] = 0.f;
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) O[w][jj] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const uint16_t* kbase = a.k + ((b * a.Hkv + hkv) * a.S) * DH;
+  const uint16_t* vbase = a.v + ((b * a.Hkv + hkv) * a.S) * DH;
+  const int32_t* tok = a.tokens + b * a.tok_ld;
+  const bool id_equal = a.seg_mode != 0;
+  int32_t id_ref[QW];
+#pragma unroll
+  for (int w = 0; w < QW; ++w) {
+    const int32_t id_q = tok[min((int64_t)c_n[w], a.tok_ld - 1)];
+    id_ref[w] = a.seg_mode ? id_q : a.pad_id;
+  }
+  const uint32_t slab_bytes = (uint32_t)a.S * DH * 2u;
+  const u32x4 rk = raw_rsrc(kbase, slab_bytes), rv = raw_rsrc(vbase, slab_bytes);
+  const u32x4 rtok = raw_rsrc(tok, (uint64_t)min(a.S, a.tok_ld) * 4);
+  // thread t requests, per 16-row half of a block, the 16 bytes that land at byte 16 t of the half:
+  // row t / 16, and of the key row the chunk (t % 16) ^ (row % 16)
+  const uint32_t krow = (uint32_t)(tid >> 4);
+  const uint32_t kreq = krow * 256u + ((uint32_t)(tid & 15) ^ krow) * 16u;
+  const uint32_t vreq = krow * 256u + (uint32_t)(tid & 15) * 16u;
+  auto request_block = [&](int i) {   // five requests per wave (the ids by every wave: same bytes, one count)
+    const uint32_t base = lds0 + (uint32_t)(i % kWgStages) * kWgStageBytes + (uint32_t)wave * 1024u;
+    const uint32_t kb_bytes = (uint32_t)(kb0_wg + 32 * i) * 256u;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      dma16(base + (uint32_t)c * 4096u, rk, kb_bytes + (uint32_t)c * 4096u + kreq, 0);
+      dma16(base + 8192u + (uint32_t)c * 4096u, rv, kb_bytes + (uint32_t)c * 4096u + vreq, 0);
+    }
+    // ids kb .. kb + 255 (the block's 32 and whatever follows them; past the row: zeros)
+    dma16(lds0 + (uint32_t)(i % kWgStages) * kWgStageBytes + 16384u, rtok, (uint32_t)(kb0_wg + 32 * i + 4 * lane) * 4u, 0);
+  };
+  auto compute_block = [&](int kb, uint32_t base) {
+    u32x4 kf[2][KS], vf[8];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int j = 0; j < KS; ++j)
+        kf[tt][j] = attn_lds128(base + (uint32_t)((tt * 16 + lm) * 256) + (((uint32_t)(j * 4 + lq) ^ (uint32_t)lm) * 16u));
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+      vf[s] = attn_lds128(base + 8192u + (uint32_t)((s < 4 ? 4 * lq + s : 12 + 4 * lq + s) * 256) + (uint32_t)lm * 16u);
+    const u32x4 t0 = attn_lds128(base + 16384u + (uint32_t)(4 * lq) * 4u);
+    const u32x4 t1 = attn_lds128(base + 16384u + (uint32_t)(16 + 4 * lq) * 4u);
+    int tk[8];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      tk[s] = (int)t0[s];
+      tk[4 + s] = (int)t1[s];
+    }
+    u32x4 pa[QW];
+#pragma unroll
+    for (int w = 0; w < QW; ++w) {
+      bool kvalid[8];
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        const int key = kb + (s < 4 ? 4 * lq + s : 16 + 4 * lq + (s - 4));
+        kvalid[s] = qvalid[w] && key >= max(k_lo, lo_n[w]) && key <= min(k_hi, c_n[w]) &&
+                    ((tk[s] == id_ref[w]) == id_equal);
+      }
+      f32x4 st[2];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        st[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < KS; ++j) st[tt] = mfma16(kf[tt][j], qf[w][j], st[tt]);
+      }
+      float sv[8];
+      float bmax = kNegBig;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        float x = rbf(st[s >> 2][s & 3]);
+        if (a.scale_bf != 0.f) x = rbf(x * a.scale_bf);
+        sv[s] = x;
+        if (kvalid[s]) bmax = fmaxf(bmax, x);
+      }
+      bmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
+      bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+      const float m_new = fmaxf(m_run[w], bmax);
+      const float alpha = __expf(m_run[w] - m_new);
+      m_run[w] = m_new;
+      float p[8], psum = 0.f;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        p[s] = kvalid[s] ? __expf(sv[s] - m_new) : 0.f;
+        psum += p[s];
+      }
+      l_run[w] = l_run[w] * alpha + psum;
+      pa[w][0] = pack2bf(p[0], p[1]);
+      pa[w][1] = pack2bf(p[2], p[3]);
+      pa[w][2] = pack2bf(p[4], p[5]);
+      pa[w][3] = pack2bf(p[6], p[7]);
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+        float ar[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ar[i] = __shfl(alpha, 4 * lq + i, 64);
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) O[w][jj][i] *= ar[i];
+      }
+    }
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) {
+      const uint32_t sel = (jj & 1) ? 0x07060302u : 0x05040100u;
+      u32x4 bfrag;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) bfrag[r] = __builtin_amdgcn_perm(vf[2 * r + 1][jj >> 1], vf[2 * r][jj >> 1], sel);
+#pragma unroll
+      for (int w = 0; w < QW; ++w) O[w][jj] = mfma16(pa[w], bfrag, O[w][jj]);
+    }
+  };
+#pragma unroll
+  for (int u = 0; u < kWgStages - 1; ++u)
+    if (u < nblk_wg) request_block(u);
+  for (int i = 0; i < nblk_wg; ++i) {
+    // this wave's share of block i has landed (behind it: the requests of blocks i + 1 ..
+    // i + stages - 2, five each; near the end, where fewer follow, everything is waited for) ...
+    if (i + kWgStages - 2 < nblk_wg) tnx_wait_vm(5 * (kWgStages - 2));
+    else tnx_wait_vm(0);
+    __syncthreads();    // ... and everyone's; every wave is also done reading block i - 1, whose stage is refilled
+    if (i + kWgStages - 1 < nblk_wg) request_block(i + kWgStages - 1);
+    const int kb = kb0_wg + 32 * i;
+    if (any && kb >= kb0 && kb <= kb_last) compute_block(kb, lds0 + (uint32_t)(i % kWgStages) * kWgStageBytes);
+  }
+#pragma unroll
+  for (int w = 0; w < QW; ++w) {
+    float lr = l_run[w];
+    lr += __shfl_xor(lr, 16, 64);
+    lr += __shfl_xor(lr, 32, 64);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = 4 * lq + i;
+      const float l = __shfl(lr, n, 64);
+      const int gi = n & (a.Gp - 1), ti = (qt0 + w) * PT + (n >> a.gp_shift);
+      if (!(gi < a.G && ti < a.T)) continue;
+      const float inv = l > 0.f ? 1.0f / l : 0.f;
+      uint16_t* o = a.out + ((b * a.T + ti) * a.Hq + hkv * a.G + gi) * DH;
+      u32x4 wv;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) wv[r] = pack2bf(O[w][2 * r][i] * inv, O[w][2 * r + 1][i] * inv);
+      *reinterpret_cast<u32x4*>(o + 8 * lm) = wv;
+    }
+  }
+}
+
 // out[qv, d] = bf16( sum_c e^{m_c - M} O_c[d] / sum_c e^{m_c - M} l_c )
 // The (m, l) pairs of all chunks are fetched at once into LDS (one round trip instead of one
 // dependent load per chunk and pass); every thread then forms M, the weights and the sums in
@@ -864,7 +1084,25 @@ extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
     if (tv) hipLaunchKernelGGL((attn_kernel<DH, FUSE, true>), grid, dim3(64), 0, st, a);         \
     else hipLaunchKernelGGL((attn_kernel<DH, FUSE, false>), grid, dim3(64), 0, st, a);           \
   } while (0)
-  // many query positions, no key split, no fused rotation: four query tiles per wave
+  // many query positions at head_dim 128, no key split, no fused rotation: keys and values through
+  // LDS, eight query tiles per work-group
+  constexpr int kWgTilesPerWave = 2;
+  if (!a.rope_sin && a.n_chunks == 1 && d->dh == 128 && tv && QT >= 2 * 4 * kWgTilesPerWave &&
+      (uint64_t)d->S * 256u < (1ull << 32)) {
+    a.QTG = (unsigned)cdiv(QT, 4 * kWgTilesPerWave);
+    dim3 wgrid(1u, (unsigned)d->Hkv, (unsigned)(d->B * a.QTG));
+    static std::once_flag wg_once;
+    static hipError_t wg_rc = hipSuccess;
+    std::call_once(wg_once, [] {
+      wg_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_wg_kernel<kWgTilesPerWave>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kWgStages * kWgStageBytes));
+    });
+    TNX_REQUIRE(wg_rc == hipSuccess, "attn: cannot raise the dynamic LDS limit");
+    hipLaunchKernelGGL((attn_wg_kernel<kWgTilesPerWave>), wgrid, dim3(256), kWgStages * kWgStageBytes, st, a);
+    TNX_CHECK_LAUNCH("gqa_attn (work-group tiles)");
+    return TNX_OK;
+  }
+  // many query positions, no key split, no fused rotation: two query tiles per wave
   constexpr int kTilesPerWave = 2;
   if (!a.rope_sin && a.n_chunks == 1 && d->dh <= 128 && QT >= 2 * kTilesPerWave) {
     a.QTG = (unsigned)cdiv(QT, kTilesPerWave);
