@@ -10,6 +10,7 @@
 #include <string.h>
 
 #include <mutex>
+#include <type_traits>
 
 #include "common.h"
 #include "gemm_tile.h"   // dma16, raw_rsrc, tnx_wait_vm
@@ -843,6 +844,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int32_t id_q = tok[min((int64_t)c_n[w], a.tok_ld - 1)];
     id_ref[w] = a.seg_mode ? id_q : a.pad_id;
   }
+  // A block that lies wholly inside every query's range of a tile, with no id to mask, takes the
+  // same arithmetic without the per-key tests: the bounds of that, uniform over the wave.
+  // (Packed batches compare ids per query and always take the general form.)
+  int lo_max[QW], hi_min[QW];
+#pragma unroll
+  for (int w = 0; w < QW; ++w) {
+    int lo = max(k_lo, lo_n[w]), hi = min(k_hi, c_n[w]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      lo = max(lo, __shfl_xor(lo, o, 64));
+      hi = min(hi, __shfl_xor(hi, o, 64));
+    }
+    const bool full = __builtin_amdgcn_ballot_w64(qvalid[w]) == ~0ull && !id_equal;
+    lo_max[w] = __builtin_amdgcn_readfirstlane(full ? lo : 0x7fffffff);
+    hi_min[w] = __builtin_amdgcn_readfirstlane(hi);
+  }
   const uint32_t slab_bytes = (uint32_t)a.S * DH * 2u;
   const u32x4 rk = raw_rsrc(kbase, slab_bytes), rv = raw_rsrc(vbase, slab_bytes);
   const u32x4 rtok = raw_rsrc(tok, (uint64_t)min(a.S, a.tok_ld) * 4);
@@ -880,15 +897,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       tk[s] = (int)t0[s];
       tk[4 + s] = (int)t1[s];
     }
-    u32x4 pa[QW];
+    // (pad mode: a key counts when its id differs from pad_id, the same test for every tile)
+    bool idok[8];
 #pragma unroll
-    for (int w = 0; w < QW; ++w) {
+    for (int s = 0; s < 8; ++s) idok[s] = (tk[s] == a.pad_id) == id_equal;
+    const bool ids_all = !id_equal && __builtin_amdgcn_ballot_w64(idok[0] && idok[1] && idok[2] && idok[3] && idok[4] &&
+                                                                  idok[5] && idok[6] && idok[7]) == ~0ull;
+    u32x4 pa[QW];
+    auto tile_step = [&](int w, auto inside_c) {
+      constexpr bool INSIDE = decltype(inside_c)::value;
       bool kvalid[8];
 #pragma unroll
       for (int s = 0; s < 8; ++s) {
         const int key = kb + (s < 4 ? 4 * lq + s : 16 + 4 * lq + (s - 4));
-        kvalid[s] = qvalid[w] && key >= max(k_lo, lo_n[w]) && key <= min(k_hi, c_n[w]) &&
-                    ((tk[s] == id_ref[w]) == id_equal);
+        kvalid[s] = INSIDE || (qvalid[w] && key >= max(k_lo, lo_n[w]) && key <= min(k_hi, c_n[w]) &&
+                               ((tk[s] == id_ref[w]) == id_equal));
       }
       f32x4 st[2];
 #pragma unroll
@@ -931,6 +954,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
           for (int i = 0; i < 4; ++i) O[w][jj][i] *= ar[i];
       }
+    };
+#pragma unroll
+    for (int w = 0; w < QW; ++w) {
+      if (ids_all && kb >= lo_max[w] && kb + 31 <= hi_min[w]) tile_step(w, std::true_type{});
+      else tile_step(w, std::false_type{});
     }
 #pragma unroll
     for (int jj = 0; jj < 8; ++jj) {
