@@ -1116,7 +1116,7 @@ extern "C" int tnx_gqa_attn(void* stream, const tnx_attn_desc* d) {
   // LDS, eight query tiles per work-group
   constexpr int kWgTilesPerWave = 2;
   if (!a.rope_sin && a.n_chunks == 1 && d->dh == 128 && tv && QT >= 2 * 4 * kWgTilesPerWave &&
-      (uint64_t)d->S * 256u < (1ull << 32)) {
+      (uint64_t)d->S * 256u < (1ull << 32) && d->B * cdiv(QT, 4 * kWgTilesPerWave) <= 65535) {
     a.QTG = (unsigned)cdiv(QT, 4 * kWgTilesPerWave);
     dim3 wgrid(1u, (unsigned)d->Hkv, (unsigned)(d->B * a.QTG));
     static std::once_flag wg_once;
