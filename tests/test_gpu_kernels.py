@@ -903,6 +903,49 @@ def test_lmhead_categorical_draw_matches_oracle(gpu, M, V, variant):
   np.testing.assert_allclose(lp.cpu().numpy(), lp2.cpu().numpy(), atol=2e-5)
 
 
+@pytest.mark.parametrize("M,V,variant,temp", [(128, 4096, 0, 0.9), (128, 8208, 1, 1.0), (40, 1040, 0, 0.7),
+                                               (7, 4096, 1, 1.3), (64, 4096, 0, 1.0)])
+def test_lmhead_categorical_draw_on_the_many_row_kernel(gpu, M, V, variant, temp):
+  """The same draw with the dense head's expanded copy, i.e. in the statistics epilogue of the
+  many-row kernel: ids equal the oracle's jax.random.categorical over the logits the kernel
+  wrote and the ids of the head kernel that reads the plain weights; log-probabilities to 2e-5."""
+  from tunix_amd import _lib as L
+  from tunix_amd import ops
+  D, step = 256, 17
+  x, w = rnd((M, D), 254), rnd((D, V), 255, 0.3)
+  gx, gw = bf(x).to(gpu), bf(w).t().contiguous().to(gpu)
+  w_exp = ops.dense_expand(gw)
+  key = TF.prng_key(4242)
+  nvb = ops.lmhead_nblocks(V)
+  stp = torch.tensor([step], dtype=torch.int32, device=gpu)
+  res = []
+  for expanded in (True, False):
+    d = L.LmHeadDesc()
+    d.M, d.D, d.V, d.x, d.w_bf16, d.temperature = M, D, V, gx.data_ptr(), gw.data_ptr(), temp
+    if expanded:
+      d.w_expanded = w_exp.data_ptr()
+    part = torch.full((M * nvb * 4,), float("nan"), dtype=torch.float32, device=gpu)
+    pdraw = torch.full((M * nvb * 3,), float("nan"), dtype=torch.float32, device=gpu)
+    lg_out = torch.empty(M, V, dtype=torch.float32, device=gpu)
+    ids = torch.full((M,), -1, dtype=torch.int32, device=gpu)
+    lp = torch.empty(M, dtype=torch.float32, device=gpu)
+    d.part, d.logits_out = part.data_ptr(), lg_out.data_ptr()
+    d.part_draw, d.draw_key0, d.draw_key1, d.draw_rng_variant = pdraw.data_ptr(), int(key[0]), int(key[1]), variant
+    d.draw_step_ptr, d.draw_id, d.draw_logp = stp.data_ptr(), ids.data_ptr(), lp.data_ptr()
+    ops.lmhead(d)
+    torch.cuda.synchronize()
+    assert not torch.isnan(pdraw).any()
+    res.append((ids.cpu(), lp.cpu(), lg_out.cpu()))
+  (ids_w, lp_w, lg_w), (ids_h, lp_h, lg_h) = res
+  assert torch.equal(lg_w, lg_h)
+  tok_ref, lp_ref = SR.sample_top_p(lg_w, TF.fold_in(key, step), temp, 1.0, None, partitionable=bool(variant))
+  assert ids_w.long().tolist() == tok_ref.tolist()
+  assert torch.equal(ids_w, ids_h)
+  np.testing.assert_allclose(lp_w.numpy(), lp_ref.numpy(), atol=2e-5)
+  np.testing.assert_allclose(lp_w.numpy(), lp_h.numpy(), atol=2e-5)
+  assert len(set(ids_w.tolist())) > 1 or M < 4
+
+
 @pytest.mark.parametrize("V", [3000, 40001])
 @pytest.mark.parametrize("segmented", [False, True])
 @pytest.mark.parametrize("k,top_p,variant", [(50, 1.0, 0), (50, 0.7, 0), (8, 0.9, 1), (0, 1.0, 0)])

@@ -686,6 +686,38 @@ void qgemm_wide_kernel(const QLArgs a, const WideHead h) {
         }
       }
     };
+    // The whole-vocabulary draw: the statistics of the general form and, per column, the logit
+    // plus the Gumbel noise of element row * N + col of rows_total * N; the block's best (first
+    // among equals: columns ascend), its id and its logit go to part_draw.
+    if (h.part_draw != nullptr) {
+      uint32_t ks0 = 0u, ks1 = (uint32_t)(*h.step_ptr);
+      threefry2x32(h.key0, h.key1, ks0, ks1);   // fold_in(key, step)
+      const uint64_t total = (uint64_t)h.rows_total * (uint64_t)a.N;
+      float gv = ninf, gl = ninf;
+      int gi = 0x7fffffff;
+      for (int ch = 0; ch < 16; ++ch) {
+        const u32x4 v = lds_ld128(base + (uint32_t)(ch * 16));
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          const int64_t col = c0 + ch * 8 + q;
+          if (col < a.N) {
+            const float raw = (q & 1) ? bfhi(v[q >> 1]) : bflo(v[q >> 1]);
+            const float l = __fdiv_rn(raw, h.temperature);
+            const float n = l + gumbel_from_bits(random_bits(ks0, ks1, (uint64_t)grow * (uint64_t)a.N + (uint64_t)col,
+                                                             total, h.variant));
+            if (n > gv) {
+              gv = n;
+              gi = (int)col;
+              gl = l;
+            }
+          }
+        }
+      }
+      float* q3 = h.part_draw + (grow * h.nvb + pb) * 3;
+      q3[0] = gv;
+      q3[1] = __int_as_float(gi);
+      q3[2] = gl;
+    }
     const bool plain = c0 + 128 <= a.N && h.part_ent == nullptr;
     if (h.temperature == 1.0f) {
       if (plain) reduce_full(std::true_type{});

@@ -6,6 +6,7 @@
 #include <mutex>
 
 #include "gemm_tile.h"
+#include "rng.h"
 
 namespace {
 
@@ -50,6 +51,13 @@ struct WideHead {
   int64_t nvb;               // 128-column blocks of the vocabulary
   float temperature;
   float* logits_out;         // optional fp32 [M, N]: the raw logits (the staged bf16 values), or null
+  // optional whole-vocabulary categorical draw (Gumbel-max with jax.random's bit stream): per
+  // (row, block) the best logit + noise, its id and its logit, as lmhead_kernel leaves them
+  float* part_draw;          // [M, nvb, 3], or null
+  uint32_t key0, key1;
+  int variant;
+  const int32_t* step_ptr;
+  int64_t rows_total;        // M of the whole call: the noise of element (row, v) is number row * V + v of M * V
 };
 
 __device__ __forceinline__ float silu_bf16(float g) {
@@ -873,7 +881,7 @@ extern "C" int tnx_qlinear_lora(void* stream, const tnx_qlinear_desc* d) {
 // the shape is not one the kernel takes (the caller then uses its own kernel), 0 when launched.
 int tnx_internal_wide_head(hipStream_t st, const tnx_lmhead_desc* d, float temperature, int64_t nvb,
                            float* part_ent) {
-  if (d->forbidden || d->draw_id || d->logits_fp32) return 1;   // (its tile is staged in bf16)
+  if (d->forbidden || d->logits_fp32) return 1;   // (its tile is staged in bf16)
   // a dense head comes here only through its expanded copy (tnx_dense_expand)
   const bool dense = d->w_bf16 != nullptr;
   const bool pre_ok = d->w_expanded && d->D % KTILE == 0 &&
@@ -900,7 +908,11 @@ int tnx_internal_wide_head(hipStream_t st, const tnx_lmhead_desc* d, float tempe
   // 128 x 128 head kernel re-reads them once per 128, as many bytes again as the weights.
   if (!wide_shape(a, dense ? 1 : 512)) return 1;
   a.y = nullptr;
-  const WideHead h{d->part, part_ent, d->targets, nvb, temperature, d->logits_out};
+  WideHead h{d->part, part_ent, d->targets, nvb, temperature, d->logits_out, nullptr, 0u, 0u, 0, nullptr, d->M};
+  if (d->draw_id) {
+    h.part_draw = d->part_draw; h.key0 = d->draw_key0; h.key1 = d->draw_key1; h.variant = d->draw_rng_variant;
+    h.step_ptr = d->draw_step_ptr;
+  }
   return scales_per_tile(a.group) == 2 ? launch_qgemm_wide<2>(st, a, h) : launch_qgemm_wide<4>(st, a, h);
 }
 
