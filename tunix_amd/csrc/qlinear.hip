@@ -601,6 +601,85 @@ __global__ __launch_bounds__(256) void lora_down_rows_kernel(const uint16_t* x, 
     }
 }
 
+// The same product with both operands requested straight into LDS (`buffer_load ... lds`, whole
+// 256-byte rows of a k-tile, chunks XOR-swizzled by the row as in the GEMM's activation tiles).
+// A work-group of four waves takes 16 MT rows x 64 NG adapter columns -- all of the adapter's
+// columns, so that x is read once -- a wave the 16-column tile `wave` of every 64-column group;
+// NS k-tiles in LDS, one computed and the others in flight.  The kernel above reads the adapter's
+// fragments from global memory in the MFMA operand layout, which the memory path serves a few
+// lanes at a time, and re-reads x once per 64 columns; here every byte arrives as part of a whole
+// kilobyte.
+template <int MT, int NG, int NS>
+__global__ __launch_bounds__(256) void lora_down_rows_lds_kernel(const uint16_t* x, int64_t M, int64_t K,
+                                                                 const uint16_t* a_t, int R, uint16_t* t,
+                                                                 int64_t t_ld) {
+  constexpr uint32_t kXBytes = MT * 16 * 256, kStage = kXBytes + NG * 64 * 256;
+  constexpr int kReq = MT + 4 * NG;   // requests per thread and k-tile
+  extern __shared__ __align__(16) unsigned char smem[];
+  const uint32_t lds0 = lds_addr(smem);
+  const int tid = threadIdx.x, lane = tid & 63, lm = lane & 15, lq = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t m0 = (int64_t)blockIdx.x * (16 * MT);
+  // rows past M / R lie beyond the resource and arrive as zeros
+  const u32x4 rx = raw_rsrc(x + m0 * K, (uint64_t)min((int64_t)(16 * MT), M - m0) * K * 2);
+  const u32x4 ra = raw_rsrc(a_t, (uint64_t)R * K * 2);
+  // thread t requests, per 16-row group of a tile, the 16 bytes that land at byte 16 t of the group:
+  // row t / 16, and of that row's 256 bytes the chunk (t % 16) ^ (row % 16)
+  const uint32_t rrow = (uint32_t)(tid >> 4);
+  const uint32_t req = rrow * (uint32_t)K * 2u + (((uint32_t)(tid & 15) ^ rrow) * 16u);
+  const uint32_t grp = 16u * (uint32_t)K * 2u;   // 16 rows further
+  const int ktiles = (int)(K / KTILE);
+  auto request = [&](int kt) {
+    const uint32_t base = lds0 + (uint32_t)(kt % NS) * kStage + (uint32_t)wave * 1024u;
+    const int ko = kt * (KTILE * 2);
+#pragma unroll
+    for (int c = 0; c < MT; ++c) dma16(base + (uint32_t)c * 4096u, rx, req + (uint32_t)c * grp, ko);
+#pragma unroll
+    for (int c = 0; c < 4 * NG; ++c) dma16(base + kXBytes + (uint32_t)c * 4096u, ra, req + (uint32_t)c * grp, ko);
+  };
+  f32x4 acc[NG][MT];
+#pragma unroll
+  for (int g = 0; g < NG; ++g)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[g][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int u = 0; u < NS - 1; ++u)
+    if (u < ktiles) request(u);
+  for (int kt = 0; kt < ktiles; ++kt) {
+    // this thread's share of k-tile kt has landed (behind it: the requests of the tiles after it) ...
+    if (kt + NS - 2 < ktiles) tnx_wait_vm(kReq * (NS - 2));
+    else tnx_wait_vm(0);
+    __syncthreads();   // ... and everyone's; every wave is done with k-tile kt - 1, whose stage is refilled
+    if (kt + NS - 1 < ktiles) request(kt + NS - 1);
+    const uint32_t base = lds0 + (uint32_t)(kt % NS) * kStage;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {   // 32 k per step: this lane's chunk 4 j + l / 16 of row l % 16
+      const uint32_t ch = ((uint32_t)(4 * j + lq) ^ (uint32_t)lm) * 16u;
+      u32x4 a[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) a[mt] = lds_ld128(base + (uint32_t)((mt * 16 + lm) * 256) + ch);
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const u32x4 b = lds_ld128(base + kXBytes + (uint32_t)((g * 64 + wave * 16 + lm) * 256) + ch);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[g][mt] = mfma16(a[mt], b, acc[g][mt]);
+      }
+    }
+  }
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
+    const int col = g * 64 + wave * 16 + lm;
+    if (col >= R) continue;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int64_t row = m0 + mt * 16 + lq * 4 + i;
+        if (row < M) t[row * t_ld + col] = f2bf(acc[g][mt][i]);
+      }
+  }
+}
+
 template <class Kern>
 int raise_lds_limit(Kern kern, size_t bytes) {
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -945,6 +1024,37 @@ extern "C" int tnx_lora_down(void* stream, const uint16_t* x, int64_t M, int64_t
   TNX_REQUIRE(x && a_t && t, "lora_down: null pointer");
   TNX_REQUIRE(M > 0 && K > 0 && K % 32 == 0, "lora_down: K=%lld must be a multiple of 32", (long long)K);
   TNX_REQUIRE(R > 0 && R % 16 == 0 && t_ld >= R, "lora_down: R=%d must be a multiple of 16 and <= t_ld", R);
+  if (M >= 512 && K % KTILE == 0 && (uint64_t)(M + 128) * (uint64_t)K * 2 < (1ull << 32) && R % 16 == 0 && R <= 192 &&
+      (uint64_t)(R + 64) * (uint64_t)K * 2 < (1ull << 32)) {
+    // many rows: both operands through LDS, all adapter columns per work-group
+    auto launch = [&](auto MTc, auto NGc, auto NSc) -> int {
+      constexpr int MT = decltype(MTc)::value, NG = decltype(NGc)::value, NS = decltype(NSc)::value;
+      constexpr size_t kSmem = (size_t)NS * (MT * 16 * 256 + NG * 64 * 256);
+      static_assert(kSmem <= 160 * 1024, "the stages fit LDS");
+      static std::once_flag once;
+      static int attr_rc = TNX_OK;
+      std::call_once(once, [] { attr_rc = raise_lds_limit(&lora_down_rows_lds_kernel<MT, NG, NS>, kSmem); });
+      if (attr_rc) return attr_rc;
+      hipLaunchKernelGGL((lora_down_rows_lds_kernel<MT, NG, NS>), dim3((unsigned)cdiv(M, 16 * MT)), dim3(256), kSmem,
+                         as_stream(stream), x, M, K, a_t, R, t, t_ld);
+      TNX_CHECK_LAUNCH("lora_down_rows_lds");
+      return TNX_OK;
+    };
+    // the tallest tile that still gives every compute unit a work-group; three k-tiles in LDS where
+    // they fit, else two
+    auto pick = [&](auto NGc) -> int {
+      constexpr int NG = decltype(NGc)::value;
+      using std::integral_constant;
+      if (cdiv(M, 128) >= 256)
+        return launch(integral_constant<int, 8>{}, NGc, integral_constant<int, (NG == 1 ? 3 : 2)>{});
+      if (cdiv(M, 64) >= 256)
+        return launch(integral_constant<int, 4>{}, NGc, integral_constant<int, (NG <= 2 ? 3 : 2)>{});
+      return launch(integral_constant<int, 2>{}, NGc, integral_constant<int, (NG <= 2 ? 3 : 2)>{});
+    };
+    if (R <= 64) return pick(std::integral_constant<int, 1>{});
+    if (R <= 128) return pick(std::integral_constant<int, 2>{});
+    if (R <= 192) return pick(std::integral_constant<int, 3>{});
+  }
   if (M >= 512 && K % KTILE == 0 && (uint64_t)(M + 128) * (uint64_t)K * 2 < (1ull << 32)) {
     // many rows: MFMA tiles of 128 rows, or of 64 / 32 where that is what it takes to fill the
     // device (32-bit buffer offsets: the activations must stay below 4 GiB)
