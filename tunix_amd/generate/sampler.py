@@ -91,7 +91,7 @@ class Sampler:
   """Sampler for transformer model."""
 
   def __init__(self, transformer: QLoRAModel, tokenizer, cache_config: CacheConfig,
-               use_graph: bool = True, prefill_rows: int = 8192):
+               use_graph: bool = True, prefill_rows: int = 16384):
     self._transformer = transformer
     self.tokenizer = tokenizer
     self.cache_config = cache_config
